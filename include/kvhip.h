@@ -1,0 +1,240 @@
+/*
+ * kvhip.h -- C interface of libkvhip.so, the MI355X (gfx950) implementation of
+ * the KV-cache hot path of mlx-swift-lm.
+ *
+ * A Swift system-library target imports this header (and nothing else) through
+ * a module map, in the way Libraries/MLXCXGrammar/include/module.modulemap
+ * exposes xgrammar_c.h.  One `kvhip_cache` handle stands behind one instance of
+ * the reference's `KVCacheSimple`, `RotatingKVCache` or `QuantizedKVCache`
+ * (Libraries/MLXLMCommon/KVCache.swift:391, :541, :923); every entry point
+ * below names the reference member it replaces.
+ *
+ * Conventions
+ *  - Every pointer named `keys`, `values`, `queries`, `out`, `dst`, `src` or
+ *    `data` is a DEVICE pointer to a dense row-major array; shapes are given in
+ *    the comment of each function.  Inputs are borrowed for the duration of the
+ *    call's enqueued work only.
+ *  - `stream` is a `hipStream_t` passed as `void *` (NULL = the default
+ *    stream).  Device work is enqueued on it; host-side counters (`offset`,
+ *    `idx`) advance when the call returns, as the reference's do while it
+ *    builds its lazy graph (KVCache.swift:438, :729-730, :1067).
+ *  - A handle is not thread-safe: like the reference's `KVCacheStorage`
+ *    (KVCachePlan.swift:104-111) it is externally serialised by its owner.
+ *  - Fallible functions return a status: 0 on success, negative on failure,
+ *    with a message readable through kvhip_last_error_message() on the calling
+ *    thread (idiom of xgrammar_c.h:39-69).
+ */
+#ifndef KVHIP_H
+#define KVHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int32_t kvhip_status;
+#define KVHIP_OK               ((int32_t)0)
+#define KVHIP_ERR_INTERNAL     ((int32_t)-1)
+#define KVHIP_ERR_INVALID_ARG  ((int32_t)-2)
+#define KVHIP_ERR_UNSUPPORTED  ((int32_t)-3) /* shape / dtype / bit width outside what the kernels cover */
+#define KVHIP_ERR_STATE        ((int32_t)-4) /* a call the reference answers with fatalError / throws */
+#define KVHIP_ERR_HIP          ((int32_t)-5) /* a HIP runtime call failed */
+#define KVHIP_ERR_NO_DEVICE    ((int32_t)-6) /* no gfx950 device visible */
+
+typedef enum {
+    KVHIP_KIND_SIMPLE = 0,    /* KVCacheSimple    KVCache.swift:391-538  */
+    KVHIP_KIND_ROTATING = 1,  /* RotatingKVCache  KVCache.swift:541-900  */
+    KVHIP_KIND_QUANTIZED = 2, /* QuantizedKVCache KVCache.swift:923-1210 */
+} kvhip_kind;
+
+typedef enum {
+    KVHIP_F16 = 0,
+    KVHIP_BF16 = 1,
+    KVHIP_F32 = 2,
+    KVHIP_U32 = 3,  /* packed codes in exported state */
+    KVHIP_BOOL = 4, /* one byte per element, for masks */
+} kvhip_dtype;
+
+/* Constructor arguments of the three cache classes.  Fields a kind does not
+ * use are ignored.  step <= 0 selects the reference default (256). */
+typedef struct {
+    int32_t kind;       /* kvhip_kind */
+    int32_t step;       /* KVCacheSimple.step :394, RotatingKVCache(step:) :565 */
+    int32_t max_size;   /* RotatingKVCache(maxSize:) */
+    int32_t keep;       /* RotatingKVCache(keep:) */
+    int32_t group_size; /* QuantizedKVCache(groupSize:) :931 */
+    int32_t bits;       /* QuantizedKVCache(bits:), affine mode; 2, 4 or 8 */
+} kvhip_config;
+
+/* MLXFast.ScaledDotProductAttentionMaskMode as the attention entry points take it. */
+typedef enum {
+    KVHIP_MASK_NONE = 0,
+    KVHIP_MASK_CAUSAL = 1, /* query i sees key j iff j <= T - L + i (KVCache.swift:2396-2400) */
+    KVHIP_MASK_ARRAY = 2,  /* bool: keep where true; float: added to the scores (:2436-2446) */
+    /* createCausalMask(n:, offset:, windowSize:, lengths:) (KVCache.swift:253-275)
+     * evaluated from indices inside the kernel instead of being materialised:
+     * keep iff offset+i >= j && (window <= 0 || offset+i < j + window)
+     *       && (lengths == NULL || j < lengths[b]) && (left_pad == NULL || j >= left_pad[b]) */
+    KVHIP_MASK_WINDOW = 3,
+} kvhip_mask_mode;
+
+typedef struct {
+    int32_t mode;       /* kvhip_mask_mode */
+    int32_t dtype;      /* ARRAY: KVHIP_BOOL, KVHIP_F16, KVHIP_BF16 or KVHIP_F32 */
+    const void *data;   /* ARRAY: device pointer, innermost (key) axis contiguous */
+    int64_t stride_b;   /* ARRAY: element strides of the batch, query-head and query-row */
+    int64_t stride_h;   /*        axes; 0 broadcasts the axis                            */
+    int64_t stride_l;
+    int32_t key_len;    /* ARRAY: extent of the key axis (must equal the presented length) */
+    int32_t offset;     /* WINDOW */
+    int32_t window;     /* WINDOW: <= 0 means no window */
+    const int32_t *lengths;  /* WINDOW: optional device [B] */
+    const int32_t *left_pad; /* WINDOW: optional device [B] */
+} kvhip_mask;
+
+/* What `makeMask(n:windowSize:returnArray:)` decides (KVCache.swift:236-250,
+ * :834-871): a symbolic mode, or the parameters of the array it would build. */
+typedef struct {
+    int32_t mode;      /* NONE, CAUSAL, or ARRAY (the reference would materialise an array) */
+    int32_t rows;      /* ARRAY: n */
+    int32_t cols;      /* ARRAY: key extent */
+    int32_t offset;    /* ARRAY from createCausalMask: its `offset` argument */
+    int32_t window;    /* ARRAY from createCausalMask: windowSize, or 0 */
+    int32_t rolled;    /* 1: the single-token rolled window mask of RotatingKVCache.makeMask :855-868 */
+    int32_t roll_shift;/* rolled: currentIdx + 1 */
+    int32_t roll_window;
+} kvhip_mask_plan_t;
+
+typedef struct kvhip_cache kvhip_cache;
+
+/* ---- library ----------------------------------------------------------- */
+const char *kvhip_version(void);
+/* Message of the last failure on this thread, or NULL. Valid until the next kvhip call. */
+const char *kvhip_last_error_message(void);
+/* Binds the library to HIP device `device` (default 0) and checks it is gfx950. */
+kvhip_status kvhip_init(int32_t device);
+/* Blocks until all work enqueued on `stream` is done (tests; `eval(cache)` LLMModel.swift:56-58). */
+kvhip_status kvhip_sync(void *stream);
+/* 0 = choose the fastest kernel for the shape (default); 1 = always the generic kernel. */
+void kvhip_set_kernel_policy(int32_t policy);
+
+/* ---- lifetime ---------------------------------------------------------- */
+/* KVCacheSimple() / RotatingKVCache(maxSize:keep:step:) / QuantizedKVCache(groupSize:bits:) */
+kvhip_status kvhip_cache_create(const kvhip_config *config, kvhip_cache **out_cache);
+/* Safe with NULL. */
+void kvhip_cache_free(kvhip_cache *cache);
+/* `copy()` (KVCache.swift:525-533, :877-885, :1177-1185): independent deep copy. */
+kvhip_status kvhip_cache_copy(const kvhip_cache *cache, void *stream, kvhip_cache **out_cache);
+/* Optional: pre-size device storage for `tokens` cached rows so later updates never reallocate. */
+kvhip_status kvhip_cache_reserve(kvhip_cache *cache, int32_t B, int32_t Hkv, int32_t Dk, int32_t Dv,
+                                 int32_t dtype, int64_t tokens);
+
+/* ---- the KVCache protocol surface (KVCache.swift:46-104) ----------------- */
+int64_t kvhip_cache_offset(const kvhip_cache *cache);          /* `offset` */
+int64_t kvhip_cache_idx(const kvhip_cache *cache);             /* RotatingKVCache.idx (metaState[4]) */
+int64_t kvhip_cache_max_size(const kvhip_cache *cache);        /* `maxSize`, -1 for nil */
+int32_t kvhip_cache_group_size(const kvhip_cache *cache);      /* QuantizedKVCacheProtocol.groupSize */
+int32_t kvhip_cache_bits(const kvhip_cache *cache);            /* QuantizedKVCacheProtocol.bits */
+int64_t kvhip_cache_capacity(const kvhip_cache *cache);        /* row extent of the reference's buffers */
+int64_t kvhip_cache_presented_length(const kvhip_cache *cache);/* key extent `update` last returned */
+int32_t kvhip_cache_is_trimmable(const kvhip_cache *cache, int64_t after_positions); /* isTrimmable(after:) */
+int64_t kvhip_cache_trim(kvhip_cache *cache, int64_t n);       /* trim(_:) -> positions trimmed */
+/* `offset` is a settable stored property in the reference (KVCache.swift:185;
+ * used by toQuantized :504 and toUnquantized :1190). */
+kvhip_status kvhip_cache_set_offset(kvhip_cache *cache, int64_t offset);
+
+/*
+ * `update(keys:values:)` (Simple :404-447, Rotating :742-750) and
+ * `updateQuantized(keys:values:)` (:1011-1102).
+ * keys [B,Hkv,L,Dk], values [B,Hkv,L,Dv] of `dtype`.  Appends / ring-writes /
+ * quantizes on the device; advances offset (and idx).  What the reference
+ * returns -- every cached row in presentation order -- stays on the device and
+ * is read by kvhip_cache_attend, or copied out by kvhip_cache_fetch*.
+ */
+kvhip_status kvhip_cache_update(kvhip_cache *cache, const void *keys, const void *values, int32_t B,
+                                int32_t Hkv, int32_t L, int32_t Dk, int32_t Dv, int32_t dtype,
+                                void *stream);
+
+/* The arrays the last `update` returned: dst_keys [B,Hkv,P,Dk], dst_values
+ * [B,Hkv,P,Dv], P = kvhip_cache_presented_length.  Not for quantized caches. */
+kvhip_status kvhip_cache_fetch(const kvhip_cache *cache, void *dst_keys, void *dst_values, void *stream);
+
+/*
+ * Attention over what the cache presents, replacing
+ * `MLXFast.scaledDotProductAttention` (AttentionUtils.swift:86-93) for Simple /
+ * Rotating caches and `quantizedScaledDotProductAttention`
+ * (KVCache.swift:2351-2447) for quantized ones.
+ * queries [B,Hq,L,Dk] and out [B,Hq,L,Dv] in the cache's dtype.
+ */
+kvhip_status kvhip_cache_attend(kvhip_cache *cache, const void *queries, int32_t B, int32_t Hq,
+                                int32_t L, int32_t D, float scale, const kvhip_mask *mask, void *out,
+                                void *stream);
+
+/* `attentionWithCacheUpdate` (AttentionUtils.swift:37-95): update, then attend. */
+kvhip_status kvhip_cache_update_attend(kvhip_cache *cache, const void *queries, const void *keys,
+                                       const void *values, int32_t B, int32_t Hq, int32_t Hkv,
+                                       int32_t L, int32_t Dk, int32_t Dv, int32_t dtype, float scale,
+                                       const kvhip_mask *mask, void *out, void *stream);
+
+/* `makeMask(n:windowSize:returnArray:)`; window_size <= 0 stands for nil. */
+kvhip_status kvhip_cache_mask_plan(const kvhip_cache *cache, int32_t n, int32_t window_size,
+                                   int32_t return_array, kvhip_mask_plan_t *out_plan);
+/* Writes the bool array the plan describes: dst [rows, cols] (or [cols] when rolled), one byte each. */
+kvhip_status kvhip_mask_materialize(const kvhip_mask_plan_t *plan, uint8_t *dst, void *stream);
+
+/* ---- state / metaState (serialisation surface) --------------------------- */
+/*
+ * `state` getter: Simple/Rotating [keys, values]; Quantized [k.wq, k.scales,
+ * k.biases, v.wq, v.scales, v.biases] (KVCache.swift:449-460, :752-763,
+ * :1113-1130), each [B,Hkv,rows,last].  Count is 0 before the first write.
+ */
+int32_t kvhip_cache_state_count(const kvhip_cache *cache);
+kvhip_status kvhip_cache_state_desc(const kvhip_cache *cache, int32_t index, int64_t shape[4],
+                                    int32_t *dtype);
+kvhip_status kvhip_cache_state_export(const kvhip_cache *cache, int32_t index, void *dst, void *stream);
+/*
+ * `state` setter (KVCache.swift:461-468, :764-773, :1131-1146): `count` arrays in
+ * the getter's order, shapes[i] = 4 extents, dtypes[i] a kvhip_dtype.  Simple
+ * sets offset to the row extent; Rotating and Quantized leave offset to metaState.
+ */
+kvhip_status kvhip_cache_state_import(kvhip_cache *cache, int32_t count, const void *const *srcs,
+                                      const int64_t *shapes, const int32_t *dtypes, void *stream);
+/* `metaState`: Simple [""]; Rotating [keep,maxSize,step,offset,idx,origin];
+ * Quantized [step,offset,groupSize,bits] (KVCache.swift:207-214, :775-815, :1148-1166). */
+int32_t kvhip_cache_meta_count(const kvhip_cache *cache);
+/* Copies entry `index` (NUL-terminated) into buf; returns its length, or a negative status. */
+int32_t kvhip_cache_meta_get(const kvhip_cache *cache, int32_t index, char *buf, int32_t buf_len);
+kvhip_status kvhip_cache_meta_set(kvhip_cache *cache, int32_t count, const char *const *values);
+
+/* ---- ring reads and conversions ------------------------------------------ */
+/*
+ * `RotatingKVCache.logicalView(tail:)` (KVCache.swift:631-658): chronological
+ * trailing entries without mutating the ring.  *out_rows receives
+ * n = max(min(max(tail,0),count), min(keep,count)); with non-NULL dst pointers
+ * the rows are written as [B,Hkv,n,D].  Returns KVHIP_ERR_STATE before the first write.
+ */
+kvhip_status kvhip_cache_logical_view(const kvhip_cache *cache, int64_t tail, int64_t *out_rows,
+                                      void *dst_keys, void *dst_values, void *stream);
+/* `KVCacheSimple.toQuantized(groupSize:bits:)` (KVCache.swift:486-523): bulk quantize on the device. */
+kvhip_status kvhip_cache_to_quantized(const kvhip_cache *cache, int32_t group_size, int32_t bits,
+                                      void *stream, kvhip_cache **out_cache);
+/* `QuantizedKVCache.toUnquantized()` (KVCache.swift:1188-1209). */
+kvhip_status kvhip_cache_to_unquantized(const kvhip_cache *cache, void *stream, kvhip_cache **out_cache);
+/* `resolvedKVQuantizationGroupSize` (KVCache.swift:902-920); 0 when none fits. */
+int32_t kvhip_resolved_group_size(int32_t requested, int32_t key_head_dim, int32_t value_head_dim);
+
+/* ---- standalone quantizer (MLX.quantized / MLX.dequantized call sites) ---- */
+/* src [rows, D] of `dtype` -> wq [rows, D*bits/32] u32, scales/biases [rows, D/group_size] of `dtype`. */
+kvhip_status kvhip_affine_quantize(const void *src, int64_t rows, int32_t D, int32_t group_size,
+                                   int32_t bits, int32_t dtype, uint32_t *wq, void *scales,
+                                   void *biases, void *stream);
+kvhip_status kvhip_affine_dequantize(const uint32_t *wq, const void *scales, const void *biases,
+                                     int64_t rows, int32_t D, int32_t group_size, int32_t bits,
+                                     int32_t dtype, void *dst, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KVHIP_H */

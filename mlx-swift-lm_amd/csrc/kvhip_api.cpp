@@ -1,0 +1,1049 @@
+// Host side of libkvhip: the three cache state machines of the reference
+// (offset / idx / capacity / ring bookkeeping as host integers, exactly as
+// Libraries/MLXLMCommon/KVCache.swift keeps them), device page storage, and the
+// extern "C" surface declared in include/kvhip.h.
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "kvhip_internal.hpp"
+
+using namespace kvhip;
+
+namespace {
+
+thread_local std::string g_err;
+thread_local bool g_has_err = false;
+int g_policy = 0;
+bool g_inited = false;
+
+kvhip_status fail(kvhip_status code, const std::string &msg) {
+    g_err = msg;
+    g_has_err = true;
+    return code;
+}
+
+#define KV_HIP(expr)                                                                         \
+    do {                                                                                     \
+        hipError_t e_ = (expr);                                                              \
+        if (e_ != hipSuccess)                                                                \
+            return fail(KVHIP_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(e_));   \
+    } while (0)
+#define KV_TRY(expr)                         \
+    do {                                     \
+        kvhip_status s_ = (expr);            \
+        if (s_ != KVHIP_OK) return s_;       \
+    } while (0)
+
+int elem_size(int dtype) { return dtype == KVHIP_F32 ? 4 : 2; }
+
+}  // namespace
+
+struct kvhip_cache {
+    int kind = 0;
+    // constructor arguments
+    int step = 256;
+    int64_t max_size = 0;
+    int64_t keep = 0;
+    int gs = 64, bits = 8;
+    std::string origin = "modelNative";
+    // reference bookkeeping
+    int64_t offset = 0;
+    int64_t idx = 0;
+    bool has_buffers = false;  // the reference's `keys != nil`
+    int64_t ref_len = 0;       // row extent of the reference's buffers
+    int64_t presented = 0;     // key extent the last update returned
+    // geometry, fixed by the first update / import / reserve
+    bool has_geom = false;
+    int B = 0, Hkv = 0;
+    Store st;
+    int64_t cap_pages = 0;
+    // rotating only: reference row -> physical slot, and slot occupancy
+    std::vector<int32_t> rows;
+    std::vector<uint8_t> used;
+    int64_t cursor = 0;
+    // scratch for attention
+    float *ws = nullptr;
+    size_t ws_bytes = 0;
+
+    int64_t cap_slots() const { return cap_pages * PAGE; }
+};
+
+namespace {
+
+void free_store(Store &st) {
+    if (st.k) (void)hipFree(st.k);
+    if (st.v) (void)hipFree(st.v);
+    if (st.ksb) (void)hipFree(st.ksb);
+    if (st.vsb) (void)hipFree(st.vsb);
+    st.k = st.v = st.ksb = st.vsb = nullptr;
+}
+
+kvhip_status set_geometry(kvhip_cache *c, int B, int Hkv, int Dk, int Dv, int dtype) {
+    if (B <= 0 || Hkv <= 0 || Dk <= 0 || Dv <= 0) return fail(KVHIP_ERR_INVALID_ARG, "non-positive shape");
+    if (dtype != KVHIP_F16 && dtype != KVHIP_BF16 && dtype != KVHIP_F32)
+        return fail(KVHIP_ERR_INVALID_ARG, "cache dtype must be float16, bfloat16 or float32");
+    if ((int64_t)B * Hkv > 65535) return fail(KVHIP_ERR_UNSUPPORTED, "B * Hkv above 65535");
+    if (c->has_geom) {
+        const Store &s = c->st;
+        if (s.BH != B * Hkv || c->B != B || s.Dk != Dk || s.Dv != Dv || s.dtype != dtype)
+            return fail(KVHIP_ERR_INVALID_ARG, "shape or dtype differs from what this cache already holds");
+        return KVHIP_OK;
+    }
+    Store &s = c->st;
+    s = Store();
+    c->B = B;
+    c->Hkv = Hkv;
+    s.BH = B * Hkv;
+    s.Dk = Dk;
+    s.Dv = Dv;
+    s.dtype = dtype;
+    s.es = elem_size(dtype);
+    if (c->kind == KVHIP_KIND_QUANTIZED) {
+        if (c->bits != 2 && c->bits != 4 && c->bits != 8)
+            return fail(KVHIP_ERR_UNSUPPORTED, "affine KV quantization is implemented for 2, 4 and 8 bits");
+        if (Dk % c->gs || Dv % c->gs) return fail(KVHIP_ERR_INVALID_ARG, "head dim not divisible by the group size");
+        s.bits = c->bits;
+        s.gs = c->gs;
+        s.k_row = (uint32_t)(Dk * c->bits / 8);
+        s.k_cell = s.k_row * PAGE;
+        s.v_cell = (uint32_t)(Dv * c->bits / 8) * PAGE;
+        s.ksb_row = (uint32_t)(Dk / c->gs * 2 * s.es);
+        s.vsb_row = (uint32_t)(Dv / c->gs * 2 * s.es);
+        s.ksb_cell = s.ksb_row * PAGE;
+        s.vsb_cell = s.vsb_row * PAGE;
+    } else {
+        s.k_row = (uint32_t)(Dk * s.es);
+        s.k_cell = s.k_row * PAGE;
+        s.v_cell = (uint32_t)(Dv * s.es) * PAGE;
+    }
+    c->has_geom = true;
+    return KVHIP_OK;
+}
+
+// Make room for `slots` physical slots.  Pages are appended; contents keep their place.
+kvhip_status ensure_slots(kvhip_cache *c, int64_t slots, hipStream_t stream, bool exact = false) {
+    const int64_t need = (slots + PAGE - 1) / PAGE;
+    if (need <= c->cap_pages) return KVHIP_OK;
+    int64_t pages = need;
+    if (!exact && c->cap_pages > 0) pages = std::max(need, c->cap_pages + (c->cap_pages + 1) / 2);
+    Store ns = c->st;
+    ns.k = ns.v = ns.ksb = ns.vsb = nullptr;
+    const size_t BH = c->st.BH;
+    struct P { char **dst; char *src; size_t cell; } planes[4] = {
+        {&ns.k, c->st.k, c->st.k_cell}, {&ns.v, c->st.v, c->st.v_cell},
+        {&ns.ksb, c->st.ksb, c->st.ksb_cell}, {&ns.vsb, c->st.vsb, c->st.vsb_cell}};
+    for (auto &p : planes) {
+        if (p.cell == 0) continue;
+        const size_t bytes = (size_t)pages * BH * p.cell;
+        hipError_t e = hipMalloc((void **)p.dst, bytes);
+        if (e != hipSuccess) {
+            free_store(ns);
+            return fail(KVHIP_ERR_HIP, std::string("hipMalloc of a cache plane failed: ") + hipGetErrorString(e));
+        }
+        const size_t old = (size_t)c->cap_pages * BH * p.cell;
+        if (old) KV_HIP(hipMemcpyAsync(*p.dst, p.src, old, hipMemcpyDeviceToDevice, stream));
+        // octet words are merged read-modify-write: start them from zero
+        KV_HIP(hipMemsetAsync(*p.dst + old, 0, bytes - old, stream));
+    }
+    if (c->cap_pages > 0) KV_HIP(hipStreamSynchronize(stream));
+    free_store(c->st);
+    c->st = ns;
+    c->cap_pages = pages;
+    if (c->kind == KVHIP_KIND_ROTATING) c->used.resize((size_t)c->cap_slots(), 0);
+    return KVHIP_OK;
+}
+
+kvhip_status ensure_ws(kvhip_cache *c, size_t bytes, hipStream_t stream) {
+    if (bytes <= c->ws_bytes) return KVHIP_OK;
+    if (c->ws) {
+        KV_HIP(hipStreamSynchronize(stream));
+        (void)hipFree(c->ws);
+        c->ws = nullptr;
+        c->ws_bytes = 0;
+    }
+    const size_t want = bytes + bytes / 4;
+    KV_HIP(hipMalloc((void **)&c->ws, want));
+    c->ws_bytes = want;
+    return KVHIP_OK;
+}
+
+// ---- run tables ------------------------------------------------------------
+struct RunList {
+    std::vector<int32_t> row0, phys0, len;
+    size_t size() const { return row0.size(); }
+};
+
+RunList runs_of(const int32_t *slots, int64_t n) {
+    RunList r;
+    for (int64_t i = 0; i < n;) {
+        int64_t j = i + 1;
+        while (j < n && slots[j] == slots[j - 1] + 1) ++j;
+        r.row0.push_back((int32_t)i);
+        r.phys0.push_back(slots[i]);
+        r.len.push_back((int32_t)(j - i));
+        i = j;
+    }
+    return r;
+}
+
+Runs pack_runs(const RunList &rl, size_t first, size_t count) {
+    Runs r;
+    r.n = (int32_t)count;
+    for (size_t i = 0; i < (size_t)MAXRUNS; ++i) {
+        const bool live = i < count;
+        r.row0[i] = live ? rl.row0[first + i] : 0;
+        r.phys0[i] = live ? rl.phys0[first + i] : 0;
+        r.len[i] = live ? rl.len[first + i] : 0;
+    }
+    return r;
+}
+
+Runs identity_runs(int64_t n) {
+    RunList rl;
+    if (n > 0) {
+        rl.row0.push_back(0);
+        rl.phys0.push_back(0);
+        rl.len.push_back((int32_t)n);
+    }
+    return pack_runs(rl, 0, rl.size());
+}
+
+// Dense export of the rows named by `slots` (any order) into [BH, n, D] arrays.
+kvhip_status export_slots(const kvhip_cache *c, const int32_t *slots, int64_t n, void *dk, void *dv,
+                          hipStream_t stream) {
+    const RunList rl = runs_of(slots, n);
+    for (size_t first = 0; first < rl.size(); first += MAXRUNS) {
+        const size_t cnt = std::min((size_t)MAXRUNS, rl.size() - first);
+        const Runs r = pack_runs(rl, first, cnt);
+        const int begin = rl.row0[first];
+        const int end = rl.row0[first + cnt - 1] + rl.len[first + cnt - 1];
+        KV_HIP(launch_export_fp(c->st, r, begin, end - begin, 0, (int)n, dk, dv, stream));
+    }
+    return KVHIP_OK;
+}
+
+// ---- rotating: physical slot management ---------------------------------------
+kvhip_status ring_alloc(kvhip_cache *c, int64_t n, std::vector<int32_t> &out, hipStream_t stream) {
+    int64_t live = 0;
+    for (uint8_t u : c->used) live += u;
+    if (live + n > c->cap_slots()) KV_TRY(ensure_slots(c, live + n, stream));
+    const int64_t C = c->cap_slots();
+    int64_t p = c->cursor % C;
+    for (int64_t got = 0, scanned = 0; got < n; ++scanned) {
+        if (scanned > 2 * C) return fail(KVHIP_ERR_INTERNAL, "ring slot allocation found no free slot");
+        if (!c->used[(size_t)p]) {
+            c->used[(size_t)p] = 1;
+            out.push_back((int32_t)p);
+            ++got;
+        }
+        p = (p + 1) % C;
+    }
+    c->cursor = p;
+    return KVHIP_OK;
+}
+
+void ring_release(kvhip_cache *c, const std::vector<int32_t> &rows, size_t lo, size_t hi) {
+    for (size_t i = lo; i < hi && i < rows.size(); ++i) c->used[(size_t)rows[i]] = 0;
+}
+
+// `trim(trimSize:_:)` (KVCache.swift:576-590) on the row map
+void ring_front_trim(kvhip_cache *c, int64_t trim) {
+    if (trim <= 0) return;
+    const size_t keep = (size_t)std::min<int64_t>(c->keep, (int64_t)c->rows.size());
+    const size_t cut_hi = std::min(c->rows.size(), keep + (size_t)trim);
+    ring_release(c, c->rows, keep, cut_hi);
+    c->rows.erase(c->rows.begin() + keep, c->rows.begin() + cut_hi);
+}
+
+// `temporalOrder(_:)` (KVCache.swift:592-606) as a permutation of the row map
+std::vector<int32_t> temporal_order(const kvhip_cache *c, std::vector<int32_t> *dropped = nullptr) {
+    const std::vector<int32_t> &a = c->rows;
+    const int64_t len = (int64_t)a.size();
+    if (c->idx == len) return a;
+    std::vector<int32_t> o;
+    if (c->idx < c->offset) {
+        const int64_t k = std::min<int64_t>(std::max<int64_t>(c->keep, 0), len);
+        const int64_t i = std::min<int64_t>(std::max<int64_t>(c->idx, k), len);
+        o.insert(o.end(), a.begin(), a.begin() + k);
+        o.insert(o.end(), a.begin() + i, a.end());
+        if (i > k) o.insert(o.end(), a.begin() + k, a.begin() + i);
+        return o;
+    }
+    const int64_t i = std::min<int64_t>(std::max<int64_t>(c->idx, 0), len);
+    o.assign(a.begin(), a.begin() + i);
+    if (dropped) dropped->assign(a.begin() + i, a.end());
+    return o;
+}
+
+// Write `n` new rows (src rows [src0, src0+n) of an [BH, L, D] pair) to the given slots.
+kvhip_status write_rows(kvhip_cache *c, const void *keys, const void *values, int L, int src0,
+                        const int32_t *slots, int64_t n, hipStream_t stream) {
+    const RunList rl = runs_of(slots, n);
+    for (size_t i = 0; i < rl.size(); ++i) {
+        if (c->kind == KVHIP_KIND_QUANTIZED)
+            KV_HIP(launch_append_quant(c->st, keys, values, L, src0 + rl.row0[i], rl.phys0[i], rl.len[i], stream));
+        else
+            KV_HIP(launch_append_fp(c->st, keys, values, L, src0 + rl.row0[i], rl.phys0[i], rl.len[i], stream));
+    }
+    return KVHIP_OK;
+}
+
+// If the presented rows are scattered over more runs than a kernel takes, gather them
+// into slot order once (ring-order gather) so later launches see a single run.
+kvhip_status ring_compact_if_needed(kvhip_cache *c, hipStream_t stream) {
+    const RunList rl = runs_of(c->rows.data(), (int64_t)c->rows.size());
+    if (rl.size() <= (size_t)MAXRUNS) return KVHIP_OK;
+    kvhip_cache tmp;
+    tmp.kind = c->kind;
+    tmp.has_geom = true;
+    tmp.B = c->B;
+    tmp.Hkv = c->Hkv;
+    tmp.st = c->st;
+    tmp.st.k = tmp.st.v = tmp.st.ksb = tmp.st.vsb = nullptr;
+    tmp.cap_pages = 0;
+    KV_TRY(ensure_slots(&tmp, c->cap_slots(), stream, true));
+    for (size_t first = 0; first < rl.size(); first += MAXRUNS) {
+        const size_t cnt = std::min((size_t)MAXRUNS, rl.size() - first);
+        KV_HIP(launch_compact_fp(c->st, pack_runs(rl, first, cnt), tmp.st, (int)c->rows.size(), stream));
+    }
+    KV_HIP(hipStreamSynchronize(stream));
+    free_store(c->st);
+    c->st = tmp.st;
+    tmp.st = Store();
+    std::fill(c->used.begin(), c->used.end(), 0);
+    for (size_t i = 0; i < c->rows.size(); ++i) {
+        c->rows[i] = (int32_t)i;
+        c->used[i] = 1;
+    }
+    c->cursor = (int64_t)c->rows.size();
+    return KVHIP_OK;
+}
+
+// ---- the three update paths ----------------------------------------------------
+kvhip_status update_simple(kvhip_cache *c, const void *k, const void *v, int L, hipStream_t stream) {
+    // KVCache.swift:404-447
+    const int64_t prev = c->offset;
+    if (!c->has_buffers || prev + L > c->ref_len) {
+        const int64_t n_steps = (c->step + L - 1) / c->step;
+        const int64_t grow = n_steps * c->step;
+        if (c->has_buffers) c->ref_len = ((prev % c->step) != 0 ? prev : c->ref_len) + grow;
+        else c->ref_len = grow;
+        c->has_buffers = true;
+    }
+    KV_TRY(ensure_slots(c, prev + L, stream));
+    c->offset += L;
+    if (c->kind == KVHIP_KIND_QUANTIZED) KV_HIP(launch_append_quant(c->st, k, v, L, 0, (int)prev, L, stream));
+    else KV_HIP(launch_append_fp(c->st, k, v, L, 0, (int)prev, L, stream));
+    c->presented = c->offset;
+    return KVHIP_OK;
+}
+
+kvhip_status update_rotating(kvhip_cache *c, const void *k, const void *v, int L, hipStream_t stream) {
+    const int64_t M = c->max_size;
+    if (L == 1) {
+        // updateInPlace, KVCache.swift:684-740
+        const int64_t prev = c->offset;
+        if (!c->has_buffers || (prev >= c->ref_len && c->ref_len < M)) {
+            const int64_t new_size = std::min<int64_t>(c->step, M - prev);
+            if (new_size > 0) KV_TRY(ring_alloc(c, new_size, c->rows, stream));
+            c->has_buffers = true;
+            c->idx = prev;
+        }
+        const int64_t trim = (int64_t)c->rows.size() - M;
+        if (trim > 0) {
+            ring_front_trim(c, trim);
+            c->idx = M;
+        }
+        if (c->idx == M) c->idx = c->keep;
+        c->ref_len = (int64_t)c->rows.size();
+        if (c->idx < 0 || c->idx >= c->ref_len)
+            return fail(KVHIP_ERR_STATE, "RotatingKVCache write cursor lies outside its buffer");
+        KV_TRY(ring_compact_if_needed(c, stream));
+        const int32_t slot = c->rows[(size_t)c->idx];
+        KV_HIP(launch_append_fp(c->st, k, v, 1, 0, slot, 1, stream));
+        c->offset += 1;
+        c->idx += 1;
+        c->presented = c->offset < M ? c->offset : c->ref_len;
+        return KVHIP_OK;
+    }
+    // updateConcat, KVCache.swift:660-682
+    if (!c->has_buffers) {
+        KV_TRY(ring_alloc(c, L, c->rows, stream));
+        c->has_buffers = true;
+        KV_TRY(write_rows(c, k, v, L, 0, c->rows.data(), L, stream));
+    } else {
+        std::vector<int32_t> dropped;
+        std::vector<int32_t> ordered = temporal_order(c, &dropped);
+        for (int32_t s : dropped) c->used[(size_t)s] = 0;
+        c->rows.swap(ordered);
+        c->idx = (int64_t)c->rows.size();
+        ring_front_trim(c, c->idx - M + 1);
+        const size_t base = c->rows.size();
+        KV_TRY(ring_alloc(c, L, c->rows, stream));
+        KV_TRY(write_rows(c, k, v, L, 0, c->rows.data() + base, L, stream));
+    }
+    c->offset += L;
+    c->ref_len = (int64_t)c->rows.size();
+    c->idx = c->ref_len;
+    c->presented = c->ref_len;
+    return ring_compact_if_needed(c, stream);
+}
+
+// rows of the current presentation as (slot list or identity)
+kvhip_status presented_runs(const kvhip_cache *c, Runs &runs, int &slots_span) {
+    if (c->kind != KVHIP_KIND_ROTATING) {
+        runs = identity_runs(c->presented);
+        slots_span = (int)c->presented;
+        return KVHIP_OK;
+    }
+    const RunList rl = runs_of(c->rows.data(), std::min<int64_t>(c->presented, (int64_t)c->rows.size()));
+    if (rl.size() > (size_t)MAXRUNS) return fail(KVHIP_ERR_INTERNAL, "ring presentation not compacted");
+    runs = pack_runs(rl, 0, rl.size());
+    slots_span = 0;
+    for (size_t i = 0; i < rl.size(); ++i) slots_span = std::max(slots_span, rl.phys0[i] + rl.len[i]);
+    return KVHIP_OK;
+}
+
+int64_t state_rows(const kvhip_cache *c) {
+    // KVCache.swift:449-460, :752-763, :1113-1130: sliced to offset when offset < extent
+    if (!c->has_buffers) return 0;
+    return c->offset < c->ref_len ? std::max<int64_t>(c->offset, 0) : c->ref_len;
+}
+
+hipStream_t S(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+kvhip_cache *new_cache_like(const kvhip_cache *c) {
+    kvhip_cache *n = new kvhip_cache();
+    n->kind = c->kind;
+    n->step = c->step;
+    n->max_size = c->max_size;
+    n->keep = c->keep;
+    n->gs = c->gs;
+    n->bits = c->bits;
+    return n;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *kvhip_version(void) { return "kvhip 0.1 (gfx950)"; }
+
+const char *kvhip_last_error_message(void) { return g_has_err ? g_err.c_str() : nullptr; }
+
+kvhip_status kvhip_init(int32_t device) {
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) return fail(KVHIP_ERR_NO_DEVICE, "no HIP device is visible");
+    if (device < 0 || device >= n) return fail(KVHIP_ERR_INVALID_ARG, "device index out of range");
+    KV_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    KV_HIP(hipGetDeviceProperties(&prop, device));
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(KVHIP_ERR_NO_DEVICE, std::string("libkvhip is built for gfx950 only, found ") + prop.gcnArchName);
+    g_inited = true;
+    return KVHIP_OK;
+}
+
+kvhip_status kvhip_sync(void *stream) {
+    KV_HIP(hipStreamSynchronize(S(stream)));
+    return KVHIP_OK;
+}
+
+void kvhip_set_kernel_policy(int32_t policy) { g_policy = policy; }
+
+kvhip_status kvhip_cache_create(const kvhip_config *cfg, kvhip_cache **out) {
+    if (!cfg || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (cfg->kind < 0 || cfg->kind > 2) return fail(KVHIP_ERR_INVALID_ARG, "unknown cache kind");
+    kvhip_cache *c = new kvhip_cache();
+    c->kind = cfg->kind;
+    c->step = cfg->step > 0 ? cfg->step : 256;
+    if (c->kind == KVHIP_KIND_ROTATING) {
+        if (cfg->max_size <= 0) {
+            delete c;
+            return fail(KVHIP_ERR_INVALID_ARG, "RotatingKVCache requires a positive maxSize");
+        }
+        c->max_size = cfg->max_size;
+        c->keep = std::max(0, cfg->keep);
+    }
+    if (c->kind == KVHIP_KIND_QUANTIZED) {
+        c->step = 256;  // `private let step` fixed at 256, KVCache.swift:934
+        c->gs = cfg->group_size > 0 ? cfg->group_size : 64;
+        c->bits = cfg->bits > 0 ? cfg->bits : 8;
+    }
+    *out = c;
+    return KVHIP_OK;
+}
+
+void kvhip_cache_free(kvhip_cache *c) {
+    if (!c) return;
+    free_store(c->st);
+    if (c->ws) (void)hipFree(c->ws);
+    delete c;
+}
+
+int64_t kvhip_cache_offset(const kvhip_cache *c) { return c ? c->offset : -1; }
+int64_t kvhip_cache_idx(const kvhip_cache *c) { return c ? c->idx : -1; }
+int64_t kvhip_cache_max_size(const kvhip_cache *c) { return (c && c->kind == KVHIP_KIND_ROTATING) ? c->max_size : -1; }
+int32_t kvhip_cache_group_size(const kvhip_cache *c) { return c ? c->gs : -1; }
+int32_t kvhip_cache_bits(const kvhip_cache *c) { return c ? c->bits : -1; }
+int64_t kvhip_cache_capacity(const kvhip_cache *c) { return c ? c->ref_len : -1; }
+int64_t kvhip_cache_presented_length(const kvhip_cache *c) { return c ? c->presented : -1; }
+
+int32_t kvhip_cache_is_trimmable(const kvhip_cache *c, int64_t after) {
+    if (!c) return 0;
+    if (c->kind == KVHIP_KIND_ROTATING) return c->offset + after < c->max_size;  // KVCache.swift:821-823
+    return 1;
+}
+
+int64_t kvhip_cache_trim(kvhip_cache *c, int64_t n) {
+    if (!c) return 0;
+    const int64_t t = std::min(c->offset, n);  // KVCache.swift:474-478, :826-831, :1171-1175
+    c->offset -= t;
+    if (c->kind == KVHIP_KIND_ROTATING) c->idx -= t;
+    return t;
+}
+
+kvhip_status kvhip_cache_set_offset(kvhip_cache *c, int64_t offset) {
+    if (!c) return fail(KVHIP_ERR_INVALID_ARG, "null cache");
+    c->offset = offset;
+    return KVHIP_OK;
+}
+
+int32_t kvhip_resolved_group_size(int32_t requested, int32_t kd, int32_t vd) {
+    // KVCache.swift:902-920
+    requested = std::max(1, requested);
+    int best = 0;
+    for (int g : {32, 64, 128}) {
+        if (kd % g || vd % g) continue;
+        if (!best || std::abs(g - requested) < std::abs(best - requested)) best = g;
+    }
+    return best;
+}
+
+kvhip_status kvhip_cache_reserve(kvhip_cache *c, int32_t B, int32_t Hkv, int32_t Dk, int32_t Dv,
+                                 int32_t dtype, int64_t tokens) {
+    if (!c) return fail(KVHIP_ERR_INVALID_ARG, "null cache");
+    if (c->kind == KVHIP_KIND_QUANTIZED && !c->has_buffers && c->offset == 0) {
+        const int eff = kvhip_resolved_group_size(c->gs, Dk, Dv);
+        if (!eff) return fail(KVHIP_ERR_STATE, "KV cache quantization requires head dimensions divisible by 32, 64 or 128");
+        c->gs = eff;
+    }
+    KV_TRY(set_geometry(c, B, Hkv, Dk, Dv, dtype));
+    return ensure_slots(c, tokens, nullptr, true);
+}
+
+kvhip_status kvhip_cache_update(kvhip_cache *c, const void *keys, const void *values, int32_t B,
+                                int32_t Hkv, int32_t L, int32_t Dk, int32_t Dv, int32_t dtype, void *stream) {
+    if (!c || !keys || !values) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (L <= 0) return fail(KVHIP_ERR_INVALID_ARG, "update needs at least one new row");
+    if (c->kind == KVHIP_KIND_QUANTIZED) {
+        // KVCache.swift:1020-1037
+        const int eff = kvhip_resolved_group_size(c->gs, Dk, Dv);
+        if (!eff)
+            return fail(KVHIP_ERR_STATE,
+                        "KV cache quantization requires head dimensions divisible by one of the supported group sizes (32, 64, 128)");
+        if (eff != c->gs && !c->has_buffers && c->offset == 0) {
+            if (c->has_geom && c->cap_pages > 0) return fail(KVHIP_ERR_STATE, "group size changed after storage was reserved");
+            c->gs = eff;
+            c->has_geom = false;
+        }
+    }
+    KV_TRY(set_geometry(c, B, Hkv, Dk, Dv, dtype));
+    if (c->kind == KVHIP_KIND_ROTATING) return update_rotating(c, keys, values, L, S(stream));
+    return update_simple(c, keys, values, L, S(stream));
+}
+
+kvhip_status kvhip_cache_fetch(const kvhip_cache *c, void *dk, void *dv, void *stream) {
+    if (!c) return fail(KVHIP_ERR_INVALID_ARG, "null cache");
+    if (c->kind == KVHIP_KIND_QUANTIZED)
+        return fail(KVHIP_ERR_STATE, "`update` was called on `QuantizedKVCache`. Use `updateQuantized` instead.");
+    if (!c->has_buffers) return fail(KVHIP_ERR_STATE, "cache is empty");
+    if (c->kind == KVHIP_KIND_ROTATING)
+        return export_slots(c, c->rows.data(), c->presented, dk, dv, S(stream));
+    std::vector<int32_t> ident((size_t)c->presented);
+    for (size_t i = 0; i < ident.size(); ++i) ident[i] = (int32_t)i;
+    return export_slots(c, ident.data(), c->presented, dk, dv, S(stream));
+}
+
+kvhip_status kvhip_cache_attend(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, int32_t L,
+                                int32_t D, float scale, const kvhip_mask *mask, void *out, void *stream) {
+    if (!c || !q || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (!c->has_geom || !c->has_buffers || c->presented <= 0) return fail(KVHIP_ERR_STATE, "attention over an empty cache");
+    if (B != c->B || D != c->st.Dk) return fail(KVHIP_ERR_INVALID_ARG, "query shape does not match the cache");
+    if (Hq <= 0 || Hq % c->Hkv) return fail(KVHIP_ERR_INVALID_ARG, "query heads must be a multiple of KV heads");
+    if (L <= 0 || L > 65535) return fail(KVHIP_ERR_INVALID_ARG, "query length out of range");
+    AttendArgs a;
+    a.st = c->st;
+    KV_TRY(presented_runs(c, a.runs, a.slots));
+    a.q = q;
+    a.out = out;
+    a.B = B;
+    a.Hq = Hq;
+    a.Hkv = c->Hkv;
+    a.L = L;
+    a.T = (int)c->presented;
+    a.scale = scale;
+    if (mask) {
+        MaskDev &m = a.mask;
+        m.mode = mask->mode;
+        if (m.mode < 0 || m.mode > 3) return fail(KVHIP_ERR_INVALID_ARG, "unknown mask mode");
+        if (m.mode == KVHIP_MASK_ARRAY) {
+            if (!mask->data) return fail(KVHIP_ERR_INVALID_ARG, "array mask without data");
+            if (mask->key_len != a.T)
+                return fail(KVHIP_ERR_INVALID_ARG, "array mask key extent differs from the presented length");
+            if (mask->dtype != KVHIP_BOOL && mask->dtype != KVHIP_F16 && mask->dtype != KVHIP_BF16 && mask->dtype != KVHIP_F32)
+                return fail(KVHIP_ERR_INVALID_ARG, "array mask dtype must be bool or a float type");
+            m.dtype = mask->dtype;
+            m.data = mask->data;
+            m.sb = mask->stride_b;
+            m.sh = mask->stride_h;
+            m.sl = mask->stride_l;
+        } else if (m.mode == KVHIP_MASK_WINDOW) {
+            m.offset = mask->offset;
+            m.window = mask->window;
+            m.lengths = mask->lengths;
+            m.left_pad = mask->left_pad;
+        }
+    }
+    hipStream_t s = S(stream);
+    const bool fast = g_policy == 0 && attend_decode_supported(a);
+    KV_TRY(ensure_ws(c, fast ? attend_decode_workspace(a) : attend_generic_workspace(a), s));
+    a.workspace = c->ws;
+    a.workspace_bytes = c->ws_bytes;
+    KV_HIP(fast ? launch_attend_decode(a, s) : launch_attend_generic(a, s));
+    return KVHIP_OK;
+}
+
+kvhip_status kvhip_cache_update_attend(kvhip_cache *c, const void *q, const void *k, const void *v,
+                                       int32_t B, int32_t Hq, int32_t Hkv, int32_t L, int32_t Dk,
+                                       int32_t Dv, int32_t dtype, float scale, const kvhip_mask *mask,
+                                       void *out, void *stream) {
+    KV_TRY(kvhip_cache_update(c, k, v, B, Hkv, L, Dk, Dv, dtype, stream));
+    return kvhip_cache_attend(c, q, B, Hq, L, Dk, scale, mask, out, stream);
+}
+
+kvhip_status kvhip_cache_mask_plan(const kvhip_cache *c, int32_t n, int32_t window, int32_t return_array,
+                                   kvhip_mask_plan_t *p) {
+    if (!c || !p) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    std::memset(p, 0, sizeof(*p));
+    const bool has_w = window > 0;
+    if (c->kind != KVHIP_KIND_ROTATING) {
+        // BaseKVCache.makeMask, KVCache.swift:236-250
+        if (n == 1) { p->mode = KVHIP_MASK_NONE; return KVHIP_OK; }
+        if (return_array || (has_w && n > window)) {
+            p->mode = KVHIP_MASK_ARRAY;
+            p->rows = n;
+            p->cols = (int32_t)c->offset + n;
+            p->offset = (int32_t)c->offset;
+            p->window = has_w ? window : 0;
+            return KVHIP_OK;
+        }
+        p->mode = KVHIP_MASK_CAUSAL;
+        return KVHIP_OK;
+    }
+    // RotatingKVCache.makeMask, KVCache.swift:834-871
+    const int64_t M = c->max_size;
+    if (n > 1) {
+        const int64_t actual = has_w ? window : M;
+        const int64_t capped = std::min(M - 1, c->offset);
+        if (capped + n > actual || return_array) {
+            p->mode = KVHIP_MASK_ARRAY;
+            p->rows = n;
+            p->cols = (int32_t)(capped + n);
+            p->offset = (int32_t)capped;
+            p->window = (int32_t)actual;
+            return KVHIP_OK;
+        }
+        p->mode = KVHIP_MASK_CAUSAL;
+        return KVHIP_OK;
+    }
+    if (!has_w) { p->mode = KVHIP_MASK_NONE; return KVHIP_OK; }
+    if (c->offset >= window && M > window) {
+        int64_t cur = c->idx;
+        if (cur >= M) cur = 0;
+        const int64_t size = c->offset < M ? c->offset + 1 : M;
+        p->mode = KVHIP_MASK_ARRAY;
+        p->rows = 1;
+        p->cols = (int32_t)size;
+        p->rolled = 1;
+        p->roll_shift = (int32_t)(cur + 1);
+        p->roll_window = window;
+        return KVHIP_OK;
+    }
+    p->mode = KVHIP_MASK_NONE;
+    return KVHIP_OK;
+}
+
+kvhip_status kvhip_mask_materialize(const kvhip_mask_plan_t *p, uint8_t *dst, void *stream) {
+    if (!p || !dst) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (p->mode != KVHIP_MASK_ARRAY) return fail(KVHIP_ERR_INVALID_ARG, "plan does not describe an array mask");
+    KV_HIP(launch_mask_materialize(*p, dst, S(stream)));
+    return KVHIP_OK;
+}
+
+// ---- state -------------------------------------------------------------------
+int32_t kvhip_cache_state_count(const kvhip_cache *c) {
+    if (!c || !c->has_buffers) return 0;
+    return c->kind == KVHIP_KIND_QUANTIZED ? 6 : 2;
+}
+
+kvhip_status kvhip_cache_state_desc(const kvhip_cache *c, int32_t i, int64_t shape[4], int32_t *dtype) {
+    if (!c || !shape || !dtype) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (i < 0 || i >= kvhip_cache_state_count(c)) return fail(KVHIP_ERR_INVALID_ARG, "state index out of range");
+    const Store &s = c->st;
+    shape[0] = c->B;
+    shape[1] = c->Hkv;
+    shape[2] = state_rows(c);
+    if (c->kind != KVHIP_KIND_QUANTIZED) {
+        shape[3] = i == 0 ? s.Dk : s.Dv;
+        *dtype = s.dtype;
+        return KVHIP_OK;
+    }
+    const int D = i < 3 ? s.Dk : s.Dv;
+    if (i % 3 == 0) {
+        shape[3] = D * s.bits / 32;
+        *dtype = KVHIP_U32;
+    } else {
+        shape[3] = D / s.gs;
+        *dtype = s.dtype;
+    }
+    return KVHIP_OK;
+}
+
+kvhip_status kvhip_cache_state_export(const kvhip_cache *c, int32_t i, void *dst, void *stream) {
+    if (!c || !dst) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (i < 0 || i >= kvhip_cache_state_count(c)) return fail(KVHIP_ERR_INVALID_ARG, "state index out of range");
+    const int64_t n = state_rows(c);
+    if (n == 0) return KVHIP_OK;
+    if (c->kind == KVHIP_KIND_QUANTIZED) {
+        KV_HIP(launch_export_quant(c->st, i, (int)n, dst, S(stream)));
+        return KVHIP_OK;
+    }
+    std::vector<int32_t> ident;
+    const int32_t *slots = c->rows.data();
+    if (c->kind != KVHIP_KIND_ROTATING) {
+        ident.resize((size_t)n);
+        for (size_t r = 0; r < ident.size(); ++r) ident[r] = (int32_t)r;
+        slots = ident.data();
+    }
+    return export_slots(c, slots, n, i == 0 ? dst : nullptr, i == 1 ? dst : nullptr, S(stream));
+}
+
+kvhip_status kvhip_cache_state_import(kvhip_cache *c, int32_t count, const void *const *srcs,
+                                      const int64_t *shapes, const int32_t *dtypes, void *stream) {
+    if (!c || !srcs || !shapes || !dtypes) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    const bool q = c->kind == KVHIP_KIND_QUANTIZED;
+    if (q ? (count != 6) : (count != 2)) {
+        if (q && count == 4) return fail(KVHIP_ERR_UNSUPPORTED, "quantized state without biases (non-affine mode) is not supported");
+        return fail(KVHIP_ERR_STATE, q ? "QuantizedKVCache state must have exactly 6 or 4 arrays"
+                                       : "cache state must have exactly 2 arrays (keys, values)");
+    }
+    const int64_t *k0 = shapes, *v0 = shapes + (q ? 12 : 4);
+    const int64_t B = k0[0], H = k0[1], n = k0[2];
+    for (int a = 0; a < count; ++a)
+        if (shapes[4 * a] != B || shapes[4 * a + 1] != H || shapes[4 * a + 2] != n)
+            return fail(KVHIP_ERR_INVALID_ARG, "state arrays disagree on batch, heads or rows");
+    int Dk, Dv, dtype;
+    if (q) {
+        if (dtypes[0] != KVHIP_U32 || dtypes[3] != KVHIP_U32) return fail(KVHIP_ERR_INVALID_ARG, "packed codes must be uint32");
+        Dk = (int)(k0[3] * 32 / c->bits);
+        Dv = (int)(v0[3] * 32 / c->bits);
+        dtype = dtypes[1];
+        if (shapes[4 * 1 + 3] * c->gs != Dk || shapes[4 * 4 + 3] * c->gs != Dv)
+            return fail(KVHIP_ERR_INVALID_ARG, "scales extent does not match head dim / group size");
+    } else {
+        Dk = (int)k0[3];
+        Dv = (int)v0[3];
+        dtype = dtypes[0];
+    }
+    // a state setter replaces the buffers wholesale
+    free_store(c->st);
+    c->st = Store();
+    c->has_geom = false;
+    c->cap_pages = 0;
+    c->rows.clear();
+    c->used.clear();
+    c->cursor = 0;
+    KV_TRY(set_geometry(c, (int)B, (int)H, Dk, Dv, dtype));
+    hipStream_t s = S(stream);
+    KV_TRY(ensure_slots(c, std::max<int64_t>(n, 1), s, true));
+    if (q) KV_HIP(launch_import_quant(c->st, srcs, (int)n, s));
+    else KV_HIP(launch_import_fp(c->st, srcs[0], srcs[1], (int)n, s));
+    c->has_buffers = true;
+    c->ref_len = n;
+    c->presented = n;
+    if (c->kind == KVHIP_KIND_SIMPLE) c->offset = n;  // KVCache.swift:467
+    if (c->kind == KVHIP_KIND_ROTATING) {
+        c->rows.resize((size_t)n);
+        for (int64_t r = 0; r < n; ++r) {
+            c->rows[(size_t)r] = (int32_t)r;
+            c->used[(size_t)r] = 1;
+        }
+        c->cursor = n;
+    }
+    return KVHIP_OK;
+}
+
+int32_t kvhip_cache_meta_count(const kvhip_cache *c) {
+    if (!c) return 0;
+    return c->kind == KVHIP_KIND_SIMPLE ? 1 : (c->kind == KVHIP_KIND_ROTATING ? 6 : 4);
+}
+
+int32_t kvhip_cache_meta_get(const kvhip_cache *c, int32_t i, char *buf, int32_t len) {
+    if (!c || !buf || len <= 0) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (i < 0 || i >= kvhip_cache_meta_count(c)) return fail(KVHIP_ERR_INVALID_ARG, "meta index out of range");
+    std::string v;
+    if (c->kind == KVHIP_KIND_ROTATING) {
+        const int64_t vals[5] = {c->keep, c->max_size, c->step, c->offset, c->idx};
+        v = i < 5 ? std::to_string(vals[i]) : c->origin;
+    } else if (c->kind == KVHIP_KIND_QUANTIZED) {
+        const int64_t vals[4] = {c->step, c->offset, c->gs, c->bits};
+        v = std::to_string(vals[i]);
+    }
+    if ((int32_t)v.size() + 1 > len) return fail(KVHIP_ERR_INVALID_ARG, "buffer too small");
+    std::memcpy(buf, v.c_str(), v.size() + 1);
+    return (int32_t)v.size();
+}
+
+static bool parse_int(const char *s, int64_t &out) {
+    if (!s || !*s) return false;
+    char *end = nullptr;
+    const long long v = std::strtoll(s, &end, 10);
+    if (*end) return false;
+    out = v;
+    return true;
+}
+
+kvhip_status kvhip_cache_meta_set(kvhip_cache *c, int32_t count, const char *const *values) {
+    if (!c || !values) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (c->kind == KVHIP_KIND_SIMPLE) {
+        if (count != 1 || !values[0] || values[0][0])
+            return fail(KVHIP_ERR_STATE, "This cache has no meta_state but a meta_state was set.");
+        return KVHIP_OK;
+    }
+    if (c->kind == KVHIP_KIND_ROTATING) {
+        // KVCache.swift:782-815
+        if (count != 5 && count != 6) return fail(KVHIP_ERR_STATE, "RotatingKVCache metaState must have 5 or 6 values");
+        int64_t keep, step, off, idx, mx;
+        if (!parse_int(values[0], keep) || !parse_int(values[2], step) || !parse_int(values[3], off) || !parse_int(values[4], idx))
+            return fail(KVHIP_ERR_STATE, "Failed to convert metaState values to integers");
+        if (values[1] && std::strcmp(values[1], "None") == 0)
+            return fail(KVHIP_ERR_STATE, "RotatingKVCache requires a non-nil maxSize. Cannot load cache with maxSize=None.");
+        if (!parse_int(values[1], mx)) return fail(KVHIP_ERR_STATE, "Failed to convert maxCacheSize to integer");
+        std::string origin = "modelNative";
+        if (count == 6) {
+            origin = values[5] ? values[5] : "";
+            if (origin != "modelNative" && origin != "requested")
+                return fail(KVHIP_ERR_STATE, "Invalid RotatingKVCache capacity origin '" + origin + "'");
+        }
+        c->keep = keep;
+        c->max_size = mx;
+        c->step = (int)step;
+        c->offset = off;
+        c->idx = idx;
+        c->origin = origin;
+        return KVHIP_OK;
+    }
+    // KVCache.swift:1148-1166
+    if (count != 4) return fail(KVHIP_ERR_STATE, "QuantizedKVCache metaState must have exactly 4 values");
+    int64_t off, gs, bits;
+    if (!parse_int(values[1], off) || !parse_int(values[2], gs) || !parse_int(values[3], bits))
+        return fail(KVHIP_ERR_STATE, "Failed to convert QuantizedKVCache metaState values to integers");
+    if (c->has_geom && c->cap_pages > 0 && (gs != c->gs || bits != c->bits))
+        return fail(KVHIP_ERR_UNSUPPORTED, "group size / bits differ from the arrays this cache already holds");
+    c->offset = off;
+    c->gs = (int)gs;
+    c->bits = (int)bits;
+    return KVHIP_OK;
+}
+
+// ---- copy / views / conversions -------------------------------------------------
+kvhip_status kvhip_cache_copy(const kvhip_cache *c, void *stream, kvhip_cache **out) {
+    if (!c || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    hipStream_t s = S(stream);
+    kvhip_cache *n = new_cache_like(c);
+    const int64_t rows = state_rows(c);
+    if (c->has_buffers) {
+        // `new.state = self.state`: the copy's buffers hold exactly the exported rows
+        n->has_geom = false;
+        kvhip_status st = set_geometry(n, c->B, c->Hkv, c->st.Dk, c->st.Dv, c->st.dtype);
+        if (st == KVHIP_OK) st = ensure_slots(n, std::max<int64_t>(rows, 1), s, true);
+        if (st != KVHIP_OK) { kvhip_cache_free(n); return st; }
+        if (c->kind == KVHIP_KIND_QUANTIZED) {
+            const int64_t pages = (rows + PAGE - 1) / PAGE;
+            const size_t BH = c->st.BH;
+            const struct { char *d; const char *s; size_t cell; } pl[4] = {
+                {n->st.k, c->st.k, c->st.k_cell}, {n->st.v, c->st.v, c->st.v_cell},
+                {n->st.ksb, c->st.ksb, c->st.ksb_cell}, {n->st.vsb, c->st.vsb, c->st.vsb_cell}};
+            for (auto &p : pl)
+                if (pages) KV_HIP(hipMemcpyAsync(p.d, p.s, (size_t)pages * BH * p.cell, hipMemcpyDeviceToDevice, s));
+        } else {
+            std::vector<int32_t> ident;
+            const int32_t *slots = c->rows.data();
+            if (c->kind != KVHIP_KIND_ROTATING) {
+                ident.resize((size_t)rows);
+                for (size_t r = 0; r < ident.size(); ++r) ident[r] = (int32_t)r;
+                slots = ident.data();
+            }
+            const RunList rl = runs_of(slots, rows);
+            for (size_t first = 0; first < rl.size(); first += MAXRUNS) {
+                const size_t cnt = std::min((size_t)MAXRUNS, rl.size() - first);
+                KV_HIP(launch_compact_fp(c->st, pack_runs(rl, first, cnt), n->st, (int)rows, s));
+            }
+        }
+        n->has_buffers = true;
+        n->ref_len = rows;
+        n->presented = rows;
+        if (c->kind == KVHIP_KIND_ROTATING) {
+            n->rows.resize((size_t)rows);
+            for (int64_t r = 0; r < rows; ++r) {
+                n->rows[(size_t)r] = (int32_t)r;
+                n->used[(size_t)r] = 1;
+            }
+            n->cursor = rows;
+        }
+    }
+    if (c->kind == KVHIP_KIND_SIMPLE) n->offset = c->has_buffers ? rows : 0;  // copy goes through state only
+    else {
+        n->offset = c->offset;
+        n->idx = c->idx;
+        n->origin = c->origin;
+    }
+    *out = n;
+    return KVHIP_OK;
+}
+
+kvhip_status kvhip_cache_logical_view(const kvhip_cache *c, int64_t tail, int64_t *out_rows, void *dk,
+                                      void *dv, void *stream) {
+    if (!c || !out_rows) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (c->kind != KVHIP_KIND_ROTATING) return fail(KVHIP_ERR_INVALID_ARG, "logicalView belongs to RotatingKVCache");
+    if (!c->has_buffers) return fail(KVHIP_ERR_STATE, "logicalView before the first write");
+    // KVCache.swift:631-658
+    std::vector<int32_t> ordered = temporal_order(c);
+    const int64_t available = (int64_t)ordered.size();
+    const int64_t requested = std::min(std::max<int64_t>(tail, 0), available);
+    const int64_t bound = std::max(requested, std::min<int64_t>(c->keep, available));
+    const int64_t trim = available - bound;
+    if (trim > 0) {
+        const int64_t k = std::min<int64_t>(c->keep, available);
+        ordered.erase(ordered.begin() + k, ordered.begin() + k + trim);
+    }
+    *out_rows = (int64_t)ordered.size();
+    if ((dk || dv) && !ordered.empty())
+        return export_slots(c, ordered.data(), (int64_t)ordered.size(), dk, dv, S(stream));
+    return KVHIP_OK;
+}
+
+kvhip_status kvhip_cache_to_quantized(const kvhip_cache *c, int32_t group_size, int32_t bits, void *stream,
+                                      kvhip_cache **out) {
+    if (!c || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (c->kind == KVHIP_KIND_ROTATING)
+        return fail(KVHIP_ERR_STATE,
+                    "RotatingKVCache quantization is not implemented because its temporal ordering requires dedicated handling.");
+    if (c->kind != KVHIP_KIND_SIMPLE) return fail(KVHIP_ERR_INVALID_ARG, "toQuantized belongs to KVCacheSimple");
+    if (group_size <= 0) group_size = 64;
+    if (bits <= 0) bits = 4;
+    hipStream_t s = S(stream);
+    kvhip_config cfg{KVHIP_KIND_QUANTIZED, 0, 0, 0, group_size, bits};
+    if (!c->has_buffers) {
+        KV_TRY(kvhip_cache_create(&cfg, out));
+        (*out)->offset = c->offset;
+        return KVHIP_OK;
+    }
+    const int eff = kvhip_resolved_group_size(group_size, c->st.Dk, c->st.Dv);
+    if (!eff)
+        return fail(KVHIP_ERR_STATE,
+                    "KV cache quantization requires head dimensions divisible by one of the supported group sizes (32, 64, 128).");
+    cfg.group_size = eff;
+    kvhip_cache *n = nullptr;
+    KV_TRY(kvhip_cache_create(&cfg, &n));
+    const int64_t rows = std::max<int64_t>(c->offset, 0);
+    kvhip_status st = set_geometry(n, c->B, c->Hkv, c->st.Dk, c->st.Dv, c->st.dtype);
+    if (st == KVHIP_OK) st = ensure_slots(n, std::max<int64_t>(rows, 1), s, true);
+    if (st != KVHIP_OK) { kvhip_cache_free(n); return st; }
+    if (rows > 0) {
+        void *tk = nullptr, *tv = nullptr;
+        const size_t bk = (size_t)c->st.BH * rows * c->st.Dk * c->st.es, bv = (size_t)c->st.BH * rows * c->st.Dv * c->st.es;
+        KV_HIP(hipMalloc(&tk, bk));
+        KV_HIP(hipMalloc(&tv, bv));
+        KV_HIP(launch_export_fp(c->st, identity_runs(rows), 0, (int)rows, 0, (int)rows, tk, tv, s));
+        KV_HIP(launch_append_quant(n->st, tk, tv, (int)rows, 0, 0, (int)rows, s));
+        KV_HIP(hipStreamSynchronize(s));
+        (void)hipFree(tk);
+        (void)hipFree(tv);
+    }
+    n->has_buffers = true;
+    n->ref_len = rows;  // the state setter keeps the arrays' extent
+    n->presented = rows;
+    n->offset = c->offset;
+    *out = n;
+    return KVHIP_OK;
+}
+
+kvhip_status kvhip_cache_to_unquantized(const kvhip_cache *c, void *stream, kvhip_cache **out) {
+    if (!c || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (c->kind != KVHIP_KIND_QUANTIZED) return fail(KVHIP_ERR_INVALID_ARG, "toUnquantized belongs to QuantizedKVCache");
+    hipStream_t s = S(stream);
+    kvhip_config cfg{KVHIP_KIND_SIMPLE, 0, 0, 0, 0, 0};
+    kvhip_cache *n = nullptr;
+    KV_TRY(kvhip_cache_create(&cfg, &n));
+    n->offset = c->offset;
+    if (!c->has_buffers) { *out = n; return KVHIP_OK; }
+    const int64_t rows = std::max<int64_t>(std::min(c->offset, c->ref_len), 0);
+    const Store &q = c->st;
+    kvhip_status st = set_geometry(n, c->B, c->Hkv, q.Dk, q.Dv, q.dtype);
+    if (st == KVHIP_OK) st = ensure_slots(n, std::max<int64_t>(rows, 1), s, true);
+    if (st != KVHIP_OK) { kvhip_cache_free(n); return st; }
+    if (rows > 0) {
+        const size_t R = (size_t)q.BH * rows;
+        void *buf[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+        const size_t bytes[6] = {R * q.Dk * q.bits / 8, R * (q.Dk / q.gs) * q.es, R * (q.Dk / q.gs) * q.es,
+                                 R * q.Dv * q.bits / 8, R * (q.Dv / q.gs) * q.es, R * (q.Dv / q.gs) * q.es};
+        void *dk = nullptr, *dv = nullptr;
+        for (int i = 0; i < 6; ++i) KV_HIP(hipMalloc(&buf[i], bytes[i]));
+        KV_HIP(hipMalloc(&dk, R * q.Dk * q.es));
+        KV_HIP(hipMalloc(&dv, R * q.Dv * q.es));
+        for (int i = 0; i < 6; ++i) KV_HIP(launch_export_quant(q, i, (int)rows, buf[i], s));
+        KV_HIP(launch_affine_dequantize((const uint32_t *)buf[0], buf[1], buf[2], (int64_t)R, q.Dk, q.gs, q.bits, q.dtype, dk, s));
+        KV_HIP(launch_affine_dequantize((const uint32_t *)buf[3], buf[4], buf[5], (int64_t)R, q.Dv, q.gs, q.bits, q.dtype, dv, s));
+        KV_HIP(launch_import_fp(n->st, dk, dv, (int)rows, s));
+        KV_HIP(hipStreamSynchronize(s));
+        for (int i = 0; i < 6; ++i) (void)hipFree(buf[i]);
+        (void)hipFree(dk);
+        (void)hipFree(dv);
+    }
+    n->has_buffers = true;
+    n->ref_len = rows;
+    n->presented = rows;
+    n->offset = rows;  // `simpleCache.state = ...` sets offset to the arrays' extent
+    *out = n;
+    return KVHIP_OK;
+}
+
+kvhip_status kvhip_affine_quantize(const void *src, int64_t rows, int32_t D, int32_t gs, int32_t bits,
+                                   int32_t dtype, uint32_t *wq, void *scales, void *biases, void *stream) {
+    if (!src || !wq || !scales || !biases) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (bits != 2 && bits != 4 && bits != 8) return fail(KVHIP_ERR_UNSUPPORTED, "bits must be 2, 4 or 8");
+    if ((gs != 32 && gs != 64 && gs != 128) || D % gs) return fail(KVHIP_ERR_INVALID_ARG, "group size must be 32, 64 or 128 and divide D");
+    if (dtype < 0 || dtype > 2) return fail(KVHIP_ERR_INVALID_ARG, "bad dtype");
+    KV_HIP(launch_affine_quantize(src, rows, D, gs, bits, dtype, wq, scales, biases, S(stream)));
+    return KVHIP_OK;
+}
+
+kvhip_status kvhip_affine_dequantize(const uint32_t *wq, const void *scales, const void *biases,
+                                     int64_t rows, int32_t D, int32_t gs, int32_t bits, int32_t dtype,
+                                     void *dst, void *stream) {
+    if (!wq || !scales || !biases || !dst) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (bits != 2 && bits != 4 && bits != 8) return fail(KVHIP_ERR_UNSUPPORTED, "bits must be 2, 4 or 8");
+    if (D % gs) return fail(KVHIP_ERR_INVALID_ARG, "group size must divide D");
+    if (dtype < 0 || dtype > 2) return fail(KVHIP_ERR_INVALID_ARG, "bad dtype");
+    KV_HIP(launch_affine_dequantize(wq, scales, biases, rows, D, gs, bits, dtype, dst, S(stream)));
+    return KVHIP_OK;
+}
+
+}  // extern "C"

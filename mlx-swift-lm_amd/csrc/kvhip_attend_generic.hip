@@ -1,0 +1,173 @@
+// Generic attention over the page layout: one workgroup per query row, any
+// dtype / bit width / head dim / mask.  It is the fallback for shapes the
+// matrix-core kernels do not cover and the in-library cross-check for them.
+//
+// Quantized caches follow the reference's unfused sequence
+// (KVCache.swift:2351-2447): q' = T(q*scale), scores = T(q' . K^), mask with
+// finfo(T).min fill (or T(scores + mask)), p = T(softmax), out = T(p . V^).
+// Full-precision caches follow the fused op (AttentionUtils.swift:86-93):
+// float32 inside, excluded keys contribute nothing, one rounding at the output.
+#include "kvhip_mask.hpp"
+
+namespace kvhip {
+
+namespace {
+
+constexpr int GT = 256;  // threads per workgroup
+
+__device__ __forceinline__ float block_reduce(float v, bool is_max, float *red) {
+    for (int off = 32; off > 0; off >>= 1) {
+        const float o = __shfl_xor(v, off);
+        v = is_max ? fmaxf(v, o) : v + o;
+    }
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float r = red[0];
+    for (int w = 1; w < GT / 64; ++w) r = is_max ? fmaxf(r, red[w]) : r + red[w];
+    return r;
+}
+
+template <int BITS> __device__ __forceinline__ uint32_t v_code(const char *cell, int unit, int e) {
+    if (BITS == 4) return (reinterpret_cast<const uint32_t *>(cell)[unit] >> (4 * e)) & 15u;
+    if (BITS == 8) return reinterpret_cast<const uint8_t *>(cell)[(size_t)unit * 8 + e];
+    return (reinterpret_cast<const uint16_t *>(cell)[unit] >> (2 * e)) & 3u;
+}
+
+// grid (L, Hq, B)
+template <int DT, int BITS>
+__global__ void __launch_bounds__(GT)
+attend_generic_kernel(AttendArgs a, int slots_pad) {
+    extern __shared__ float smem[];  // q' [Dk] | red [4]
+    float *qs = smem;
+    float *red = smem + a.st.Dk;
+    const Store &st = a.st;
+    const int l = blockIdx.x, hq = blockIdx.y, b = blockIdx.z;
+    const int r = a.Hq / a.Hkv;
+    const int bh = b * a.Hkv + hq / r;
+    const size_t qrow = ((size_t)(b * a.Hq + hq) * a.L + l);
+    float *p = a.workspace + qrow * slots_pad;
+    constexpr bool Q = BITS != 0;
+    constexpr int BB = Q ? BITS : 4;
+    const float fill = finfo_min_dt(DT);
+
+    for (int d = threadIdx.x; d < st.Dk; d += GT) {
+        const float qv = Elem<DT>::load(a.q, qrow * st.Dk + d) * a.scale;
+        qs[d] = Q ? round_dt<DT>(qv) : qv;
+    }
+    __syncthreads();
+
+    // ---- scores -------------------------------------------------------------
+    float mx = -INFINITY;
+    for (int slot = threadIdx.x; slot < slots_pad; slot += GT) {
+        const int row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
+        float s = -INFINITY;
+        if (row >= 0 && row < a.T) {
+            float sum = 0.f;
+            if (Q) {
+                constexpr int per = 32 / BB;
+                const uint32_t *w = reinterpret_cast<const uint32_t *>(k_row_ptr(st, bh, slot));
+                const char *sb = ksb_row_ptr(st, bh, slot);
+                for (int g = 0; g < st.Dk / st.gs; ++g) {
+                    const float sc = Elem<DT>::load(sb, 2 * g), bi = Elem<DT>::load(sb, 2 * g + 1);
+                    for (int jj = 0; jj < st.gs; ++jj) {
+                        const int d = g * st.gs + jj;
+                        const uint32_t c = (w[d / per] >> ((d % per) * BB)) & ((1u << BB) - 1u);
+                        sum += qs[d] * (sc * (float)c + bi);
+                    }
+                }
+                s = round_dt<DT>(sum);
+            } else {
+                const char *krow = k_row_ptr(st, bh, slot);
+                for (int d = 0; d < st.Dk; ++d) sum += qs[d] * Elem<DT>::load(krow, d);
+                s = sum;
+            }
+            float add;
+            const bool keep = mask_keep(a.mask, b, hq, l, row, a.L, a.T, add);
+            if (Q) {
+                if (!keep) s = fill;
+                else if (a.mask.mode == KVHIP_MASK_ARRAY && a.mask.dtype != KVHIP_BOOL) s = round_dt<DT>(s + add);
+            } else {
+                s = keep ? s + add : -INFINITY;
+            }
+        }
+        p[slot] = s;
+        mx = fmaxf(mx, s);
+    }
+    mx = block_reduce(mx, true, red);
+
+    // ---- softmax ------------------------------------------------------------
+    float den = 0.f;
+    for (int slot = threadIdx.x; slot < slots_pad; slot += GT) {
+        const float s = p[slot];
+        const float e = (s == -INFINITY) ? 0.f : expf(s - mx);
+        p[slot] = e;
+        den += e;
+    }
+    den = block_reduce(den, false, red);
+    const float inv = den > 0.f ? 1.0f / den : 0.f;
+    for (int slot = threadIdx.x; slot < slots_pad; slot += GT) {
+        const float w = Q ? round_dt<DT>(__fdiv_rn(p[slot], den > 0.f ? den : 1.f)) : p[slot] * inv;
+        p[slot] = w;
+    }
+    __syncthreads();
+
+    // ---- out = p . V^ ---------------------------------------------------------
+    for (int d = threadIdx.x; d < st.Dv; d += GT) {
+        float acc = 0.f;
+        for (int blk = 0; blk * 32 < slots_pad; ++blk) {
+            const char *cell = v_cell_ptr(st, bh, blk * 32);
+            const int bip = ((blk * 32) & (PAGE - 1)) >> 5;
+            for (int j = 0; j < 4; ++j) {
+                const int unit = (bip * 4 + j) * st.Dv + d;
+                for (int e = 0; e < 8; ++e) {
+                    const int slot = blk * 32 + 4 * j + (e & 3) + 16 * (e >> 2);
+                    const float w = p[slot];
+                    if (w == 0.f) continue;
+                    float v;
+                    if (Q) {
+                        const char *sb = vsb_row_ptr(st, bh, slot);
+                        const int g = d / st.gs;
+                        v = Elem<DT>::load(sb, 2 * g) * (float)v_code<BB>(cell, unit, e) + Elem<DT>::load(sb, 2 * g + 1);
+                    } else {
+                        v = Elem<DT>::load(cell, (size_t)unit * 8 + e);
+                    }
+                    acc += w * v;
+                }
+            }
+        }
+        Elem<DT>::store(a.out, qrow * st.Dv + d, acc);
+    }
+}
+
+}  // namespace
+
+static int pad32(int n) { return (n + 31) & ~31; }
+
+size_t attend_generic_workspace(const AttendArgs &a) {
+    return (size_t)a.B * a.Hq * a.L * pad32(a.slots) * sizeof(float);
+}
+
+hipError_t launch_attend_generic(const AttendArgs &a, hipStream_t s) {
+    dim3 grid(a.L, a.Hq, a.B), block(GT);
+    const size_t lds = (a.st.Dk + 8) * sizeof(float);
+    const int sp = pad32(a.slots);
+#define GEN(DT, BITS) hipLaunchKernelGGL((attend_generic_kernel<DT, BITS>), grid, block, lds, s, a, sp)
+#define GEN_DT(BITS)                                        \
+    do {                                                    \
+        if (a.st.dtype == 0) GEN(0, BITS);                  \
+        else if (a.st.dtype == 1) GEN(1, BITS);             \
+        else GEN(2, BITS);                                  \
+    } while (0)
+    switch (a.st.bits) {
+        case 0: GEN_DT(0); break;
+        case 2: GEN_DT(2); break;
+        case 4: GEN_DT(4); break;
+        default: GEN_DT(8); break;
+    }
+#undef GEN_DT
+#undef GEN
+    return hipGetLastError();
+}
+
+}  // namespace kvhip

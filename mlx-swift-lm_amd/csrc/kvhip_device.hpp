@@ -1,0 +1,96 @@
+// Device-side element conversion and the affine quantizer core shared by the
+// append, import/export and standalone quantize kernels.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include "kvhip_internal.hpp"
+
+namespace kvhip {
+
+// DT: 0 float16, 1 bfloat16, 2 float32 (kvhip_dtype)
+template <int DT> struct Elem;
+template <> struct Elem<0> {
+    using type = uint16_t;
+    static __device__ __forceinline__ float load(const void *p, size_t i) {
+        return __half2float(reinterpret_cast<const __half *>(p)[i]);
+    }
+    static __device__ __forceinline__ void store(void *p, size_t i, float v) {
+        reinterpret_cast<__half *>(p)[i] = __float2half_rn(v);
+    }
+};
+template <> struct Elem<1> {
+    using type = uint16_t;
+    static __device__ __forceinline__ float load(const void *p, size_t i) {
+        return __uint_as_float((uint32_t) reinterpret_cast<const uint16_t *>(p)[i] << 16);
+    }
+    static __device__ __forceinline__ uint16_t bits(float v) {
+        uint32_t x = __float_as_uint(v);
+        if ((x & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
+        return (uint16_t)((x + (((x >> 16) & 1u) + 0x7fffu)) >> 16);
+    }
+    static __device__ __forceinline__ void store(void *p, size_t i, float v) {
+        reinterpret_cast<uint16_t *>(p)[i] = bits(v);
+    }
+};
+template <> struct Elem<2> {
+    using type = float;
+    static __device__ __forceinline__ float load(const void *p, size_t i) {
+        return reinterpret_cast<const float *>(p)[i];
+    }
+    static __device__ __forceinline__ void store(void *p, size_t i, float v) {
+        reinterpret_cast<float *>(p)[i] = v;
+    }
+};
+
+// Round a float to dtype DT and back (the value an array of that dtype holds).
+template <int DT> __device__ __forceinline__ float round_dt(float v) {
+    if (DT == 0) return __half2float(__float2half_rn(v));
+    if (DT == 1) return __uint_as_float((uint32_t)Elem<1>::bits(v) << 16);
+    return v;
+}
+
+__device__ __forceinline__ float finfo_min_dt(int dt) {
+    return dt == 0 ? -65504.0f : (dt == 1 ? -3.3895313892515355e38f : -3.4028234663852886e38f);
+}
+
+// Affine parameters of one group from its extrema, in float32, step for step as
+// MLX's CPU quantizer computes them (call sites KVCache.swift:1069-1070).
+__device__ __forceinline__ void affine_params(float w_min, float w_max, float n_bins, float &scale,
+                                              float &bias) {
+    const float eps = 1e-7f;
+    const bool mask = fabsf(w_min) > fabsf(w_max);
+    float s = fmaxf(__fdiv_rn(__fsub_rn(w_max, w_min), n_bins), eps);
+    s = mask ? s : -s;
+    const float edge = mask ? w_min : w_max;
+    const float q0 = rintf(__fdiv_rn(edge, s));
+    bias = 0.0f;
+    if (q0 != 0.0f) {
+        s = __fdiv_rn(edge, q0);
+        bias = edge;
+    }
+    scale = s;
+}
+
+__device__ __forceinline__ uint32_t affine_code(float w, float scale, float bias, float n_bins) {
+    float q = rintf(__fdiv_rn(__fsub_rn(w, bias), scale));
+    q = fminf(fmaxf(q, 0.0f), n_bins);
+    return (uint32_t)q;
+}
+
+// Min/max over a group of `width` (<= 64, power of two) adjacent lanes.
+__device__ __forceinline__ void group_minmax(float &mn, float &mx, int width) {
+    for (int off = 1; off < width; off <<= 1) {
+        mn = fminf(mn, __shfl_xor(mn, off));
+        mx = fmaxf(mx, __shfl_xor(mx, off));
+    }
+}
+
+// OR-combine `v` across `width` adjacent lanes (power of two).
+__device__ __forceinline__ uint32_t group_or(uint32_t v, int width) {
+    for (int off = 1; off < width; off <<= 1) v |= __shfl_xor(v, off);
+    return v;
+}
+
+}  // namespace kvhip

@@ -1,0 +1,167 @@
+// Shared definitions of libkvhip: the device-resident page layout, the
+// row-to-slot run table kernels receive, and the kernel launcher prototypes.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kvhip.h"
+
+namespace kvhip {
+
+// ---------------------------------------------------------------------------
+// Page layout
+//
+// Cached rows live in fixed pages of PAGE tokens.  A plane (K data, V data and,
+// for quantized caches, K and V scale/bias pairs) is one allocation laid out
+// page-major: [page][b*Hkv + h][PAGE rows].  Growing a cache appends pages;
+// nothing already written moves relative to its page.
+//
+//  K plane   rows in natural order: row s of a page holds Dk elements (fp) or
+//            Dk*bits/32 packed uint32 words in MLX's order (quantized).
+//  V plane   "octet transposed" so that the PV contraction can feed matrix-core
+//            operands without shuffles.  A page is 8 blocks of 32 tokens.  In a
+//            block, token tl (0..31) belongs to octet j = (tl & 15) >> 2 at
+//            position e = (tl & 3) + 4 * (tl >> 4); for every (block, j, d) the
+//            8 values of the octet are contiguous:
+//              fp        8 elements                     (16 B for 16-bit types)
+//              quantized 8 codes of `bits` bits, LSB first (one uint32 at 4 bits)
+//            unit index inside a page = (block * 4 + j) * Dv + d.
+//  sb planes per row and group one (scale, bias) pair of the cache dtype.
+// ---------------------------------------------------------------------------
+constexpr int PAGE = 256;
+constexpr int PAGE_SHIFT = 8;
+constexpr int MAXRUNS = 8;
+
+struct Store {
+    char *k = nullptr;    // K plane
+    char *v = nullptr;    // V plane
+    char *ksb = nullptr;  // K (scale,bias) plane, quantized only
+    char *vsb = nullptr;  // V (scale,bias) plane, quantized only
+    int32_t BH = 0;       // B * Hkv
+    int32_t Dk = 0, Dv = 0;
+    int32_t dtype = 0;    // kvhip_dtype of cached values / of scales and biases
+    int32_t es = 2;       // bytes per element of dtype
+    int32_t bits = 0;     // 0: full precision
+    int32_t gs = 0;
+    // bytes one (page, bh) cell occupies in each plane
+    uint32_t k_cell = 0, v_cell = 0, ksb_cell = 0, vsb_cell = 0;
+    uint32_t k_row = 0;   // bytes per K row
+    uint32_t ksb_row = 0, vsb_row = 0;
+};
+
+// Contiguous pieces of the presented order: rows [row0, row0+len) live in
+// physical slots [phys0, phys0+len).
+struct Runs {
+    int32_t n = 0;
+    int32_t row0[MAXRUNS];
+    int32_t phys0[MAXRUNS];
+    int32_t len[MAXRUNS];
+};
+
+struct MaskDev {
+    int32_t mode = 0;   // kvhip_mask_mode
+    int32_t dtype = 0;
+    const void *data = nullptr;
+    int64_t sb = 0, sh = 0, sl = 0;
+    int32_t offset = 0, window = 0;
+    const int32_t *lengths = nullptr;
+    const int32_t *left_pad = nullptr;
+};
+
+#if defined(__HIPCC__)
+// ---- device-side address helpers -------------------------------------------
+__device__ __forceinline__ const char *k_row_ptr(const Store &st, int bh, int slot) {
+    return st.k + ((size_t)(slot >> PAGE_SHIFT) * st.BH + bh) * st.k_cell + (size_t)(slot & (PAGE - 1)) * st.k_row;
+}
+__device__ __forceinline__ const char *ksb_row_ptr(const Store &st, int bh, int slot) {
+    return st.ksb + ((size_t)(slot >> PAGE_SHIFT) * st.BH + bh) * st.ksb_cell + (size_t)(slot & (PAGE - 1)) * st.ksb_row;
+}
+__device__ __forceinline__ const char *vsb_row_ptr(const Store &st, int bh, int slot) {
+    return st.vsb + ((size_t)(slot >> PAGE_SHIFT) * st.BH + bh) * st.vsb_cell + (size_t)(slot & (PAGE - 1)) * st.vsb_row;
+}
+__device__ __forceinline__ const char *v_cell_ptr(const Store &st, int bh, int slot) {
+    return st.v + ((size_t)(slot >> PAGE_SHIFT) * st.BH + bh) * st.v_cell;
+}
+// octet coordinates of a slot inside its page
+__device__ __forceinline__ int v_unit_base(int slot, int Dv) {  // (block*4 + j) * Dv
+    const int s = slot & (PAGE - 1);
+    const int tl = s & 31;
+    return (((s >> 5) << 2) + ((tl & 15) >> 2)) * Dv;
+}
+__device__ __forceinline__ int v_pos(int slot) {
+    const int tl = slot & 31;
+    return (tl & 3) + ((tl >> 4) << 2);
+}
+// presented row of a physical slot, or -1
+__device__ __forceinline__ int slot_to_row(const Runs &r, int slot) {
+    int row = -1;
+#pragma unroll
+    for (int i = 0; i < MAXRUNS; ++i) {
+        if (i < r.n) {
+            const int d = slot - r.phys0[i];
+            if (d >= 0 && d < r.len[i]) row = r.row0[i] + d;
+        }
+    }
+    return row;
+}
+__device__ __forceinline__ int row_to_slot(const Runs &r, int row) {
+    int slot = -1;
+#pragma unroll
+    for (int i = 0; i < MAXRUNS; ++i) {
+        if (i < r.n) {
+            const int d = row - r.row0[i];
+            if (d >= 0 && d < r.len[i]) slot = r.phys0[i] + d;
+        }
+    }
+    return slot;
+}
+#endif
+
+// ---- kernel launchers (defined in the .hip files) ---------------------------
+// New rows src[l] for l in [src0, src0+n) go to physical slots [slot0, slot0+n).
+hipError_t launch_append_fp(const Store &st, const void *keys, const void *values, int L, int src0,
+                            int slot0, int n, hipStream_t s);
+hipError_t launch_append_quant(const Store &st, const void *keys, const void *values, int L, int src0,
+                               int slot0, int n, hipStream_t s);
+// Copy rows [row_begin, row_begin+count) of `runs` out to dense [BH, dst_rows, D] arrays whose
+// row 0 corresponds to row dst_row0 of `runs`.  Either destination may be NULL.
+hipError_t launch_export_fp(const Store &st, const Runs &runs, int row_begin, int count, int dst_row0,
+                            int dst_rows, void *dst_k, void *dst_v, hipStream_t s);
+// which: 0 k.wq 1 k.scales 2 k.biases 3 v.wq 4 v.scales 5 v.biases
+hipError_t launch_export_quant(const Store &st, int which, int nrows, void *dst, hipStream_t s);
+// Dense [BH, nrows, D] arrays into slots [0, nrows).
+hipError_t launch_import_fp(const Store &st, const void *src_k, const void *src_v, int nrows, hipStream_t s);
+hipError_t launch_import_quant(const Store &st, const void *const srcs[6], int nrows, hipStream_t s);
+// Device-to-device copy of slots between two stores of identical geometry, through a row map:
+// dst slot i <- src slot of presented row i.
+hipError_t launch_compact_fp(const Store &src, const Runs &runs, const Store &dst, int nrows, hipStream_t s);
+hipError_t launch_affine_quantize(const void *src, int64_t rows, int D, int gs, int bits, int dtype,
+                                  uint32_t *wq, void *scales, void *biases, hipStream_t s);
+hipError_t launch_affine_dequantize(const uint32_t *wq, const void *scales, const void *biases,
+                                    int64_t rows, int D, int gs, int bits, int dtype, void *dst,
+                                    hipStream_t s);
+hipError_t launch_mask_materialize(const kvhip_mask_plan_t &plan, uint8_t *dst, hipStream_t s);
+
+struct AttendArgs {
+    Store st;
+    Runs runs;
+    const void *q = nullptr;  // [B, Hq, L, Dk]
+    void *out = nullptr;      // [B, Hq, L, Dv]
+    int32_t B = 0, Hq = 0, Hkv = 0, L = 0;
+    int32_t T = 0;            // presented length
+    int32_t slots = 0;        // physical slots in use span [0, slots)
+    float scale = 1.f;
+    MaskDev mask;
+    float *workspace = nullptr;
+    size_t workspace_bytes = 0;
+};
+// Bytes of scratch each kernel family needs for these arguments.
+size_t attend_generic_workspace(const AttendArgs &a);
+hipError_t launch_attend_generic(const AttendArgs &a, hipStream_t s);
+// Fast split-sequence decode kernels; `supported` says whether the shape is covered.
+bool attend_decode_supported(const AttendArgs &a);
+size_t attend_decode_workspace(const AttendArgs &a);
+hipError_t launch_attend_decode(const AttendArgs &a, hipStream_t s);
+
+}  // namespace kvhip

@@ -1,0 +1,36 @@
+// Mask evaluation shared by the attention kernels.
+#pragma once
+#include "kvhip_device.hpp"
+
+namespace kvhip {
+
+// Decides whether query row l (of L) of batch b / query head hq may see presented
+// key row j (of T).  `add` receives the additive term of a float array mask.
+__device__ __forceinline__ bool mask_keep(const MaskDev &m, int b, int hq, int l, int j, int L, int T,
+                                          float &add) {
+    add = 0.0f;
+    switch (m.mode) {
+        case KVHIP_MASK_CAUSAL:
+            return j <= T - L + l;
+        case KVHIP_MASK_ARRAY: {
+            const size_t i = (size_t)(b * m.sb + hq * m.sh + l * m.sl) + j;
+            if (m.dtype == KVHIP_BOOL) return reinterpret_cast<const uint8_t *>(m.data)[i] != 0;
+            if (m.dtype == KVHIP_F16) add = Elem<0>::load(m.data, i);
+            else if (m.dtype == KVHIP_BF16) add = Elem<1>::load(m.data, i);
+            else add = Elem<2>::load(m.data, i);
+            return true;
+        }
+        case KVHIP_MASK_WINDOW: {
+            const int li = m.offset + l;
+            bool keep = li >= j;
+            if (m.window > 0) keep = keep && (li < j + m.window);
+            if (m.lengths) keep = keep && (j < m.lengths[b]);
+            if (m.left_pad) keep = keep && (j >= m.left_pad[b]);
+            return keep;
+        }
+        default:
+            return true;
+    }
+}
+
+}  // namespace kvhip

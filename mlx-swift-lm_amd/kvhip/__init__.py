@@ -1,0 +1,5 @@
+"""kvhip: MI355X (gfx950) KV-cache hot path behind the reference's KVCache surface."""
+from ._lib import KVHipError, LIB_PATH, SIGNATURES, load  # noqa: F401
+from .attention import attention_with_cache_update, quantized_scaled_dot_product_attention  # noqa: F401
+from .cache import (KVCacheSimple, MaskMode, QuantizedKVCache, RotatingKVCache, affine_dequantize,  # noqa: F401
+                    affine_quantize, resolved_kv_quantization_group_size, trim_prompt_cache)

@@ -1,0 +1,383 @@
+"""Host-side mirror of the reference's cache classes over libkvhip.
+
+Class and member names follow Libraries/MLXLMCommon/KVCache.swift
+(`KVCacheSimple` :391, `RotatingKVCache` :541, `QuantizedKVCache` :923); the
+arrays are torch tensors on the GPU, used only as device memory.  Every method
+is a thin call into the C ABI: the cached rows never leave the device unless a
+caller asks for `state`, `fetch()` or `logical_view()`.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+
+from . import _lib as L
+
+_DT = {torch.float16: L.F16, torch.bfloat16: L.BF16, torch.float32: L.F32}
+_TORCH = {L.F16: torch.float16, L.BF16: torch.bfloat16, L.F32: torch.float32, L.U32: torch.int32,
+          L.BOOL: torch.bool}
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr())
+
+
+class MaskMode:
+    """`MLXFast.ScaledDotProductAttentionMaskMode`: .none / .causal / .array(mask),
+    plus .window -- createCausalMask evaluated from indices inside the kernel."""
+
+    def __init__(self, mode, array=None, offset=0, window=0, lengths=None, left_pad=None):
+        self.mode, self.array = mode, array
+        self.offset, self.window, self.lengths, self.left_pad = offset, window, lengths, left_pad
+
+    @staticmethod
+    def none():
+        return MaskMode(L.MASK_NONE)
+
+    @staticmethod
+    def causal():
+        return MaskMode(L.MASK_CAUSAL)
+
+    @staticmethod
+    def from_array(a):
+        return MaskMode(L.MASK_ARRAY, array=a)
+
+    @staticmethod
+    def window_mask(offset, window=0, lengths=None, left_pad=None):
+        return MaskMode(L.MASK_WINDOW, offset=offset, window=window, lengths=lengths, left_pad=left_pad)
+
+    def to_c(self, B, Hq, Lq):
+        m = L.Mask()
+        m.mode = self.mode
+        keep = []
+        if self.mode == L.MASK_ARRAY:
+            a = self.array
+            if a.dtype == torch.bool:
+                a8 = a.to(torch.uint8).contiguous()
+                m.dtype = L.BOOL
+            else:
+                a8 = a.contiguous()
+                m.dtype = _DT[a.dtype]
+            while a8.dim() < 4:
+                a8 = a8.unsqueeze(0)
+            assert a8.shape[2] == Lq, "mask query extent"
+            assert a8.shape[0] in (1, B) and a8.shape[1] in (1, Hq)
+            st = a8.stride()
+            m.stride_b = 0 if a8.shape[0] == 1 else st[0]
+            m.stride_h = 0 if a8.shape[1] == 1 else st[1]
+            m.stride_l = st[2]
+            m.key_len = a8.shape[3]
+            m.data = a8.data_ptr()
+            keep.append(a8)
+        elif self.mode == L.MASK_WINDOW:
+            m.offset, m.window = int(self.offset), int(self.window or 0)
+            for name in ("lengths", "left_pad"):
+                t = getattr(self, name)
+                if t is not None:
+                    t = t.to(device="cuda", dtype=torch.int32).contiguous()
+                    setattr(m, name, t.data_ptr())
+                    keep.append(t)
+        return m, keep
+
+
+class _Cache:
+    kind = None
+
+    def __init__(self, handle=None, **cfg):
+        L.init()
+        self._lib = L.load()
+        if handle is None:
+            c = L.Config(kind=self.kind, step=cfg.get("step", 0), max_size=cfg.get("max_size", 0),
+                         keep=cfg.get("keep", 0), group_size=cfg.get("group_size", 0), bits=cfg.get("bits", 0))
+            h = C.c_void_p()
+            L.check(self._lib.kvhip_cache_create(C.byref(c), C.byref(h)))
+            handle = h
+        self._h = handle
+        self._shape = None  # (B, Hkv, Dk, Dv, torch dtype) once known
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self._lib.kvhip_cache_free(h)
+
+    # ---- protocol surface -------------------------------------------------
+    @property
+    def offset(self):
+        return self._lib.kvhip_cache_offset(self._h)
+
+    @offset.setter
+    def offset(self, v):
+        L.check(self._lib.kvhip_cache_set_offset(self._h, int(v)))
+
+    @property
+    def max_size(self):
+        v = self._lib.kvhip_cache_max_size(self._h)
+        return None if v < 0 else v
+
+    @property
+    def capacity(self):
+        return self._lib.kvhip_cache_capacity(self._h)
+
+    @property
+    def presented_length(self):
+        return self._lib.kvhip_cache_presented_length(self._h)
+
+    @property
+    def is_trimmable(self):
+        return bool(self._lib.kvhip_cache_is_trimmable(self._h, 0))
+
+    def is_trimmable_after(self, positions):
+        return bool(self._lib.kvhip_cache_is_trimmable(self._h, int(positions)))
+
+    def trim(self, n):
+        return self._lib.kvhip_cache_trim(self._h, int(n))
+
+    def reserve(self, B, Hkv, Dk, Dv, dtype, tokens):
+        L.check(self._lib.kvhip_cache_reserve(self._h, B, Hkv, Dk, Dv, _DT[dtype], int(tokens)))
+
+    def _note_shape(self, keys, values):
+        B, H, _, Dk = keys.shape
+        self._shape = (B, H, Dk, values.shape[3], keys.dtype)
+
+    def _update(self, keys, values):
+        assert keys.is_cuda and values.is_cuda and keys.dtype == values.dtype
+        keys, values = keys.contiguous(), values.contiguous()
+        B, H, Lq, Dk = keys.shape
+        L.check(self._lib.kvhip_cache_update(self._h, _ptr(keys), _ptr(values), B, H, Lq, Dk,
+                                             values.shape[3], _DT[keys.dtype], _stream()))
+        self._note_shape(keys, values)
+
+    def attend(self, queries, scale, mask=None):
+        """Attention of `queries` [B,Hq,L,D] over what the cache presents."""
+        q = queries.contiguous()
+        B, Hq, Lq, D = q.shape
+        Dv = self._shape[3]
+        out = torch.empty((B, Hq, Lq, Dv), dtype=q.dtype, device=q.device)
+        mask = mask or MaskMode.none()
+        m, keep = mask.to_c(B, Hq, Lq)
+        L.check(self._lib.kvhip_cache_attend(self._h, _ptr(q), B, Hq, Lq, D, float(scale), C.byref(m),
+                                             _ptr(out), _stream()))
+        del keep
+        return out
+
+    def update_attend(self, queries, keys, values, scale, mask=None):
+        """`attentionWithCacheUpdate` for this cache (AttentionUtils.swift:37-95)."""
+        q, k, v = queries.contiguous(), keys.contiguous(), values.contiguous()
+        B, Hq, Lq, D = q.shape
+        H = k.shape[1]
+        out = torch.empty((B, Hq, Lq, v.shape[3]), dtype=q.dtype, device=q.device)
+        mask = mask or MaskMode.none()
+        m, keep = mask.to_c(B, Hq, Lq)
+        L.check(self._lib.kvhip_cache_update_attend(self._h, _ptr(q), _ptr(k), _ptr(v), B, Hq, H, Lq, D,
+                                                    v.shape[3], _DT[k.dtype], float(scale), C.byref(m),
+                                                    _ptr(out), _stream()))
+        self._note_shape(k, v)
+        del keep
+        return out
+
+    def make_mask(self, n, window_size=None, return_array=False):
+        """`makeMask(n:windowSize:returnArray:)`; array masks are built on the device."""
+        p = L.MaskPlan()
+        L.check(self._lib.kvhip_cache_mask_plan(self._h, int(n), int(window_size or 0), int(return_array), C.byref(p)))
+        if p.mode == L.MASK_NONE:
+            return MaskMode.none()
+        if p.mode == L.MASK_CAUSAL:
+            return MaskMode.causal()
+        shape = (p.cols,) if p.rolled else (p.rows, p.cols)
+        buf = torch.empty(shape, dtype=torch.uint8, device="cuda")
+        L.check(self._lib.kvhip_mask_materialize(C.byref(p), _ptr(buf), _stream()))
+        return MaskMode.from_array(buf.bool())
+
+    # ---- state / metaState ---------------------------------------------------
+    @property
+    def state(self):
+        n = self._lib.kvhip_cache_state_count(self._h)
+        out = []
+        for i in range(n):
+            shape = (C.c_int64 * 4)()
+            dt = C.c_int32()
+            L.check(self._lib.kvhip_cache_state_desc(self._h, i, C.byref(shape), C.byref(dt)))
+            t = torch.empty(tuple(shape), dtype=_TORCH[dt.value], device="cuda")
+            L.check(self._lib.kvhip_cache_state_export(self._h, i, _ptr(t), _stream()))
+            out.append(t)
+        return out
+
+    @state.setter
+    def state(self, arrays):
+        arrays = [a.contiguous() for a in arrays]
+        n = len(arrays)
+        ptrs = (C.c_void_p * max(n, 1))(*[a.data_ptr() for a in arrays])
+        shapes = (C.c_int64 * (4 * max(n, 1)))(*[d for a in arrays for d in a.shape])
+        dts = (C.c_int32 * max(n, 1))(*[L.U32 if a.dtype in (torch.int32, torch.uint32) else _DT[a.dtype] for a in arrays])
+        L.check(self._lib.kvhip_cache_state_import(self._h, n, ptrs, shapes, dts, _stream()))
+        torch.cuda.current_stream().synchronize()
+        if self.kind == L.KIND_QUANTIZED:
+            per = 32 // self.bits
+            self._shape = (arrays[0].shape[0], arrays[0].shape[1], arrays[0].shape[3] * per,
+                           arrays[3].shape[3] * per, arrays[1].dtype)
+        else:
+            self._shape = (arrays[0].shape[0], arrays[0].shape[1], arrays[0].shape[3], arrays[1].shape[3],
+                           arrays[0].dtype)
+
+    @property
+    def meta_state(self):
+        out = []
+        buf = C.create_string_buffer(64)
+        for i in range(self._lib.kvhip_cache_meta_count(self._h)):
+            L.check(self._lib.kvhip_cache_meta_get(self._h, i, buf, 64))
+            out.append(buf.value.decode())
+        return out
+
+    @meta_state.setter
+    def meta_state(self, values):
+        arr = (C.c_char_p * len(values))(*[v.encode() for v in values])
+        L.check(self._lib.kvhip_cache_meta_set(self._h, len(values), arr))
+
+    def copy(self):
+        h = C.c_void_p()
+        L.check(self._lib.kvhip_cache_copy(self._h, _stream(), C.byref(h)))
+        new = type(self).__new__(type(self))
+        _Cache.__init__(new, handle=h)
+        new._shape = self._shape
+        return new
+
+
+class KVCacheSimple(_Cache):
+    """`KVCacheSimple` (KVCache.swift:391-538)."""
+    kind = L.KIND_SIMPLE
+
+    def __init__(self, step=256, handle=None):
+        super().__init__(handle=handle, step=step)
+
+    def update(self, keys, values, fetch=True):
+        """`update(keys:values:)`: returns all cached keys/values (copied out of the
+        page layout when `fetch` is true; attention does not need that copy)."""
+        self._update(keys, values)
+        return self.fetch() if fetch else None
+
+    def fetch(self):
+        B, H, Dk, Dv, dt = self._shape
+        n = self.presented_length
+        k = torch.empty((B, H, n, Dk), dtype=dt, device="cuda")
+        v = torch.empty((B, H, n, Dv), dtype=dt, device="cuda")
+        L.check(self._lib.kvhip_cache_fetch(self._h, _ptr(k), _ptr(v), _stream()))
+        return k, v
+
+    def to_quantized(self, group_size=64, bits=4):
+        h = C.c_void_p()
+        L.check(self._lib.kvhip_cache_to_quantized(self._h, group_size, bits, _stream(), C.byref(h)))
+        q = QuantizedKVCache.__new__(QuantizedKVCache)
+        _Cache.__init__(q, handle=h)
+        q._shape = self._shape
+        return q
+
+
+class RotatingKVCache(KVCacheSimple):
+    """`RotatingKVCache` (KVCache.swift:541-900)."""
+    kind = L.KIND_ROTATING
+
+    def __init__(self, max_size, keep=0, step=256, handle=None):
+        _Cache.__init__(self, handle=handle, max_size=max_size, keep=keep, step=step)
+
+    @property
+    def idx(self):
+        return self._lib.kvhip_cache_idx(self._h)
+
+    def logical_view(self, tail):
+        """`logicalView(tail:)` (KVCache.swift:631-658); None before the first write."""
+        if self._shape is None:
+            return None
+        n = C.c_int64()
+        L.check(self._lib.kvhip_cache_logical_view(self._h, int(tail), C.byref(n), None, None, _stream()))
+        B, H, Dk, Dv, dt = self._shape
+        k = torch.empty((B, H, n.value, Dk), dtype=dt, device="cuda")
+        v = torch.empty((B, H, n.value, Dv), dtype=dt, device="cuda")
+        if n.value:
+            L.check(self._lib.kvhip_cache_logical_view(self._h, int(tail), C.byref(n), _ptr(k), _ptr(v), _stream()))
+        return k, v
+
+
+class QuantizedKVCache(_Cache):
+    """`QuantizedKVCache` (KVCache.swift:923-1210), affine mode."""
+    kind = L.KIND_QUANTIZED
+
+    def __init__(self, group_size=64, bits=8, handle=None):
+        super().__init__(handle=handle, group_size=group_size, bits=bits)
+
+    @property
+    def group_size(self):
+        return self._lib.kvhip_cache_group_size(self._h)
+
+    @property
+    def bits(self):
+        return self._lib.kvhip_cache_bits(self._h)
+
+    def update(self, keys, values):
+        raise RuntimeError("`update` was called on `QuantizedKVCache`. Use `updateQuantized` instead.")
+
+    def update_quantized(self, keys, values, fetch=True):
+        """`updateQuantized(keys:values:)`: ((wq, scales, biases), (wq, scales, biases))."""
+        self._update(keys, values)
+        return self.get_quantized_state() if fetch else None
+
+    def get_quantized_state(self):
+        s = self.state
+        if not s:
+            return None
+        n = self.offset
+        s = [a[:, :, :n] for a in s]
+        return (s[0], s[1], s[2]), (s[3], s[4], s[5])
+
+    def to_unquantized(self):
+        h = C.c_void_p()
+        L.check(self._lib.kvhip_cache_to_unquantized(self._h, _stream(), C.byref(h)))
+        s = KVCacheSimple.__new__(KVCacheSimple)
+        _Cache.__init__(s, handle=h)
+        s._shape = self._shape
+        return s
+
+
+def resolved_kv_quantization_group_size(requested, key_head_dim, value_head_dim):
+    """`resolvedKVQuantizationGroupSize` (KVCache.swift:902-920)."""
+    g = L.load().kvhip_resolved_group_size(requested, key_head_dim, value_head_dim)
+    return g or None
+
+
+def trim_prompt_cache(caches, num_tokens):
+    """`trimPromptCache` (KVCache.swift:2302-2306)."""
+    if not caches or not all(c.is_trimmable for c in caches):
+        return 0
+    for c in caches[1:]:
+        c.trim(num_tokens)
+    return caches[0].trim(num_tokens)
+
+
+def affine_quantize(w, group_size=64, bits=4):
+    """`MLX.quantized(w, groupSize:, bits:)` on the device: (wq int32-as-u32, scales, biases)."""
+    L.init()
+    w = w.contiguous()
+    D = w.shape[-1]
+    rows = w.numel() // D
+    wq = torch.empty(w.shape[:-1] + (D * bits // 32,), dtype=torch.int32, device=w.device)
+    s = torch.empty(w.shape[:-1] + (D // group_size,), dtype=w.dtype, device=w.device)
+    b = torch.empty_like(s)
+    L.check(L.load().kvhip_affine_quantize(_ptr(w), rows, D, group_size, bits, _DT[w.dtype], _ptr(wq),
+                                           _ptr(s), _ptr(b), _stream()))
+    return wq, s, b
+
+
+def affine_dequantize(wq, scales, biases, group_size=64, bits=4):
+    """`MLX.dequantized` on the device."""
+    L.init()
+    wq, scales, biases = wq.contiguous(), scales.contiguous(), biases.contiguous()
+    D = wq.shape[-1] * 32 // bits
+    rows = wq.numel() // wq.shape[-1]
+    out = torch.empty(wq.shape[:-1] + (D,), dtype=scales.dtype, device=wq.device)
+    L.check(L.load().kvhip_affine_dequantize(_ptr(wq), _ptr(scales), _ptr(biases), rows, D, group_size, bits,
+                                             _DT[scales.dtype], _ptr(out), _stream()))
+    return out

@@ -1,0 +1,253 @@
+"""GPU parity tests of attention over the device caches against the CPU oracle.
+
+Tolerance (BASELINE north star): max-abs <= 1e-2 and mean-abs <= 1e-3 against
+the oracle's restatement of the reference path.  Every case runs twice: with the
+library's default kernel choice and with the generic kernel forced, so the
+matrix-core kernels are checked against both the oracle and the generic kernel.
+"""
+import numpy as np
+import pytest
+import torch
+
+import kvhip
+from kvhip import _lib as L
+from oracle import c_oracle as CO
+from oracle import kv_oracle as O
+from tests.util import NAME, dev, err_stats, np32, randn
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS = 1e-2, 1e-3
+
+
+@pytest.fixture(params=[0, 1], ids=["auto", "generic"])
+def policy(request):
+    kvhip.load().kvhip_set_kernel_policy(request.param)
+    yield request.param
+    kvhip.load().kvhip_set_kernel_policy(0)
+
+
+def check(out, ref, what=""):
+    mx, mean = err_stats(np32(out), ref)
+    assert np.isfinite(np32(out)).all(), what
+    assert mx <= MAX_ABS and mean <= MEAN_ABS, f"{what}: max-abs {mx:.3e} mean-abs {mean:.3e}"
+
+
+def omask(mask, dtype):
+    """kvhip MaskMode -> oracle Mask"""
+    if mask is None or mask.mode == L.MASK_NONE:
+        return O.Mask.NONE
+    if mask.mode == L.MASK_CAUSAL:
+        return O.Mask.CAUSAL
+    a = mask.array
+    return O.Mask("array", a.cpu().numpy() if a.dtype == torch.bool else np32(a))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("bits,gs,D", [(8, 64, 64), (4, 64, 128), (4, 32, 64), (2, 64, 128)])
+@pytest.mark.parametrize("r", [1, 4])
+def test_quantized_attention_modes(policy, dtype, bits, gs, D, r):
+    rng = np.random.default_rng(bits + D + r)
+    B, Hkv, T0, Lq = 2, 2, 83, 4
+    name = NAME[dtype]
+    c = kvhip.QuantizedKVCache(gs, bits)
+    o = O.QuantizedKVCache(gs, bits, name)
+    k, kd = randn(rng, (B, Hkv, T0, D), dtype)
+    v, vd = randn(rng, (B, Hkv, T0, D), dtype)
+    c.update_quantized(kd, vd, fetch=False)
+    o.update_quantized(k, v)
+    scale = 1.0 / np.sqrt(D)
+    # multi-token step with .causal, then an array mask, then single-token .none
+    k, kd = randn(rng, (B, Hkv, Lq, D), dtype)
+    v, vd = randn(rng, (B, Hkv, Lq, D), dtype)
+    q, qd = randn(rng, (B, Hkv * r, Lq, D), dtype)
+    out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, kvhip.MaskMode.causal())
+    ref = O.attention_with_cache_update(q, k, v, o, scale, O.Mask.CAUSAL, name)
+    check(out, ref, "causal")
+    T = c.offset
+    m = torch.from_numpy(O.create_causal_mask(Lq, T - Lq, 16)).cuda()
+    out = c.attend(qd, scale, kvhip.MaskMode.from_array(m))
+    ref = O.quantized_sdpa(q, *o.get_quantized_state(), scale, O.Mask("array", m.cpu().numpy()), gs if D % gs == 0 else 32, bits, name)
+    check(out, ref, "bool array")
+    lens = torch.tensor([T - 7, T], dtype=torch.int32)
+    mb = torch.from_numpy(O.create_causal_mask(Lq, T - Lq, None, lens.numpy())).cuda()  # [B,1,L,T]
+    out = c.attend(qd, scale, kvhip.MaskMode.from_array(mb))
+    ref = O.quantized_sdpa(q, *o.get_quantized_state(), scale, O.Mask("array", mb.cpu().numpy()), o.group_size, bits, name)
+    check(out, ref, "batched bool array")
+    add = O.round_to(rng.standard_normal((B, Hkv * r, Lq, T)).astype(np.float32), name)
+    out = c.attend(qd, scale, kvhip.MaskMode.from_array(dev(add, dtype)))
+    ref = O.quantized_sdpa(q, *o.get_quantized_state(), scale, O.Mask("array", add), o.group_size, bits, name)
+    check(out, ref, "additive array")
+    # the symbolic window mask equals the materialised createCausalMask
+    outw = c.attend(qd, scale, kvhip.MaskMode.window_mask(T - Lq, 16))
+    refw = O.quantized_sdpa(q, *o.get_quantized_state(), scale, O.Mask("array", O.create_causal_mask(Lq, T - Lq, 16)), o.group_size, bits, name)
+    check(outw, refw, "window")
+    k, kd = randn(rng, (B, Hkv, 1, D), dtype)
+    v, vd = randn(rng, (B, Hkv, 1, D), dtype)
+    q, qd = randn(rng, (B, Hkv * r, 1, D), dtype)
+    out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale)
+    ref = O.attention_with_cache_update(q, k, v, o, scale, O.Mask.NONE, name)
+    assert out.dtype == dtype  # KVCacheTests.swift:1219-1242
+    check(out, ref, "decode")
+
+
+@pytest.mark.parametrize("r", [1, 2])
+def test_quantized_causal_close_to_full_precision(policy, r):
+    # KVCacheTests.swift:1185-1217: 8-bit g64 causal vs fp SDPA, rtol .05 / atol .1
+    rng = np.random.default_rng(0)
+    B, Hkv, Lq, D = 1, 2, 4, 64
+    scale = 1.0 / np.sqrt(D)
+    q, qd = randn(rng, (B, Hkv * r, Lq, D), torch.float32)
+    k, kd = randn(rng, (B, Hkv, Lq, D), torch.float32)
+    v, vd = randn(rng, (B, Hkv, Lq, D), torch.float32)
+    c = kvhip.QuantizedKVCache(64, 8)
+    out = np32(kvhip.attention_with_cache_update(qd, kd, vd, c, scale, kvhip.MaskMode.causal()))
+    ref = O.sdpa(q, k, v, scale, O.Mask.CAUSAL, "float32")
+    assert np.allclose(out, ref, rtol=0.05, atol=0.1)
+    s = kvhip.KVCacheSimple()
+    out_fp = np32(kvhip.attention_with_cache_update(qd, kd, vd, s, scale, kvhip.MaskMode.causal()))
+    assert np.allclose(out_fp, ref, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("Dk,Dv,r", [(128, 128, 4), (64, 32, 1), (256, 256, 2), (80, 80, 2)])
+def test_simple_cache_attention(policy, dtype, Dk, Dv, r):
+    rng = np.random.default_rng(Dk + r)
+    B, Hkv = 2, 2
+    name = NAME[dtype]
+    c = kvhip.KVCacheSimple()
+    o = O.KVCacheSimple(name)
+    scale = 1.0 / np.sqrt(Dk)
+    for Lq, mode in [(70, "causal"), (1, "none"), (3, "causal"), (1, "none"), (260, "array"), (1, "none")]:
+        k, kd = randn(rng, (B, Hkv, Lq, Dk), dtype)
+        v, vd = randn(rng, (B, Hkv, Lq, Dv), dtype)
+        q, qd = randn(rng, (B, Hkv * r, Lq, Dk), dtype)
+        if mode == "array":
+            mask = c.make_mask(Lq, 64, True)
+            om = o.make_mask(Lq, 64, True)
+            assert np.array_equal(mask.array.cpu().numpy(), om.array)
+        else:
+            mask = kvhip.MaskMode.causal() if mode == "causal" else kvhip.MaskMode.none()
+            om = O.Mask.CAUSAL if mode == "causal" else O.Mask.NONE
+        out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
+        ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
+        check(out, ref, f"L={Lq} {mode}")
+
+
+def test_rotating_attention_past_wrap_matches_never_rotated_reference(policy):
+    # KVCacheTests.swift:1451-1491 (rtol = atol = 1e-5, float32)
+    rng = np.random.default_rng(0)
+    window, history, nq, heads, hd = 8, 20, 4, 2, 4
+    scale = 1.0 / np.sqrt(hd)
+    ak, akd = randn(rng, (1, heads, history + nq, hd), torch.float32)
+    av, avd = randn(rng, (1, heads, history + nq, hd), torch.float32)
+    q, qd = randn(rng, (1, heads, nq, hd), torch.float32)
+    c = kvhip.RotatingKVCache(window)
+    for p in range(history):
+        c.update(akd[:, :, p:p + 1], avd[:, :, p:p + 1], fetch=False)
+    mask = c.make_mask(nq, window, False)
+    out = kvhip.attention_with_cache_update(qd, akd[:, :, history:], avd[:, :, history:], c, scale, mask)
+    qp = np.arange(history, history + nq)[:, None]
+    kp = np.arange(history + nq)[None, :]
+    ref = O.sdpa(q, ak, av, scale, O.Mask("array", (qp >= kp) & (qp < kp + window)), "float32")
+    assert np.allclose(np32(out), ref, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rotating_cfg4_reduced(policy, dtype):
+    """BASELINE config 4 scaled down (maxSize 512, keep 4, D 256, 64-token chunks):
+    chunked prefill wraps the ring, windowed array masks, then single-token decode."""
+    rng = np.random.default_rng(4)
+    B, Hq, Hkv, D, M, chunk = 2, 4, 2, 256, 512, 64
+    name = NAME[dtype]
+    scale = 1.0 / np.sqrt(D)
+    c = kvhip.RotatingKVCache(M, keep=4)
+    o = O.RotatingKVCache(M, keep=4, dtype=name)
+    for i in range(20):
+        k, kd = randn(rng, (B, Hkv, chunk, D), dtype)
+        v, vd = randn(rng, (B, Hkv, chunk, D), dtype)
+        q, qd = randn(rng, (B, Hq, chunk, D), dtype)
+        mask = c.make_mask(chunk, M, False)
+        om = o.make_mask(chunk, M, False)
+        assert mask.mode == {"none": 0, "causal": 1, "array": 2}[om.mode]
+        out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
+        ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
+        if i in (0, 7, 8, 9, 19):
+            check(out, ref, f"chunk {i}")
+    for i in range(40):
+        k, kd = randn(rng, (B, Hkv, 1, D), dtype)
+        v, vd = randn(rng, (B, Hkv, 1, D), dtype)
+        q, qd = randn(rng, (B, Hq, 1, D), dtype)
+        out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, c.make_mask(1, M, False))
+        ref = O.attention_with_cache_update(q, k, v, o, scale, o.make_mask(1, M, False), name)
+        check(out, ref, f"decode {i}")
+        assert c.meta_state == o.get_meta_state()
+
+
+def test_cfg1_quantized_prefill_then_decode(policy):
+    """BASELINE config 1 at full size: B1, 16q/4kv heads, D64, fp16, 8-bit g64; prefill
+    512 with .causal, then 128 single-token appends each followed by quantized SDPA."""
+    rng = np.random.default_rng(0)
+    B, Hq, Hkv, D = 1, 16, 4, 64
+    scale = 0.125
+    dtype = torch.float16
+    c = kvhip.QuantizedKVCache(64, 8)
+    o = O.QuantizedKVCache(64, 8, "float16")
+    q, qd = randn(rng, (B, Hq, 512, D), dtype)
+    k, kd = randn(rng, (B, Hkv, 512, D), dtype)
+    v, vd = randn(rng, (B, Hkv, 512, D), dtype)
+    out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, c.make_mask(512))
+    qk, qv = o.update_quantized(k, v)
+    ref = CO.qsdpa(q, qk, qv, scale, "causal", 64, 8, "float16")
+    check(out, ref, "prefill")
+    for step in range(128):
+        q, qd = randn(rng, (B, Hq, 1, D), dtype)
+        k, kd = randn(rng, (B, Hkv, 1, D), dtype)
+        v, vd = randn(rng, (B, Hkv, 1, D), dtype)
+        out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, c.make_mask(1))
+        qk, qv = o.update_quantized(k, v)
+        ref = CO.qsdpa(q, qk, qv, scale, None, 64, 8, "float16")
+        check(out, ref, f"decode {step}")
+    assert c.offset == 640 and c.meta_state == ["256", "640", "64", "8"]
+    for a, b in zip(c.state, o.get_state()):
+        if a.dtype == torch.int32:
+            assert np.array_equal(np32(a), b)
+        else:
+            assert np.array_equal(O.to_bits(np32(a), "float16"), O.to_bits(b, "float16"))
+
+
+def test_cfg5_ragged_speculative_rollback_reduced(policy):
+    """BASELINE config 5 scaled down: ragged left-padded batch, rounds of 4 draft tokens
+    scored under causal AND left-padding masks, then trim(n)."""
+    rng = np.random.default_rng(0)
+    B, Hq, Hkv, D, Lq = 4, 8, 2, 128, 4
+    dtype = torch.float16
+    lens = rng.integers(40, 300, size=B)
+    Tmax = int(lens.max())
+    pad = (Tmax - lens).astype(np.int32)
+    c = kvhip.QuantizedKVCache(64, 4)
+    o = O.QuantizedKVCache(64, 4, "float16")
+    k, kd = randn(rng, (B, Hkv, Tmax, D), dtype)
+    v, vd = randn(rng, (B, Hkv, Tmax, D), dtype)
+    c.update_quantized(kd, vd, fetch=False)
+    o.update_quantized(k, v)
+    scale = 1.0 / np.sqrt(D)
+    trims = np.random.default_rng(1).integers(0, 5, size=12)
+    for rnd in range(12):
+        k, kd = randn(rng, (B, Hkv, Lq, D), dtype)
+        v, vd = randn(rng, (B, Hkv, Lq, D), dtype)
+        q, qd = randn(rng, (B, Hq, Lq, D), dtype)
+        T = c.offset + Lq
+        m = O.create_causal_mask(Lq, T - Lq)[None, None] & (np.arange(T)[None, None, None, :] >= pad[:, None, None, None])
+        if rnd % 2 == 0:
+            mask = kvhip.MaskMode.from_array(torch.from_numpy(m).cuda())
+        else:
+            mask = kvhip.MaskMode.window_mask(T - Lq, 0, left_pad=torch.from_numpy(pad))
+        out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
+        ref = O.attention_with_cache_update(q, k, v, o, scale, O.Mask("array", m), "float16")
+        check(out, ref, f"round {rnd}")
+        n = int(trims[rnd])
+        assert c.trim(n) == o.trim(n) and c.offset == o.offset
+    for a, b in zip(c.state, o.get_state()):
+        if a.dtype == torch.int32:
+            assert np.array_equal(np32(a), b)

@@ -1,0 +1,326 @@
+"""GPU parity tests of the cache write/read path through the C ABI: packed
+codes, scales/biases, ring indices, trim offsets and state layouts are compared
+bit for bit with the CPU oracle on the same seeded inputs."""
+import numpy as np
+import pytest
+import torch
+
+import kvhip
+from oracle import kv_oracle as O
+from tests.util import NAME, bits_equal, dev, np32, randn
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float16, torch.bfloat16, torch.float32]
+
+
+def positioned(lo, hi, D=2, dtype=torch.float16):
+    p = np.arange(lo, hi, dtype=np.float32)
+    k = np.broadcast_to(p[None, None, :, None], (1, 1, hi - lo, D)).copy()
+    return (k, -k), (dev(k, dtype), dev(-k, dtype))
+
+
+# ------------------------------------------------------------------ quantizer
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("gs", [32, 64, 128])
+def test_affine_quantize_bit_exact(dtype, bits, gs):
+    rng = np.random.default_rng(bits * 100 + gs)
+    w = rng.standard_normal((2, 3, 19, 128)).astype(np.float32)
+    w *= (10.0 ** rng.uniform(-1, 1, size=(128,))).astype(np.float32)
+    w[0, 0, 0] = 0.0
+    w[0, 0, 1] = 3.25
+    w[0, 0, 2, :64] = -w[0, 0, 2, 64:]
+    w[0, 0, 3] = np.abs(w[0, 0, 3])
+    w[0, 0, 4] = -np.abs(w[0, 0, 4])
+    w = O.round_to(w, NAME[dtype])
+    wq, s, b = kvhip.affine_quantize(dev(w, dtype), gs, bits)
+    owq, os_, ob = O.affine_quantize(w, gs, bits, NAME[dtype])
+    assert np.array_equal(np32(wq), owq)
+    assert bits_equal(s, os_, dtype) and bits_equal(b, ob, dtype)
+    deq = kvhip.affine_dequantize(wq, s, b, gs, bits)
+    assert bits_equal(deq, O.affine_dequantize(owq, os_, ob, gs, bits, NAME[dtype]), dtype)
+
+
+def check_quantized_state(cache, ocache, dtype):
+    st = cache.state
+    ost = ocache.get_state()
+    assert len(st) == len(ost) == 6
+    for i, (a, o) in enumerate(zip(st, ost)):
+        assert tuple(a.shape) == tuple(o.shape), (i, a.shape, o.shape)
+        if i % 3 == 0:
+            assert np.array_equal(np32(a), o), f"packed codes differ in state[{i}]"
+        else:
+            assert bits_equal(a, o, dtype), f"scales/biases differ in state[{i}]"
+    assert cache.meta_state == ocache.get_meta_state()
+    assert cache.capacity == ocache.capacity
+
+
+@pytest.mark.parametrize("dtype,bits,gs,D", [
+    (torch.float16, 4, 64, 128), (torch.float16, 8, 64, 64), (torch.bfloat16, 4, 32, 64),
+    (torch.float32, 8, 64, 128), (torch.float16, 2, 64, 128), (torch.float16, 4, 128, 256),
+])
+def test_quantized_cache_append_trim_state(dtype, bits, gs, D):
+    rng = np.random.default_rng(11)
+    B, H = 2, 3
+    cache = kvhip.QuantizedKVCache(gs, bits)
+    ocache = O.QuantizedKVCache(gs, bits, NAME[dtype])
+    # ragged schedule: crosses octets, 32-token blocks, pages and step growth; trims between
+    for L, trim in [(5, 0), (1, 0), (1, 0), (37, 2), (1, 1), (300, 0), (1, 0), (4, 3), (4, 4), (4, 0), (250, 7), (1, 0)]:
+        k, kd = randn(rng, (B, H, L, D), dtype, 2.0)
+        v, vd = randn(rng, (B, H, L, D), dtype, 0.5)
+        cache.update_quantized(kd, vd, fetch=False)
+        ocache.update_quantized(k, v)
+        assert cache.offset == ocache.offset
+        check_quantized_state(cache, ocache, dtype)
+        assert cache.trim(trim) == ocache.trim(trim)
+        assert cache.offset == ocache.offset
+    check_quantized_state(cache, ocache, dtype)
+    # copy is independent and equal
+    cp = cache.copy()
+    k, kd = randn(rng, (B, H, 3, D), dtype)
+    cache.update_quantized(kd, kd, fetch=False)
+    check_quantized_state(cp, ocache, dtype)
+    ocache.update_quantized(k, k)
+    check_quantized_state(cache, ocache, dtype)
+    # state round trip into a fresh cache (restore order: state, then metaState)
+    fresh = kvhip.QuantizedKVCache(gs, bits)
+    fresh.state = cache.state
+    fresh.meta_state = cache.meta_state
+    assert fresh.offset == cache.offset
+    for a, b in zip(fresh.state, cache.state):
+        assert torch.equal(a, b)
+    # and it keeps working after the restore
+    k, kd = randn(rng, (B, H, 2, D), dtype)
+    fresh.update_quantized(kd, kd, fetch=False)
+    ocache2 = ocache.copy()
+    ocache2.update_quantized(k, k)
+    check_quantized_state(fresh, ocache2, dtype)
+
+
+def test_quantized_group_size_fallback_and_errors():
+    # KVCacheTests.swift:477-501: QuantizedKVCache(64, 4) fed D=32 -> groupSize 32
+    rng = np.random.default_rng(0)
+    c = kvhip.QuantizedKVCache(64, 4)
+    k, kd = randn(rng, (1, 2, 3, 32), torch.float16)
+    c.update_quantized(kd, kd, fetch=False)
+    assert c.group_size == 32
+    c.update_quantized(kd, kd, fetch=False)
+    assert c.group_size == 32 and c.offset == 6 and c.meta_state == ["256", "6", "32", "4"]
+    with pytest.raises(RuntimeError):
+        c.update(kd, kd)
+    bad = kvhip.QuantizedKVCache(64, 4)
+    _, k5 = randn(rng, (1, 1, 2, 5), torch.float16)
+    with pytest.raises(kvhip.KVHipError) as e:
+        bad.update_quantized(k5, k5, fetch=False)
+    assert "group sizes" in str(e.value)
+
+
+# ------------------------------------------------------------------ simple
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_simple_cache_update_fetch_state(dtype):
+    rng = np.random.default_rng(5)
+    B, H, Dk, Dv = 2, 2, 64, 32
+    c = kvhip.KVCacheSimple()
+    o = O.KVCacheSimple(NAME[dtype])
+    for L, trim in [(3, 0), (1, 0), (260, 1), (1, 0), (31, 30), (5, 0), (1, 0), (512, 0)]:
+        k, kd = randn(rng, (B, H, L, Dk), dtype)
+        v, vd = randn(rng, (B, H, L, Dv), dtype)
+        gk, gv = c.update(kd, vd)
+        ok, ov = o.update(k, v)
+        assert np.array_equal(np32(gk), ok) and np.array_equal(np32(gv), ov)
+        assert (c.offset, c.capacity) == (o.offset, o.capacity)
+        assert c.trim(trim) == o.trim(trim)
+    st, ost = c.state, o.get_state()
+    assert all(np.array_equal(np32(a), b) for a, b in zip(st, ost))
+    assert c.meta_state == [""] and c.is_trimmable and c.max_size is None
+    cp = c.copy()
+    assert cp.offset == c.offset and all(torch.equal(a, b) for a, b in zip(cp.state, c.state))
+    _, kd = randn(rng, (B, H, 1, Dk), dtype)
+    _, vd = randn(rng, (B, H, 1, Dv), dtype)
+    c.update(kd, vd, fetch=False)
+    assert cp.offset == c.offset - 1
+    fresh = kvhip.KVCacheSimple()
+    fresh.state = st
+    assert fresh.offset == st[0].shape[2]
+    assert all(torch.equal(a, b) for a, b in zip(fresh.state, st))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_simple_to_quantized_and_back(dtype):
+    rng = np.random.default_rng(9)
+    c = kvhip.KVCacheSimple()
+    o = O.KVCacheSimple(NAME[dtype])
+    for L in (70, 1, 1):
+        k, kd = randn(rng, (2, 2, L, 64), dtype)
+        v, vd = randn(rng, (2, 2, L, 64), dtype)
+        c.update(kd, vd, fetch=False)
+        o.update(k, v)
+    c.trim(1)
+    o.trim(1)
+    q = c.to_quantized(64, 4)
+    oq = o.to_quantized(64, 4)
+    check_quantized_state(q, oq, dtype)
+    # empty Simple, offset 7, toQuantized(128, 4) -> ["256","7","128","4"] (KVCacheTests.swift:526-536)
+    e = kvhip.KVCacheSimple()
+    e.offset = 7
+    assert e.to_quantized(128, 4).meta_state == ["256", "7", "128", "4"]
+    # D=5 cannot be quantized; RotatingKVCache never can (KVCacheTests.swift:538-551)
+    s5 = kvhip.KVCacheSimple()
+    _, k5 = randn(rng, (1, 1, 2, 5), dtype)
+    s5.update(k5, k5, fetch=False)
+    with pytest.raises(kvhip.KVHipError):
+        s5.to_quantized()
+    r = kvhip.RotatingKVCache(8)
+    with pytest.raises(kvhip.KVHipError):
+        r.to_quantized()
+    # back to full precision
+    u = q.to_unquantized()
+    ou = oq.to_unquantized()
+    assert u.offset == ou.offset
+    for a, b in zip(u.state, ou.get_state()):
+        assert bits_equal(a, b, dtype)
+
+
+# ------------------------------------------------------------------ rotating
+def drive_pair(c, o, ks, vs, dtype):
+    gk, gv = c.update(dev(ks, dtype), dev(vs, dtype))
+    ok, ov = o.update(ks, vs)
+    assert np.array_equal(np32(gk), ok), "presented keys differ"
+    assert np.array_equal(np32(gv), ov), "presented values differ"
+    assert c.meta_state == o.get_meta_state()
+    assert c.presented_length == ok.shape[2]
+
+
+@pytest.mark.parametrize("keep", [0, 2])
+def test_rotating_single_token_ring_and_logical_view(keep):
+    # KVCacheTests.swift:1312-1404
+    dtype = torch.float16
+    c = kvhip.RotatingKVCache(8, keep=keep)
+    o = O.RotatingKVCache(8, keep=keep)
+    assert c.logical_view(8) is None
+    for p in range(20):
+        (k, v), _ = positioned(p, p + 1)
+        drive_pair(c, o, k, v, dtype)
+        assert c.idx == o.idx and c.offset == o.offset
+    for tail in (8, 7, 5, 3, 2, 1, 0, -1, 99):
+        gk, gv = c.logical_view(tail)
+        ok, ov = o.logical_view(tail)
+        assert np.array_equal(np32(gk), ok) and np.array_equal(np32(gv), ov), tail
+    if keep == 0:
+        assert [int(x) for x in np32(c.logical_view(8)[0])[0, 0, :, 0]] == list(range(12, 20))
+        assert [int(x) for x in np32(c.logical_view(3)[0])[0, 0, :, 0]] == [17, 18, 19]
+    else:
+        assert [int(x) for x in np32(c.logical_view(5)[0])[0, 0, :, 0]] == [0, 1, 17, 18, 19]
+        assert [int(x) for x in np32(c.logical_view(1)[0])[0, 0, :, 0]] == [0, 1]
+    # reads leave the ring untouched
+    before = (c.meta_state, [a.clone() for a in c.state])
+    c.logical_view(7)
+    assert before[0] == c.meta_state and all(torch.equal(a, b) for a, b in zip(before[1], c.state))
+    assert not c.is_trimmable and c.max_size == 8
+
+
+def test_rotating_view_plus_new_rows_equals_write_presentation():
+    # KVCacheTests.swift:1409-1446
+    dtype = torch.float16
+    c = kvhip.RotatingKVCache(8)
+    o = O.RotatingKVCache(8)
+    for p in range(20):
+        (k, v), _ = positioned(p, p + 1)
+        drive_pair(c, o, k, v, dtype)
+    vk, vv = c.logical_view(7)
+    mask = c.make_mask(4, 8, False)
+    omask = o.make_mask(4, 8, False)
+    (k, v), (kd, vd) = positioned(20, 24)
+    pk, pv = c.update(kd, vd)
+    assert torch.equal(pk, torch.cat([vk, kd], 2)) and torch.equal(pv, torch.cat([vv, vd], 2))
+    assert mask.array.shape == (4, 11) and np.array_equal(mask.array.cpu().numpy(), omask.array)
+
+
+@pytest.mark.parametrize("M,keep,step,schedule", [
+    (8, 0, 256, [1, 1, 1, 4, 1, 1, 6, 1, 1, 1, 1, 1, 1, 1, 1, 1, 3, 9, 1, 1, 12, 1, 1]),
+    (8, 2, 4, [3, 1, 1, 1, 1, 1, 1, 1, 1, 5, 1, 1, 1, 1, 1, 1, 1, 1, 1, 2, 1]),
+    (16, 4, 3, [1] * 5 + [7] + [1] * 30 + [20] + [1] * 20 + [2, 2, 2] + [1] * 20),
+    (64, 4, 256, [32, 32, 32, 32, 1, 1, 1, 32, 1] + [1] * 70 + [40, 1, 1]),
+    (300, 4, 256, [128, 128, 128, 128, 128] + [1] * 310 + [128, 1, 1]),
+])
+def test_rotating_mixed_updates_match_reference_buffers(M, keep, step, schedule):
+    """Every update's presentation, metaState (offset, idx) and state equal the
+    reference's buffers row for row, through growth, wrap, front-trim and re-linearisation."""
+    dtype = torch.float16
+    c = kvhip.RotatingKVCache(M, keep=keep, step=step)
+    o = O.RotatingKVCache(M, keep=keep, step=step)
+    pos = 0
+    for L in schedule:
+        (k, v), _ = positioned(pos, pos + L, D=4)
+        drive_pair(c, o, k, v, dtype)
+        pos += L
+        assert c.is_trimmable == o.is_trimmable
+    st, ost = c.state, o.get_state()
+    assert all(np.array_equal(np32(a), b) for a, b in zip(st, ost))
+    # copy + state/meta restore
+    cp = c.copy()
+    assert cp.meta_state == c.meta_state and all(torch.equal(a, b) for a, b in zip(cp.state, st))
+    fresh = kvhip.RotatingKVCache(M)
+    fresh.state = st
+    fresh.meta_state = c.meta_state
+    (k, v), _ = positioned(pos, pos + 1, D=4)
+    o2 = o.copy()
+    drive_pair(fresh, o, k, v, dtype)
+    drive_pair(cp, o2, k, v, dtype)
+
+
+def test_rotating_trim_then_write():
+    # trim is pure bookkeeping: offset -= n, idx -= n (KVCache.swift:826-831)
+    dtype = torch.float16
+    c = kvhip.RotatingKVCache(32)
+    o = O.RotatingKVCache(32)
+    pos = 0
+    for L, trim in [(5, 0), (4, 3), (4, 4), (4, 0), (1, 0), (4, 2), (1, 1), (1, 0)]:
+        (k, v), _ = positioned(pos, pos + L, D=4)
+        drive_pair(c, o, k, v, dtype)
+        pos += L
+        assert c.is_trimmable_after(L) == o.is_trimmable_after(L)
+        assert c.trim(trim) == o.trim(trim)
+        pos -= trim
+        assert c.meta_state == o.get_meta_state()
+
+
+def test_rotating_cfg4_trace_reduced():
+    """BASELINE config 4 at reduced batch/heads: maxSize 4096, keep 4, 512-token chunks
+    wrap the ring three times, then single-token decode (lengths from KVCache.swift:660-740)."""
+    dtype = torch.bfloat16
+    c = kvhip.RotatingKVCache(4096, keep=4)
+    o = O.RotatingKVCache(4096, keep=4, dtype="bfloat16")
+    rng = np.random.default_rng(4)
+    lens = []
+    for i in range(24):
+        k, kd = randn(rng, (1, 1, 512, 8), dtype)
+        c.update(kd, kd, fetch=False)
+        o.update(k, k)
+        lens.append(c.presented_length)
+        assert c.meta_state == o.get_meta_state()
+    assert lens[:8] == [512 * i for i in range(1, 9)] and all(n == 4607 for n in lens[8:])
+    gk, _ = c.fetch()
+    assert np.array_equal(np32(gk), o.keys)
+    for i in range(5):
+        k, kd = randn(rng, (1, 1, 1, 8), dtype)
+        gk, _ = c.update(kd, kd)
+        ok, _ = o.update(k, k)
+        assert np.array_equal(np32(gk), ok) and c.meta_state == o.get_meta_state()
+    assert c.presented_length == 4096 and (c.offset, c.idx) == (12293, 9)
+
+
+def test_mask_materialize_matches_create_causal_mask():
+    c = kvhip.KVCacheSimple()
+    c.offset = 37
+    for n, w, ra in [(5, None, True), (9, 4, False), (3, 8, True)]:
+        m = c.make_mask(n, w, ra)
+        om = O.base_make_mask(37, n, w, ra)
+        assert np.array_equal(m.array.cpu().numpy(), om.array)
+    r = kvhip.RotatingKVCache(16)
+    o = O.RotatingKVCache(16)
+    r.meta_state = ["0", "16", "256", "21", "5"]
+    o.set_meta_state(["0", "16", "256", "21", "5"])
+    m, om = r.make_mask(1, 8), o.make_mask(1, 8)
+    assert np.array_equal(m.array.cpu().numpy(), om.array)
