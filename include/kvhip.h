@@ -119,6 +119,16 @@ kvhip_status kvhip_init(int32_t device);
 kvhip_status kvhip_sync(void *stream);
 /* 0 = choose the fastest kernel for the shape (default); 1 = always the generic kernel. */
 void kvhip_set_kernel_policy(int32_t policy);
+/*
+ * Measurement hooks (no counterpart in the reference, which times whole
+ * generations with wall clocks, Evaluate.swift:2467).  While enabled, every
+ * launch of the split-sequence decode attention kernel is bracketed by HIP
+ * events on the stream it is launched on.  kvhip_profile_read waits for those
+ * events, returns the number of launches and their summed duration in
+ * milliseconds, and clears the record.
+ */
+void kvhip_profile_enable(int32_t on);
+kvhip_status kvhip_profile_read(int32_t *out_launches, double *out_total_ms);
 
 /* ---- lifetime ---------------------------------------------------------- */
 /* KVCacheSimple() / RotatingKVCache(maxSize:keep:step:) / QuantizedKVCache(groupSize:bits:) */

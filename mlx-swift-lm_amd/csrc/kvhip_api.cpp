@@ -456,6 +456,16 @@ kvhip_status kvhip_sync(void *stream) {
 
 void kvhip_set_kernel_policy(int32_t policy) { g_policy = policy; }
 
+void kvhip_profile_enable(int32_t on) { profile_enable(on != 0); }
+
+kvhip_status kvhip_profile_read(int32_t *out_launches, double *out_total_ms) {
+    if (!out_launches || !out_total_ms) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    int n = 0;
+    KV_HIP(profile_read(&n, out_total_ms));
+    *out_launches = n;
+    return KVHIP_OK;
+}
+
 kvhip_status kvhip_cache_create(const kvhip_config *cfg, kvhip_cache **out) {
     if (!cfg || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
     if (cfg->kind < 0 || cfg->kind > 2) return fail(KVHIP_ERR_INVALID_ARG, "unknown cache kind");

@@ -74,7 +74,8 @@ def test_quantized_attention_modes(policy, dtype, bits, gs, D, r):
     out = c.attend(qd, scale, kvhip.MaskMode.from_array(mb))
     ref = O.quantized_sdpa(q, *o.get_quantized_state(), scale, O.Mask("array", mb.cpu().numpy()), o.group_size, bits, name)
     check(out, ref, "batched bool array")
-    add = O.round_to(rng.standard_normal((B, Hkv * r, Lq, T)).astype(np.float32), name)
+    # per-head masks only line up in the reference without GQA (KVCache.swift:2436-2440)
+    add = O.round_to(rng.standard_normal((B, Hkv if r == 1 else 1, Lq, T)).astype(np.float32), name)
     out = c.attend(qd, scale, kvhip.MaskMode.from_array(dev(add, dtype)))
     ref = O.quantized_sdpa(q, *o.get_quantized_state(), scale, O.Mask("array", add), o.group_size, bits, name)
     check(out, ref, "additive array")

@@ -78,9 +78,10 @@ def test_quantized_cache_append_trim_state(dtype, bits, gs, D):
     check_quantized_state(cache, ocache, dtype)
     # copy is independent and equal
     cp = cache.copy()
+    ocp = ocache.copy()
     k, kd = randn(rng, (B, H, 3, D), dtype)
     cache.update_quantized(kd, kd, fetch=False)
-    check_quantized_state(cp, ocache, dtype)
+    check_quantized_state(cp, ocp, dtype)
     ocache.update_quantized(k, k)
     check_quantized_state(cache, ocache, dtype)
     # state round trip into a fresh cache (restore order: state, then metaState)
