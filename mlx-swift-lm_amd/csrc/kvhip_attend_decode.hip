@@ -1,26 +1,32 @@
-// Split-sequence decode attention on the matrix cores (gfx950 MFMA 16x16x32).
+// Split-sequence decode attention on the matrix cores (gfx950).
 //
 // One workgroup (4 wavefronts) owns a contiguous span of physical slots of one
 // (batch, kv-head) pair and leaves an unnormalised partial (max, sum, out[D]) per
-// query row; a second small kernel merges the partials of all spans.  The r*L
-// (<= 4) query rows that share a kv head ride in the M dimension of the QK^T
-// tile, so K and V are read from HBM exactly once per step.
+// query row; a second small kernel merges the partials of all spans.  All query
+// rows that share a kv head (r = Hq/Hkv heads times L new tokens, up to 16) are
+// served from one pass over K and V, which are read from HBM exactly once.
 //
-// Per 64-slot tile and wavefront:
-//   QK^T   four 16-token sub-tiles are multiplied by four copies of the query
-//          block placed in different row groups of the A operand, so that the
-//          accumulator of lane l ends up holding the scores of token l for all
-//          query rows.  Packed codes become MFMA operands without a dequantize
-//          pass: a 4-bit (8-bit) code masked in place is the fp16 subnormal
-//          code * 2^-24 (high nibbles: * 2^-20, compensated by queries
-//          pre-scaled by 1/16), so q.(scale*code + bias) is evaluated as
-//          scale * 2^24 * mfma(q, masked words) + bias * sum(q).
-//   softmax online, running maximum per wavefront, rescaling only when a tile
-//          raises it.
-//   PV     P (times the per-token V scale of the column's group) goes through LDS
-//          into the A operand; the octet-transposed V words are the B operand
-//          as stored.  V biases are accumulated on the side: sum_t p_t * bias_t.
+// The contraction uses v_mfma_f32_4x4x4_16B_f16: sixteen independent 4x4x4 blocks
+// per instruction.  With CBSZ=4 the A operand of ONE block (chosen by ABID) is
+// broadcast to all sixteen, so the small operand (4 query rows / 4 probability
+// rows) costs two registers while the large one (K, V) fills the B side:
+//
+//   QK^T  block b covers tokens 4b..4b+3: lane l supplies four head-dim elements
+//         of token l's K row (B); the accumulator of lane l receives the scores of
+//         token l for the 4 query rows.  The query operands of 16 successive steps
+//         live in the 16 lane groups of one register pair; ABID picks the step.
+//   PV    block b covers head-dim columns 4b..4b+3 (+64h): lane l supplies, for
+//         column l, four consecutive tokens of the transposed V tile (B); the
+//         probabilities of step s (tokens 4s..4s+3) sit in lane group s after a
+//         4x4 transpose inside each quad of lanes and are broadcast with ABID = s.
+//
+// Packed codes become operands without a dequantize pass: a code masked in place
+// is the fp16 subnormal code * 2^-24 (high nibbles: * 2^-20, compensated by
+// operands pre-scaled by 1/16), which the matrix core multiplies exactly.  So
+//   q . (scale*code + bias)            = scale * 2^24 * mfma(q, masked K words) + bias * sum(q)
+//   sum_t p_t (scale_t*code_t + bias_t) = 2^24 * mfma(p*scale, masked V words) + sum_t p_t bias_t
 #include <cstdlib>
+#include <utility>
 #include <vector>
 
 #include "kvhip_mask.hpp"
@@ -29,65 +35,34 @@ namespace kvhip {
 
 namespace {
 
-typedef _Float16 h8 __attribute__((ext_vector_type(8)));
-typedef __bf16 b8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef short s4 __attribute__((ext_vector_type(4)));
 typedef float f4 __attribute__((ext_vector_type(4)));
-union Op {
-    h8 h;
-    b8 b;
-    uint32_t u[4];
-    uint4 v;
+union Op {  // one 4-element 16-bit operand
+    h4 h;
+    s4 s;
+    uint32_t u[2];
 };
 
 constexpr int WAVES = 4;
-constexpr int TILE = 64;
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float TWO24 = 16777216.0f;
 
-// element position inside an 8-element operand chunk for operand slot kk
-template <int BITS> __device__ __forceinline__ constexpr int elem_of(int kk) {
-    return BITS == 4 ? ((kk >> 1) + 4 * (kk & 1)) : (BITS == 8 ? ((kk & 4) + ((kk >> 1) & 1) + 2 * (kk & 1)) : kk);
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
 }
-// operand slot of octet position e (inverse of elem_of)
-template <int BITS> __device__ __forceinline__ int slot_of(int e) {
-    return BITS == 4 ? (2 * (e & 3) + (e >> 2)) : (BITS == 8 ? ((e & 4) + 2 * (e & 1) + ((e >> 1) & 1)) : e);
-}
-// slots whose masked value carries an extra factor 16 (high nibbles)
-template <int BITS> __device__ __forceinline__ constexpr bool hi_slot(int kk) { return BITS == 4 && (kk & 2); }
-
-template <int BITS> struct Words;  // raw 8-element chunk as loaded
-template <> struct Words<4> { uint32_t w; };
-template <> struct Words<8> { uint2 w; };
-template <> struct Words<0> { uint4 w; };
-
-template <int BITS> __device__ __forceinline__ Op to_operand(const Words<BITS> &x);
-template <> __device__ __forceinline__ Op to_operand<4>(const Words<4> &x) {
-    Op o;
-    const uint32_t w8 = x.w >> 8;
-    o.u[0] = x.w & 0x000f000fu;
-    o.u[1] = x.w & 0x00f000f0u;
-    o.u[2] = w8 & 0x000f000fu;
-    o.u[3] = w8 & 0x00f000f0u;
-    return o;
-}
-template <> __device__ __forceinline__ Op to_operand<8>(const Words<8> &x) {
-    Op o;
-    o.u[0] = x.w.x & 0x00ff00ffu;
-    o.u[1] = (x.w.x >> 8) & 0x00ff00ffu;
-    o.u[2] = x.w.y & 0x00ff00ffu;
-    o.u[3] = (x.w.y >> 8) & 0x00ff00ffu;
-    return o;
-}
-template <> __device__ __forceinline__ Op to_operand<0>(const Words<0> &x) {
-    Op o;
-    o.v = x.w;
-    return o;
+// f(std::integral_constant<int, i>) for i = 0..N-1, fully unrolled with compile-time i
+template <int N, class F> __device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
-template <bool BF> __device__ __forceinline__ f4 mfma(const Op &a, const Op &b, f4 c) {
-    if (BF) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, c, 0, 0, 0);
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, c, 0, 0, 0);
+template <int ABID> __device__ __forceinline__ f4 mfma444(const Op &a, const Op &b, f4 c) {
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(a.h, b.h, c, 4, ABID, 0);
 }
+
+// v_exp_f32 without the denormal-range fix-up (results below 2^-126 flush to zero)
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __device__ __forceinline__ float wave_max(float v) {
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
@@ -97,265 +72,326 @@ __device__ __forceinline__ float wave_sum(float v) {
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
     return v;
 }
-
-__device__ __forceinline__ uint16_t f2h_bits(float v) {
-    return __builtin_bit_cast(uint16_t, (_Float16)v);
+__device__ __forceinline__ uint16_t f2h_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+__device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
+    return (uint32_t)f2h_bits(lo) | ((uint32_t)f2h_bits(hi) << 16);
 }
-__device__ __forceinline__ uint16_t f2bf_bits(float v) { return Elem<1>::bits(v); }
 
-// One tile's worth of raw operand data held in registers.
-template <int BITS, int D, int G> struct TileRegs {
-    Words<BITS> k[4][D / 32];  // [sub-tile u][step]
-    Words<BITS> v[2][D / 16];  // [32-token block][d tile]
-    float ks[G], kb[G], vs[G], vb[G];
-    int row;                   // presented row of this lane's token, -1 if none
+// value held by lane (l ^ 1) / (l ^ 2) of the same quad
+__device__ __forceinline__ uint32_t quad_xor1(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+}
+__device__ __forceinline__ uint32_t quad_xor2(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+}
+// 4x4 transpose inside each quad: before, lane c holds x[i]; after, lane i holds in
+// x[k] what lane k held in x[i].
+__device__ __forceinline__ void quad_transpose(uint32_t x[4], int lane) {
+    const bool b0 = lane & 1, b1 = lane & 2;
+    {
+        const uint32_t s01 = b0 ? x[0] : x[1], s23 = b0 ? x[2] : x[3];
+        const uint32_t r01 = quad_xor1(s01), r23 = quad_xor1(s23);
+        x[0] = b0 ? r01 : x[0];
+        x[1] = b0 ? x[1] : r01;
+        x[2] = b0 ? r23 : x[2];
+        x[3] = b0 ? x[3] : r23;
+    }
+    {
+        const uint32_t s02 = b1 ? x[0] : x[2], s13 = b1 ? x[1] : x[3];
+        const uint32_t r02 = quad_xor2(s02), r13 = quad_xor2(s13);
+        x[0] = b1 ? r02 : x[0];
+        x[2] = b1 ? x[2] : r02;
+        x[1] = b1 ? r13 : x[1];
+        x[3] = b1 ? x[3] : r13;
+    }
+}
+
+// load N consecutive dwords with the widest vector accesses
+template <int N> __device__ __forceinline__ void load_words(uint32_t *dst, const char *p) {
+    if constexpr (N % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < N / 4; ++i) {
+            const uint4 v = reinterpret_cast<const uint4 *>(p)[i];
+            dst[4 * i] = v.x; dst[4 * i + 1] = v.y; dst[4 * i + 2] = v.z; dst[4 * i + 3] = v.w;
+        }
+    } else if constexpr (N % 2 == 0) {
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i) {
+            const uint2 v = reinterpret_cast<const uint2 *>(p)[i];
+            dst[2 * i] = v.x; dst[2 * i + 1] = v.y;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) dst[i] = reinterpret_cast<const uint32_t *>(p)[i];
+    }
+}
+
+// ---- operand geometry --------------------------------------------------------------
+// A "step" contracts 4 elements; one packed 32-bit word yields WSTEPS steps.
+//   4 bit: 8 codes -> 2 steps taking nibbles (0,4,1,5) and (2,6,3,7); the last two
+//          of each are high nibbles (value x16)
+//   8 bit: 4 codes -> 1 step taking bytes (0,2,1,3)
+template <int BITS> struct Geo;
+template <> struct Geo<4> {
+    static constexpr int WSTEPS = 2, EPW = 8;
+    static __device__ __forceinline__ constexpr int elem(int h, int k) { return 2 * h + (k >> 1) + 4 * (k & 1); }
+    static __device__ __forceinline__ constexpr bool hi(int k) { return k >= 2; }
+    static __device__ __forceinline__ void unpack(uint32_t w, Op *o) {
+        const uint32_t w8 = w >> 8;
+        o[0].u[0] = w & 0x000f000fu;
+        o[0].u[1] = w & 0x00f000f0u;
+        o[1].u[0] = w8 & 0x000f000fu;
+        o[1].u[1] = w8 & 0x00f000f0u;
+    }
+};
+template <> struct Geo<8> {
+    static constexpr int WSTEPS = 1, EPW = 4;
+    static __device__ __forceinline__ constexpr int elem(int, int k) { return (k >> 1) + 2 * (k & 1); }
+    static __device__ __forceinline__ constexpr bool hi(int) { return false; }
+    static __device__ __forceinline__ void unpack(uint32_t w, Op *o) {
+        o[0].u[0] = w & 0x00ff00ffu;
+        o[0].u[1] = (w >> 8) & 0x00ff00ffu;
+    }
 };
 
-// partial layout in the workspace: per (bh, split, query row): m, l, out[D]
-template <int D> constexpr int part_stride() { return D + 2; }
+// One tile (64 slots) of raw operand data in registers; lane l owns token l of the tile
+// for K and head-dim column l (+64h) for V.
+template <int BITS, int D, int G> struct TileRegs {
+    static constexpr int KW = D * BITS / 32;   // dwords of one K row
+    static constexpr int VW = 64 * BITS / 32;  // dwords of one V tile row
+    uint32_t k[KW];
+    uint32_t v[D / 64][VW];
+    float ks[G], kb[G], vs[G], vb[G];
+    int row;  // presented row of this lane's token, -1 if none
+};
 
-template <int BITS, int D, int GS, int DT>
+// RG = groups of 4 query rows handled per pass (R <= 4 RG)
+template <int BITS, int D, int GS, int DT, int RG>
 __global__ void __launch_bounds__(WAVES * 64, 2)
 decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
-    constexpr bool Q = BITS != 0;
-    constexpr bool BF = !Q && DT == 1;  // quantized caches always use fp16 operands
-    constexpr int S = D / 32;            // MFMA steps over the head dim
-    constexpr int G = Q ? D / GS : 1;    // quantization groups per row
-    constexpr int NT = D / 16;           // output column tiles
+    using GEO = Geo<BITS>;
+    constexpr int G = D / GS;      // quantization groups per row (1 or 2)
+    constexpr int NH = D / 64;     // 64-column halves of the output
+    constexpr int NQA = D / 64;    // query operand register pairs (16 steps of 4 elements each)
+    constexpr int RR = 4 * RG;     // query rows carried
+    using T = TileRegs<BITS, D, G>;
     const Store &st = a.st;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n = lane & 15, j = lane >> 4;
+    const int blk = lane >> 2, qi = lane & 3;  // lane group (MFMA block) and position in it
     const int bh = blockIdx.y, split = blockIdx.x;
     const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
     const int r = a.Hq / a.Hkv;
-    const int R = r * a.L;  // query rows sharing this kv head (<= 4)
+    const int R = r * a.L;
 
-    __shared__ __attribute__((aligned(16))) uint16_t pbuf[WAVES][2][G][4][TILE];  // [wave][hi/lo][group][row][slot]
-    __shared__ float cbuf[WAVES][4][D + 2];
+    __shared__ float cbuf[WAVES][RR][D + 2];
 
-    // ---- query operands: built once per workgroup, kept in LDS ------------------
-    // qlds[u][s][lane] is the A operand of sub-tile u at step s: the query block sits in
-    // row group u (rows 4u..4u+3) and every other row is zero.
-    __shared__ uint4 qlds[4][S][64];
-    float qsum[G][4];
+    // ---- query operands: lane (blk, qi) holds row qi's 4 elements of step 16 x + blk ----
+    Op qa[RG][NQA];
+    float qsum[RG][G][4];
 #pragma unroll
-    for (int g = 0; g < G; ++g)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) qsum[g][i] = 0.f;
-    {
-        const int i = n & 3;  // query row this lane feeds
+    for (int rg = 0; rg < RG; ++rg) {
+        const int i = 4 * rg + qi;
         const int rep = i / a.L, l = i - rep * a.L;
         const size_t qoff = ((size_t)(b * a.Hq + hk * r + rep) * a.L + l) * D;
-        const int u = wave;   // wavefront w fills the operands of sub-tile w
-        const bool on = (n >> 2) == u && i < R;
 #pragma unroll
-        for (int s = 0; s < S; ++s) {
-            Op base;
+        for (int x = 0; x < NQA; ++x) {
+            const int step = 16 * x + blk;
+            const int w = step / GEO::WSTEPS, h = step % GEO::WSTEPS;
+            float qv[4];
 #pragma unroll
-            for (int w = 0; w < 4; ++w) base.u[w] = 0u;
-            if (on) {
-#pragma unroll
-                for (int kk = 0; kk < 8; ++kk) {
-                    const int d = 32 * s + 8 * j + elem_of<BITS>(kk);
-                    float qv = Elem<DT>::load(a.q, qoff + d);
-                    if (Q) qv = round_dt<DT>(qv * a.scale);
-                    const uint16_t hb = BF ? f2bf_bits(qv) : f2h_bits(hi_slot<BITS>(kk) ? qv * 0.0625f : qv);
-                    base.u[kk >> 1] |= (uint32_t)hb << (16 * (kk & 1));
-                }
+            for (int k = 0; k < 4; ++k) {
+                const int d = w * GEO::EPW + GEO::elem(h, k);
+                float v = 0.f;
+                if (i < R) v = round_dt<DT>(Elem<DT>::load(a.q, qoff + d) * a.scale);
+                qv[k] = GEO::hi(k) ? v * 0.0625f : v;
             }
-            qlds[u][s][lane] = base.v;
+            qa[rg][x].u[0] = pack_h2(qv[0], qv[1]);
+            qa[rg][x].u[1] = pack_h2(qv[2], qv[3]);
         }
-        if (Q) {
-            // sum of the (rounded, fp16-held) queries per group, for the bias term
 #pragma unroll
-            for (int g = 0; g < G; ++g)
+        for (int g = 0; g < G; ++g)
 #pragma unroll
-                for (int ii = 0; ii < 4; ++ii) {
-                    float sacc = 0.f;
-                    if (ii < R) {
-                        const int rep2 = ii / a.L, l2 = ii - rep2 * a.L;
-                        const size_t qo = ((size_t)(b * a.Hq + hk * r + rep2) * a.L + l2) * D;
-                        for (int d = g * GS + lane; d < (g + 1) * GS; d += 64)
-                            sacc += (float)(_Float16)round_dt<DT>(Elem<DT>::load(a.q, qo + d) * a.scale);
-                    }
-                    qsum[g][ii] = wave_sum(sacc);
+            for (int ii = 0; ii < 4; ++ii) {
+                float sacc = 0.f;
+                const int i2 = 4 * rg + ii;
+                if (i2 < R) {
+                    // sum of the (rounded, fp16-held) queries of the group, for the bias term
+                    const int rep2 = i2 / a.L, l2 = i2 - rep2 * a.L;
+                    const size_t qo = ((size_t)(b * a.Hq + hk * r + rep2) * a.L + l2) * D;
+                    for (int d = g * GS + lane; d < (g + 1) * GS; d += 64)
+                        sacc += (float)(_Float16)round_dt<DT>(Elem<DT>::load(a.q, qo + d) * a.scale);
                 }
-        }
+                qsum[rg][g][ii] = wave_sum(sacc);
+            }
     }
-    __syncthreads();
 
-    // ---- running state ---------------------------------------------------------
-    float m_run[4], l_part[4], bacc[G][4];
-    f4 oacc[NT];
+    // ---- running state ---------------------------------------------------------------
+    float m_run[RG][4], l_part[RG][4], bacc[RG][G][4];
+    f4 oacc[RG][NH];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) { m_run[i] = -INFINITY; l_part[i] = 0.f; }
+    for (int rg = 0; rg < RG; ++rg) {
 #pragma unroll
-    for (int g = 0; g < G; ++g)
+        for (int i = 0; i < 4; ++i) { m_run[rg][i] = -INFINITY; l_part[rg][i] = 0.f; }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) bacc[g][i] = 0.f;
+        for (int g = 0; g < G; ++g)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) oacc[t] = f4{0.f, 0.f, 0.f, 0.f};
+            for (int i = 0; i < 4; ++i) bacc[rg][g][i] = 0.f;
+#pragma unroll
+        for (int h = 0; h < NH; ++h) oacc[rg][h] = f4{0.f, 0.f, 0.f, 0.f};
+    }
 
     const int tile_begin = split * tiles_per_wg;
     const int tile_end = min(tiles_total, tile_begin + tiles_per_wg);
     const float fill = finfo_min_dt(DT);
-    // LDS position of this lane's token inside the P staging row
-    const int tl = lane & 31;
-    const int e_tok = (tl & 3) + ((tl >> 4) << 2);
-    const int ppos = (lane & 32) + 8 * ((tl & 15) >> 2) + slot_of<BITS>(e_tok);
-    const float vfac = (BITS == 4 && (e_tok & 1)) ? 0.0625f : 1.0f;
+    // tokens whose V code sits in a high nibble carry 1/16 on the probability side
+    const float vfac = (BITS == 4 && (lane & 2)) ? 0.0625f : 1.0f;
 
-    auto load_tile = [&](int tile, TileRegs<BITS, D, G> &t) {
-        const int slot0 = tile * TILE;
-        // K: sub-tile u, token n, chunk j
-        const char *kbase = k_row_ptr(st, bh, slot0 + n);
-        constexpr int CH = Q ? BITS : 16;  // bytes per 8-element chunk
+    const bool identity = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
+    const size_t k_page = (size_t)st.BH * st.k_cell, v_page = (size_t)st.BH * st.v_cell;
+    const size_t ksb_page = (size_t)st.BH * st.ksb_cell, vsb_page = (size_t)st.BH * st.vsb_cell;
+    constexpr int VROW = T::VW * 4;  // bytes of one V tile row
+
+    auto load_tile = [&](int tile_, T &t) {
+        const int tile = __builtin_amdgcn_readfirstlane(tile_);
+        const int page = tile >> 2, tip = tile & 3;  // 4 tiles per page
+        const char *kt = st.k + page * k_page + (size_t)bh * st.k_cell + (size_t)(tip * TILE + lane) * st.k_row;
+        load_words<T::KW>(t.k, kt);
+        const char *vt = st.v + page * v_page + (size_t)bh * st.v_cell + ((size_t)tip * D + lane) * VROW;
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int h = 0; h < NH; ++h) load_words<T::VW>(t.v[h], vt + (size_t)h * 64 * VROW);
+        const char *ksb = st.ksb + page * ksb_page + (size_t)bh * st.ksb_cell + (size_t)(tip * TILE + lane) * st.ksb_row;
+        const char *vsb = st.vsb + page * vsb_page + (size_t)bh * st.vsb_cell + (size_t)(tip * TILE + lane) * st.vsb_row;
+        uint32_t kraw[G], vraw[G];  // (scale, bias) pairs of a 16-bit dtype
+        load_words<G>(kraw, ksb);
+        load_words<G>(vraw, vsb);
 #pragma unroll
-            for (int s = 0; s < S; ++s) {
-                const char *p = kbase + (size_t)u * 16 * st.k_row + (4 * s + j) * CH;
-                if constexpr (BITS == 4) t.k[u][s].w = *reinterpret_cast<const uint32_t *>(p);
-                else if constexpr (BITS == 8) *reinterpret_cast<uint2 *>(&t.k[u][s].w) = *reinterpret_cast<const uint2 *>(p);
-                else *reinterpret_cast<uint4 *>(&t.k[u][s].w) = *reinterpret_cast<const uint4 *>(p);
-            }
-        // V: block blk, octet j, column tile dt, column n
-        const char *vcell = v_cell_ptr(st, bh, slot0);
-        const int bip = (slot0 & (PAGE - 1)) >> 5;
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-            for (int dt = 0; dt < NT; ++dt) {
-                const size_t unit = (size_t)((bip + blk) * 4 + j) * D + 16 * dt + n;
-                const char *p = vcell + unit * CH;
-                if constexpr (BITS == 4) t.v[blk][dt].w = *reinterpret_cast<const uint32_t *>(p);
-                else if constexpr (BITS == 8) *reinterpret_cast<uint2 *>(&t.v[blk][dt].w) = *reinterpret_cast<const uint2 *>(p);
-                else *reinterpret_cast<uint4 *>(&t.v[blk][dt].w) = *reinterpret_cast<const uint4 *>(p);
-            }
-        const int slot = slot0 + lane;
-        if (Q) {
-            const char *ksb = ksb_row_ptr(st, bh, slot);
-            const char *vsb = vsb_row_ptr(st, bh, slot);
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-                t.ks[g] = Elem<DT>::load(ksb, 2 * g);
-                t.kb[g] = Elem<DT>::load(ksb, 2 * g + 1);
-                t.vs[g] = Elem<DT>::load(vsb, 2 * g);
-                t.vb[g] = Elem<DT>::load(vsb, 2 * g + 1);
+        for (int g = 0; g < G; ++g) {
+            if (DT == 0) {
+                t.ks[g] = (float)__builtin_bit_cast(_Float16, (uint16_t)kraw[g]);
+                t.kb[g] = (float)__builtin_bit_cast(_Float16, (uint16_t)(kraw[g] >> 16));
+                t.vs[g] = (float)__builtin_bit_cast(_Float16, (uint16_t)vraw[g]);
+                t.vb[g] = (float)__builtin_bit_cast(_Float16, (uint16_t)(vraw[g] >> 16));
+            } else {
+                t.ks[g] = __uint_as_float(kraw[g] << 16);
+                t.kb[g] = __uint_as_float(kraw[g] & 0xffff0000u);
+                t.vs[g] = __uint_as_float(vraw[g] << 16);
+                t.vb[g] = __uint_as_float(vraw[g] & 0xffff0000u);
             }
         }
-        const int row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
+        const int slot = tile * TILE + lane;
+        int row;
+        if (identity) row = slot;
+        else row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
         t.row = (row >= 0 && row < a.T) ? row : -1;
     };
 
-    auto compute_tile = [&](const TileRegs<BITS, D, G> &t) {
-        // ---- scores -------------------------------------------------------------
-        f4 sacc[G];
-#pragma unroll
-        for (int g = 0; g < G; ++g) sacc[g] = f4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int u = 0; u < 4; ++u)
-#pragma unroll
-            for (int s = 0; s < S; ++s) {
-                const int g = Q ? (32 * s) / GS : 0;
-                Op qa;
-                qa.v = qlds[u][s][lane];
-                sacc[g] = mfma<BF>(qa, to_operand<BITS>(t.k[u][s]), sacc[g]);
-            }
-        float sc[4];
+    auto compute_tile = [&](const T &t) {
         const bool live = t.row >= 0;
+        // ---- QK^T: scores of token `lane` for every query row ---------------------------
+        f4 sacc[RG][G];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float s_;
-            if (Q) {
-                s_ = 0.f;
+        for (int rg = 0; rg < RG; ++rg)
 #pragma unroll
-                for (int g = 0; g < G; ++g) s_ += (t.ks[g] * TWO24) * sacc[g][i] + t.kb[g] * qsum[g][i];
+            for (int g = 0; g < G; ++g) sacc[rg][g] = f4{0.f, 0.f, 0.f, 0.f};
+        static_for<T::KW>([&](auto W) {
+            constexpr int w = decltype(W)::value;
+            constexpr int g = (w * GEO::EPW) / GS;
+            Op o[GEO::WSTEPS];
+            GEO::unpack(t.k[w], o);
+            static_for<GEO::WSTEPS>([&](auto H) {
+                constexpr int h = decltype(H)::value;
+                constexpr int step = w * GEO::WSTEPS + h;
+#pragma unroll
+                for (int rg = 0; rg < RG; ++rg)
+                    sacc[rg][g] = mfma444<step % 16>(qa[rg][step / 16], o[h], sacc[rg][g]);
+            });
+        });
+
+        // ---- online softmax per row group; probabilities become PV A operands ------------
+        Op pa[RG][G];
+#pragma unroll
+        for (int rg = 0; rg < RG; ++rg) {
+            float sc[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float s_ = 0.f;
+#pragma unroll
+                for (int g = 0; g < G; ++g) s_ += (t.ks[g] * TWO24) * sacc[rg][g][i] + t.kb[g] * qsum[rg][g][i];
                 s_ = round_dt<DT>(s_);
-            } else {
-                s_ = sacc[0][i] * a.scale;
-            }
-            if (live && i < R && a.mask.mode != KVHIP_MASK_NONE) {
-                const int rep = i / a.L, l = i - rep * a.L;
-                float add;
-                const bool keep = mask_keep(a.mask, b, hk * r + rep, l, t.row, a.L, a.T, add);
-                if (Q) {
+                const int row_i = 4 * rg + i;
+                if (a.mask.mode != KVHIP_MASK_NONE && live && row_i < R) {
+                    const int rep = row_i / a.L, l = row_i - rep * a.L;
+                    float add;
+                    const bool keep = mask_keep(a.mask, b, hk * r + rep, l, t.row, a.L, a.T, add);
                     if (!keep) s_ = fill;
                     else if (a.mask.mode == KVHIP_MASK_ARRAY && a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
-                } else {
-                    s_ = keep ? s_ + add : -INFINITY;
+                }
+                sc[i] = live ? s_ : -INFINITY;
+            }
+            // raise the running maximum only when this tile exceeds it
+            bool need = false;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) need = need || (sc[i] > m_run[rg][i]);
+            if (__any(need)) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float mn = fmaxf(m_run[rg][i], wave_max(sc[i]));
+                    const float alpha = (mn == -INFINITY) ? 1.f : fast_exp2((m_run[rg][i] - mn) * LOG2E);
+                    m_run[rg][i] = mn;
+                    l_part[rg][i] *= alpha;
+#pragma unroll
+                    for (int g = 0; g < G; ++g) bacc[rg][g][i] *= alpha;
+#pragma unroll
+                    for (int h = 0; h < NH; ++h) oacc[rg][h][i] *= alpha;
                 }
             }
-            sc[i] = live ? s_ : -INFINITY;
-        }
-        // ---- online softmax: raise the running maximum only when a tile exceeds it
-        bool need = false;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) need = need || (sc[i] > m_run[i]);
-        if (__any(need)) {
+            uint32_t x[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float mn = fmaxf(m_run[i], wave_max(sc[i]));
-                const float alpha = (mn == -INFINITY) ? 1.f : exp2f((m_run[i] - mn) * LOG2E);
-                m_run[i] = mn;
-                l_part[i] *= alpha;
+                const float p = (sc[i] == -INFINITY) ? 0.f : fast_exp2((sc[i] - m_run[rg][i]) * LOG2E);
+                l_part[rg][i] += p;
+                float pv[2] = {0.f, 0.f};
 #pragma unroll
-                for (int g = 0; g < G; ++g) bacc[g][i] *= alpha;
-#pragma unroll
-                for (int tt = 0; tt < NT; ++tt) oacc[tt][i] *= alpha;
-            }
-        }
-        float p[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            p[i] = (sc[i] == -INFINITY) ? 0.f : exp2f((sc[i] - m_run[i]) * LOG2E);
-            l_part[i] += p[i];
-        }
-        // ---- stage P (x per-token V scale) into LDS in A-operand order --------------
-#pragma unroll
-        for (int g = 0; g < G; ++g)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if (Q) {
-                    bacc[g][i] += p[i] * t.vb[g];
-                    pbuf[wave][0][g][i][ppos] = f2h_bits(p[i] * (t.vs[g] * vfac));
-                } else if (BF) {
-                    const uint16_t hi = f2bf_bits(p[i]);
-                    const float rest = p[i] - __uint_as_float((uint32_t)hi << 16);
-                    pbuf[wave][0][g][i][ppos] = hi;
-                    pbuf[wave][1][g][i][ppos] = f2bf_bits(rest);
-                } else {
-                    pbuf[wave][0][g][i][ppos] = f2h_bits(p[i]);
+                for (int g = 0; g < G; ++g) {
+                    bacc[rg][g][i] += p * t.vb[g];
+                    pv[g] = p * (t.vs[g] * vfac);
                 }
+                x[i] = pack_h2(pv[0], pv[1]);
             }
-        __builtin_amdgcn_wave_barrier();
-        // ---- out += P . V ---------------------------------------------------------------
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk) {
-            Op pa[G], pl[G];
-#pragma unroll
-            for (int g = 0; g < G; ++g) {
-                pa[g].v = *reinterpret_cast<const uint4 *>(&pbuf[wave][0][g][n & 3][blk * 32 + 8 * j]);
-                if (BF) pl[g].v = *reinterpret_cast<const uint4 *>(&pbuf[wave][1][g][n & 3][blk * 32 + 8 * j]);
-            }
-#pragma unroll
-            for (int dt = 0; dt < NT; ++dt) {
-                const int g = Q ? (16 * dt) / GS : 0;
-                const Op vb_ = to_operand<BITS>(t.v[blk][dt]);
-                oacc[dt] = mfma<BF>(pa[g], vb_, oacc[dt]);
-                if (BF) oacc[dt] = mfma<BF>(pl[g], vb_, oacc[dt]);
+            // lane (blk, i) now gets, in x[k], row i's value for token 4 blk + k
+            quad_transpose(x, lane);
+            pa[rg][0].u[0] = __builtin_amdgcn_perm(x[1], x[0], 0x05040100u);
+            pa[rg][0].u[1] = __builtin_amdgcn_perm(x[3], x[2], 0x05040100u);
+            if (G > 1) {
+                pa[rg][G - 1].u[0] = __builtin_amdgcn_perm(x[1], x[0], 0x07060302u);
+                pa[rg][G - 1].u[1] = __builtin_amdgcn_perm(x[3], x[2], 0x07060302u);
             }
         }
-        __builtin_amdgcn_wave_barrier();
+
+        // ---- out += P . V: lane supplies column lane (+64 h), step s = tokens 4s..4s+3 ------
+        static_for<NH>([&](auto HH) {
+            constexpr int h = decltype(HH)::value;
+            constexpr int g = (64 * h) / GS;
+            static_for<T::VW>([&](auto W) {
+                constexpr int w = decltype(W)::value;
+                Op o[GEO::WSTEPS];
+                GEO::unpack(t.v[h][w], o);
+                static_for<GEO::WSTEPS>([&](auto S2) {
+                    constexpr int s = w * GEO::WSTEPS + decltype(S2)::value;
+#pragma unroll
+                    for (int rg = 0; rg < RG; ++rg)
+                        oacc[rg][h] = mfma444<s>(pa[rg][g], o[decltype(S2)::value], oacc[rg][h]);
+                });
+            });
+        });
     };
 
-    // ---- main loop: this wavefront takes every WAVES-th tile of the span, one tile
-    // of loads in flight ahead of the arithmetic
-    // (variants whose tile does not fit twice in the register file run single-buffered
-    // and lean on the second resident wavefront to cover the load latency)
-    constexpr bool PREFETCH = !(D == 128 && (BITS == 8 || G > 2));
+    // ---- main loop: this wavefront takes every WAVES-th tile of the span, one tile of
+    // loads in flight ahead of the arithmetic (variants whose tile does not fit twice in
+    // the register file run single-buffered and lean on the other resident wavefronts)
+    constexpr bool PREFETCH = (RG == 1 && !(BITS == 8 && D == 128)) || (RG == 2 && BITS == 4 && D == 64);
     if constexpr (PREFETCH) {
-        TileRegs<BITS, D, G> bufA, bufB;
+        T bufA, bufB;
         int tile = tile_begin + wave;
         if (tile < tile_end) load_tile(tile, bufA);
         while (tile < tile_end) {
@@ -370,7 +406,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             tile = next2;
         }
     } else {
-        TileRegs<BITS, D, G> buf;
+        T buf;
         for (int tile = tile_begin + wave; tile < tile_end; tile += WAVES) {
             load_tile(tile, buf);
             compute_tile(buf);
@@ -379,31 +415,30 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 
     // ---- wavefront partial -> LDS ---------------------------------------------------
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        l_part[i] = wave_sum(l_part[i]);
+    for (int rg = 0; rg < RG; ++rg) {
 #pragma unroll
-        for (int g = 0; g < G; ++g) bacc[g][i] = wave_sum(bacc[g][i]);
-    }
-    if (j == 0) {
+        for (int i = 0; i < 4; ++i) {
+            l_part[rg][i] = wave_sum(l_part[rg][i]);
 #pragma unroll
-        for (int dt = 0; dt < NT; ++dt) {
-            const int g = Q ? (16 * dt) / GS : 0;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float o = oacc[dt][i];
-                if (Q) o = o * TWO24 + bacc[g][i];
-                cbuf[wave][i][16 * dt + n] = o;
-            }
+            for (int g = 0; g < G; ++g) bacc[rg][g][i] = wave_sum(bacc[rg][g][i]);
         }
-    }
-    if (lane < 4) {
-        cbuf[wave][lane][D] = m_run[lane];
-        cbuf[wave][lane][D + 1] = l_part[lane];
+#pragma unroll
+        for (int h = 0; h < NH; ++h) {
+            constexpr int dummy = 0;
+            (void)dummy;
+            const int g = (64 * h) / GS;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) cbuf[wave][4 * rg + i][64 * h + lane] = oacc[rg][h][i] * TWO24 + bacc[rg][g][i];
+        }
+        if (lane < 4) {
+            cbuf[wave][4 * rg + lane][D] = m_run[rg][lane];
+            cbuf[wave][4 * rg + lane][D + 1] = l_part[rg][lane];
+        }
     }
     __syncthreads();
     // ---- merge the 4 wavefronts, write the span's partial ------------------------------
-    float *part = a.workspace + ((size_t)bh * nsplit + split) * 4 * (D + 2);
-    for (int idx = threadIdx.x; idx < 4 * (D + 2); idx += WAVES * 64) {
+    float *part = a.workspace + ((size_t)bh * nsplit + split) * RR * (D + 2);
+    for (int idx = threadIdx.x; idx < RR * (D + 2); idx += WAVES * 64) {
         const int i = idx / (D + 2), c = idx - i * (D + 2);
         float mx = -INFINITY;
 #pragma unroll
@@ -416,7 +451,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 #pragma unroll
             for (int w = 0; w < WAVES; ++w) {
                 const float mw = cbuf[w][i][D];
-                const float wgt = (mw == -INFINITY) ? 0.f : exp2f((mw - mx) * LOG2E);
+                const float wgt = (mw == -INFINITY) ? 0.f : fast_exp2((mw - mx) * LOG2E);
                 v += wgt * cbuf[w][i][c];
             }
         }
@@ -427,20 +462,21 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 // grid (R, BH): merge the span partials of one query row and write the output row
 template <int D, int DT>
 __global__ void __launch_bounds__(D)
-combine_kernel(AttendArgs a, int nsplit) {
+combine_kernel(AttendArgs a, int nsplit, int rr) {
     const int i = blockIdx.x, bh = blockIdx.y;
     const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
     const int r = a.Hq / a.Hkv;
     const int rep = i / a.L, l = i - rep * a.L;
-    const float *part = a.workspace + (size_t)bh * nsplit * 4 * (D + 2) + (size_t)i * (D + 2);
+    const size_t sstride = (size_t)rr * (D + 2);
+    const float *part = a.workspace + (size_t)bh * nsplit * sstride + (size_t)i * (D + 2);
     const int d = threadIdx.x;
     float mx = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, part[(size_t)s * 4 * (D + 2) + D]);
+    for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, part[s * sstride + D]);
     float num = 0.f, den = 0.f;
     for (int s = 0; s < nsplit; ++s) {
-        const float *p = part + (size_t)s * 4 * (D + 2);
+        const float *p = part + s * sstride;
         const float mw = p[D];
-        const float w = (mw == -INFINITY) ? 0.f : exp2f((mw - mx) * LOG2E);
+        const float w = (mw == -INFINITY) ? 0.f : fast_exp2((mw - mx) * LOG2E);
         num += w * p[d];
         den += w * p[D + 1];
     }
@@ -449,12 +485,14 @@ combine_kernel(AttendArgs a, int nsplit) {
 }
 
 struct Plan {
-    int tiles_total, tiles_per_wg, nsplit;
+    int tiles_total, tiles_per_wg, nsplit, rg;
 };
 
 Plan plan_for(const AttendArgs &a) {
     Plan p;
     p.tiles_total = (a.slots + TILE - 1) / TILE;
+    const int R = (a.Hq / a.Hkv) * a.L;
+    p.rg = R <= 4 ? 1 : (R <= 8 ? 2 : 4);
     const int BH = a.st.BH;
     // enough workgroups to fill 256 CUs several times over; a span is a multiple of
     // WAVES tiles so every wavefront of a workgroup gets the same share
@@ -468,11 +506,9 @@ Plan plan_for(const AttendArgs &a) {
     return p;
 }
 
-}  // namespace
-
-namespace {
 bool g_profile = false;
 std::vector<hipEvent_t> g_events;  // begin/end pairs
+
 }  // namespace
 
 void profile_enable(bool on) { g_profile = on; }
@@ -507,16 +543,16 @@ bool attend_decode_supported(const AttendArgs &a) {
     if (s.dtype != KVHIP_F16 && s.dtype != KVHIP_BF16) return false;
     if (s.Dk != s.Dv) return false;
     const int R = (a.Hq / a.Hkv) * a.L;
-    if (R > 4) return false;
-    if (s.bits == 0) return false;  // full-precision caches: generic kernel for now
-    if (s.bits != 4 && s.bits != 8) return false;
-    if (s.Dk != 64 && s.Dk != 128) return false;
-    return s.gs == 32 || s.gs == 64 || (s.gs == 128 && s.Dk == 128);
+    if (R > 16) return false;
+    if (s.bits != 4 && s.bits != 8) return false;  // full-precision caches: other kernels
+    if (s.Dk == 64) return s.gs == 64;
+    if (s.Dk == 128) return s.gs == 64 || s.gs == 128;
+    return false;
 }
 
 size_t attend_decode_workspace(const AttendArgs &a) {
     const Plan p = plan_for(a);
-    return (size_t)a.st.BH * p.nsplit * 4 * (a.st.Dk + 2) * sizeof(float);
+    return (size_t)a.st.BH * p.nsplit * 4 * p.rg * (a.st.Dk + 2) * sizeof(float);
 }
 
 hipError_t launch_attend_decode(const AttendArgs &a, hipStream_t s) {
@@ -524,35 +560,37 @@ hipError_t launch_attend_decode(const AttendArgs &a, hipStream_t s) {
     const Store &st = a.st;
     dim3 grid(p.nsplit, st.BH), block(WAVES * 64);
     const int R = (a.Hq / a.Hkv) * a.L;
-#define DEC(BITS, D, GS, DT)                                                                              \
+#define DEC(BITS, D, GS, DT, RG)                                                                          \
     do {                                                                                                  \
         profile_mark(s, true);                                                                            \
-        hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT>), grid, block, 0, s, a, p.tiles_total,         \
+        hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG>), grid, block, 0, s, a, p.tiles_total,     \
                            p.tiles_per_wg, p.nsplit);                                                     \
         profile_mark(s, false);                                                                           \
-        hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit);   \
+        hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG);  \
     } while (0)
-#define DEC_DT(BITS, D, GS)                      \
-    do {                                         \
-        if (st.dtype == KVHIP_F16) DEC(BITS, D, GS, 0); \
-        else DEC(BITS, D, GS, 1);                \
+#define DEC_RG(BITS, D, GS, DT)                       \
+    do {                                              \
+        if (p.rg == 1) DEC(BITS, D, GS, DT, 1);       \
+        else if (p.rg == 2) DEC(BITS, D, GS, DT, 2);  \
+        else DEC(BITS, D, GS, DT, 4);                 \
     } while (0)
-#define DEC_Q(BITS)                                               \
-    do {                                                          \
-        if (st.Dk == 64) {                                        \
-            if (st.gs == 32) DEC_DT(BITS, 64, 32);                \
-            else DEC_DT(BITS, 64, 64);                            \
-        } else {                                                  \
-            if (st.gs == 32) DEC_DT(BITS, 128, 32);               \
-            else if (st.gs == 64) DEC_DT(BITS, 128, 64);          \
-            else DEC_DT(BITS, 128, 128);                          \
-        }                                                         \
+#define DEC_DT(BITS, D, GS)                                \
+    do {                                                   \
+        if (st.dtype == KVHIP_F16) DEC_RG(BITS, D, GS, 0); \
+        else DEC_RG(BITS, D, GS, 1);                       \
+    } while (0)
+#define DEC_Q(BITS)                                 \
+    do {                                            \
+        if (st.Dk == 64) DEC_DT(BITS, 64, 64);      \
+        else if (st.gs == 64) DEC_DT(BITS, 128, 64); \
+        else DEC_DT(BITS, 128, 128);                \
     } while (0)
     if (st.bits == 4) DEC_Q(4);
     else if (st.bits == 8) DEC_Q(8);
     else return hipErrorNotSupported;
 #undef DEC_Q
 #undef DEC_DT
+#undef DEC_RG
 #undef DEC
     return hipGetLastError();
 }

@@ -28,12 +28,6 @@ __device__ __forceinline__ float block_reduce(float v, bool is_max, float *red) 
     return r;
 }
 
-template <int BITS> __device__ __forceinline__ uint32_t v_code(const char *cell, int unit, int e) {
-    if (BITS == 4) return (reinterpret_cast<const uint32_t *>(cell)[unit] >> (4 * e)) & 15u;
-    if (BITS == 8) return reinterpret_cast<const uint8_t *>(cell)[(size_t)unit * 8 + e];
-    return (reinterpret_cast<const uint16_t *>(cell)[unit] >> (2 * e)) & 3u;
-}
-
 // grid (L, Hq, B)
 template <int DT, int BITS>
 __global__ void __launch_bounds__(GT)
@@ -66,14 +60,16 @@ attend_generic_kernel(AttendArgs a, int slots_pad) {
             float sum = 0.f;
             if (Q) {
                 constexpr int per = 32 / BB;
-                const uint32_t *w = reinterpret_cast<const uint32_t *>(k_row_ptr(st, bh, slot));
+                const uint32_t *krow = reinterpret_cast<const uint32_t *>(k_row_ptr(st, bh, slot));
                 const char *sb = ksb_row_ptr(st, bh, slot);
                 for (int g = 0; g < st.Dk / st.gs; ++g) {
                     const float sc = Elem<DT>::load(sb, 2 * g), bi = Elem<DT>::load(sb, 2 * g + 1);
-                    for (int jj = 0; jj < st.gs; ++jj) {
-                        const int d = g * st.gs + jj;
-                        const uint32_t c = (w[d / per] >> ((d % per) * BB)) & ((1u << BB) - 1u);
-                        sum += qs[d] * (sc * (float)c + bi);
+                    for (int w0 = g * st.gs / per; w0 < (g + 1) * st.gs / per; ++w0) {
+                        const uint32_t word = krow[w0];
+                        for (int i = 0; i < per; ++i) {
+                            const uint32_t c = (word >> (i * BB)) & ((1u << BB) - 1u);
+                            sum += qs[w0 * per + i] * (sc * (float)c + bi);
+                        }
                     }
                 }
                 s = round_dt<DT>(sum);
@@ -115,25 +111,22 @@ attend_generic_kernel(AttendArgs a, int slots_pad) {
     // ---- out = p . V^ ---------------------------------------------------------
     for (int d = threadIdx.x; d < st.Dv; d += GT) {
         float acc = 0.f;
-        for (int blk = 0; blk * 32 < slots_pad; ++blk) {
-            const char *cell = v_cell_ptr(st, bh, blk * 32);
-            const int bip = ((blk * 32) & (PAGE - 1)) >> 5;
-            for (int j = 0; j < 4; ++j) {
-                const int unit = (bip * 4 + j) * st.Dv + d;
-                for (int e = 0; e < 8; ++e) {
-                    const int slot = blk * 32 + 4 * j + (e & 3) + 16 * (e >> 2);
-                    const float w = p[slot];
-                    if (w == 0.f) continue;
-                    float v;
-                    if (Q) {
-                        const char *sb = vsb_row_ptr(st, bh, slot);
-                        const int g = d / st.gs;
-                        v = Elem<DT>::load(sb, 2 * g) * (float)v_code<BB>(cell, unit, e) + Elem<DT>::load(sb, 2 * g + 1);
-                    } else {
-                        v = Elem<DT>::load(cell, (size_t)unit * 8 + e);
-                    }
-                    acc += w * v;
+        for (int slot0 = 0; slot0 < slots_pad; slot0 += TILE) {
+            const char *vrow = v_cell_ptr(st, bh, slot0) + v_row_off(st, slot0, d);
+            const int nt = min(TILE, slots_pad - slot0);
+            for (int t = 0; t < nt; ++t) {
+                const int slot = slot0 + t;
+                const float w = p[slot];
+                if (w == 0.f) continue;
+                float v;
+                if (Q) {
+                    const char *sb = vsb_row_ptr(st, bh, slot);
+                    const int g = d / st.gs;
+                    v = Elem<DT>::load(sb, 2 * g) * (float)v_code_load<BB>(vrow, t) + Elem<DT>::load(sb, 2 * g + 1);
+                } else {
+                    v = Elem<DT>::load(vrow, t);
                 }
+                acc += w * v;
             }
         }
         Elem<DT>::store(a.out, qrow * st.Dv + d, acc);

@@ -17,20 +17,25 @@ namespace kvhip {
 // page-major: [page][b*Hkv + h][PAGE rows].  Growing a cache appends pages;
 // nothing already written moves relative to its page.
 //
-//  K plane   rows in natural order: row s of a page holds Dk elements (fp) or
-//            Dk*bits/32 packed uint32 words in MLX's order (quantized).
-//  V plane   "octet transposed" so that the PV contraction can feed matrix-core
-//            operands without shuffles.  A page is 8 blocks of 32 tokens.  In a
-//            block, token tl (0..31) belongs to octet j = (tl & 15) >> 2 at
-//            position e = (tl & 3) + 4 * (tl >> 4); for every (block, j, d) the
-//            8 values of the octet are contiguous:
-//              fp        8 elements                     (16 B for 16-bit types)
-//              quantized 8 codes of `bits` bits, LSB first (one uint32 at 4 bits)
-//            unit index inside a page = (block * 4 + j) * Dv + d.
+//  K plane   one row per token in the reference's own order: Dk elements (full
+//            precision) or Dk*bits/32 packed uint32 words in MLX's bit order.  A
+//            wavefront lane that owns one token reads its whole row as vectors.
+//  V plane   transposed per tile of TILE = 64 tokens, so that the PV contraction
+//            reads, for one head-dim column, the values of consecutive tokens as
+//            one vector: a page cell is [tile 0..3][d 0..Dv-1][64 tokens].
+//              full precision  64 elements, token t at index t
+//              8 bit   16 words; word t >> 2 holds tokens 4q..4q+3 at byte
+//                      positions {0, 2, 1, 3}
+//              4 bit   8 words; word t >> 3 holds an octet of tokens at nibble
+//                      positions {0, 4, 1, 5, 2, 6, 3, 7}
+//              2 bit   4 words; word t >> 4, token t & 15 at bits [2(t&15), +2)
+//            The 4/8-bit positions are the order in which a masked word splits into
+//            fp16 operand pairs (see kvhip_attend_decode.hip).
 //  sb planes per row and group one (scale, bias) pair of the cache dtype.
 // ---------------------------------------------------------------------------
 constexpr int PAGE = 256;
 constexpr int PAGE_SHIFT = 8;
+constexpr int TILE = 64;       // tokens per V tile; 4 tiles per page
 constexpr int MAXRUNS = 8;
 
 struct Store {
@@ -83,15 +88,20 @@ __device__ __forceinline__ const char *vsb_row_ptr(const Store &st, int bh, int 
 __device__ __forceinline__ const char *v_cell_ptr(const Store &st, int bh, int slot) {
     return st.v + ((size_t)(slot >> PAGE_SHIFT) * st.BH + bh) * st.v_cell;
 }
-// octet coordinates of a slot inside its page
-__device__ __forceinline__ int v_unit_base(int slot, int Dv) {  // (block*4 + j) * Dv
-    const int s = slot & (PAGE - 1);
-    const int tl = s & 31;
-    return (((s >> 5) << 2) + ((tl & 15) >> 2)) * Dv;
+// bit position of token t (0..63 inside its tile) within the V tile row of a column
+template <int BITS> __device__ __forceinline__ int v_bitpos(int t) {
+    if (BITS == 4) return 32 * (t >> 3) + 4 * (((t & 7) >> 1) + 4 * (t & 1));
+    if (BITS == 8) return 32 * (t >> 2) + 8 * (((t & 3) >> 1) + 2 * (t & 1));
+    return 2 * t;  // BITS == 2
 }
-__device__ __forceinline__ int v_pos(int slot) {
-    const int tl = slot & 31;
-    return (tl & 3) + ((tl >> 4) << 2);
+// byte offset, inside the page cell, of the V tile row (tile of `slot`, column d)
+__device__ __forceinline__ size_t v_row_off(const Store &st, int slot, int d) {
+    const size_t row_bytes = st.bits ? (size_t)TILE * st.bits / 8 : (size_t)TILE * st.es;
+    return ((size_t)((slot & (PAGE - 1)) >> 6) * st.Dv + d) * row_bytes;
+}
+template <int BITS> __device__ __forceinline__ uint32_t v_code_load(const char *vrow, int t) {
+    const int bp = v_bitpos<BITS>(t);
+    return (reinterpret_cast<const uint32_t *>(vrow)[bp >> 5] >> (bp & 31)) & ((1u << BITS) - 1u);
 }
 // presented row of a physical slot, or -1
 __device__ __forceinline__ int slot_to_row(const Runs &r, int slot) {

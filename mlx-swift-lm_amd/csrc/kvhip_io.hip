@@ -7,12 +7,6 @@ namespace kvhip {
 
 namespace {
 
-template <int BITS> __device__ __forceinline__ uint32_t read_v_code(const char *cell, int unit, int e) {
-    if (BITS == 4) return (reinterpret_cast<const uint32_t *>(cell)[unit] >> (4 * e)) & 15u;
-    if (BITS == 8) return reinterpret_cast<const uint8_t *>(cell)[(size_t)unit * 8 + e];
-    return (reinterpret_cast<const uint16_t *>(cell)[unit] >> (2 * e)) & 3u;
-}
-
 // One wavefront quantizes one row of D elements.  Optional outputs:
 //   k_words   packed codes in MLX order (D*BITS/32 words)
 //   code_out  one byte per element (for the transposed V assembly)
@@ -78,23 +72,23 @@ __global__ void append_fp_kernel(Store st, const char *keys, const char *values,
     E *kd = reinterpret_cast<E *>(const_cast<char *>(k_row_ptr(st, bh, slot)));
     for (int d = threadIdx.x; d < st.Dk; d += blockDim.x) kd[d] = ks[d];
     const E *vs = reinterpret_cast<const E *>(values) + ((size_t)bh * L + l) * st.Dv;
-    E *vd = reinterpret_cast<E *>(const_cast<char *>(v_cell_ptr(st, bh, slot)));
-    const int ub = v_unit_base(slot, st.Dv);
-    const int e = v_pos(slot);
-    for (int d = threadIdx.x; d < st.Dv; d += blockDim.x) vd[(size_t)(ub + d) * 8 + e] = vs[d];
+    char *vc = const_cast<char *>(v_cell_ptr(st, bh, slot));
+    const int t = slot & (TILE - 1);
+    for (int d = threadIdx.x; d < st.Dv; d += blockDim.x)
+        reinterpret_cast<E *>(vc + v_row_off(st, slot, d))[t] = vs[d];
 }
 
-// grid (32-token blocks touched, BH), 256 threads.  Each wavefront quantizes rows
-// of the block; V codes are staged as bytes in LDS and then merged into the
-// octet words, touching only the positions this append writes.
+// grid (64-token tiles touched, BH), 256 threads.  Each wavefront quantizes rows of
+// the tile; V codes are staged as bytes in LDS and then merged into the transposed
+// tile rows, touching only the token positions this append writes.
 template <int DT, int BITS>
 __global__ void __launch_bounds__(256)
 append_quant_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, int n) {
-    extern __shared__ uint8_t vcodes[];  // [32][Dv]
+    extern __shared__ uint8_t vcodes[];  // [64][Dv]
     const int bh = blockIdx.y;
-    const int blk = (slot0 >> 5) + blockIdx.x;
-    const int lo = max(slot0, blk * 32);
-    const int hi = min(slot0 + n, blk * 32 + 32);
+    const int tile = (slot0 >> 6) + blockIdx.x;
+    const int lo = max(slot0, tile * TILE);
+    const int hi = min(slot0 + n, tile * TILE + TILE);
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     for (int slot = lo + wave; slot < hi; slot += 4) {
@@ -104,38 +98,28 @@ append_quant_kernel(Store st, const char *keys, const char *values, int L, int s
         quantize_row_wave<DT, BITS>(krow, st.Dk, st.gs, lane,
                                     reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot))),
                                     nullptr, const_cast<char *>(ksb_row_ptr(st, bh, slot)), nullptr, nullptr);
-        quantize_row_wave<DT, BITS>(vrow, st.Dv, st.gs, lane, nullptr, vcodes + (slot & 31) * st.Dv,
+        quantize_row_wave<DT, BITS>(vrow, st.Dv, st.gs, lane, nullptr, vcodes + (slot & (TILE - 1)) * st.Dv,
                                     const_cast<char *>(vsb_row_ptr(st, bh, slot)), nullptr, nullptr);
     }
     __syncthreads();
-    char *cell = const_cast<char *>(v_cell_ptr(st, bh, blk * 32));
-    const int blk_in_page = ((blk * 32) & (PAGE - 1)) >> 5;
-    const int units = 4 * st.Dv;
-    for (int u = threadIdx.x; u < units; u += blockDim.x) {
-        const int j = u / st.Dv, d = u - j * st.Dv;
-        uint64_t nbits = 0, mbits = 0;
-        for (int e = 0; e < 8; ++e) {
-            const int tl = 4 * j + (e & 3) + 16 * (e >> 2);
-            const int slot = blk * 32 + tl;
-            if (slot >= lo && slot < hi) {
-                nbits |= (uint64_t)vcodes[tl * st.Dv + d] << (e * BITS);
-                mbits |= (uint64_t)((1u << BITS) - 1u) << (e * BITS);
+    char *cell = const_cast<char *>(v_cell_ptr(st, bh, lo));
+    constexpr int TPW = 32 / BITS;          // tokens per word
+    constexpr int WPR = TILE / TPW;         // words per tile row
+    const int t_lo = lo & (TILE - 1), t_hi = t_lo + (hi - lo);
+    for (int u = threadIdx.x; u < st.Dv * WPR; u += blockDim.x) {
+        const int d = u / WPR, w = u - d * WPR;
+        if ((w + 1) * TPW <= t_lo || w * TPW >= t_hi) continue;
+        uint32_t nbits = 0, mbits = 0;
+        for (int tt = 0; tt < TPW; ++tt) {
+            const int t = w * TPW + tt;
+            if (t >= t_lo && t < t_hi) {
+                const int bp = v_bitpos<BITS>(t) & 31;
+                nbits |= (uint32_t)vcodes[t * st.Dv + d] << bp;
+                mbits |= ((1u << BITS) - 1u) << bp;
             }
         }
-        if (mbits == 0) continue;
-        const int unit = (blk_in_page * 4 + j) * st.Dv + d;
-        if (BITS == 4) {
-            uint32_t *p = reinterpret_cast<uint32_t *>(cell) + unit;
-            const uint32_t m = (uint32_t)mbits;
-            *p = (m == 0xffffffffu) ? (uint32_t)nbits : ((*p & ~m) | (uint32_t)nbits);
-        } else if (BITS == 8) {
-            uint64_t *p = reinterpret_cast<uint64_t *>(cell) + unit;
-            *p = (mbits == ~0ull) ? nbits : ((*p & ~mbits) | nbits);
-        } else {
-            uint16_t *p = reinterpret_cast<uint16_t *>(cell) + unit;
-            const uint16_t m = (uint16_t)mbits;
-            *p = (uint16_t)((*p & ~m) | (uint16_t)nbits);
-        }
+        uint32_t *p = reinterpret_cast<uint32_t *>(cell + v_row_off(st, lo, d)) + w;
+        *p = (mbits == 0xffffffffu) ? nbits : ((*p & ~mbits) | nbits);
     }
 }
 
@@ -152,11 +136,11 @@ __global__ void export_fp_kernel(Store st, Runs runs, int row_begin, int dst_row
         for (int d = threadIdx.x; d < st.Dk; d += blockDim.x) kd[d] = ks[d];
     }
     if (dst_v) {
-        const E *vs = reinterpret_cast<const E *>(v_cell_ptr(st, bh, slot));
+        const char *vc = v_cell_ptr(st, bh, slot);
         E *vd = reinterpret_cast<E *>(dst_v) + ((size_t)bh * nrows + i) * st.Dv;
-        const int ub = v_unit_base(slot, st.Dv);
-        const int e = v_pos(slot);
-        for (int d = threadIdx.x; d < st.Dv; d += blockDim.x) vd[d] = vs[(size_t)(ub + d) * 8 + e];
+        const int t = slot & (TILE - 1);
+        for (int d = threadIdx.x; d < st.Dv; d += blockDim.x)
+            vd[d] = reinterpret_cast<const E *>(vc + v_row_off(st, slot, d))[t];
     }
 }
 
@@ -169,10 +153,10 @@ __global__ void import_fp_kernel(Store st, const char *src_k, const char *src_v,
     E *kd = reinterpret_cast<E *>(const_cast<char *>(k_row_ptr(st, bh, slot)));
     for (int d = threadIdx.x; d < st.Dk; d += blockDim.x) kd[d] = ks[d];
     const E *vs = reinterpret_cast<const E *>(src_v) + ((size_t)bh * nrows + slot) * st.Dv;
-    E *vd = reinterpret_cast<E *>(const_cast<char *>(v_cell_ptr(st, bh, slot)));
-    const int ub = v_unit_base(slot, st.Dv);
-    const int e = v_pos(slot);
-    for (int d = threadIdx.x; d < st.Dv; d += blockDim.x) vd[(size_t)(ub + d) * 8 + e] = vs[d];
+    char *vc = const_cast<char *>(v_cell_ptr(st, bh, slot));
+    const int t = slot & (TILE - 1);
+    for (int d = threadIdx.x; d < st.Dv; d += blockDim.x)
+        reinterpret_cast<E *>(vc + v_row_off(st, slot, d))[t] = vs[d];
 }
 
 template <int ES>
@@ -185,11 +169,11 @@ __global__ void compact_fp_kernel(Store src, Runs runs, Store dst, int nrows) {
     const E *ks = reinterpret_cast<const E *>(k_row_ptr(src, bh, slot));
     E *kd = reinterpret_cast<E *>(const_cast<char *>(k_row_ptr(dst, bh, i)));
     for (int d = threadIdx.x; d < src.Dk; d += blockDim.x) kd[d] = ks[d];
-    const E *vs = reinterpret_cast<const E *>(v_cell_ptr(src, bh, slot));
-    E *vd = reinterpret_cast<E *>(const_cast<char *>(v_cell_ptr(dst, bh, i)));
-    const int ubs = v_unit_base(slot, src.Dv), es = v_pos(slot);
-    const int ubd = v_unit_base(i, src.Dv), ed = v_pos(i);
-    for (int d = threadIdx.x; d < src.Dv; d += blockDim.x) vd[(size_t)(ubd + d) * 8 + ed] = vs[(size_t)(ubs + d) * 8 + es];
+    const char *vs = v_cell_ptr(src, bh, slot);
+    char *vd = const_cast<char *>(v_cell_ptr(dst, bh, i));
+    const int ts = slot & (TILE - 1), td = i & (TILE - 1);
+    for (int d = threadIdx.x; d < src.Dv; d += blockDim.x)
+        reinterpret_cast<E *>(vd + v_row_off(dst, i, d))[td] = reinterpret_cast<const E *>(vs + v_row_off(src, slot, d))[ts];
 }
 
 // which: 0 k.wq 1 k.scales 2 k.biases 3 v.wq 4 v.scales 5 v.biases; grid (nrows, BH)
@@ -207,11 +191,12 @@ __global__ void export_quant_kernel(Store st, int which, int nrows, char *dst) {
         constexpr int per = 32 / BITS;
         const int W = st.Dv / per;
         const char *cell = v_cell_ptr(st, bh, slot);
-        const int ub = v_unit_base(slot, st.Dv), e = v_pos(slot);
+        const int t = slot & (TILE - 1);
         uint32_t *d = reinterpret_cast<uint32_t *>(dst) + ((size_t)bh * nrows + slot) * W;
         for (int w = threadIdx.x; w < W; w += blockDim.x) {
             uint32_t word = 0;
-            for (int i = 0; i < per; ++i) word |= read_v_code<BITS>(cell, ub + w * per + i, e) << (i * BITS);
+            for (int i = 0; i < per; ++i)
+                word |= v_code_load<BITS>(cell + v_row_off(st, slot, w * per + i), t) << (i * BITS);
             d[w] = word;
         }
     } else {
@@ -229,13 +214,12 @@ __global__ void export_quant_kernel(Store st, int which, int nrows, char *dst) {
     }
 }
 
-// grid (32-token blocks, BH): dense reference arrays into slots [0, nrows)
+// grid (64-token tiles, BH): dense reference arrays into slots [0, nrows)
 template <int BITS>
 __global__ void import_quant_kernel(Store st, const uint32_t *kw, const char *ks, const char *kb,
                                     const uint32_t *vw, const char *vs, const char *vb, int nrows) {
     const int bh = blockIdx.y;
-    const int blk = blockIdx.x;
-    const int lo = blk * 32, hi = min(nrows, lo + 32);
+    const int lo = blockIdx.x * TILE, hi = min(nrows, lo + TILE);
     const int es = st.es;
     constexpr int per = 32 / BITS;
     const int Wk = st.Dk / per, Wv = st.Dv / per, Gk = st.Dk / st.gs, Gv = st.Dv / st.gs;
@@ -265,22 +249,19 @@ __global__ void import_quant_kernel(Store st, const uint32_t *kw, const char *ks
         }
     }
     char *cell = const_cast<char *>(v_cell_ptr(st, bh, lo));
-    const int blk_in_page = (lo & (PAGE - 1)) >> 5;
-    const int units = 4 * st.Dv;
-    for (int u = threadIdx.x; u < units; u += blockDim.x) {
-        const int j = u / st.Dv, d = u - j * st.Dv;
-        uint64_t nbits = 0;
-        for (int e = 0; e < 8; ++e) {
-            const int slot = lo + 4 * j + (e & 3) + 16 * (e >> 2);
-            if (slot < hi) {
-                const uint32_t word = vw[((size_t)bh * nrows + slot) * Wv + d / per];
-                nbits |= (uint64_t)((word >> ((d % per) * BITS)) & ((1u << BITS) - 1u)) << (e * BITS);
+    constexpr int TPW = 32 / BITS;
+    constexpr int WPR = TILE / TPW;
+    for (int u = threadIdx.x; u < st.Dv * WPR; u += blockDim.x) {
+        const int d = u / WPR, w = u - d * WPR;
+        uint32_t nbits = 0;
+        for (int tt = 0; tt < TPW; ++tt) {
+            const int t = w * TPW + tt;
+            if (lo + t < hi) {
+                const uint32_t word = vw[((size_t)bh * nrows + lo + t) * Wv + d / per];
+                nbits |= ((word >> ((d % per) * BITS)) & ((1u << BITS) - 1u)) << (v_bitpos<BITS>(t) & 31);
             }
         }
-        const int unit = (blk_in_page * 4 + j) * st.Dv + d;
-        if (BITS == 4) reinterpret_cast<uint32_t *>(cell)[unit] = (uint32_t)nbits;
-        else if (BITS == 8) reinterpret_cast<uint64_t *>(cell)[unit] = nbits;
-        else reinterpret_cast<uint16_t *>(cell)[unit] = (uint16_t)nbits;
+        reinterpret_cast<uint32_t *>(cell + v_row_off(st, lo, d))[w] = nbits;
     }
 }
 
@@ -350,9 +331,9 @@ hipError_t launch_append_fp(const Store &st, const void *keys, const void *value
 hipError_t launch_append_quant(const Store &st, const void *keys, const void *values, int L, int src0,
                                int slot0, int n, hipStream_t s) {
     if (n <= 0) return hipSuccess;
-    const int nblk = ((slot0 + n - 1) >> 5) - (slot0 >> 5) + 1;
-    dim3 grid(nblk, st.BH), block(256);
-    const size_t lds = (size_t)32 * st.Dv;
+    const int ntile = ((slot0 + n - 1) >> 6) - (slot0 >> 6) + 1;
+    dim3 grid(ntile, st.BH), block(256);
+    const size_t lds = (size_t)TILE * st.Dv;
 #define CALL(DT, BITS)                                                                           \
     hipLaunchKernelGGL((append_quant_kernel<DT, BITS>), grid, block, lds, s, st, (const char *)keys, \
                        (const char *)values, L, src0, slot0, n)
@@ -403,7 +384,7 @@ hipError_t launch_export_quant(const Store &st, int which, int nrows, void *dst,
 
 hipError_t launch_import_quant(const Store &st, const void *const srcs[6], int nrows, hipStream_t s) {
     if (nrows <= 0) return hipSuccess;
-    dim3 grid((nrows + 31) / 32, st.BH), block(256);
+    dim3 grid((nrows + TILE - 1) / TILE, st.BH), block(256);
 #define IMP(BITS)                                                                                     \
     hipLaunchKernelGGL(import_quant_kernel<BITS>, grid, block, 0, s, st, (const uint32_t *)srcs[0],   \
                        (const char *)srcs[1], (const char *)srcs[2], (const uint32_t *)srcs[3],       \
