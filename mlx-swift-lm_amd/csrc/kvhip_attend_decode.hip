@@ -165,8 +165,11 @@ template <int BITS, int D, int G> struct TileRegs {
     int row;  // presented row of this lane's token, -1 if none
 };
 
-// RG = groups of 4 query rows handled per pass (R <= 4 RG)
-template <int BITS, int D, int GS, int DT, int RG>
+// RG = groups of 4 query rows handled per pass (R <= 4 RG).  MASKED = false compiles the
+// mask evaluation out, which keeps the tile loop free of branches (and of the
+// conservative load waits they force).  Slots map to presented rows one to one: only
+// RotatingKVCache remaps slots, and it is never quantized.
+template <int BITS, int D, int GS, int DT, int RG, bool MASKED>
 __global__ void __launch_bounds__(WAVES * 64, 2)
 decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     using GEO = Geo<BITS>;
@@ -176,7 +179,8 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     constexpr int RR = 4 * RG;     // query rows carried
     using T = TileRegs<BITS, D, G>;
     const Store &st = a.st;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform
     const int blk = lane >> 2, qi = lane & 3;  // lane group (MFMA block) and position in it
     const int bh = blockIdx.y, split = blockIdx.x;
     const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
@@ -246,24 +250,33 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     // tokens whose V code sits in a high nibble carry 1/16 on the probability side
     const float vfac = (BITS == 4 && (lane & 2)) ? 0.0625f : 1.0f;
 
-    const bool identity = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
-    const size_t k_page = (size_t)st.BH * st.k_cell, v_page = (size_t)st.BH * st.v_cell;
-    const size_t ksb_page = (size_t)st.BH * st.ksb_cell, vsb_page = (size_t)st.BH * st.vsb_cell;
     constexpr int VROW = T::VW * 4;  // bytes of one V tile row
 
-    auto load_tile = [&](int tile_, T &t) {
-        const int tile = __builtin_amdgcn_readfirstlane(tile_);
-        const int page = tile >> 2, tip = tile & 3;  // 4 tiles per page
-        const char *kt = st.k + page * k_page + (size_t)bh * st.k_cell + (size_t)(tip * TILE + lane) * st.k_row;
-        load_words<T::KW>(t.k, kt);
-        const char *vt = st.v + page * v_page + (size_t)bh * st.v_cell + ((size_t)tip * D + lane) * VROW;
+    // This wavefront takes tiles tile0, tile0 + 4, ...: always the same tile of
+    // successive pages, so its four plane pointers advance by one page cell stride.
+    const int tile0 = tile_begin + wave;
+    const int my_tiles = tile0 < tile_end ? (tile_end - tile0 + WAVES - 1) / WAVES : 0;
+    const size_t k_step = (size_t)st.BH * st.k_cell, v_step = (size_t)st.BH * st.v_cell;
+    const size_t ksb_step = (size_t)st.BH * st.ksb_cell, vsb_step = (size_t)st.BH * st.vsb_cell;
+    const int page0 = tile0 >> 2, tip = tile0 & 3;  // 4 tiles per page
+    const char *kp = st.k + ((size_t)page0 * st.BH + bh) * st.k_cell + (size_t)tip * TILE * st.k_row;
+    const char *vp = st.v + ((size_t)page0 * st.BH + bh) * st.v_cell + (size_t)tip * D * VROW;
+    const char *ksp = st.ksb + ((size_t)page0 * st.BH + bh) * st.ksb_cell + (size_t)tip * TILE * st.ksb_row;
+    const char *vsp = st.vsb + ((size_t)page0 * st.BH + bh) * st.vsb_cell + (size_t)tip * TILE * st.vsb_row;
+    const uint32_t k_lane = lane * st.k_row, v_lane = lane * VROW;
+    const uint32_t ksb_lane = lane * st.ksb_row, vsb_lane = lane * st.vsb_row;
+    int slot_next = tile0 * TILE + lane;  // slot of this lane's token in the tile loaded next
+    int loaded = 0;                       // tiles loaded so far
+
+    // Loads tile number `loaded` of this wavefront (clamped to its last tile, so the
+    // prefetch past the end stays unconditional and in bounds).
+    auto load_tile = [&](T &t) {
+        load_words<T::KW>(t.k, kp + k_lane);
 #pragma unroll
-        for (int h = 0; h < NH; ++h) load_words<T::VW>(t.v[h], vt + (size_t)h * 64 * VROW);
-        const char *ksb = st.ksb + page * ksb_page + (size_t)bh * st.ksb_cell + (size_t)(tip * TILE + lane) * st.ksb_row;
-        const char *vsb = st.vsb + page * vsb_page + (size_t)bh * st.vsb_cell + (size_t)(tip * TILE + lane) * st.vsb_row;
+        for (int h = 0; h < NH; ++h) load_words<T::VW>(t.v[h], vp + v_lane + (size_t)h * 64 * VROW);
         uint32_t kraw[G], vraw[G];  // (scale, bias) pairs of a 16-bit dtype
-        load_words<G>(kraw, ksb);
-        load_words<G>(vraw, vsb);
+        load_words<G>(kraw, ksp + ksb_lane);
+        load_words<G>(vraw, vsp + vsb_lane);
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             if (DT == 0) {
@@ -278,11 +291,15 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 t.vb[g] = __uint_as_float(vraw[g] & 0xffff0000u);
             }
         }
-        const int slot = tile * TILE + lane;
-        int row;
-        if (identity) row = slot;
-        else row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
-        t.row = (row >= 0 && row < a.T) ? row : -1;
+        t.row = slot_next < a.T ? slot_next : -1;
+        ++loaded;
+        if (loaded < my_tiles) {  // wave-uniform: step to the same tile of the next page
+            kp += k_step;
+            vp += v_step;
+            ksp += ksb_step;
+            vsp += vsb_step;
+            slot_next += PAGE;
+        }
     };
 
     auto compute_tile = [&](const T &t) {
@@ -318,13 +335,15 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 #pragma unroll
                 for (int g = 0; g < G; ++g) s_ += (t.ks[g] * TWO24) * sacc[rg][g][i] + t.kb[g] * qsum[rg][g][i];
                 s_ = round_dt<DT>(s_);
-                const int row_i = 4 * rg + i;
-                if (a.mask.mode != KVHIP_MASK_NONE && live && row_i < R) {
-                    const int rep = row_i / a.L, l = row_i - rep * a.L;
-                    float add;
-                    const bool keep = mask_keep(a.mask, b, hk * r + rep, l, t.row, a.L, a.T, add);
-                    if (!keep) s_ = fill;
-                    else if (a.mask.mode == KVHIP_MASK_ARRAY && a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
+                [[maybe_unused]] const int row_i = 4 * rg + i;
+                if constexpr (MASKED) {
+                    if (live && row_i < R) {
+                        const int rep = row_i / a.L, l = row_i - rep * a.L;
+                        float add;
+                        const bool keep = mask_keep(a.mask, b, hk * r + rep, l, t.row, a.L, a.T, add);
+                        if (!keep) s_ = fill;
+                        else if (a.mask.mode == KVHIP_MASK_ARRAY && a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
+                    }
                 }
                 sc[i] = live ? s_ : -INFINITY;
             }
@@ -386,30 +405,28 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         });
     };
 
-    // ---- main loop: this wavefront takes every WAVES-th tile of the span, one tile of
-    // loads in flight ahead of the arithmetic (variants whose tile does not fit twice in
-    // the register file run single-buffered and lean on the other resident wavefronts)
+    // ---- main loop: one tile of loads in flight ahead of the arithmetic (variants whose
+    // tile does not fit twice in the register file run single-buffered and lean on the
+    // other resident wavefronts)
     constexpr bool PREFETCH = (RG == 1 && !(BITS == 8 && D == 128)) || (RG == 2 && BITS == 4 && D == 64);
-    if constexpr (PREFETCH) {
-        T bufA, bufB;
-        int tile = tile_begin + wave;
-        if (tile < tile_end) load_tile(tile, bufA);
-        while (tile < tile_end) {
-            const int next = tile + WAVES;
-            if (next < tile_end) load_tile(next, bufB);
-            compute_tile(bufA);
-            tile = next;
-            if (tile >= tile_end) break;
-            const int next2 = tile + WAVES;
-            if (next2 < tile_end) load_tile(next2, bufA);
-            compute_tile(bufB);
-            tile = next2;
-        }
-    } else {
-        T buf;
-        for (int tile = tile_begin + wave; tile < tile_end; tile += WAVES) {
-            load_tile(tile, buf);
-            compute_tile(buf);
+    if (my_tiles > 0) {
+        if constexpr (PREFETCH) {
+            T bufA, bufB;
+            load_tile(bufA);
+            for (int done = 0;;) {
+                load_tile(bufB);
+                compute_tile(bufA);
+                if (++done == my_tiles) break;
+                load_tile(bufA);
+                compute_tile(bufB);
+                if (++done == my_tiles) break;
+            }
+        } else {
+            T buf;
+            for (int done = 0; done < my_tiles; ++done) {
+                load_tile(buf);
+                compute_tile(buf);
+            }
         }
     }
 
@@ -494,9 +511,11 @@ Plan plan_for(const AttendArgs &a) {
     const int R = (a.Hq / a.Hkv) * a.L;
     p.rg = R <= 4 ? 1 : (R <= 8 ? 2 : 4);
     const int BH = a.st.BH;
-    // enough workgroups to fill 256 CUs several times over; a span is a multiple of
-    // WAVES tiles so every wavefront of a workgroup gets the same share
-    int want = (256 * 16 + BH - 1) / BH;
+    // Spans are sized so that all workgroups are resident at once (2 per CU): every
+    // wavefront streams for the whole kernel and no second scheduling round leaves CUs
+    // idle.  A span is a multiple of WAVES tiles so each wavefront gets the same share.
+    int want = (256 * 2) / BH;
+    if (want < 1) want = 1;
     int per = (p.tiles_total + want - 1) / want;
     if (const char *e = getenv("KVHIP_DECODE_TILES")) per = atoi(e);
     per = per < WAVES ? WAVES : per;
@@ -544,6 +563,7 @@ bool attend_decode_supported(const AttendArgs &a) {
     if (s.Dk != s.Dv) return false;
     const int R = (a.Hq / a.Hkv) * a.L;
     if (R > 16) return false;
+    if (a.runs.n != 1 || a.runs.row0[0] != 0 || a.runs.phys0[0] != 0) return false;
     if (s.bits != 4 && s.bits != 8) return false;  // full-precision caches: other kernels
     if (s.Dk == 64) return s.gs == 64;
     if (s.Dk == 128) return s.gs == 64 || s.gs == 128;
@@ -563,8 +583,12 @@ hipError_t launch_attend_decode(const AttendArgs &a, hipStream_t s) {
 #define DEC(BITS, D, GS, DT, RG)                                                                          \
     do {                                                                                                  \
         profile_mark(s, true);                                                                            \
-        hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG>), grid, block, 0, s, a, p.tiles_total,     \
-                           p.tiles_per_wg, p.nsplit);                                                     \
+        if (a.mask.mode == KVHIP_MASK_NONE)                                                               \
+            hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG, false>), grid, block, 0, s, a,         \
+                               p.tiles_total, p.tiles_per_wg, p.nsplit);                                  \
+        else                                                                                              \
+            hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG, true>), grid, block, 0, s, a,          \
+                               p.tiles_total, p.tiles_per_wg, p.nsplit);                                  \
         profile_mark(s, false);                                                                           \
         hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG);  \
     } while (0)
