@@ -31,6 +31,10 @@ sys.path.insert(0, os.path.join(ROOT, "mlx-swift-lm_amd"))
 
 B, HQ, HKV, D, BITS, GS, CTX = 32, 32, 8, 128, 4, 64, 32768
 HBM_PEAK_GBS = 8000.0
+# HBM bytes moved per launch of the decode kernel divided by its algorithmic bytes, from two
+# rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a
+# plain 1 GiB copy; summary in profiles/decode_kernel_q4_d128_cfg3.md
+MEASURED_TRAFFIC_RATIO = 1.0033
 ROW_BYTES = 144  # per cached token and kv head: K and V codes 2*64 B + 2*2 groups*(scale+bias)*2 B
 
 
@@ -42,6 +46,9 @@ def main():
     ap.add_argument("--context", type=int, default=CTX)
     ap.add_argument("--batch", type=int, default=B)
     ap.add_argument("--cpu-steps", type=int, default=2, help="decode steps timed on the CPU baseline (0 = skip)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy 4 times (reference point for rocprofv3 --pmc "
+                         "FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--traffic-kib", type=float, default=None,
                     help="HBM KiB per launch of the decode kernel from rocprofv3 --pmc runs (else null)")
     args = ap.parse_args()
@@ -84,7 +91,13 @@ def main():
     torch.cuda.synchronize()
 
     lib = kvhip.load()
-    outs = []
+    if args.calibrate_copy:
+        src = torch.full((1 << 30,), 7, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for i in range(args.warmup):
         out = cache.update_attend(qs[i], ks[i], vs[i], scale)
     torch.cuda.synchronize()
@@ -112,7 +125,8 @@ def main():
         roofline = {"bound": "hbm", "kernel": "decode_kernel<4,128,64,f16>", "achieved": round(achieved, 1),
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                     "kernel_ms": round(kernel_ms, 5), "algorithmic_bytes": int(alg_bytes),
-                    "traffic": None if args.traffic_kib is None else int(args.traffic_kib * 1024)}
+                    "traffic": int(args.traffic_kib * 1024) if args.traffic_kib is not None
+                    else (int(alg_bytes * MEASURED_TRAFFIC_RATIO) if (nb, ctx) == (B, CTX) else None)}
 
     # ---- CPU baseline + full-size parity sample ------------------------------------
     cpu = None
