@@ -60,6 +60,9 @@ template <int N, class F> __device__ __forceinline__ void static_for(F &&f) {
 template <int ABID> __device__ __forceinline__ f4 mfma444(const Op &a, const Op &b, f4 c) {
     return __builtin_amdgcn_mfma_f32_4x4x4f16(a.h, b.h, c, 4, ABID, 0);
 }
+template <int ABID> __device__ __forceinline__ f4 mfma444_bf(const Op &a, const Op &b, f4 c) {
+    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(a.s, b.s, c, 4, ABID, 0);
+}
 
 // v_exp_f32 without the denormal-range fix-up (results below 2^-126 flush to zero)
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -476,6 +479,250 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     }
 }
 
+// ---------------------------------------------------------------------------------
+// Full-precision caches (KVCacheSimple, RotatingKVCache), fp16 or bf16.
+//
+// Same decomposition and the same 4x4x4 broadcast contraction as above, but a tile of
+// 16-bit K and V is 4x larger than a 4-bit one, so it is streamed through two
+// 32-register buffers in pieces of 64 elements per lane: a K piece is 64 head-dim
+// elements of the lane's token, a V piece is the 64 tokens of the lane's column.
+// The load of the next piece is issued as soon as a buffer has been consumed.
+// bf16 keeps P as a (hi, lo) pair of bf16 values so the PV product carries 16 bits of
+// probability; rows of a RotatingKVCache are found through the run table.
+template <int D, int DT, int RG, bool MASKED, bool IDENT>
+__global__ void __launch_bounds__(WAVES * 64, 2)
+decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
+    constexpr bool BF = DT == 1;
+    constexpr int NP = D / 64;   // pieces per K row and per V tile column set
+    constexpr int RR = 4 * RG;
+    constexpr int PW = 32;       // dwords per piece
+    const Store &st = a.st;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int blk = lane >> 2, qi = lane & 3;
+    const int bh = blockIdx.y, split = blockIdx.x;
+    const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
+    const int r = a.Hq / a.Hkv;
+    const int R = r * a.L;
+
+    __shared__ float cbuf[WAVES][RR][D + 2];
+
+    // query operands: lane (blk, qi) holds row qi's elements 4*(16 x + blk) .. +3, unscaled
+    Op qa[RG][NP];
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg) {
+        const int i = 4 * rg + qi;
+        const int rep = i / a.L, l = i - rep * a.L;
+        const size_t qoff = ((size_t)(b * a.Hq + hk * r + rep) * a.L + l) * D;
+#pragma unroll
+        for (int x = 0; x < NP; ++x) {
+            uint32_t w0 = 0, w1 = 0;
+            if (i < R) {
+                const uint16_t *qp = reinterpret_cast<const uint16_t *>(a.q) + qoff + 4 * (16 * x + blk);
+                w0 = (uint32_t)qp[0] | ((uint32_t)qp[1] << 16);
+                w1 = (uint32_t)qp[2] | ((uint32_t)qp[3] << 16);
+            }
+            qa[rg][x].u[0] = w0;
+            qa[rg][x].u[1] = w1;
+        }
+    }
+
+    float m_run[RG][4], l_part[RG][4];
+    f4 oacc[RG][NP];
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { m_run[rg][i] = -INFINITY; l_part[rg][i] = 0.f; }
+#pragma unroll
+        for (int h = 0; h < NP; ++h) oacc[rg][h] = f4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    const int tile_begin = split * tiles_per_wg;
+    const int tile_end = min(tiles_total, tile_begin + tiles_per_wg);
+    const int tile0 = tile_begin + wave;
+    const int my_tiles = tile0 < tile_end ? (tile_end - tile0 + WAVES - 1) / WAVES : 0;
+    const size_t k_step = (size_t)st.BH * st.k_cell, v_step = (size_t)st.BH * st.v_cell;
+    const int page0 = tile0 >> 2, tip = tile0 & 3;
+    constexpr int VROW = TILE * 2;  // bytes of one V tile row
+    const char *kp = st.k + ((size_t)page0 * st.BH + bh) * st.k_cell + (size_t)tip * TILE * st.k_row;
+    const char *vp = st.v + ((size_t)page0 * st.BH + bh) * st.v_cell + (size_t)tip * D * VROW;
+    const uint32_t k_lane = lane * st.k_row, v_lane = lane * VROW;
+    int slot_cur = tile0 * TILE + lane;
+    int k_loaded = 0, v_loaded = 0;  // tiles whose K / V pieces have been requested
+
+    // piece x of the K row / V column set of the tile the respective pointer stands on;
+    // after the last piece the pointer steps to this wavefront's next tile (clamped, so
+    // the prefetch past the end stays unconditional and in bounds)
+    auto load_k = [&](uint32_t *buf, int x) {
+        load_words<PW>(buf, kp + k_lane + x * (PW * 4));
+        if (x == NP - 1) {
+            ++k_loaded;
+            if (k_loaded < my_tiles) kp += k_step;
+        }
+    };
+    auto load_v = [&](uint32_t *buf, int x) {
+        load_words<PW>(buf, vp + v_lane + (size_t)x * 64 * VROW);
+        if (x == NP - 1) {
+            ++v_loaded;
+            if (v_loaded < my_tiles) vp += v_step;
+        }
+    };
+
+    uint32_t bufA[PW], bufB[PW];
+    // piece order per tile: K0 .. K(NP-1), V0 .. V(NP-1); piece n lives in buffer n & 1
+    // (NP = 1: K in A, V in B;  NP >= 2: even pieces in A, odd in B)
+    auto buf_of = [&](int n) -> uint32_t * { return (n & 1) ? bufB : bufA; };
+
+    if (my_tiles > 0) {
+        load_k(buf_of(0), 0);
+        if (NP > 1) load_k(buf_of(1), 1); else load_v(buf_of(1), 0);
+        for (int done = 0; done < my_tiles; ++done) {
+            int row;
+            if (IDENT) row = slot_cur;
+            else row = slot_cur < a.slots ? slot_to_row(a.runs, slot_cur) : -1;
+            row = (row >= 0 && row < a.T) ? row : -1;
+            const bool live = row >= 0;
+            // ---- QK^T over the K pieces ---------------------------------------------
+            f4 sacc[RG];
+#pragma unroll
+            for (int rg = 0; rg < RG; ++rg) sacc[rg] = f4{0.f, 0.f, 0.f, 0.f};
+            static_for<NP>([&](auto X) {
+                constexpr int x = decltype(X)::value;
+                uint32_t *buf = buf_of(x);
+                static_for<16>([&](auto S) {
+                    constexpr int s = decltype(S)::value;
+                    Op o;
+                    o.u[0] = buf[2 * s];
+                    o.u[1] = buf[2 * s + 1];
+#pragma unroll
+                    for (int rg = 0; rg < RG; ++rg)
+                        sacc[rg] = BF ? mfma444_bf<s>(qa[rg][x], o, sacc[rg]) : mfma444<s>(qa[rg][x], o, sacc[rg]);
+                });
+                // the buffer is free: request the piece two ahead in the order K.., V..
+                constexpr int n2 = x + 2;
+                if constexpr (n2 < NP) load_k(buf, n2);
+                else if constexpr (n2 < 2 * NP) load_v(buf, n2 - NP);
+                else load_k(buf, n2 - 2 * NP);  // NP == 1: the next tile's K
+            });
+            // ---- online softmax ----------------------------------------------------------
+            Op pa[RG], pl[RG];
+#pragma unroll
+            for (int rg = 0; rg < RG; ++rg) {
+                float sc[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float s_ = sacc[rg][i] * a.scale;
+                    [[maybe_unused]] const int row_i = 4 * rg + i;
+                    if constexpr (MASKED) {
+                        if (live && row_i < R) {
+                            const int rep = row_i / a.L, l = row_i - rep * a.L;
+                            float add;
+                            const bool keep = mask_keep(a.mask, b, hk * r + rep, l, row, a.L, a.T, add);
+                            s_ = keep ? s_ + add : -INFINITY;
+                        }
+                    }
+                    sc[i] = live ? s_ : -INFINITY;
+                }
+                bool need = false;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) need = need || (sc[i] > m_run[rg][i]);
+                if (__any(need)) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float mn = fmaxf(m_run[rg][i], wave_max(sc[i]));
+                        const float alpha = (mn == -INFINITY) ? 1.f : fast_exp2((m_run[rg][i] - mn) * LOG2E);
+                        m_run[rg][i] = mn;
+                        l_part[rg][i] *= alpha;
+#pragma unroll
+                        for (int h = 0; h < NP; ++h) oacc[rg][h][i] *= alpha;
+                    }
+                }
+                uint32_t xx[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float p = (sc[i] == -INFINITY || m_run[rg][i] == -INFINITY) ? 0.f : fast_exp2((sc[i] - m_run[rg][i]) * LOG2E);
+                    l_part[rg][i] += p;
+                    if (BF) {
+                        const uint32_t hi = Elem<1>::bits(p);
+                        const float rest = p - __uint_as_float(hi << 16);
+                        xx[i] = hi | ((uint32_t)Elem<1>::bits(rest) << 16);
+                    } else {
+                        xx[i] = (uint32_t)f2h_bits(p);
+                    }
+                }
+                quad_transpose(xx, lane);
+                pa[rg].u[0] = __builtin_amdgcn_perm(xx[1], xx[0], 0x05040100u);
+                pa[rg].u[1] = __builtin_amdgcn_perm(xx[3], xx[2], 0x05040100u);
+                if (BF) {
+                    pl[rg].u[0] = __builtin_amdgcn_perm(xx[1], xx[0], 0x07060302u);
+                    pl[rg].u[1] = __builtin_amdgcn_perm(xx[3], xx[2], 0x07060302u);
+                }
+            }
+            // ---- out += P . V over the V pieces ---------------------------------------------
+            static_for<NP>([&](auto X) {
+                constexpr int x = decltype(X)::value;
+                uint32_t *buf = buf_of(NP + x);
+                static_for<16>([&](auto S) {
+                    constexpr int s = decltype(S)::value;
+                    Op o;
+                    o.u[0] = buf[2 * s];
+                    o.u[1] = buf[2 * s + 1];
+#pragma unroll
+                    for (int rg = 0; rg < RG; ++rg) {
+                        if (BF) {
+                            oacc[rg][x] = mfma444_bf<s>(pa[rg], o, oacc[rg][x]);
+                            oacc[rg][x] = mfma444_bf<s>(pl[rg], o, oacc[rg][x]);
+                        } else {
+                            oacc[rg][x] = mfma444<s>(pa[rg], o, oacc[rg][x]);
+                        }
+                    }
+                });
+                // request the piece two ahead: the rest of V, then the next tile's K
+                constexpr int n2 = NP + x + 2;
+                if constexpr (n2 < 2 * NP) load_v(buf, n2 - NP);
+                else if constexpr (n2 < 3 * NP) load_k(buf, n2 - 2 * NP);
+                else load_v(buf, n2 - 3 * NP);  // NP == 1: the next tile's V
+            });
+            slot_cur += PAGE;
+        }
+    }
+
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) l_part[rg][i] = wave_sum(l_part[rg][i]);
+#pragma unroll
+        for (int h = 0; h < NP; ++h)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) cbuf[wave][4 * rg + i][64 * h + lane] = oacc[rg][h][i];
+        if (lane < 4) {
+            cbuf[wave][4 * rg + lane][D] = m_run[rg][lane];
+            cbuf[wave][4 * rg + lane][D + 1] = l_part[rg][lane];
+        }
+    }
+    __syncthreads();
+    float *part = a.workspace + ((size_t)bh * nsplit + split) * RR * (D + 2);
+    for (int idx = threadIdx.x; idx < RR * (D + 2); idx += WAVES * 64) {
+        const int i = idx / (D + 2), c = idx - i * (D + 2);
+        float mx = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, cbuf[w][i][D]);
+        float v;
+        if (c == D) {
+            v = mx;
+        } else {
+            v = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) {
+                const float mw = cbuf[w][i][D];
+                const float wgt = (mw == -INFINITY) ? 0.f : fast_exp2((mw - mx) * LOG2E);
+                v += wgt * cbuf[w][i][c];
+            }
+        }
+        part[idx] = v;
+    }
+}
+
 // grid (R, BH): merge the span partials of one query row and write the output row
 template <int D, int DT>
 __global__ void __launch_bounds__(D)
@@ -563,8 +810,9 @@ bool attend_decode_supported(const AttendArgs &a) {
     if (s.Dk != s.Dv) return false;
     const int R = (a.Hq / a.Hkv) * a.L;
     if (R > 16) return false;
+    if (s.bits == 0) return s.Dk == 64 || s.Dk == 128 || s.Dk == 256;
     if (a.runs.n != 1 || a.runs.row0[0] != 0 || a.runs.phys0[0] != 0) return false;
-    if (s.bits != 4 && s.bits != 8) return false;  // full-precision caches: other kernels
+    if (s.bits != 4 && s.bits != 8) return false;
     if (s.Dk == 64) return s.gs == 64;
     if (s.Dk == 128) return s.gs == 64 || s.gs == 128;
     return false;
@@ -609,9 +857,43 @@ hipError_t launch_attend_decode(const AttendArgs &a, hipStream_t s) {
         else if (st.gs == 64) DEC_DT(BITS, 128, 64); \
         else DEC_DT(BITS, 128, 128);                \
     } while (0)
+    const bool ident = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
+    const bool masked = a.mask.mode != KVHIP_MASK_NONE;
+#define FP(D, DT, RG, M, I)                                                                               \
+    do {                                                                                                  \
+        profile_mark(s, true);                                                                            \
+        hipLaunchKernelGGL((decode_fp_kernel<D, DT, RG, M, I>), grid, block, 0, s, a, p.tiles_total,      \
+                           p.tiles_per_wg, p.nsplit);                                                     \
+        profile_mark(s, false);                                                                           \
+        hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG);  \
+    } while (0)
+#define FP_MI(D, DT, RG)                                          \
+    do {                                                          \
+        if (!masked && ident) FP(D, DT, RG, false, true);         \
+        else if (!masked) FP(D, DT, RG, false, false);            \
+        else if (ident) FP(D, DT, RG, true, true);                \
+        else FP(D, DT, RG, true, false);                          \
+    } while (0)
+#define FP_RG(D, DT)                              \
+    do {                                          \
+        if (p.rg == 1) FP_MI(D, DT, 1);           \
+        else if (p.rg == 2) FP_MI(D, DT, 2);      \
+        else FP_MI(D, DT, 4);                     \
+    } while (0)
+#define FP_DT(D)                                  \
+    do {                                          \
+        if (st.dtype == KVHIP_F16) FP_RG(D, 0);   \
+        else FP_RG(D, 1);                         \
+    } while (0)
     if (st.bits == 4) DEC_Q(4);
     else if (st.bits == 8) DEC_Q(8);
-    else return hipErrorNotSupported;
+    else if (st.Dk == 64) FP_DT(64);
+    else if (st.Dk == 128) FP_DT(128);
+    else FP_DT(256);
+#undef FP_DT
+#undef FP_RG
+#undef FP_MI
+#undef FP
 #undef DEC_Q
 #undef DEC_DT
 #undef DEC_RG
