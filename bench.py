@@ -46,6 +46,9 @@ def main():
     ap.add_argument("--context", type=int, default=CTX)
     ap.add_argument("--batch", type=int, default=B)
     ap.add_argument("--cpu-steps", type=int, default=2, help="decode steps timed on the CPU baseline (0 = skip)")
+    ap.add_argument("--workload", default="cfg3", choices=["cfg3", "cfg2", "cfg4", "cfg5"],
+                    help="cfg3 (default) is the configuration the metric is quoted on; the others are the "
+                         "remaining BASELINE.json configs, measured for DESIGN.md")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy 4 times (reference point for rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -68,6 +71,9 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
     dev = torch.device("cuda:0")
+    if args.workload != "cfg3":
+        print(json.dumps(other_workload(args, torch, kvhip, L, dev)))
+        return
     nb, ctx = args.batch, args.context
     g = torch.Generator(device=dev)
     g.manual_seed(0)
@@ -163,6 +169,137 @@ def main():
         "hbm_gbs_whole_step": round(alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
     }
     print(json.dumps(line))
+
+
+def _timed(torch, fn, steps):
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fn(i)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def other_workload(args, torch, kvhip, L, dev):
+    """BASELINE.json configs[1], [3], [4] on synthetic data; returns one JSON-able dict."""
+    import ctypes as C
+    lib = kvhip.load()
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+
+    def kernel_ms():
+        n, ms = C.c_int32(), C.c_double()
+        L.check(lib.kvhip_profile_read(C.byref(n), C.byref(ms)))
+        return ms.value / max(n.value, 1), n.value
+
+    if args.workload == "cfg2":
+        # KVCacheSimple fp16 append + SDPA decode, B8, 32q/8kv, D128, grow to 8192 one token per step
+        Bn, Hq, Hkv, D = 8, 32, 8, 128
+        res = {}
+        for dtype, name in ((torch.float16, "f16"), (torch.bfloat16, "bf16")):
+            cache = kvhip.KVCacheSimple()
+            cache.reserve(Bn, Hkv, D, D, dtype, 8192 + 64)
+            ch = torch.ones(D, device=dev)
+            ch[torch.randperm(D, generator=g, device=dev)[:max(1, D // 100)]] = 8.0
+            q = torch.randn(64, Bn, Hq, 1, D, generator=g, device=dev).to(dtype)
+            kv = (torch.randn(64, 2, Bn, Hkv, 1, D, generator=g, device=dev) * 0.5 * ch).to(dtype)
+            scale = D ** -0.5
+            t_total0 = time.perf_counter()
+            points = {}
+            t = 0
+            for target in (1024, 2048, 4096, 8192):
+                while t < target - 32:
+                    cache.update_attend(q[t % 64], kv[t % 64, 0], kv[t % 64, 1], scale)
+                    t += 1
+                lib.kvhip_profile_enable(1)
+                dt = _timed(torch, lambda i: cache.update_attend(q[i], kv[i, 0], kv[i, 1], scale), 32)
+                lib.kvhip_profile_enable(0)
+                kms, _ = kernel_ms()
+                t += 32
+                alg = Bn * Hkv * (target - 16) * D * 2 * 2
+                points[str(target)] = {"step_us": round(dt * 1e6, 2), "kernel_us": round(kms * 1e3, 2),
+                                       "kernel_GBs": round(alg / (kms * 1e-3) / 1e9, 1),
+                                       "frac_of_8TBs": round(alg / (kms * 1e-3) / 8e12, 4)}
+            torch.cuda.synchronize()
+            res[name] = {"sweep_seconds_1_to_8192": round(time.perf_counter() - t_total0, 3), "at_length": points}
+        return {"workload": "configs[1]: KVCacheSimple append + SDPA decode, B8 32q/8kv D128, 1..8192", "results": res}
+
+    if args.workload == "cfg4":
+        # RotatingKVCache 4096 keep 4, B4 8q/4kv D256 bf16: 24 x 512-token chunks, then 512 decode steps
+        Bn, Hq, Hkv, D, M = 4, 8, 4, 256, 4096
+        dtype = torch.bfloat16
+        cache = kvhip.RotatingKVCache(M, keep=4)
+        scale = D ** -0.5
+        chunk_ms = []
+        for c in range(24):
+            q = torch.randn(Bn, Hq, 512, D, generator=g, device=dev).to(dtype)
+            k = torch.randn(Bn, Hkv, 512, D, generator=g, device=dev).to(dtype)
+            v = torch.randn(Bn, Hkv, 512, D, generator=g, device=dev).to(dtype)
+            off = min(M - 1, cache.offset)
+            # the reference's [512, off+512] causal-and-window array mask, evaluated from indices
+            mask = kvhip.MaskMode.window_mask(off, M) if off + 512 > M else kvhip.MaskMode.causal()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            cache.update_attend(q, k, v, scale, mask)
+            torch.cuda.synchronize()
+            chunk_ms.append((time.perf_counter() - t0) * 1e3)
+        tk = cache.presented_length
+        flops = Bn * Hq * 512 * tk * D * 4
+        steady = sorted(chunk_ms[10:])[len(chunk_ms[10:]) // 2]
+        q = torch.randn(64, Bn, Hq, 1, D, generator=g, device=dev).to(dtype)
+        kv = torch.randn(64, 2, Bn, Hkv, 1, D, generator=g, device=dev).to(dtype)
+        for i in range(8):
+            cache.update_attend(q[i], kv[i, 0], kv[i, 1], scale)
+        lib.kvhip_profile_enable(1)
+        dt = _timed(torch, lambda i: cache.update_attend(q[i % 64], kv[i % 64, 0], kv[i % 64, 1], scale), 504)
+        lib.kvhip_profile_enable(0)
+        kms, _ = kernel_ms()
+        alg = Bn * Hkv * M * D * 2 * 2
+        return {"workload": "configs[3]: RotatingKVCache 4096 keep 4, B4 8q/4kv D256 bf16",
+                "prefill_chunk_ms_steady": round(steady, 4), "prefill_keys": int(tk),
+                "prefill_TFLOPs": round(flops / (steady * 1e-3) / 1e12, 1),
+                "prefill_frac_of_2.5PF": round(flops / (steady * 1e-3) / 2.5e15, 4),
+                "decode_step_us": round(dt * 1e6, 2), "decode_kernel_us": round(kms * 1e3, 2),
+                "decode_kernel_GBs": round(alg / (kms * 1e-3) / 1e9, 1),
+                "decode_frac_of_8TBs": round(alg / (kms * 1e-3) / 8e12, 4),
+                "offset": int(cache.offset), "idx": int(cache.idx)}
+
+    # cfg5: speculative rollback on a ragged left-padded batch, 4-bit g64, Llama-3-8B shape
+    import numpy as np
+    Bn, Hq, Hkv, D, Lq = 16, 32, 8, 128, 4
+    rng = np.random.default_rng(0)
+    lens = rng.integers(1024, 16385, size=Bn)
+    tmax = int(lens.max())
+    pad = torch.from_numpy((tmax - lens).astype(np.int32)).to(dev)
+    cache = kvhip.QuantizedKVCache(64, 4)
+    cache.reserve(Bn, Hkv, D, D, torch.float16, tmax + 256 * 4 + 64)
+    for t0 in range(0, tmax, 2048):
+        nn = min(2048, tmax - t0)
+        k = torch.randn(Bn, Hkv, nn, D, generator=g, device=dev).to(torch.float16)
+        cache.update_quantized(k, k.flip(-1), fetch=False)
+    q = torch.randn(16, Bn, Hq, Lq, D, generator=g, device=dev).to(torch.float16)
+    kv = torch.randn(16, 2, Bn, Hkv, Lq, D, generator=g, device=dev).to(torch.float16)
+    trims = np.random.default_rng(1).integers(0, 5, size=256)
+    scale = D ** -0.5
+
+    def rnd(i):
+        mask = kvhip.MaskMode.window_mask(cache.offset, 0, left_pad=pad)
+        cache.update_attend(q[i % 16], kv[i % 16, 0], kv[i % 16, 1], scale, mask)
+        cache.trim(int(trims[i]))
+
+    for i in range(4):
+        rnd(i)
+    lib.kvhip_profile_enable(1)
+    dt = _timed(torch, rnd, 256)
+    lib.kvhip_profile_enable(0)
+    kms, _ = kernel_ms()
+    valid = float(lens.sum()) + Bn * (cache.offset - tmax)
+    return {"workload": "configs[4]: 4-bit QuantizedKVCache, B16 ragged U[1024,16384] left-padded, 256 rounds of "
+                        "append 4 + SDPA + trim(0..4)",
+            "round_us": round(dt * 1e6, 2), "kernel_us": round(kms * 1e3, 2), "padded_len": int(cache.offset),
+            "valid_bytes_per_round": int(Hkv * 144 * valid), "dense_bytes_per_round": int(Bn * Hkv * 144 * cache.offset),
+            "kernel_GBs_dense": round(Bn * Hkv * 144 * cache.offset / (kms * 1e-3) / 1e9, 1),
+            "kernel_GBs_valid": round(Hkv * 144 * valid / (kms * 1e-3) / 1e9, 1), "final_offset": int(cache.offset)}
 
 
 if __name__ == "__main__":

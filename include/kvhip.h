@@ -127,6 +127,10 @@ void kvhip_set_kernel_policy(int32_t policy);
  * events, returns the number of launches and their summed duration in
  * milliseconds, and clears the record.
  */
+/* Which kernel family the last attention call on this thread's library state used:
+ * 0 generic, 1 matrix-core decode (quantized), 2 matrix-core decode (full precision),
+ * 3 matrix-core chunked-prefill tile; -1 before the first call.  For tests and reports. */
+int32_t kvhip_last_attend_kernel(void);
 void kvhip_profile_enable(int32_t on);
 kvhip_status kvhip_profile_read(int32_t *out_launches, double *out_total_ms);
 

@@ -18,6 +18,7 @@ namespace {
 thread_local std::string g_err;
 thread_local bool g_has_err = false;
 int g_policy = 0;
+int g_last_kernel = -1;
 bool g_inited = false;
 
 kvhip_status fail(kvhip_status code, const std::string &msg) {
@@ -456,6 +457,8 @@ kvhip_status kvhip_sync(void *stream) {
 
 void kvhip_set_kernel_policy(int32_t policy) { g_policy = policy; }
 
+int32_t kvhip_last_attend_kernel(void) { return g_last_kernel; }
+
 void kvhip_profile_enable(int32_t on) { profile_enable(on != 0); }
 
 kvhip_status kvhip_profile_read(int32_t *out_launches, double *out_total_ms) {
@@ -621,11 +624,22 @@ kvhip_status kvhip_cache_attend(kvhip_cache *c, const void *q, int32_t B, int32_
         }
     }
     hipStream_t s = S(stream);
-    const bool fast = g_policy == 0 && attend_decode_supported(a);
-    KV_TRY(ensure_ws(c, fast ? attend_decode_workspace(a) : attend_generic_workspace(a), s));
-    a.workspace = c->ws;
-    a.workspace_bytes = c->ws_bytes;
-    KV_HIP(fast ? launch_attend_decode(a, s) : launch_attend_generic(a, s));
+    if (g_policy == 0 && attend_decode_supported(a)) {
+        KV_TRY(ensure_ws(c, attend_decode_workspace(a), s));
+        a.workspace = c->ws;
+        a.workspace_bytes = c->ws_bytes;
+        KV_HIP(launch_attend_decode(a, s));
+        g_last_kernel = a.st.bits ? 1 : 2;
+    } else if (g_policy == 0 && attend_prefill_supported(a)) {
+        KV_HIP(launch_attend_prefill(a, s));
+        g_last_kernel = 3;
+    } else {
+        g_last_kernel = 0;
+        KV_TRY(ensure_ws(c, attend_generic_workspace(a), s));
+        a.workspace = c->ws;
+        a.workspace_bytes = c->ws_bytes;
+        KV_HIP(launch_attend_generic(a, s));
+    }
     return KVHIP_OK;
 }
 

@@ -1,0 +1,364 @@
+// Chunked-prefill attention tile on the matrix cores (gfx950, v_mfma_f32_16x16x32_f16).
+//
+// Many query rows per kv head (r = Hq/Hkv heads times L new tokens).  One workgroup
+// (4 wavefronts) owns 128 query rows of one (batch, kv-head) pair -- 32 per wavefront
+// -- and walks the cached keys in tiles of 32 physical slots.  A tile is staged once
+// per workgroup in LDS as fp16 (packed codes are dequantised here, bf16 is converted),
+// K as [token][d] and V as [d][token], which is how the page layout already stores
+// them; the dense contractions then run as
+//   S^T   = K . Q^T      A = K rows from LDS, B = query rows held in registers
+//   out^T += V^T . P^T   A = V^T rows from LDS, B = the probabilities exactly where the
+//                        S^T accumulators left them (lane (q, j) holds tokens 4j..4j+3 of
+//                        both 16-token halves), so P never moves between lanes
+// with the online softmax in fp32 between them.  Masks are evaluated from indices
+// (causal, window, lengths, left padding) or read from the caller's array; for the
+// symbolic ones whole key tiles outside the visible range are skipped.
+#include "kvhip_mask.hpp"
+
+namespace kvhip {
+
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+union Op8 {
+    h8 h;
+    uint32_t u[4];
+    uint2 d2[2];
+    uint4 v;
+};
+
+constexpr int BM = 128;   // query rows per workgroup
+constexpr int BN = 32;    // key slots per tile
+constexpr float LOG2E = 1.4426950408889634f;
+
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ uint16_t h_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+__device__ __forceinline__ uint32_t h2_bits(float lo, float hi) { return (uint32_t)h_bits(lo) | ((uint32_t)h_bits(hi) << 16); }
+
+// BITS 0: full precision (DT 0 fp16 / 1 bf16); 4 / 8: quantized (scales of dtype DT)
+template <int BITS, int D, int DT, bool IDENT>
+__global__ void __launch_bounds__(256, 2)
+prefill_kernel(AttendArgs a) {
+    constexpr bool Q = BITS != 0;
+    constexpr int KS = D + 8;    // halves per K row in LDS (padded against bank conflicts)
+    constexpr int VS = BN + 4;   // halves per V^T row in LDS
+    constexpr int S = D / 32;    // contraction steps over the head dim
+    constexpr int NDT = D / 16;  // 16-row tiles of out^T
+    __shared__ __attribute__((aligned(16))) _Float16 Ks[BN * KS];
+    __shared__ __attribute__((aligned(16))) _Float16 Vs[D * VS];
+    __shared__ int rows_s[BN];
+    __shared__ float sb_s[Q ? BN * 2 * (D / 32) : 1];  // V (scale, bias) per token and group
+
+    const Store &st = a.st;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, jj = lane >> 4;
+    const int bh = blockIdx.y;
+    const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
+    const int r = a.Hq / a.Hkv;
+    const int R = r * a.L;
+    const int row0 = blockIdx.x * BM + wave * 32;  // first query row of this wavefront
+    const float fill = finfo_min_dt(DT);
+
+    // ---- query operands: B of S^T = K . Q^T; lane (n, jj) holds q[row][32 s + 8 jj ..] ----
+    Op8 qop[2][S];
+    int q_l[2], q_h[2];
+    bool q_ok[2];
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+        const int i = row0 + 16 * qt + n;
+        q_ok[qt] = i < R;
+        const int rep = q_ok[qt] ? i / a.L : 0;
+        q_l[qt] = q_ok[qt] ? i - rep * a.L : 0;
+        q_h[qt] = hk * r + rep;
+        const size_t qoff = ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D;
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                float v0 = 0.f, v1 = 0.f;
+                if (q_ok[qt]) {
+                    v0 = Elem<DT>::load(a.q, qoff + 32 * s + 8 * jj + 2 * w);
+                    v1 = Elem<DT>::load(a.q, qoff + 32 * s + 8 * jj + 2 * w + 1);
+                    if (Q) {
+                        v0 = round_dt<DT>(v0 * a.scale);
+                        v1 = round_dt<DT>(v1 * a.scale);
+                    }
+                }
+                qop[qt][s].u[w] = h2_bits(v0, v1);
+            }
+        }
+    }
+
+    f4 oacc[2][NDT];
+    float m_run[2], l_run[2];
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+        m_run[qt] = -INFINITY;
+        l_run[qt] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) oacc[qt][dt] = f4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // ---- visible slot range for symbolic masks (only when slots are presented rows) -------
+    int tile_lo = 0, tile_hi = (a.slots + BN - 1) / BN;
+    if (IDENT) {
+        const int i_first = blockIdx.x * BM, i_last = min(R, i_first + BM) - 1;
+        const bool spans = (i_first / a.L) != (i_last / a.L);
+        const int l_min = spans ? 0 : i_first % a.L, l_max = spans ? a.L - 1 : i_last % a.L;
+        if (a.mask.mode == KVHIP_MASK_CAUSAL) {
+            tile_hi = min(tile_hi, (a.T - a.L + l_max) / BN + 1);
+        } else if (a.mask.mode == KVHIP_MASK_WINDOW) {
+            tile_hi = min(tile_hi, (a.mask.offset + l_max) / BN + 1);
+            if (a.mask.window > 0) tile_lo = max(0, (a.mask.offset + l_min - a.mask.window + 1) / BN);
+        }
+        tile_hi = min(tile_hi, (a.T + BN - 1) / BN);
+    }
+
+    for (int tile = tile_lo; tile < tile_hi; ++tile) {
+        const int slot0 = tile * BN;
+        // ---- stage the tile: K -> Ks[token][d], V -> Vs[d][token], rows -> rows_s ---------
+        if (tid < BN) {
+            const int slot = slot0 + tid;
+            int row;
+            if (IDENT) row = slot;
+            else row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
+            rows_s[tid] = (row >= 0 && row < a.T) ? row : -1;
+        }
+        if constexpr (!Q) {
+            {   // K: 8 threads per token row, D/8 elements each
+                const int t = tid >> 3, part = tid & 7;
+                const uint16_t *src = reinterpret_cast<const uint16_t *>(k_row_ptr(st, bh, slot0 + t)) + part * (D / 8);
+                _Float16 *dst = Ks + t * KS + part * (D / 8);
+#pragma unroll
+                for (int e = 0; e < D / 8; e += 8) {
+                    uint4 raw = *reinterpret_cast<const uint4 *>(src + e);
+                    if (DT == 1) {
+                        uint32_t *w = reinterpret_cast<uint32_t *>(&raw);
+#pragma unroll
+                        for (int x = 0; x < 4; ++x)
+                            w[x] = h2_bits(__uint_as_float(w[x] << 16), __uint_as_float(w[x] & 0xffff0000u));
+                    }
+                    *reinterpret_cast<uint4 *>(dst + e) = raw;
+                }
+            }
+            {   // V: the tile is one 32-token half of a 64-token page tile; 2 threads per column
+                const char *cell = v_cell_ptr(st, bh, slot0);
+                const int half = (slot0 & 32) ? 1 : 0;
+                for (int c = tid; c < 2 * D; c += 256) {
+                    const int d = c >> 1, part = c & 1;
+                    const uint16_t *src = reinterpret_cast<const uint16_t *>(cell + v_row_off(st, slot0, d)) + half * 32 + part * 16;
+                    _Float16 *dst = Vs + d * VS + part * 16;
+#pragma unroll
+                    for (int e = 0; e < 16; e += 8) {
+                        uint4 raw = *reinterpret_cast<const uint4 *>(src + e);
+                        if (DT == 1) {
+                            uint32_t *w = reinterpret_cast<uint32_t *>(&raw);
+#pragma unroll
+                            for (int x = 0; x < 4; ++x)
+                                w[x] = h2_bits(__uint_as_float(w[x] << 16), __uint_as_float(w[x] & 0xffff0000u));
+                        }
+                        *reinterpret_cast<uint2 *>(dst + e) = make_uint2(raw.x, raw.y);
+                        *reinterpret_cast<uint2 *>(dst + e + 4) = make_uint2(raw.z, raw.w);
+                    }
+                }
+            }
+        } else {
+            constexpr int BB = Q ? BITS : 4;
+            constexpr int per = 32 / BB;
+            const int G = D / st.gs;
+            {   // K: 8 threads per token row, D/8 codes each, dequantised as scale*code + bias
+                const int t = tid >> 3, part = tid & 7;
+                const uint32_t *w = reinterpret_cast<const uint32_t *>(k_row_ptr(st, bh, slot0 + t));
+                const char *sb = ksb_row_ptr(st, bh, slot0 + t);
+                _Float16 *dst = Ks + t * KS;
+                for (int d = part * (D / 8); d < (part + 1) * (D / 8); d += 2) {
+                    const int g = d / st.gs;
+                    const float sc = Elem<DT>::load(sb, 2 * g), bi = Elem<DT>::load(sb, 2 * g + 1);
+                    const uint32_t word = w[d / per];
+                    const float c0 = (float)((word >> ((d % per) * BB)) & ((1u << BB) - 1u));
+                    const float c1 = (float)((word >> (((d + 1) % per) * BB)) & ((1u << BB) - 1u));
+                    *reinterpret_cast<uint32_t *>(dst + d) = h2_bits(sc * c0 + bi, sc * c1 + bi);
+                }
+            }
+            if (tid < BN) {  // V (scale, bias) of the tile's tokens
+                const char *sb = vsb_row_ptr(st, bh, slot0 + tid);
+                for (int g = 0; g < G; ++g) {
+                    sb_s[(tid * 2) * (D / 32) + g] = Elem<DT>::load(sb, 2 * g);
+                    sb_s[(tid * 2 + 1) * (D / 32) + g] = Elem<DT>::load(sb, 2 * g + 1);
+                }
+            }
+            __syncthreads();
+            {   // V: column d, 16 tokens per thread
+                const char *cell = v_cell_ptr(st, bh, slot0);
+                const int tbase = slot0 & 32;  // first token of this half inside the 64-token tile
+                for (int c = tid; c < 2 * D; c += 256) {
+                    const int d = c >> 1, part = c & 1;
+                    const int g = d / st.gs;
+                    const char *vrow = cell + v_row_off(st, slot0, d);
+                    _Float16 *dst = Vs + d * VS + part * 16;
+#pragma unroll
+                    for (int e = 0; e < 16; e += 2) {
+                        const int t0 = part * 16 + e;
+                        const float c0 = (float)v_code_load<BB>(vrow, tbase + t0);
+                        const float c1 = (float)v_code_load<BB>(vrow, tbase + t0 + 1);
+                        const float v0 = sb_s[(t0 * 2) * (D / 32) + g] * c0 + sb_s[(t0 * 2 + 1) * (D / 32) + g];
+                        const float v1 = sb_s[((t0 + 1) * 2) * (D / 32) + g] * c1 + sb_s[((t0 + 1) * 2 + 1) * (D / 32) + g];
+                        *reinterpret_cast<uint32_t *>(dst + e) = h2_bits(v0, v1);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+
+        // ---- S^T = K . Q^T: acc[qt][mt] rows = tokens 16 mt + 4 jj + i, column = query n -----
+        f4 sacc[2][2];
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) sacc[qt][mt] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < S; ++s)
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) {
+                Op8 ka;
+                ka.v = *reinterpret_cast<const uint4 *>(Ks + (16 * mt + n) * KS + 32 * s + 8 * jj);
+#pragma unroll
+                for (int qt = 0; qt < 2; ++qt)
+                    sacc[qt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka.h, qop[qt][s].h, sacc[qt][mt], 0, 0, 0);
+            }
+        int trow[2][4];
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) trow[mt][i] = rows_s[16 * mt + 4 * jj + i];
+
+        // ---- online softmax per query column; P^T stays in place as the PV B operand ------
+        Op8 pb[2];
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+            float sc[2][4];
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float s_ = Q ? round_dt<DT>(sacc[qt][mt][i]) : sacc[qt][mt][i] * a.scale;
+                    const int row = trow[mt][i];
+                    if (row >= 0 && q_ok[qt]) {
+                        if (a.mask.mode != KVHIP_MASK_NONE) {
+                            float add;
+                            const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
+                            if (Q) {
+                                if (!keep) s_ = fill;
+                                else if (a.mask.mode == KVHIP_MASK_ARRAY && a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
+                            } else {
+                                s_ = keep ? s_ + add : -INFINITY;
+                            }
+                        }
+                    } else {
+                        s_ = -INFINITY;
+                    }
+                    sc[mt][i] = s_;
+                    tmax = fmaxf(tmax, s_);
+                }
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+            const float mn = fmaxf(m_run[qt], tmax);
+            const float alpha = (mn == -INFINITY) ? 1.f : exp2_fast((m_run[qt] - mn) * LOG2E);
+            m_run[qt] = mn;
+            float psum = 0.f;
+            float p[2][4];
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    p[mt][i] = (sc[mt][i] == -INFINITY) ? 0.f : exp2_fast((sc[mt][i] - mn) * LOG2E);
+                    psum += p[mt][i];
+                }
+            l_run[qt] = l_run[qt] * alpha + psum;
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) oacc[qt][dt][i] *= alpha;
+            pb[qt].u[0] = h2_bits(p[0][0], p[0][1]);
+            pb[qt].u[1] = h2_bits(p[0][2], p[0][3]);
+            pb[qt].u[2] = h2_bits(p[1][0], p[1][1]);
+            pb[qt].u[3] = h2_bits(p[1][2], p[1][3]);
+        }
+
+        // ---- out^T += V^T . P^T: A = V^T rows (tokens 4jj..4jj+3 and 16+4jj..) from LDS -------
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+            Op8 va;
+            const _Float16 *vrow = Vs + (16 * dt + n) * VS;
+            va.d2[0] = *reinterpret_cast<const uint2 *>(vrow + 4 * jj);
+            va.d2[1] = *reinterpret_cast<const uint2 *>(vrow + 16 + 4 * jj);
+#pragma unroll
+            for (int qt = 0; qt < 2; ++qt)
+                oacc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va.h, pb[qt].h, oacc[qt][dt], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // ---- normalise and store: lane (n, jj) holds out[q = n][d = 16 dt + 4 jj + i] ------------
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+        float l = l_run[qt];
+        l += __shfl_xor(l, 16);
+        l += __shfl_xor(l, 32);
+        if (!q_ok[qt]) continue;
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        const size_t ooff = ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) Elem<DT>::store(a.out, ooff + 16 * dt + 4 * jj + i, oacc[qt][dt][i] * inv);
+    }
+}
+
+}  // namespace
+
+bool attend_prefill_supported(const AttendArgs &a) {
+    const Store &s = a.st;
+    if (s.dtype != KVHIP_F16 && s.dtype != KVHIP_BF16) return false;
+    if (s.Dk != s.Dv) return false;
+    if (s.Dk != 64 && s.Dk != 128 && s.Dk != 256) return false;
+    if (s.bits != 0 && s.bits != 4 && s.bits != 8) return false;
+    if (s.bits != 0 && (s.gs < 32 || s.Dk > 128)) return false;
+    return (a.Hq / a.Hkv) * a.L > 16;
+}
+
+hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
+    const Store &st = a.st;
+    const int R = (a.Hq / a.Hkv) * a.L;
+    dim3 grid((R + BM - 1) / BM, st.BH), block(256);
+    const bool ident = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
+#define PF(BITS, D, DT)                                                                                  \
+    do {                                                                                                 \
+        if (ident) hipLaunchKernelGGL((prefill_kernel<BITS, D, DT, true>), grid, block, 0, s, a);        \
+        else hipLaunchKernelGGL((prefill_kernel<BITS, D, DT, false>), grid, block, 0, s, a);             \
+    } while (0)
+#define PF_DT(BITS, D)                           \
+    do {                                         \
+        if (st.dtype == KVHIP_F16) PF(BITS, D, 0); \
+        else PF(BITS, D, 1);                     \
+    } while (0)
+#define PF_D(BITS)                               \
+    do {                                         \
+        if (st.Dk == 64) PF_DT(BITS, 64);        \
+        else PF_DT(BITS, 128);                   \
+    } while (0)
+    if (st.bits == 4) PF_D(4);
+    else if (st.bits == 8) PF_D(8);
+    else if (st.Dk == 64) PF_DT(0, 64);
+    else if (st.Dk == 128) PF_DT(0, 128);
+    else PF_DT(0, 256);
+#undef PF_D
+#undef PF_DT
+#undef PF
+    return hipGetLastError();
+}
+
+}  // namespace kvhip

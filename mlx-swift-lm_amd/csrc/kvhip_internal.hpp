@@ -173,6 +173,9 @@ hipError_t launch_attend_generic(const AttendArgs &a, hipStream_t s);
 bool attend_decode_supported(const AttendArgs &a);
 size_t attend_decode_workspace(const AttendArgs &a);
 hipError_t launch_attend_decode(const AttendArgs &a, hipStream_t s);
+// Matrix-core chunked-prefill tile (many query rows per kv head).
+bool attend_prefill_supported(const AttendArgs &a);
+hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s);
 // Event bracket around the dominant kernel while profiling is enabled.
 void profile_enable(bool on);
 void profile_mark(hipStream_t s, bool begin);

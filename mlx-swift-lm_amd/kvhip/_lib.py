@@ -49,6 +49,7 @@ SIGNATURES = {
     "kvhip_init": (_I32, [_I32]),
     "kvhip_sync": (_I32, [_P]),
     "kvhip_set_kernel_policy": (None, [_I32]),
+    "kvhip_last_attend_kernel": (_I32, []),
     "kvhip_profile_enable": (None, [_I32]),
     "kvhip_profile_read": (_I32, [C.POINTER(_I32), C.POINTER(C.c_double)]),
     "kvhip_cache_create": (_I32, [C.POINTER(Config), C.POINTER(_P)]),

@@ -182,6 +182,7 @@ def test_rotating_cfg4_reduced(policy, dtype):
         out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, c.make_mask(1, M, False))
         ref = O.attention_with_cache_update(q, k, v, o, scale, o.make_mask(1, M, False), name)
         check(out, ref, f"decode {i}")
+        assert kvhip.load().kvhip_last_attend_kernel() == (2 if policy == 0 else 0)  # MFMA fp decode
         assert c.meta_state == o.get_meta_state()
 
 
@@ -201,6 +202,7 @@ def test_cfg1_quantized_prefill_then_decode(policy):
     qk, qv = o.update_quantized(k, v)
     ref = CO.qsdpa(q, qk, qv, scale, "causal", 64, 8, "float16")
     check(out, ref, "prefill")
+    assert kvhip.load().kvhip_last_attend_kernel() == (3 if policy == 0 else 0)  # MFMA prefill tile
     for step in range(128):
         q, qd = randn(rng, (B, Hq, 1, D), dtype)
         k, kd = randn(rng, (B, Hkv, 1, D), dtype)
@@ -209,6 +211,7 @@ def test_cfg1_quantized_prefill_then_decode(policy):
         qk, qv = o.update_quantized(k, v)
         ref = CO.qsdpa(q, qk, qv, scale, None, 64, 8, "float16")
         check(out, ref, f"decode {step}")
+    assert kvhip.load().kvhip_last_attend_kernel() == (1 if policy == 0 else 0)  # MFMA quantized decode
     assert c.offset == 640 and c.meta_state == ["256", "640", "64", "8"]
     for a, b in zip(c.state, o.get_state()):
         if a.dtype == torch.int32:
@@ -247,6 +250,7 @@ def test_cfg5_ragged_speculative_rollback_reduced(policy):
         out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
         ref = O.attention_with_cache_update(q, k, v, o, scale, O.Mask("array", m), "float16")
         check(out, ref, f"round {rnd}")
+        assert kvhip.load().kvhip_last_attend_kernel() == (1 if policy == 0 else 0)  # 16 query rows per kv head
         n = int(trims[rnd])
         assert c.trim(n) == o.trim(n) and c.offset == o.offset
     for a, b in zip(c.state, o.get_state()):
