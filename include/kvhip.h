@@ -122,7 +122,7 @@ void kvhip_set_kernel_policy(int32_t policy);
 /*
  * Measurement hooks (no counterpart in the reference, which times whole
  * generations with wall clocks, Evaluate.swift:2467).  While enabled, every
- * launch of the split-sequence decode attention kernel is bracketed by HIP
+ * launch of the dominant attention kernel (split-sequence decode or prefill tile) is bracketed by HIP
  * events on the stream it is launched on.  kvhip_profile_read waits for those
  * events, returns the number of launches and their summed duration in
  * milliseconds, and clears the record.

@@ -168,11 +168,12 @@ template <int BITS, int D, int G> struct TileRegs {
     int row;  // presented row of this lane's token, -1 if none
 };
 
-// RG = groups of 4 query rows handled per pass (R <= 4 RG).  MASKED = false compiles the
-// mask evaluation out, which keeps the tile loop free of branches (and of the
-// conservative load waits they force).  Slots map to presented rows one to one: only
+// RG = groups of 4 query rows handled per pass (R <= 4 RG).  MM selects the mask code:
+// 0 none (the tile loop is branch free), 1 index-only masks (causal / window, per-batch
+// bounds preloaded: no memory access in the loop), 2 array masks (loads in the loop, which
+// force conservative waits on the prefetch).  Slots map to presented rows one to one: only
 // RotatingKVCache remaps slots, and it is never quantized.
-template <int BITS, int D, int GS, int DT, int RG, bool MASKED>
+template <int BITS, int D, int GS, int DT, int RG, int MM>
 __global__ void __launch_bounds__(WAVES * 64, 2)
 decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     using GEO = Geo<BITS>;
@@ -250,6 +251,12 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     const int tile_begin = split * tiles_per_wg;
     const int tile_end = min(tiles_total, tile_begin + tiles_per_wg);
     const float fill = finfo_min_dt(DT);
+    const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
+    int mrow_l[RG][4];  // query position l of each carried row
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mrow_l[rg][i] = (4 * rg + i) % a.L;
     // tokens whose V code sits in a high nibble carry 1/16 on the probability side
     const float vfac = (BITS == 4 && (lane & 2)) ? 0.0625f : 1.0f;
 
@@ -339,13 +346,15 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 for (int g = 0; g < G; ++g) s_ += (t.ks[g] * TWO24) * sacc[rg][g][i] + t.kb[g] * qsum[rg][g][i];
                 s_ = round_dt<DT>(s_);
                 [[maybe_unused]] const int row_i = 4 * rg + i;
-                if constexpr (MASKED) {
+                if constexpr (MM == 1) {
+                    if (!sym_mask_keep(sym, mrow_l[rg][i], t.row)) s_ = fill;
+                } else if constexpr (MM == 2) {
                     if (live && row_i < R) {
                         const int rep = row_i / a.L, l = row_i - rep * a.L;
                         float add;
                         const bool keep = mask_keep(a.mask, b, hk * r + rep, l, t.row, a.L, a.T, add);
                         if (!keep) s_ = fill;
-                        else if (a.mask.mode == KVHIP_MASK_ARRAY && a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
+                        else if (a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
                     }
                 }
                 sc[i] = live ? s_ : -INFINITY;
@@ -489,7 +498,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 // The load of the next piece is issued as soon as a buffer has been consumed.
 // bf16 keeps P as a (hi, lo) pair of bf16 values so the PV product carries 16 bits of
 // probability; rows of a RotatingKVCache are found through the run table.
-template <int D, int DT, int RG, bool MASKED, bool IDENT>
+template <int D, int DT, int RG, int MM, bool IDENT>
 __global__ void __launch_bounds__(WAVES * 64, 2)
 decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     constexpr bool BF = DT == 1;
@@ -537,6 +546,12 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         for (int h = 0; h < NP; ++h) oacc[rg][h] = f4{0.f, 0.f, 0.f, 0.f};
     }
 
+    const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
+    int mrow_l[RG][4];
+#pragma unroll
+    for (int rg = 0; rg < RG; ++rg)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mrow_l[rg][i] = (4 * rg + i) % a.L;
     const int tile_begin = split * tiles_per_wg;
     const int tile_end = min(tiles_total, tile_begin + tiles_per_wg);
     const int tile0 = tile_begin + wave;
@@ -613,7 +628,9 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 for (int i = 0; i < 4; ++i) {
                     float s_ = sacc[rg][i] * a.scale;
                     [[maybe_unused]] const int row_i = 4 * rg + i;
-                    if constexpr (MASKED) {
+                    if constexpr (MM == 1) {
+                        if (!sym_mask_keep(sym, mrow_l[rg][i], row)) s_ = -INFINITY;
+                    } else if constexpr (MM == 2) {
                         if (live && row_i < R) {
                             const int rep = row_i / a.L, l = row_i - rep * a.L;
                             float add;
@@ -828,14 +845,18 @@ hipError_t launch_attend_decode(const AttendArgs &a, hipStream_t s) {
     const Store &st = a.st;
     dim3 grid(p.nsplit, st.BH), block(WAVES * 64);
     const int R = (a.Hq / a.Hkv) * a.L;
+    const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
 #define DEC(BITS, D, GS, DT, RG)                                                                          \
     do {                                                                                                  \
         profile_mark(s, true);                                                                            \
-        if (a.mask.mode == KVHIP_MASK_NONE)                                                               \
-            hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG, false>), grid, block, 0, s, a,         \
+        if (mm == 0)                                                                                      \
+            hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG, 0>), grid, block, 0, s, a,             \
+                               p.tiles_total, p.tiles_per_wg, p.nsplit);                                  \
+        else if (mm == 1)                                                                                 \
+            hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG, 1>), grid, block, 0, s, a,             \
                                p.tiles_total, p.tiles_per_wg, p.nsplit);                                  \
         else                                                                                              \
-            hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG, true>), grid, block, 0, s, a,          \
+            hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG, 2>), grid, block, 0, s, a,             \
                                p.tiles_total, p.tiles_per_wg, p.nsplit);                                  \
         profile_mark(s, false);                                                                           \
         hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG);  \
@@ -858,7 +879,6 @@ hipError_t launch_attend_decode(const AttendArgs &a, hipStream_t s) {
         else DEC_DT(BITS, 128, 128);                \
     } while (0)
     const bool ident = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
-    const bool masked = a.mask.mode != KVHIP_MASK_NONE;
 #define FP(D, DT, RG, M, I)                                                                               \
     do {                                                                                                  \
         profile_mark(s, true);                                                                            \
@@ -869,10 +889,12 @@ hipError_t launch_attend_decode(const AttendArgs &a, hipStream_t s) {
     } while (0)
 #define FP_MI(D, DT, RG)                                          \
     do {                                                          \
-        if (!masked && ident) FP(D, DT, RG, false, true);         \
-        else if (!masked) FP(D, DT, RG, false, false);            \
-        else if (ident) FP(D, DT, RG, true, true);                \
-        else FP(D, DT, RG, true, false);                          \
+        if (mm == 0 && ident) FP(D, DT, RG, 0, true);             \
+        else if (mm == 0) FP(D, DT, RG, 0, false);                \
+        else if (mm == 1 && ident) FP(D, DT, RG, 1, true);        \
+        else if (mm == 1) FP(D, DT, RG, 1, false);                \
+        else if (ident) FP(D, DT, RG, 2, true);                   \
+        else FP(D, DT, RG, 2, false);                             \
     } while (0)
 #define FP_RG(D, DT)                              \
     do {                                          \

@@ -28,7 +28,6 @@ union Op8 {
     uint4 v;
 };
 
-constexpr int BM = 128;   // query rows per workgroup
 constexpr int BN = 32;    // key slots per tile
 constexpr float LOG2E = 1.4426950408889634f;
 
@@ -36,11 +35,15 @@ __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ uint16_t h_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
 __device__ __forceinline__ uint32_t h2_bits(float lo, float hi) { return (uint32_t)h_bits(lo) | ((uint32_t)h_bits(hi) << 16); }
 
-// BITS 0: full precision (DT 0 fp16 / 1 bf16); 4 / 8: quantized (scales of dtype DT)
-template <int BITS, int D, int DT, bool IDENT>
+// BITS 0: full precision (DT 0 fp16 / 1 bf16); 4 / 8: quantized (scales of dtype DT).
+// QT = 16-row query tiles per wavefront (2: 128 rows per workgroup, 1: 64 rows, chosen by
+// the launcher so that the grid fills the chip).  MM: 0 no mask, 1 index-only mask
+// (causal / window, no memory access in the loop), 2 array mask.
+template <int BITS, int D, int DT, bool IDENT, int QT, int MM>
 __global__ void __launch_bounds__(256, 2)
 prefill_kernel(AttendArgs a) {
     constexpr bool Q = BITS != 0;
+    constexpr int BM = 64 * QT;
     constexpr int KS = D + 8;    // halves per K row in LDS (padded against bank conflicts)
     constexpr int VS = BN + 4;   // halves per V^T row in LDS
     constexpr int S = D / 32;    // contraction steps over the head dim
@@ -58,15 +61,16 @@ prefill_kernel(AttendArgs a) {
     const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
     const int r = a.Hq / a.Hkv;
     const int R = r * a.L;
-    const int row0 = blockIdx.x * BM + wave * 32;  // first query row of this wavefront
+    const int row0 = blockIdx.x * BM + wave * 16 * QT;  // first query row of this wavefront
     const float fill = finfo_min_dt(DT);
+    const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
 
     // ---- query operands: B of S^T = K . Q^T; lane (n, jj) holds q[row][32 s + 8 jj ..] ----
-    Op8 qop[2][S];
-    int q_l[2], q_h[2];
-    bool q_ok[2];
+    Op8 qop[QT][S];
+    int q_l[QT], q_h[QT];
+    bool q_ok[QT];
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
+    for (int qt = 0; qt < QT; ++qt) {
         const int i = row0 + 16 * qt + n;
         q_ok[qt] = i < R;
         const int rep = q_ok[qt] ? i / a.L : 0;
@@ -91,10 +95,10 @@ prefill_kernel(AttendArgs a) {
         }
     }
 
-    f4 oacc[2][NDT];
-    float m_run[2], l_run[2];
+    f4 oacc[QT][NDT];
+    float m_run[QT], l_run[QT];
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
+    for (int qt = 0; qt < QT; ++qt) {
         m_run[qt] = -INFINITY;
         l_run[qt] = 0.f;
 #pragma unroll
@@ -116,118 +120,178 @@ prefill_kernel(AttendArgs a) {
         tile_hi = min(tile_hi, (a.T + BN - 1) / BN);
     }
 
-    for (int tile = tile_lo; tile < tile_hi; ++tile) {
+    // ---- staging: a tile is fetched from global memory into registers one iteration ahead
+    // (in flight while the current tile is contracted), then converted and written to LDS.
+    constexpr int BB = Q ? BITS : 4;
+    constexpr int KU = Q ? 1 : D / 64;            // uint4 per thread for K (fp); quantized: words below
+    constexpr int KQW = (D / 8) * BB / 32;        // quantized: packed words per thread for K (D/8 codes)
+    constexpr int VQW = 16 * BB / 32;             // quantized: packed words per thread and column for V
+    constexpr int VCOLS = (2 * D + 255) / 256;    // (column, half) items per thread for V
+    uint4 kreg[Q ? 1 : KU];
+    uint4 vreg[Q ? 1 : 2 * VCOLS];
+    uint32_t kq[Q ? KQW : 1], vq[Q ? VCOLS * VQW : 1], ksb_raw = 0;
+    uint32_t vsb_raw[Q ? D / 32 : 1];
+    int row_reg = -1;
+    const int kt = tid >> 3, kpart = tid & 7;     // K: 8 threads per token row
+
+    auto fetch = [&](int tile) {
         const int slot0 = tile * BN;
-        // ---- stage the tile: K -> Ks[token][d], V -> Vs[d][token], rows -> rows_s ---------
         if (tid < BN) {
             const int slot = slot0 + tid;
             int row;
             if (IDENT) row = slot;
             else row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
-            rows_s[tid] = (row >= 0 && row < a.T) ? row : -1;
+            row_reg = (row >= 0 && row < a.T) ? row : -1;
         }
+        const char *cell = v_cell_ptr(st, bh, slot0);
         if constexpr (!Q) {
-            {   // K: 8 threads per token row, D/8 elements each
-                const int t = tid >> 3, part = tid & 7;
-                const uint16_t *src = reinterpret_cast<const uint16_t *>(k_row_ptr(st, bh, slot0 + t)) + part * (D / 8);
-                _Float16 *dst = Ks + t * KS + part * (D / 8);
+            const uint4 *src = reinterpret_cast<const uint4 *>(k_row_ptr(st, bh, slot0 + kt)) + kpart * KU;
 #pragma unroll
-                for (int e = 0; e < D / 8; e += 8) {
-                    uint4 raw = *reinterpret_cast<const uint4 *>(src + e);
-                    if (DT == 1) {
-                        uint32_t *w = reinterpret_cast<uint32_t *>(&raw);
+            for (int e = 0; e < KU; ++e) kreg[e] = src[e];
+            const int half = (slot0 & 32) ? 1 : 0;
 #pragma unroll
-                        for (int x = 0; x < 4; ++x)
-                            w[x] = h2_bits(__uint_as_float(w[x] << 16), __uint_as_float(w[x] & 0xffff0000u));
-                    }
-                    *reinterpret_cast<uint4 *>(dst + e) = raw;
-                }
-            }
-            {   // V: the tile is one 32-token half of a 64-token page tile; 2 threads per column
-                const char *cell = v_cell_ptr(st, bh, slot0);
-                const int half = (slot0 & 32) ? 1 : 0;
-                for (int c = tid; c < 2 * D; c += 256) {
+            for (int ci = 0; ci < VCOLS; ++ci) {
+                const int c = tid + 256 * ci;
+                if (c < 2 * D) {
                     const int d = c >> 1, part = c & 1;
-                    const uint16_t *src = reinterpret_cast<const uint16_t *>(cell + v_row_off(st, slot0, d)) + half * 32 + part * 16;
-                    _Float16 *dst = Vs + d * VS + part * 16;
-#pragma unroll
-                    for (int e = 0; e < 16; e += 8) {
-                        uint4 raw = *reinterpret_cast<const uint4 *>(src + e);
-                        if (DT == 1) {
-                            uint32_t *w = reinterpret_cast<uint32_t *>(&raw);
-#pragma unroll
-                            for (int x = 0; x < 4; ++x)
-                                w[x] = h2_bits(__uint_as_float(w[x] << 16), __uint_as_float(w[x] & 0xffff0000u));
-                        }
-                        *reinterpret_cast<uint2 *>(dst + e) = make_uint2(raw.x, raw.y);
-                        *reinterpret_cast<uint2 *>(dst + e + 4) = make_uint2(raw.z, raw.w);
-                    }
+                    const uint4 *vs = reinterpret_cast<const uint4 *>(cell + v_row_off(st, slot0, d) + half * 64 + part * 32);
+                    vreg[2 * ci] = vs[0];
+                    vreg[2 * ci + 1] = vs[1];
                 }
             }
         } else {
-            constexpr int BB = Q ? BITS : 4;
-            constexpr int per = 32 / BB;
-            const int G = D / st.gs;
-            {   // K: 8 threads per token row, D/8 codes each, dequantised as scale*code + bias
-                const int t = tid >> 3, part = tid & 7;
-                const uint32_t *w = reinterpret_cast<const uint32_t *>(k_row_ptr(st, bh, slot0 + t));
-                const char *sb = ksb_row_ptr(st, bh, slot0 + t);
-                _Float16 *dst = Ks + t * KS;
-                for (int d = part * (D / 8); d < (part + 1) * (D / 8); d += 2) {
-                    const int g = d / st.gs;
-                    const float sc = Elem<DT>::load(sb, 2 * g), bi = Elem<DT>::load(sb, 2 * g + 1);
-                    const uint32_t word = w[d / per];
-                    const float c0 = (float)((word >> ((d % per) * BB)) & ((1u << BB) - 1u));
-                    const float c1 = (float)((word >> (((d + 1) % per) * BB)) & ((1u << BB) - 1u));
-                    *reinterpret_cast<uint32_t *>(dst + d) = h2_bits(sc * c0 + bi, sc * c1 + bi);
-                }
-            }
-            if (tid < BN) {  // V (scale, bias) of the tile's tokens
-                const char *sb = vsb_row_ptr(st, bh, slot0 + tid);
-                for (int g = 0; g < G; ++g) {
-                    sb_s[(tid * 2) * (D / 32) + g] = Elem<DT>::load(sb, 2 * g);
-                    sb_s[(tid * 2 + 1) * (D / 32) + g] = Elem<DT>::load(sb, 2 * g + 1);
-                }
-            }
-            __syncthreads();
-            {   // V: column d, 16 tokens per thread
-                const char *cell = v_cell_ptr(st, bh, slot0);
-                const int tbase = slot0 & 32;  // first token of this half inside the 64-token tile
-                for (int c = tid; c < 2 * D; c += 256) {
-                    const int d = c >> 1, part = c & 1;
-                    const int g = d / st.gs;
-                    const char *vrow = cell + v_row_off(st, slot0, d);
-                    _Float16 *dst = Vs + d * VS + part * 16;
+            const uint32_t *w = reinterpret_cast<const uint32_t *>(k_row_ptr(st, bh, slot0 + kt)) + kpart * KQW;
 #pragma unroll
-                    for (int e = 0; e < 16; e += 2) {
-                        const int t0 = part * 16 + e;
-                        const float c0 = (float)v_code_load<BB>(vrow, tbase + t0);
-                        const float c1 = (float)v_code_load<BB>(vrow, tbase + t0 + 1);
+            for (int e = 0; e < KQW; ++e) kq[e] = w[e];
+            // the D/8 codes of this thread lie in one group (group sizes are >= 32 >= D/8)
+            const int g = (kpart * (D / 8)) / st.gs;
+            ksb_raw = reinterpret_cast<const uint32_t *>(ksb_row_ptr(st, bh, slot0 + kt))[g];
+            if (tid < BN) {
+                const uint32_t *sb = reinterpret_cast<const uint32_t *>(vsb_row_ptr(st, bh, slot0 + tid));
+#pragma unroll
+                for (int gg = 0; gg < D / 32; ++gg)
+                    if (gg < D / st.gs) vsb_raw[gg] = sb[gg];
+            }
+            const int tbase = slot0 & 32;
+#pragma unroll
+            for (int ci = 0; ci < VCOLS; ++ci) {
+                const int c = tid + 256 * ci;
+                if (c < 2 * D) {
+                    const int d = c >> 1, part = c & 1;
+                    const uint32_t *vw = reinterpret_cast<const uint32_t *>(cell + v_row_off(st, slot0, d)) + (tbase + part * 16) * BB / 32;
+#pragma unroll
+                    for (int e = 0; e < VQW; ++e) vq[ci * VQW + e] = vw[e];
+                }
+            }
+        }
+    };
+    auto sb_pair = [&](uint32_t raw, float &sc, float &bi) {  // (scale, bias) of a 16-bit dtype
+        if (DT == 0) {
+            sc = (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+            bi = (float)__builtin_bit_cast(_Float16, (uint16_t)(raw >> 16));
+        } else {
+            sc = __uint_as_float(raw << 16);
+            bi = __uint_as_float(raw & 0xffff0000u);
+        }
+    };
+    auto to_h2 = [&](uint32_t w) -> uint32_t {  // two cache-dtype elements -> two fp16
+        if (DT == 1) return h2_bits(__uint_as_float(w << 16), __uint_as_float(w & 0xffff0000u));
+        return w;
+    };
+    auto stage_k = [&]() {  // K, row indices and (quantized) the V scale/bias table
+        if (tid < BN) rows_s[tid] = row_reg;
+        if constexpr (!Q) {
+            _Float16 *dst = Ks + kt * KS + kpart * (D / 8);
+#pragma unroll
+            for (int e = 0; e < KU; ++e) {
+                uint4 r_ = kreg[e];
+                r_.x = to_h2(r_.x); r_.y = to_h2(r_.y); r_.z = to_h2(r_.z); r_.w = to_h2(r_.w);
+                *reinterpret_cast<uint4 *>(dst + 8 * e) = r_;
+            }
+        } else {
+            constexpr int per = 32 / BB;
+            float sc, bi;
+            sb_pair(ksb_raw, sc, bi);
+            _Float16 *dst = Ks + kt * KS + kpart * (D / 8);
+#pragma unroll
+            for (int e = 0; e < KQW; ++e)
+#pragma unroll
+                for (int x = 0; x < per; x += 2) {
+                    const float c0 = (float)((kq[e] >> (x * BB)) & ((1u << BB) - 1u));
+                    const float c1 = (float)((kq[e] >> ((x + 1) * BB)) & ((1u << BB) - 1u));
+                    *reinterpret_cast<uint32_t *>(dst + e * per + x) = h2_bits(sc * c0 + bi, sc * c1 + bi);
+                }
+            if (tid < BN) {
+#pragma unroll
+                for (int gg = 0; gg < D / 32; ++gg)
+                    if (gg < D / st.gs) {
+                        float s2, b2;
+                        sb_pair(vsb_raw[gg], s2, b2);
+                        sb_s[(tid * 2) * (D / 32) + gg] = s2;
+                        sb_s[(tid * 2 + 1) * (D / 32) + gg] = b2;
+                    }
+            }
+        }
+    };
+    auto stage_v = [&]() {
+#pragma unroll
+        for (int ci = 0; ci < VCOLS; ++ci) {
+            const int c = tid + 256 * ci;
+            if (c < 2 * D) {
+                const int d = c >> 1, part = c & 1;
+                _Float16 *dst = Vs + d * VS + part * 16;
+                if constexpr (!Q) {
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        const uint4 r_ = vreg[2 * ci + e];
+                        *reinterpret_cast<uint2 *>(dst + 8 * e) = make_uint2(to_h2(r_.x), to_h2(r_.y));
+                        *reinterpret_cast<uint2 *>(dst + 8 * e + 4) = make_uint2(to_h2(r_.z), to_h2(r_.w));
+                    }
+                } else {
+                    const int g = d / st.gs;
+                    // token tt of the 16 sits at code position p(tt) of its word (V tile order)
+#pragma unroll
+                    for (int tt = 0; tt < 16; tt += 2) {
+                        const int bp0 = v_bitpos<BB>(tt), bp1 = v_bitpos<BB>(tt + 1);
+                        const float c0 = (float)((vq[ci * VQW + (bp0 >> 5)] >> (bp0 & 31)) & ((1u << BB) - 1u));
+                        const float c1 = (float)((vq[ci * VQW + (bp1 >> 5)] >> (bp1 & 31)) & ((1u << BB) - 1u));
+                        const int t0 = part * 16 + tt;
                         const float v0 = sb_s[(t0 * 2) * (D / 32) + g] * c0 + sb_s[(t0 * 2 + 1) * (D / 32) + g];
                         const float v1 = sb_s[((t0 + 1) * 2) * (D / 32) + g] * c1 + sb_s[((t0 + 1) * 2 + 1) * (D / 32) + g];
-                        *reinterpret_cast<uint32_t *>(dst + e) = h2_bits(v0, v1);
+                        *reinterpret_cast<uint32_t *>(dst + tt) = h2_bits(v0, v1);
                     }
                 }
             }
         }
+    };
+
+    if (tile_lo < tile_hi) fetch(tile_lo);
+    for (int tile = tile_lo; tile < tile_hi; ++tile) {
+        if (tile > tile_lo) __syncthreads();  // everyone is done reading the previous tile
+        stage_k();
+        if constexpr (Q) __syncthreads();     // the V dequantisation reads the scale/bias table
+        stage_v();
         __syncthreads();
+        if (tile + 1 < tile_hi) fetch(tile + 1);
 
         // ---- S^T = K . Q^T: acc[qt][mt] rows = tokens 16 mt + 4 jj + i, column = query n -----
-        f4 sacc[2][2];
+        f4 sacc[QT][2];
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt)
+        for (int qt = 0; qt < QT; ++qt)
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt) sacc[qt][mt] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s = 0; s < S; ++s)
+        for (int mt = 0; mt < 2; ++mt) {
+            Op8 ka[S];  // all K operands of this 16-token half first, then the MFMAs back to back
 #pragma unroll
-            for (int mt = 0; mt < 2; ++mt) {
-                Op8 ka;
-                ka.v = *reinterpret_cast<const uint4 *>(Ks + (16 * mt + n) * KS + 32 * s + 8 * jj);
+            for (int s = 0; s < S; ++s)
+                ka[s].v = *reinterpret_cast<const uint4 *>(Ks + (16 * mt + n) * KS + 32 * s + 8 * jj);
 #pragma unroll
-                for (int qt = 0; qt < 2; ++qt)
-                    sacc[qt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka.h, qop[qt][s].h, sacc[qt][mt], 0, 0, 0);
-            }
+            for (int s = 0; s < S; ++s)
+#pragma unroll
+                for (int qt = 0; qt < QT; ++qt)
+                    sacc[qt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka[s].h, qop[qt][s].h, sacc[qt][mt], 0, 0, 0);
+        }
         int trow[2][4];
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
@@ -235,9 +299,9 @@ prefill_kernel(AttendArgs a) {
             for (int i = 0; i < 4; ++i) trow[mt][i] = rows_s[16 * mt + 4 * jj + i];
 
         // ---- online softmax per query column; P^T stays in place as the PV B operand ------
-        Op8 pb[2];
+        Op8 pb[QT];
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
+        for (int qt = 0; qt < QT; ++qt) {
             float sc[2][4];
             float tmax = -INFINITY;
 #pragma unroll
@@ -247,12 +311,14 @@ prefill_kernel(AttendArgs a) {
                     float s_ = Q ? round_dt<DT>(sacc[qt][mt][i]) : sacc[qt][mt][i] * a.scale;
                     const int row = trow[mt][i];
                     if (row >= 0 && q_ok[qt]) {
-                        if (a.mask.mode != KVHIP_MASK_NONE) {
+                        if constexpr (MM == 1) {
+                            if (!sym_mask_keep(sym, q_l[qt], row)) s_ = Q ? fill : -INFINITY;
+                        } else if constexpr (MM == 2) {
                             float add;
                             const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
                             if (Q) {
                                 if (!keep) s_ = fill;
-                                else if (a.mask.mode == KVHIP_MASK_ARRAY && a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
+                                else if (a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
                             } else {
                                 s_ = keep ? s_ + add : -INFINITY;
                             }
@@ -290,21 +356,25 @@ prefill_kernel(AttendArgs a) {
 
         // ---- out^T += V^T . P^T: A = V^T rows (tokens 4jj..4jj+3 and 16+4jj..) from LDS -------
 #pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-            Op8 va;
-            const _Float16 *vrow = Vs + (16 * dt + n) * VS;
-            va.d2[0] = *reinterpret_cast<const uint2 *>(vrow + 4 * jj);
-            va.d2[1] = *reinterpret_cast<const uint2 *>(vrow + 16 + 4 * jj);
+        for (int d0 = 0; d0 < NDT; d0 += 4) {
+            Op8 va[4];  // four V^T operands per batch of LDS reads
 #pragma unroll
-            for (int qt = 0; qt < 2; ++qt)
-                oacc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va.h, pb[qt].h, oacc[qt][dt], 0, 0, 0);
+            for (int x = 0; x < 4; ++x) {
+                const _Float16 *vrow = Vs + (16 * (d0 + x) + n) * VS;
+                va[x].d2[0] = *reinterpret_cast<const uint2 *>(vrow + 4 * jj);
+                va[x].d2[1] = *reinterpret_cast<const uint2 *>(vrow + 16 + 4 * jj);
+            }
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+#pragma unroll
+                for (int qt = 0; qt < QT; ++qt)
+                    oacc[qt][d0 + x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[x].h, pb[qt].h, oacc[qt][d0 + x], 0, 0, 0);
         }
-        __syncthreads();
     }
 
     // ---- normalise and store: lane (n, jj) holds out[q = n][d = 16 dt + 4 jj + i] ------------
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
+    for (int qt = 0; qt < QT; ++qt) {
         float l = l_run[qt];
         l += __shfl_xor(l, 16);
         l += __shfl_xor(l, 32);
@@ -333,17 +403,35 @@ bool attend_prefill_supported(const AttendArgs &a) {
 hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
     const Store &st = a.st;
     const int R = (a.Hq / a.Hkv) * a.L;
-    dim3 grid((R + BM - 1) / BM, st.BH), block(256);
+    // 128 query rows per workgroup reuse each staged tile twice as often; 64 rows are used
+    // when that would leave the grid too small to fill 256 CUs twice over
+    const bool wide = (size_t)((R + 127) / 128) * st.BH >= 512 && st.Dk <= 128;
+    const int bm = wide ? 128 : 64;
+    dim3 grid((R + bm - 1) / bm, st.BH), block(256);
     const bool ident = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
-#define PF(BITS, D, DT)                                                                                  \
-    do {                                                                                                 \
-        if (ident) hipLaunchKernelGGL((prefill_kernel<BITS, D, DT, true>), grid, block, 0, s, a);        \
-        else hipLaunchKernelGGL((prefill_kernel<BITS, D, DT, false>), grid, block, 0, s, a);             \
+    const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
+#define PF_M(BITS, D, DT, QT, MM)                                                                         \
+    do {                                                                                                  \
+        profile_mark(s, true);                                                                            \
+        if (ident) hipLaunchKernelGGL((prefill_kernel<BITS, D, DT, true, QT, MM>), grid, block, 0, s, a); \
+        else hipLaunchKernelGGL((prefill_kernel<BITS, D, DT, false, QT, MM>), grid, block, 0, s, a);      \
+        profile_mark(s, false);                                                                           \
+    } while (0)
+#define PF(BITS, D, DT, QT)                      \
+    do {                                         \
+        if (mm == 0) PF_M(BITS, D, DT, QT, 0);   \
+        else if (mm == 1) PF_M(BITS, D, DT, QT, 1); \
+        else PF_M(BITS, D, DT, QT, 2);           \
+    } while (0)
+#define PF_QT(BITS, D, DT)                       \
+    do {                                         \
+        if (wide) PF(BITS, D, DT, 2);            \
+        else PF(BITS, D, DT, 1);                 \
     } while (0)
 #define PF_DT(BITS, D)                           \
     do {                                         \
-        if (st.dtype == KVHIP_F16) PF(BITS, D, 0); \
-        else PF(BITS, D, 1);                     \
+        if (st.dtype == KVHIP_F16) PF_QT(BITS, D, 0); \
+        else PF_QT(BITS, D, 1);                  \
     } while (0)
 #define PF_D(BITS)                               \
     do {                                         \
@@ -354,10 +442,13 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
     else if (st.bits == 8) PF_D(8);
     else if (st.Dk == 64) PF_DT(0, 64);
     else if (st.Dk == 128) PF_DT(0, 128);
-    else PF_DT(0, 256);
+    else if (st.dtype == KVHIP_F16) PF(0, 256, 0, 1);
+    else PF(0, 256, 1, 1);
 #undef PF_D
 #undef PF_DT
+#undef PF_QT
 #undef PF
+#undef PF_M
     return hipGetLastError();
 }
 

@@ -33,4 +33,28 @@ __device__ __forceinline__ bool mask_keep(const MaskDev &m, int b, int hq, int l
     }
 }
 
+// Index-only masks (causal, window with optional per-batch bounds) with the per-batch
+// bounds already in registers: no memory access, so kernels can keep loads in flight.
+struct SymMask {
+    int mode, offset, window, len_b, pad_b, T, L;
+};
+__device__ __forceinline__ SymMask sym_mask_init(const MaskDev &m, int b, int L, int T) {
+    SymMask s;
+    s.mode = m.mode;
+    s.offset = m.offset;
+    s.window = m.window;
+    s.len_b = (m.mode == KVHIP_MASK_WINDOW && m.lengths) ? m.lengths[b] : 0x7fffffff;
+    s.pad_b = (m.mode == KVHIP_MASK_WINDOW && m.left_pad) ? m.left_pad[b] : 0;
+    s.T = T;
+    s.L = L;
+    return s;
+}
+__device__ __forceinline__ bool sym_mask_keep(const SymMask &s, int l, int j) {
+    if (s.mode == KVHIP_MASK_CAUSAL) return j <= s.T - s.L + l;
+    const int li = s.offset + l;
+    bool keep = li >= j && j < s.len_b && j >= s.pad_b;
+    if (s.window > 0) keep = keep && (li < j + s.window);
+    return keep;
+}
+
 }  // namespace kvhip
