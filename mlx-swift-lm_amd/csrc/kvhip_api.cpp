@@ -631,6 +631,9 @@ kvhip_status kvhip_cache_attend(kvhip_cache *c, const void *q, int32_t B, int32_
         KV_HIP(launch_attend_decode(a, s));
         g_last_kernel = a.st.bits ? 1 : 2;
     } else if (g_policy == 0 && attend_prefill_supported(a)) {
+        KV_TRY(ensure_ws(c, attend_prefill_workspace(a), s));
+        a.workspace = c->ws;
+        a.workspace_bytes = c->ws_bytes;
         KV_HIP(launch_attend_prefill(a, s));
         g_last_kernel = 3;
     } else {

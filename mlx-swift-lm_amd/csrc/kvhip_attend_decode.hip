@@ -821,6 +821,21 @@ hipError_t profile_read(int *launches, double *total_ms) {
     return hipSuccess;
 }
 
+hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s) {
+    const int R = (a.Hq / a.Hkv) * a.L;
+    dim3 grid(R, a.st.BH);
+#define CMB(D)                                                                                       \
+    do {                                                                                             \
+        if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL((combine_kernel<D, 0>), grid, dim3(D), 0, s, a, nsplit, rows); \
+        else hipLaunchKernelGGL((combine_kernel<D, 1>), grid, dim3(D), 0, s, a, nsplit, rows);       \
+    } while (0)
+    if (a.st.Dk == 64) CMB(64);
+    else if (a.st.Dk == 128) CMB(128);
+    else CMB(256);
+#undef CMB
+    return hipGetLastError();
+}
+
 bool attend_decode_supported(const AttendArgs &a) {
     const Store &s = a.st;
     if (s.dtype != KVHIP_F16 && s.dtype != KVHIP_BF16) return false;

@@ -41,7 +41,7 @@ __device__ __forceinline__ uint32_t h2_bits(float lo, float hi) { return (uint32
 // (causal / window, no memory access in the loop), 2 array mask.
 template <int BITS, int D, int DT, bool IDENT, int QT, int MM>
 __global__ void __launch_bounds__(256, 2)
-prefill_kernel(AttendArgs a) {
+prefill_kernel(AttendArgs a, int nsplit) {
     constexpr bool Q = BITS != 0;
     constexpr int BM = 64 * QT;
     constexpr int KS = D + 8;    // halves per K row in LDS (padded against bank conflicts)
@@ -118,6 +118,15 @@ prefill_kernel(AttendArgs a) {
             if (a.mask.window > 0) tile_lo = max(0, (a.mask.offset + l_min - a.mask.window + 1) / BN);
         }
         tile_hi = min(tile_hi, (a.T + BN - 1) / BN);
+    }
+
+    // ---- optional split of the key range over blockIdx.z (small grids): each part leaves an
+    // unnormalised partial per query row, merged by the decode path's combine kernel
+    const int split = blockIdx.z;
+    if (nsplit > 1) {
+        const int span = (tile_hi - tile_lo + nsplit - 1) / nsplit;
+        tile_lo = tile_lo + split * span;
+        tile_hi = min(tile_hi, tile_lo + span);
     }
 
     // ---- staging: a tile is fetched from global memory into registers one iteration ahead
@@ -379,6 +388,18 @@ prefill_kernel(AttendArgs a) {
         l += __shfl_xor(l, 16);
         l += __shfl_xor(l, 32);
         if (!q_ok[qt]) continue;
+        if (nsplit > 1) {
+            const int i = row0 + 16 * qt + n;
+            float *part = a.workspace + (((size_t)bh * nsplit + split) * R + i) * (D + 2);
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt)
+                *reinterpret_cast<f4 *>(part + 16 * dt + 4 * jj) = oacc[qt][dt];
+            if (jj == 0) {
+                part[D] = m_run[qt];
+                part[D + 1] = l;
+            }
+            continue;
+        }
         const float inv = l > 0.f ? 1.0f / l : 0.f;
         const size_t ooff = ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D;
 #pragma unroll
@@ -400,6 +421,27 @@ bool attend_prefill_supported(const AttendArgs &a) {
     return (a.Hq / a.Hkv) * a.L > 16;
 }
 
+// Key-range parts per query block: only when the grid would leave most CUs without a
+// second workgroup, and only while the partials stay small.
+static int prefill_splits(const AttendArgs &a) {
+    const int R = (a.Hq / a.Hkv) * a.L;
+    const bool wide = (size_t)((R + 127) / 128) * a.st.BH >= 512 && a.st.Dk <= 128;
+    const size_t wgs = (size_t)((R + (wide ? 127 : 63)) / (wide ? 128 : 64)) * a.st.BH;
+    int n = (int)(768 / (wgs ? wgs : 1));
+    const int tiles = (a.slots + BN - 1) / BN;
+    if (n > tiles / 8) n = tiles / 8;
+    if (n > 8) n = 8;
+    if (n < 2) return 1;
+    if ((size_t)a.st.BH * n * R * (a.st.Dk + 2) * sizeof(float) > ((size_t)256 << 20)) return 1;
+    return n;
+}
+
+size_t attend_prefill_workspace(const AttendArgs &a) {
+    const int n = prefill_splits(a);
+    if (n <= 1) return 0;
+    return (size_t)a.st.BH * n * (a.Hq / a.Hkv) * a.L * (a.st.Dk + 2) * sizeof(float);
+}
+
 hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
     const Store &st = a.st;
     const int R = (a.Hq / a.Hkv) * a.L;
@@ -407,14 +449,15 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
     // when that would leave the grid too small to fill 256 CUs twice over
     const bool wide = (size_t)((R + 127) / 128) * st.BH >= 512 && st.Dk <= 128;
     const int bm = wide ? 128 : 64;
-    dim3 grid((R + bm - 1) / bm, st.BH), block(256);
+    const int nsplit = prefill_splits(a);
+    dim3 grid((R + bm - 1) / bm, st.BH, nsplit), block(256);
     const bool ident = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
     const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
 #define PF_M(BITS, D, DT, QT, MM)                                                                         \
     do {                                                                                                  \
         profile_mark(s, true);                                                                            \
-        if (ident) hipLaunchKernelGGL((prefill_kernel<BITS, D, DT, true, QT, MM>), grid, block, 0, s, a); \
-        else hipLaunchKernelGGL((prefill_kernel<BITS, D, DT, false, QT, MM>), grid, block, 0, s, a);      \
+        if (ident) hipLaunchKernelGGL((prefill_kernel<BITS, D, DT, true, QT, MM>), grid, block, 0, s, a, nsplit); \
+        else hipLaunchKernelGGL((prefill_kernel<BITS, D, DT, false, QT, MM>), grid, block, 0, s, a, nsplit);      \
         profile_mark(s, false);                                                                           \
     } while (0)
 #define PF(BITS, D, DT, QT)                      \
@@ -449,6 +492,10 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
 #undef PF_QT
 #undef PF
 #undef PF_M
+    if (nsplit > 1) {
+        hipError_t e = launch_combine(a, nsplit, R, s);
+        if (e != hipSuccess) return e;
+    }
     return hipGetLastError();
 }
 

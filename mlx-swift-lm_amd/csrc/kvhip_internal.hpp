@@ -175,6 +175,10 @@ size_t attend_decode_workspace(const AttendArgs &a);
 hipError_t launch_attend_decode(const AttendArgs &a, hipStream_t s);
 // Matrix-core chunked-prefill tile (many query rows per kv head).
 bool attend_prefill_supported(const AttendArgs &a);
+size_t attend_prefill_workspace(const AttendArgs &a);
+// Merge `nsplit` partials per query row, laid out [bh][split][rows][D+2] in a.workspace
+// (out[D] unnormalised, running max, running sum), and write the normalised rows to a.out.
+hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s);
 hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s);
 // Event bracket around the dominant kernel while profiling is enabled.
 void profile_enable(bool on);
