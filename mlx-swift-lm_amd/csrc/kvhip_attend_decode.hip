@@ -194,6 +194,10 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     __shared__ float cbuf[WAVES][RR][D + 2];
 
     // ---- query operands: lane (blk, qi) holds row qi's 4 elements of step 16 x + blk ----
+    // qsum[rg][g][i] = sum over group g of the (rounded, fp16-held) query row 4 rg + i, for
+    // the bias term; built from the same registers: the 16 steps of one operand pair lie in
+    // one group (group sizes are multiples of 64), so a lane sums its 4 elements, the 16
+    // lane groups are added up by shuffles and the four rows are read out of their quad.
     Op qa[RG][NQA];
     float qsum[RG][G][4];
 #pragma unroll
@@ -201,6 +205,9 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         const int i = 4 * rg + qi;
         const int rep = i / a.L, l = i - rep * a.L;
         const size_t qoff = ((size_t)(b * a.Hq + hk * r + rep) * a.L + l) * D;
+        float part[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) part[g] = 0.f;
 #pragma unroll
         for (int x = 0; x < NQA; ++x) {
             const int step = 16 * x + blk;
@@ -210,27 +217,21 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             for (int k = 0; k < 4; ++k) {
                 const int d = w * GEO::EPW + GEO::elem(h, k);
                 float v = 0.f;
-                if (i < R) v = round_dt<DT>(Elem<DT>::load(a.q, qoff + d) * a.scale);
+                if (i < R) v = (float)(_Float16)round_dt<DT>(Elem<DT>::load(a.q, qoff + d) * a.scale);
+                part[(64 * x) / GS] += v;
                 qv[k] = GEO::hi(k) ? v * 0.0625f : v;
             }
             qa[rg][x].u[0] = pack_h2(qv[0], qv[1]);
             qa[rg][x].u[1] = pack_h2(qv[2], qv[3]);
         }
 #pragma unroll
-        for (int g = 0; g < G; ++g)
+        for (int g = 0; g < G; ++g) {
+            float v = part[g];
+            for (int off = 4; off < 64; off <<= 1) v += __shfl_xor(v, off);  // over the 16 lane groups
 #pragma unroll
-            for (int ii = 0; ii < 4; ++ii) {
-                float sacc = 0.f;
-                const int i2 = 4 * rg + ii;
-                if (i2 < R) {
-                    // sum of the (rounded, fp16-held) queries of the group, for the bias term
-                    const int rep2 = i2 / a.L, l2 = i2 - rep2 * a.L;
-                    const size_t qo = ((size_t)(b * a.Hq + hk * r + rep2) * a.L + l2) * D;
-                    for (int d = g * GS + lane; d < (g + 1) * GS; d += 64)
-                        sacc += (float)(_Float16)round_dt<DT>(Elem<DT>::load(a.q, qo + d) * a.scale);
-                }
-                qsum[rg][g][ii] = wave_sum(sacc);
-            }
+            for (int ii = 0; ii < 4; ++ii)  // wave-uniform: keep it in a scalar register
+                qsum[rg][g][ii] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), ii));
+        }
     }
 
     // ---- running state ---------------------------------------------------------------
@@ -248,10 +249,23 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         for (int h = 0; h < NH; ++h) oacc[rg][h] = f4{0.f, 0.f, 0.f, 0.f};
     }
 
-    const int tile_begin = split * tiles_per_wg;
-    const int tile_end = min(tiles_total, tile_begin + tiles_per_wg);
     const float fill = finfo_min_dt(DT);
     const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
+    int tile_begin = split * tiles_per_wg;
+    int tile_end = min(tiles_total, tile_begin + tiles_per_wg);
+    if constexpr (MM == 1) {
+        // length-aware partition: an index-only mask bounds the rows this (batch) can see
+        // (left padding, lengths, causal/window reach); spans of equal size start at the first
+        // visible tile, so a ragged batch gets workgroups in proportion to each length
+        int vis_lo, vis_hi;
+        sym_mask_row_range(sym, vis_lo, vis_hi);
+        const int t_lo = max(0, vis_lo) >> 6, t_hi = min(tiles_total, (min(vis_hi, a.T - 1) >> 6) + 1);
+        // tiles_per_wg == 0: divide this batch row's own visible range over the spans
+        const int per = tiles_per_wg > 0 ? tiles_per_wg
+                                         : (max(t_hi - t_lo, 1) + nsplit * WAVES - 1) / (nsplit * WAVES) * WAVES;
+        tile_begin = t_lo + split * per;  // spans past t_hi are empty
+        tile_end = min(t_hi, tile_begin + per);
+    }
     int mrow_l[RG][4];  // query position l of each carried row
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg)
@@ -366,7 +380,8 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             if (__any(need)) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const float mn = fmaxf(m_run[rg][i], wave_max(sc[i]));
+                    const float mn = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(
+                        __builtin_bit_cast(int, fmaxf(m_run[rg][i], wave_max(sc[i])))));
                     const float alpha = (mn == -INFINITY) ? 1.f : fast_exp2((m_run[rg][i] - mn) * LOG2E);
                     m_run[rg][i] = mn;
                     l_part[rg][i] *= alpha;
@@ -552,8 +567,18 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     for (int rg = 0; rg < RG; ++rg)
 #pragma unroll
         for (int i = 0; i < 4; ++i) mrow_l[rg][i] = (4 * rg + i) % a.L;
-    const int tile_begin = split * tiles_per_wg;
-    const int tile_end = min(tiles_total, tile_begin + tiles_per_wg);
+    int tile_begin = split * tiles_per_wg;
+    int tile_end = min(tiles_total, tile_begin + tiles_per_wg);
+    if constexpr (MM == 1 && IDENT) {
+        int vis_lo, vis_hi;
+        sym_mask_row_range(sym, vis_lo, vis_hi);
+        const int t_lo = max(0, vis_lo) >> 6, t_hi = min(tiles_total, (min(vis_hi, a.T - 1) >> 6) + 1);
+        // tiles_per_wg == 0: divide this batch row's own visible range over the spans
+        const int per = tiles_per_wg > 0 ? tiles_per_wg
+                                         : (max(t_hi - t_lo, 1) + nsplit * WAVES - 1) / (nsplit * WAVES) * WAVES;
+        tile_begin = t_lo + split * per;  // spans past t_hi are empty
+        tile_end = min(t_hi, tile_begin + per);
+    }
     const int tile0 = tile_begin + wave;
     const int my_tiles = tile0 < tile_end ? (tile_end - tile0 + WAVES - 1) / WAVES : 0;
     const size_t k_step = (size_t)st.BH * st.k_cell, v_step = (size_t)st.BH * st.v_cell;
@@ -786,6 +811,12 @@ Plan plan_for(const AttendArgs &a) {
     per = (per + WAVES - 1) / WAVES * WAVES;
     p.tiles_per_wg = per;
     p.nsplit = (p.tiles_total + per - 1) / per;
+    // ragged batches (per-batch bounds): the same number of spans for every batch row, each
+    // row's visible range divided among them in the kernel (all workgroups stay resident
+    // and none is empty; measured faster than equal-sized spans with more of them for the
+    // long rows)
+    if (a.mask.mode == KVHIP_MASK_WINDOW && (a.mask.left_pad || a.mask.lengths) && !getenv("KVHIP_DECODE_TILES"))
+        p.tiles_per_wg = 0;
     return p;
 }
 

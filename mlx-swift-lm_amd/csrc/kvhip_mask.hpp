@@ -57,4 +57,16 @@ __device__ __forceinline__ bool sym_mask_keep(const SymMask &s, int l, int j) {
     return keep;
 }
 
+// Inclusive range of key rows any query position l in [0, L) may see under an index-only mask.
+__device__ __forceinline__ void sym_mask_row_range(const SymMask &s, int &lo, int &hi) {
+    if (s.mode == KVHIP_MASK_CAUSAL) {
+        lo = 0;
+        hi = s.T - 1;
+        return;
+    }
+    lo = s.pad_b;
+    hi = min(s.offset + s.L - 1, s.len_b - 1);
+    if (s.window > 0) lo = max(lo, s.offset - s.window + 1);
+}
+
 }  // namespace kvhip
