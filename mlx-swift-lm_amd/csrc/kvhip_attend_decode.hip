@@ -67,13 +67,37 @@ template <int ABID> __device__ __forceinline__ f4 mfma444_bf(const Op &a, const 
 // v_exp_f32 without the denormal-range fix-up (results below 2^-126 flush to zero)
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Wavefront reductions on the data-parallel-primitive path (no LDS round trips): two quad
+// permutes and two row mirrors leave each row of 16 lanes reduced, two row broadcasts
+// carry the rows into lane 63, which is read out as a wave-uniform scalar.
+template <int CTRL, int ROWS>
+__device__ __forceinline__ float dpp_take(float v) {  // v of the lane CTRL names; own v outside ROWS
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v),
+                                                                 CTRL, ROWS, 0xF, false));
+}
 __device__ __forceinline__ float wave_max(float v) {
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    return v;
+    v = fmaxf(v, dpp_take<0xB1, 0xF>(v));   // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_take<0x4E, 0xF>(v));   // quad_perm [2,3,0,1]
+    v = fmaxf(v, dpp_take<0x141, 0xF>(v));  // row_half_mirror
+    v = fmaxf(v, dpp_take<0x140, 0xF>(v));  // row_mirror
+    v = fmaxf(v, dpp_take<0x142, 0xA>(v));  // row_bcast15 into rows 1 and 3
+    v = fmaxf(v, dpp_take<0x143, 0xC>(v));  // row_bcast31 into rows 2 and 3
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 __device__ __forceinline__ float wave_sum(float v) {
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-    return v;
+    v += dpp_take<0xB1, 0xF>(v);
+    v += dpp_take<0x4E, 0xF>(v);
+    v += dpp_take<0x141, 0xF>(v);
+    v += dpp_take<0x140, 0xF>(v);
+    // the broadcast steps must add only into the rows they target
+    const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xA, 0xF, false));
+    v += r1;
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xC, 0xF, false));
+    v += r2;
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+__device__ __forceinline__ float uniform(float v) {  // v is the same in every lane
+    return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
 }
 __device__ __forceinline__ uint16_t f2h_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
 __device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
@@ -165,7 +189,8 @@ template <int BITS, int D, int G> struct TileRegs {
     uint32_t k[KW];
     uint32_t v[D / 64][VW];
     float ks[G], kb[G], vs[G], vb[G];
-    int row;  // presented row of this lane's token, -1 if none
+    int row;    // presented row of this lane's token, -1 if none
+    bool edge;  // wave-uniform: some token of the tile is dead or masked for some query row
 };
 
 // RG = groups of 4 query rows handled per pass (R <= 4 RG).  MM selects the mask code:
@@ -235,12 +260,13 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     }
 
     // ---- running state ---------------------------------------------------------------
-    float m_run[RG][4], l_part[RG][4], bacc[RG][G][4];
+    // m_use = m_run, or 0 while m_run is still -inf, so exp2((s - m_use) log2 e) needs no guard
+    float m_run[RG][4], m_use[RG][4], l_part[RG][4], bacc[RG][G][4];
     f4 oacc[RG][NH];
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { m_run[rg][i] = -INFINITY; l_part[rg][i] = 0.f; }
+        for (int i = 0; i < 4; ++i) { m_run[rg][i] = -INFINITY; m_use[rg][i] = 0.f; l_part[rg][i] = 0.f; }
 #pragma unroll
         for (int g = 0; g < G; ++g)
 #pragma unroll
@@ -290,7 +316,14 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     const uint32_t k_lane = lane * st.k_row, v_lane = lane * VROW;
     const uint32_t ksb_lane = lane * st.ksb_row, vsb_lane = lane * st.vsb_row;
     int slot_next = tile0 * TILE + lane;  // slot of this lane's token in the tile loaded next
+    int base_next = tile0 * TILE;         // its first slot (wave-uniform)
     int loaded = 0;                       // tiles loaded so far
+    // rows every query row keeps: tiles inside [full_lo, full_hi] need no mask or bound test
+    int full_lo = 0, full_hi = a.T - 1;
+    if constexpr (MM == 1) {
+        sym_mask_full_range(sym, full_lo, full_hi);
+        full_hi = min(full_hi, a.T - 1);
+    }
 
     // Loads tile number `loaded` of this wavefront (clamped to its last tile, so the
     // prefetch past the end stays unconditional and in bounds).
@@ -316,6 +349,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             }
         }
         t.row = slot_next < a.T ? slot_next : -1;
+        t.edge = base_next < full_lo || base_next + (TILE - 1) > full_hi;
         ++loaded;
         if (loaded < my_tiles) {  // wave-uniform: step to the same tile of the next page
             kp += k_step;
@@ -323,6 +357,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             ksp += ksb_step;
             vsp += vsb_step;
             slot_next += PAGE;
+            base_next += PAGE;
         }
     };
 
@@ -349,41 +384,61 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         });
 
         // ---- online softmax per row group; probabilities become PV A operands ------------
+        // Interior tiles (every token live and visible to every query row: the common case,
+        // decided per wavefront when the tile was loaded) skip all mask and bound tests.
         Op pa[RG][G];
+        float ks24[G], vsf[G];
 #pragma unroll
-        for (int rg = 0; rg < RG; ++rg) {
+        for (int g = 0; g < G; ++g) {
+            ks24[g] = t.ks[g] * TWO24;
+            vsf[g] = t.vs[g] * vfac;
+        }
+        auto softmax_rg = [&](auto RGC) {
+            constexpr int rg = decltype(RGC)::value;
             float sc[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float s_ = 0.f;
+                float s_ = t.kb[0] * qsum[rg][0][i];
 #pragma unroll
-                for (int g = 0; g < G; ++g) s_ += (t.ks[g] * TWO24) * sacc[rg][g][i] + t.kb[g] * qsum[rg][g][i];
-                s_ = round_dt<DT>(s_);
-                [[maybe_unused]] const int row_i = 4 * rg + i;
-                if constexpr (MM == 1) {
-                    if (!sym_mask_keep(sym, mrow_l[rg][i], t.row)) s_ = fill;
-                } else if constexpr (MM == 2) {
-                    if (live && row_i < R) {
-                        const int rep = row_i / a.L, l = row_i - rep * a.L;
-                        float add;
-                        const bool keep = mask_keep(a.mask, b, hk * r + rep, l, t.row, a.L, a.T, add);
-                        if (!keep) s_ = fill;
-                        else if (a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
-                    }
-                }
-                sc[i] = live ? s_ : -INFINITY;
+                for (int g = 1; g < G; ++g) s_ = __builtin_fmaf(t.kb[g], qsum[rg][g][i], s_);
+#pragma unroll
+                for (int g = 0; g < G; ++g) s_ = __builtin_fmaf(ks24[g], sacc[rg][g][i], s_);
+                sc[i] = round_dt<DT>(s_);
             }
-            // raise the running maximum only when this tile exceeds it
+            if (MM == 2 || t.edge) {  // wave-uniform
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float s_ = sc[i];
+                    [[maybe_unused]] const int row_i = 4 * rg + i;
+                    if constexpr (MM == 1) {
+                        if (!sym_mask_keep(sym, mrow_l[rg][i], t.row)) s_ = fill;
+                    } else if constexpr (MM == 2) {
+                        if (live && row_i < R) {
+                            const int rep = row_i / a.L, l = row_i - rep * a.L;
+                            float add;
+                            const bool keep = mask_keep(a.mask, b, hk * r + rep, l, t.row, a.L, a.T, add);
+                            if (!keep) s_ = fill;
+                            else if (a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
+                        }
+                    }
+                    sc[i] = live ? s_ : -INFINITY;
+                }
+            }
+            // raise the running maximum only when this tile exceeds it (rare after the first
+            // few tiles; the empty asm keeps the reductions inside the branch)
             bool need = false;
 #pragma unroll
             for (int i = 0; i < 4; ++i) need = need || (sc[i] > m_run[rg][i]);
             if (__any(need)) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const float mn = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(
-                        __builtin_bit_cast(int, fmaxf(m_run[rg][i], wave_max(sc[i])))));
+                    float x_ = sc[i];
+                    asm volatile("" : "+v"(x_));
+                    // wave-uniform values, kept in scalar registers
+                    const float mn = uniform(fmaxf(m_run[rg][i], wave_max(x_)));
                     const float alpha = (mn == -INFINITY) ? 1.f : fast_exp2((m_run[rg][i] - mn) * LOG2E);
                     m_run[rg][i] = mn;
+                    m_use[rg][i] = uniform((mn == -INFINITY) ? 0.f : mn);
                     l_part[rg][i] *= alpha;
 #pragma unroll
                     for (int g = 0; g < G; ++g) bacc[rg][g][i] *= alpha;
@@ -394,13 +449,14 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             uint32_t x[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const float p = (sc[i] == -INFINITY) ? 0.f : fast_exp2((sc[i] - m_run[rg][i]) * LOG2E);
+                // exp2(-inf) = 0 covers dead lanes; m_use is finite even before any live token
+                const float p = fast_exp2((sc[i] - m_use[rg][i]) * LOG2E);
                 l_part[rg][i] += p;
                 float pv[2] = {0.f, 0.f};
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
-                    bacc[rg][g][i] += p * t.vb[g];
-                    pv[g] = p * (t.vs[g] * vfac);
+                    bacc[rg][g][i] = __builtin_fmaf(p, t.vb[g], bacc[rg][g][i]);
+                    pv[g] = p * vsf[g];
                 }
                 x[i] = pack_h2(pv[0], pv[1]);
             }
@@ -412,7 +468,8 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 pa[rg][G - 1].u[0] = __builtin_amdgcn_perm(x[1], x[0], 0x07060302u);
                 pa[rg][G - 1].u[1] = __builtin_amdgcn_perm(x[3], x[2], 0x07060302u);
             }
-        }
+        };
+        static_for<RG>([&](auto RGC) { softmax_rg(RGC); });
 
         // ---- out += P . V: lane supplies column lane (+64 h), step s = tokens 4s..4s+3 ------
         static_for<NH>([&](auto HH) {
@@ -671,7 +728,9 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 if (__any(need)) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
-                        const float mn = fmaxf(m_run[rg][i], wave_max(sc[i]));
+                        float x_ = sc[i];
+                        asm volatile("" : "+v"(x_));  // keeps the reduction inside the branch
+                        const float mn = fmaxf(m_run[rg][i], wave_max(x_));
                         const float alpha = (mn == -INFINITY) ? 1.f : fast_exp2((m_run[rg][i] - mn) * LOG2E);
                         m_run[rg][i] = mn;
                         l_part[rg][i] *= alpha;

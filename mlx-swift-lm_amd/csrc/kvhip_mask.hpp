@@ -69,4 +69,16 @@ __device__ __forceinline__ void sym_mask_row_range(const SymMask &s, int &lo, in
     if (s.window > 0) lo = max(lo, s.offset - s.window + 1);
 }
 
+// Inclusive range of key rows EVERY query position l in [0, L) sees (empty if lo > hi).
+__device__ __forceinline__ void sym_mask_full_range(const SymMask &s, int &lo, int &hi) {
+    if (s.mode == KVHIP_MASK_CAUSAL) {
+        lo = 0;
+        hi = s.T - s.L;
+        return;
+    }
+    lo = s.pad_b;
+    hi = min(s.offset, s.len_b - 1);
+    if (s.window > 0) lo = max(lo, s.offset + s.L - s.window);
+}
+
 }  // namespace kvhip
