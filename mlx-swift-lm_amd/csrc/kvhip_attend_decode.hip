@@ -317,7 +317,6 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     const uint32_t ksb_lane = lane * st.ksb_row, vsb_lane = lane * st.vsb_row;
     int slot_next = tile0 * TILE + lane;  // slot of this lane's token in the tile loaded next
     int base_next = tile0 * TILE;         // its first slot (wave-uniform)
-    int loaded = 0;                       // tiles loaded so far
     // rows every query row keeps: tiles inside [full_lo, full_hi] need no mask or bound test
     int full_lo = 0, full_hi = a.T - 1;
     if constexpr (MM == 1) {
@@ -325,43 +324,62 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         full_hi = min(full_hi, a.T - 1);
     }
 
-    // Loads tile number `loaded` of this wavefront (clamped to its last tile, so the
-    // prefetch past the end stays unconditional and in bounds).
-    auto load_tile = [&](T &t) {
+    // The K half (codes, scales, row bookkeeping) and the V half of tile number k_loaded /
+    // v_loaded of this wavefront (clamped to its last tile, so loads past the end stay
+    // unconditional and in bounds).
+    int k_loaded = 0, v_loaded = 0;
+    auto load_k = [&](T &t) {
         load_words<T::KW>(t.k, kp + k_lane);
-#pragma unroll
-        for (int h = 0; h < NH; ++h) load_words<T::VW>(t.v[h], vp + v_lane + (size_t)h * 64 * VROW);
-        uint32_t kraw[G], vraw[G];  // (scale, bias) pairs of a 16-bit dtype
+        uint32_t kraw[G];  // (scale, bias) pairs of a 16-bit dtype
         load_words<G>(kraw, ksp + ksb_lane);
-        load_words<G>(vraw, vsp + vsb_lane);
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             if (DT == 0) {
                 t.ks[g] = (float)__builtin_bit_cast(_Float16, (uint16_t)kraw[g]);
                 t.kb[g] = (float)__builtin_bit_cast(_Float16, (uint16_t)(kraw[g] >> 16));
-                t.vs[g] = (float)__builtin_bit_cast(_Float16, (uint16_t)vraw[g]);
-                t.vb[g] = (float)__builtin_bit_cast(_Float16, (uint16_t)(vraw[g] >> 16));
             } else {
                 t.ks[g] = __uint_as_float(kraw[g] << 16);
                 t.kb[g] = __uint_as_float(kraw[g] & 0xffff0000u);
-                t.vs[g] = __uint_as_float(vraw[g] << 16);
-                t.vb[g] = __uint_as_float(vraw[g] & 0xffff0000u);
             }
         }
         t.row = slot_next < a.T ? slot_next : -1;
         t.edge = base_next < full_lo || base_next + (TILE - 1) > full_hi;
-        ++loaded;
-        if (loaded < my_tiles) {  // wave-uniform: step to the same tile of the next page
+        ++k_loaded;
+        if (k_loaded < my_tiles) {  // wave-uniform: step to the same tile of the next page
             kp += k_step;
-            vp += v_step;
             ksp += ksb_step;
-            vsp += vsb_step;
             slot_next += PAGE;
             base_next += PAGE;
         }
     };
+    auto load_v = [&](T &t) {
+#pragma unroll
+        for (int h = 0; h < NH; ++h) load_words<T::VW>(t.v[h], vp + v_lane + (size_t)h * 64 * VROW);
+        uint32_t vraw[G];
+        load_words<G>(vraw, vsp + vsb_lane);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            if (DT == 0) {
+                t.vs[g] = (float)__builtin_bit_cast(_Float16, (uint16_t)vraw[g]);
+                t.vb[g] = (float)__builtin_bit_cast(_Float16, (uint16_t)(vraw[g] >> 16));
+            } else {
+                t.vs[g] = __uint_as_float(vraw[g] << 16);
+                t.vb[g] = __uint_as_float(vraw[g] & 0xffff0000u);
+            }
+        }
+        ++v_loaded;
+        if (v_loaded < my_tiles) {
+            vp += v_step;
+            vsp += vsb_step;
+        }
+    };
+    auto load_tile = [&](T &t) {
+        load_k(t);
+        load_v(t);
+    };
 
-    auto compute_tile = [&](const T &t) {
+    Op pa[RG][G];  // probabilities of the tile in flight, as PV operands
+    auto compute_qk_softmax = [&](const T &t) {
         const bool live = t.row >= 0;
         // ---- QK^T: scores of token `lane` for every query row ---------------------------
         f4 sacc[RG][G];
@@ -386,7 +404,6 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         // ---- online softmax per row group; probabilities become PV A operands ------------
         // Interior tiles (every token live and visible to every query row: the common case,
         // decided per wavefront when the tile was loaded) skip all mask and bound tests.
-        Op pa[RG][G];
         float ks24[G], vsf[G];
 #pragma unroll
         for (int g = 0; g < G; ++g) {
@@ -470,8 +487,10 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             }
         };
         static_for<RG>([&](auto RGC) { softmax_rg(RGC); });
+    };
 
-        // ---- out += P . V: lane supplies column lane (+64 h), step s = tokens 4s..4s+3 ------
+    // ---- out += P . V: lane supplies column lane (+64 h), step s = tokens 4s..4s+3 ----------
+    auto compute_pv = [&](const T &t) {
         static_for<NH>([&](auto HH) {
             constexpr int h = decltype(HH)::value;
             constexpr int g = (64 * h) / GS;
@@ -489,10 +508,16 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         });
     };
 
-    // ---- main loop: one tile of loads in flight ahead of the arithmetic (variants whose
-    // tile does not fit twice in the register file run single-buffered and lean on the
-    // other resident wavefronts)
-    constexpr bool PREFETCH = (RG == 1 && !(BITS == 8 && D == 128)) || (RG == 2 && BITS == 4 && D == 64);
+    auto compute_tile = [&](const T &t) {
+        compute_qk_softmax(t);
+        compute_pv(t);
+    };
+
+    // ---- main loop.  Variants whose tile fits twice in the register file keep one whole
+    // tile of loads in flight ahead of the arithmetic.  The others run one buffer with the
+    // halves skewed: V of a tile is requested before its QK^T and softmax, K of the next
+    // tile before its PV, so each half has the other half's arithmetic to arrive in.
+    constexpr bool PREFETCH = (RG == 1 && !(BITS == 8 && D == 128)) || (BITS == 4 && (RG == 2 || D == 64));
     if (my_tiles > 0) {
         if constexpr (PREFETCH) {
             T bufA, bufB;
@@ -507,9 +532,12 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             }
         } else {
             T buf;
+            load_k(buf);
             for (int done = 0; done < my_tiles; ++done) {
-                load_tile(buf);
-                compute_tile(buf);
+                load_v(buf);
+                compute_qk_softmax(buf);
+                load_k(buf);
+                compute_pv(buf);
             }
         }
     }
@@ -945,11 +973,21 @@ size_t attend_decode_workspace(const AttendArgs &a) {
     return (size_t)a.st.BH * p.nsplit * 4 * p.rg * (a.st.Dk + 2) * sizeof(float);
 }
 
-hipError_t launch_attend_decode(const AttendArgs &a, hipStream_t s) {
+hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
+    AttendArgs a = a_in;
     const Plan p = plan_for(a);
     const Store &st = a.st;
     dim3 grid(p.nsplit, st.BH), block(WAVES * 64);
     const int R = (a.Hq / a.Hkv) * a.L;
+    if (st.bits != 0 && p.rg == 4 && a.mask.mode == KVHIP_MASK_NONE) {
+        // the 16-row unmasked variants need more registers than the index-mask ones (which
+        // the compiler schedules tighter); an all-visible window is the same computation
+        a.mask.mode = KVHIP_MASK_WINDOW;
+        a.mask.offset = 1 << 30;
+        a.mask.window = 0;
+        a.mask.lengths = nullptr;
+        a.mask.left_pad = nullptr;
+    }
     const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
 #define DEC(BITS, D, GS, DT, RG)                                                                          \
     do {                                                                                                  \
