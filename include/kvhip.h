@@ -222,6 +222,39 @@ int32_t kvhip_cache_meta_count(const kvhip_cache *cache);
 int32_t kvhip_cache_meta_get(const kvhip_cache *cache, int32_t index, char *buf, int32_t buf_len);
 kvhip_status kvhip_cache_meta_set(kvhip_cache *cache, int32_t count, const char *const *values);
 
+/* ---- staged rounds on a ring ------------------------------------------------ */
+/*
+ * `RotatingStagedKVCache` (RotatingStagedKVCache.swift:12-132) and the rotating leaf of a
+ * speculative round (`RotatingRoundStrategy`, KVCacheRound.swift:128-156), folded into the
+ * ring's own handle.  Between `stage_begin` and `stage_commit` the handle behaves as the
+ * staged wrapper:
+ *   - `kvhip_cache_update` stages its rows (device copy into spare slots; the ring and its
+ *     offset / idx stay untouched) and the presentation becomes
+ *     logicalView(tail: min(offset, maxSize-1)) ++ staged (RotatingStagedKVCache.swift:78-91),
+ *     which `kvhip_cache_fetch` exports and `kvhip_cache_attend` reads in place;
+ *   - offset, idx, is_trimmable, trim, state export, meta_get and `kvhip_cache_mask_plan`
+ *     keep answering for the live ring, which does not move (:49-58, :95-111); the
+ *     wrapper's own `offset` is kvhip_cache_offset + kvhip_cache_stage_count (:33-37), its
+ *     `isTrimmable` is false and its `trim` returns 0 (:113-119) -- the host shim says so
+ *     without a call;
+ *   - state import, meta_set and copy fail with KVHIP_ERR_STATE (the reference traps).
+ * Only KVHIP_KIND_ROTATING stages; the other kinds are written through and trimmed
+ * (`AppendOnlyRoundStrategy`, KVCacheRound.swift:99-125) and get KVHIP_ERR_INVALID_ARG here.
+ */
+kvhip_status kvhip_cache_stage_begin(kvhip_cache *cache);
+int32_t kvhip_cache_stage_is_open(const kvhip_cache *cache);
+/* `stagedCount` (RotatingStagedKVCache.swift:23). */
+int64_t kvhip_cache_stage_count(const kvhip_cache *cache);
+/* `stagedArrays` (RotatingStagedKVCache.swift:27-30): the staged rows as [B,Hkv,n,D] pairs. */
+kvhip_status kvhip_cache_stage_fetch(const kvhip_cache *cache, void *dst_keys, void *dst_values, void *stream);
+/*
+ * `commit(retaining:)` (RotatingStagedKVCache.swift:62-76): the first
+ * min(max(retaining,0), staged) rows are appended to the ring through the normal write
+ * path (`kvhip_cache_update` semantics for that many rows), the rest are dropped, and the
+ * round closes.  retaining = 0 is a rollback.
+ */
+kvhip_status kvhip_cache_stage_commit(kvhip_cache *cache, int64_t retaining, void *stream);
+
 /* ---- ring reads and conversions ------------------------------------------ */
 /*
  * `RotatingKVCache.logicalView(tail:)` (KVCache.swift:631-658): chronological

@@ -66,6 +66,14 @@ struct kvhip_cache {
     std::vector<int32_t> rows;
     std::vector<uint8_t> used;
     int64_t cursor = 0;
+    // rotating only: an open staged round (RotatingStagedKVCache.swift:12-132).  Staged rows
+    // sit in spare slots of the same page store; the ring's own rows are untouched until commit.
+    bool staging = false;
+    std::vector<int32_t> staged;      // slots of the staged rows, in write order
+    std::vector<int32_t> stage_view;  // slots of the presentation: trailing window ++ staged
+    int64_t presented_live = 0;       // `presented` of the live ring when the round opened
+    void *stage_tmp_k = nullptr, *stage_tmp_v = nullptr;  // dense copy of the rows a commit keeps
+    size_t stage_tmp_rows = 0;
     // scratch for attention
     float *ws = nullptr;
     size_t ws_bytes = 0;
@@ -293,11 +301,12 @@ kvhip_status write_rows(kvhip_cache *c, const void *keys, const void *values, in
     return KVHIP_OK;
 }
 
-// If the presented rows are scattered over more runs than a kernel takes, gather them
-// into slot order once (ring-order gather) so later launches see a single run.
-kvhip_status ring_compact_if_needed(kvhip_cache *c, hipStream_t stream) {
-    const RunList rl = runs_of(c->rows.data(), (int64_t)c->rows.size());
-    if (rl.size() <= (size_t)MAXRUNS) return KVHIP_OK;
+// Gather every live row (ring rows, then staged rows) into slot order in a fresh store, so
+// that later launches see single runs.
+kvhip_status compact_store(kvhip_cache *c, hipStream_t stream) {
+    std::vector<int32_t> all(c->rows);
+    all.insert(all.end(), c->staged.begin(), c->staged.end());
+    const RunList rl = runs_of(all.data(), (int64_t)all.size());
     kvhip_cache tmp;
     tmp.kind = c->kind;
     tmp.has_geom = true;
@@ -309,19 +318,25 @@ kvhip_status ring_compact_if_needed(kvhip_cache *c, hipStream_t stream) {
     KV_TRY(ensure_slots(&tmp, c->cap_slots(), stream, true));
     for (size_t first = 0; first < rl.size(); first += MAXRUNS) {
         const size_t cnt = std::min((size_t)MAXRUNS, rl.size() - first);
-        KV_HIP(launch_compact_fp(c->st, pack_runs(rl, first, cnt), tmp.st, (int)c->rows.size(), stream));
+        KV_HIP(launch_compact_fp(c->st, pack_runs(rl, first, cnt), tmp.st, (int)all.size(), stream));
     }
     KV_HIP(hipStreamSynchronize(stream));
     free_store(c->st);
     c->st = tmp.st;
     tmp.st = Store();
     std::fill(c->used.begin(), c->used.end(), 0);
-    for (size_t i = 0; i < c->rows.size(); ++i) {
-        c->rows[i] = (int32_t)i;
-        c->used[i] = 1;
-    }
-    c->cursor = (int64_t)c->rows.size();
+    for (size_t i = 0; i < all.size(); ++i) c->used[i] = 1;
+    for (size_t i = 0; i < c->rows.size(); ++i) c->rows[i] = (int32_t)i;
+    for (size_t i = 0; i < c->staged.size(); ++i) c->staged[i] = (int32_t)(c->rows.size() + i);
+    c->cursor = (int64_t)all.size();
     return KVHIP_OK;
+}
+
+// If the ring's rows are scattered over more runs than a kernel takes, compact.
+kvhip_status ring_compact_if_needed(kvhip_cache *c, hipStream_t stream) {
+    const RunList rl = runs_of(c->rows.data(), (int64_t)c->rows.size());
+    if (rl.size() <= (size_t)MAXRUNS) return KVHIP_OK;
+    return compact_store(c, stream);
 }
 
 // ---- the three update paths ----------------------------------------------------
@@ -401,11 +416,51 @@ kvhip_status presented_runs(const kvhip_cache *c, Runs &runs, int &slots_span) {
         slots_span = (int)c->presented;
         return KVHIP_OK;
     }
-    const RunList rl = runs_of(c->rows.data(), std::min<int64_t>(c->presented, (int64_t)c->rows.size()));
+    const bool staged_view = c->staging && !c->stage_view.empty();
+    const std::vector<int32_t> &list = staged_view ? c->stage_view : c->rows;
+    const RunList rl = runs_of(list.data(), std::min<int64_t>(c->presented, (int64_t)list.size()));
     if (rl.size() > (size_t)MAXRUNS) return fail(KVHIP_ERR_INTERNAL, "ring presentation not compacted");
     runs = pack_runs(rl, 0, rl.size());
     slots_span = 0;
     for (size_t i = 0; i < rl.size(); ++i) slots_span = std::max(slots_span, rl.phys0[i] + rl.len[i]);
+    return KVHIP_OK;
+}
+
+// `logicalView(tail:)` (KVCache.swift:631-658) as a list of slots
+std::vector<int32_t> logical_rows(const kvhip_cache *c, int64_t tail) {
+    std::vector<int32_t> ordered = temporal_order(c);
+    const int64_t available = (int64_t)ordered.size();
+    const int64_t requested = std::min(std::max<int64_t>(tail, 0), available);
+    const int64_t bound = std::max(requested, std::min<int64_t>(c->keep, available));
+    const int64_t trim = available - bound;
+    if (trim > 0) {
+        const int64_t k = std::min<int64_t>(c->keep, available);
+        ordered.erase(ordered.begin() + k, ordered.begin() + k + trim);
+    }
+    return ordered;
+}
+
+// `presentation(stagedKeys:stagedValues:)` (RotatingStagedKVCache.swift:78-91)
+void stage_build_view(kvhip_cache *c) {
+    c->stage_view.clear();
+    const int64_t bound = std::min<int64_t>(c->offset, c->max_size - 1);
+    if (bound > 0 && c->has_buffers) c->stage_view = logical_rows(c, bound);
+    c->stage_view.insert(c->stage_view.end(), c->staged.begin(), c->staged.end());
+}
+
+// `RotatingStagedKVCache.update` (RotatingStagedKVCache.swift:41-47): the rows go to spare
+// slots, the ring stays as it is, and the presentation is the trailing window plus
+// everything staged so far -- read in place by the attention kernels, never concatenated.
+kvhip_status stage_update(kvhip_cache *c, const void *k, const void *v, int L, hipStream_t stream) {
+    const size_t base = c->staged.size();
+    KV_TRY(ring_alloc(c, L, c->staged, stream));
+    KV_TRY(write_rows(c, k, v, L, 0, c->staged.data() + base, L, stream));
+    stage_build_view(c);
+    if (runs_of(c->stage_view.data(), (int64_t)c->stage_view.size()).size() > (size_t)MAXRUNS) {
+        KV_TRY(compact_store(c, stream));
+        stage_build_view(c);
+    }
+    c->presented = (int64_t)c->stage_view.size();
     return KVHIP_OK;
 }
 
@@ -496,6 +551,8 @@ void kvhip_cache_free(kvhip_cache *c) {
     if (!c) return;
     free_store(c->st);
     if (c->ws) (void)hipFree(c->ws);
+    if (c->stage_tmp_k) (void)hipFree(c->stage_tmp_k);
+    if (c->stage_tmp_v) (void)hipFree(c->stage_tmp_v);
     delete c;
 }
 
@@ -567,6 +624,7 @@ kvhip_status kvhip_cache_update(kvhip_cache *c, const void *keys, const void *va
         }
     }
     KV_TRY(set_geometry(c, B, Hkv, Dk, Dv, dtype));
+    if (c->staging) return stage_update(c, keys, values, L, S(stream));
     if (c->kind == KVHIP_KIND_ROTATING) return update_rotating(c, keys, values, L, S(stream));
     return update_simple(c, keys, values, L, S(stream));
 }
@@ -575,6 +633,8 @@ kvhip_status kvhip_cache_fetch(const kvhip_cache *c, void *dk, void *dv, void *s
     if (!c) return fail(KVHIP_ERR_INVALID_ARG, "null cache");
     if (c->kind == KVHIP_KIND_QUANTIZED)
         return fail(KVHIP_ERR_STATE, "`update` was called on `QuantizedKVCache`. Use `updateQuantized` instead.");
+    if (c->staging && !c->stage_view.empty())
+        return export_slots(c, c->stage_view.data(), (int64_t)c->stage_view.size(), dk, dv, S(stream));
     if (!c->has_buffers) return fail(KVHIP_ERR_STATE, "cache is empty");
     if (c->kind == KVHIP_KIND_ROTATING)
         return export_slots(c, c->rows.data(), c->presented, dk, dv, S(stream));
@@ -586,7 +646,9 @@ kvhip_status kvhip_cache_fetch(const kvhip_cache *c, void *dk, void *dv, void *s
 kvhip_status kvhip_cache_attend(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, int32_t L,
                                 int32_t D, float scale, const kvhip_mask *mask, void *out, void *stream) {
     if (!c || !q || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
-    if (!c->has_geom || !c->has_buffers || c->presented <= 0) return fail(KVHIP_ERR_STATE, "attention over an empty cache");
+    const bool staged_view = c->staging && !c->stage_view.empty();
+    if (!c->has_geom || (!c->has_buffers && !staged_view) || c->presented <= 0)
+        return fail(KVHIP_ERR_STATE, "attention over an empty cache");
     if (B != c->B || D != c->st.Dk) return fail(KVHIP_ERR_INVALID_ARG, "query shape does not match the cache");
     if (Hq <= 0 || Hq % c->Hkv) return fail(KVHIP_ERR_INVALID_ARG, "query heads must be a multiple of KV heads");
     if (L <= 0 || L > 65535) return fail(KVHIP_ERR_INVALID_ARG, "query length out of range");
@@ -764,6 +826,8 @@ kvhip_status kvhip_cache_state_export(const kvhip_cache *c, int32_t i, void *dst
 kvhip_status kvhip_cache_state_import(kvhip_cache *c, int32_t count, const void *const *srcs,
                                       const int64_t *shapes, const int32_t *dtypes, void *stream) {
     if (!c || !srcs || !shapes || !dtypes) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (c->staging)  // RotatingStagedKVCache.swift:95-103
+        return fail(KVHIP_ERR_STATE, "RotatingStagedKVCache is round-scoped and cannot be restored from state");
     const bool q = c->kind == KVHIP_KIND_QUANTIZED;
     if (q ? (count != 6) : (count != 2)) {
         if (q && count == 4) return fail(KVHIP_ERR_UNSUPPORTED, "quantized state without biases (non-affine mode) is not supported");
@@ -848,6 +912,8 @@ static bool parse_int(const char *s, int64_t &out) {
 
 kvhip_status kvhip_cache_meta_set(kvhip_cache *c, int32_t count, const char *const *values) {
     if (!c || !values) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (c->staging)  // RotatingStagedKVCache.swift:105-111
+        return fail(KVHIP_ERR_STATE, "RotatingStagedKVCache is round-scoped and cannot be restored from metaState");
     if (c->kind == KVHIP_KIND_SIMPLE) {
         if (count != 1 || !values[0] || values[0][0])
             return fail(KVHIP_ERR_STATE, "This cache has no meta_state but a meta_state was set.");
@@ -892,6 +958,8 @@ kvhip_status kvhip_cache_meta_set(kvhip_cache *c, int32_t count, const char *con
 // ---- copy / views / conversions -------------------------------------------------
 kvhip_status kvhip_cache_copy(const kvhip_cache *c, void *stream, kvhip_cache **out) {
     if (!c || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (c->staging)  // RotatingStagedKVCache.swift:123-125
+        return fail(KVHIP_ERR_STATE, "RotatingStagedKVCache is round-scoped and cannot be copied");
     hipStream_t s = S(stream);
     kvhip_cache *n = new_cache_like(c);
     const int64_t rows = state_rows(c);
@@ -945,21 +1013,68 @@ kvhip_status kvhip_cache_copy(const kvhip_cache *c, void *stream, kvhip_cache **
     return KVHIP_OK;
 }
 
+// ---- staged rounds on a ring (RotatingStagedKVCache.swift, KVCacheRound.swift:128-156) ------
+kvhip_status kvhip_cache_stage_begin(kvhip_cache *c) {
+    if (!c) return fail(KVHIP_ERR_INVALID_ARG, "null cache");
+    if (c->kind != KVHIP_KIND_ROTATING)
+        return fail(KVHIP_ERR_INVALID_ARG, "only RotatingKVCache stages a round; append-only caches are written through and trimmed");
+    if (c->staging) return fail(KVHIP_ERR_STATE, "a staged round is already open on this cache");
+    c->staging = true;
+    c->staged.clear();
+    c->stage_view.clear();
+    c->presented_live = c->presented;
+    return KVHIP_OK;
+}
+
+int32_t kvhip_cache_stage_is_open(const kvhip_cache *c) { return c && c->staging; }
+
+int64_t kvhip_cache_stage_count(const kvhip_cache *c) { return c ? (int64_t)c->staged.size() : -1; }
+
+kvhip_status kvhip_cache_stage_fetch(const kvhip_cache *c, void *dk, void *dv, void *stream) {
+    if (!c) return fail(KVHIP_ERR_INVALID_ARG, "null cache");
+    if (!c->staging || c->staged.empty()) return fail(KVHIP_ERR_STATE, "nothing is staged");
+    return export_slots(c, c->staged.data(), (int64_t)c->staged.size(), dk, dv, S(stream));
+}
+
+kvhip_status kvhip_cache_stage_commit(kvhip_cache *c, int64_t retaining, void *stream) {
+    if (!c) return fail(KVHIP_ERR_INVALID_ARG, "null cache");
+    if (!c->staging) return fail(KVHIP_ERR_STATE, "no staged round is open on this cache");
+    hipStream_t s = S(stream);
+    // RotatingStagedKVCache.swift:62-76: the first `keep` staged rows go to the ring through
+    // the normal write path, the rest are dropped.  The kept rows are first gathered into a
+    // dense pair (a few rows), because the normal write path may reuse their slots.
+    const int64_t keep = std::min<int64_t>(std::max<int64_t>(retaining, 0), (int64_t)c->staged.size());
+    kvhip_status st = KVHIP_OK;
+    if (keep > 0) {
+        if ((size_t)keep > c->stage_tmp_rows) {
+            KV_HIP(hipStreamSynchronize(s));
+            if (c->stage_tmp_k) (void)hipFree(c->stage_tmp_k);
+            if (c->stage_tmp_v) (void)hipFree(c->stage_tmp_v);
+            c->stage_tmp_k = c->stage_tmp_v = nullptr;
+            c->stage_tmp_rows = 0;
+            const size_t rows = (size_t)std::max<int64_t>(keep, 16);
+            KV_HIP(hipMalloc(&c->stage_tmp_k, (size_t)c->st.BH * rows * c->st.Dk * c->st.es));
+            KV_HIP(hipMalloc(&c->stage_tmp_v, (size_t)c->st.BH * rows * c->st.Dv * c->st.es));
+            c->stage_tmp_rows = rows;
+        }
+        st = export_slots(c, c->staged.data(), keep, c->stage_tmp_k, c->stage_tmp_v, s);
+    }
+    for (int32_t slot : c->staged) c->used[(size_t)slot] = 0;
+    c->staged.clear();
+    c->stage_view.clear();
+    c->staging = false;
+    c->presented = c->presented_live;
+    if (st != KVHIP_OK) return st;
+    if (keep > 0) return update_rotating(c, c->stage_tmp_k, c->stage_tmp_v, (int)keep, s);
+    return KVHIP_OK;
+}
+
 kvhip_status kvhip_cache_logical_view(const kvhip_cache *c, int64_t tail, int64_t *out_rows, void *dk,
                                       void *dv, void *stream) {
     if (!c || !out_rows) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
     if (c->kind != KVHIP_KIND_ROTATING) return fail(KVHIP_ERR_INVALID_ARG, "logicalView belongs to RotatingKVCache");
     if (!c->has_buffers) return fail(KVHIP_ERR_STATE, "logicalView before the first write");
-    // KVCache.swift:631-658
-    std::vector<int32_t> ordered = temporal_order(c);
-    const int64_t available = (int64_t)ordered.size();
-    const int64_t requested = std::min(std::max<int64_t>(tail, 0), available);
-    const int64_t bound = std::max(requested, std::min<int64_t>(c->keep, available));
-    const int64_t trim = available - bound;
-    if (trim > 0) {
-        const int64_t k = std::min<int64_t>(c->keep, available);
-        ordered.erase(ordered.begin() + k, ordered.begin() + k + trim);
-    }
+    const std::vector<int32_t> ordered = logical_rows(c, tail);
     *out_rows = (int64_t)ordered.size();
     if ((dk || dv) && !ordered.empty())
         return export_slots(c, ordered.data(), (int64_t)ordered.size(), dk, dv, S(stream));

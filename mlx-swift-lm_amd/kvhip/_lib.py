@@ -80,6 +80,11 @@ SIGNATURES = {
     "kvhip_cache_meta_count": (_I32, [_P]),
     "kvhip_cache_meta_get": (_I32, [_P, _I32, C.c_char_p, _I32]),
     "kvhip_cache_meta_set": (_I32, [_P, _I32, C.POINTER(C.c_char_p)]),
+    "kvhip_cache_stage_begin": (_I32, [_P]),
+    "kvhip_cache_stage_is_open": (_I32, [_P]),
+    "kvhip_cache_stage_count": (_I64, [_P]),
+    "kvhip_cache_stage_fetch": (_I32, [_P, _P, _P, _P]),
+    "kvhip_cache_stage_commit": (_I32, [_P, _I64, _P]),
     "kvhip_cache_logical_view": (_I32, [_P, _I64, C.POINTER(_I64), _P, _P, _P]),
     "kvhip_cache_to_quantized": (_I32, [_P, _I32, _I32, _P, C.POINTER(_P)]),
     "kvhip_cache_to_unquantized": (_I32, [_P, _P, C.POINTER(_P)]),

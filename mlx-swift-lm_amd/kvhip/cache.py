@@ -290,7 +290,7 @@ class RotatingKVCache(KVCacheSimple):
 
     def logical_view(self, tail):
         """`logicalView(tail:)` (KVCache.swift:631-658); None before the first write."""
-        if self._shape is None:
+        if self._shape is None or self._lib.kvhip_cache_state_count(self._h) == 0:
             return None
         n = C.c_int64()
         L.check(self._lib.kvhip_cache_logical_view(self._h, int(tail), C.byref(n), None, None, _stream()))
