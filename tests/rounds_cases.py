@@ -352,7 +352,45 @@ def case_rewind_refused_after_replacement(be):
     assert_unchanged(be, replacement, snap, "after a rewind against a replaced entry")
 
 
+def case_long_random_schedule(be):
+    """A long seeded schedule (rounds of random width and acceptance, single-token writes in
+    between, a pinned prefix) against an accepted-only replay: exercises slot reuse and, on
+    the device, compaction of a fragmented page store."""
+    rng = np.random.default_rng(7)
+    window, keep = 48, 3
+    live, ref = be.rotating(window, keep), be.rotating(window, keep)
+    fill(be, live, 0, 11, one_by_one=False)
+    fill(be, ref, 0, 11, one_by_one=False)
+    nxt = 11
+    st = be.storage([live])
+    for i in range(160):
+        if rng.integers(0, 3) == 0:
+            k, v = be.kv(nxt, nxt + 1)
+            be.update(live, k, v)
+            be.update(ref, k, v)
+            be.commit_tokens(st, 1)
+            nxt += 1
+            continue
+        written = int(rng.integers(1, 9))
+        accepted = int(rng.integers(0, written + 1))
+        rnd = be.begin(st, written)
+        pk, pv = stage(be, rnd, nxt, nxt + written)[0]
+        got = be.positions(pk)
+        assert got[-written:] == list(range(nxt, nxt + written)), f"step {i}"
+        assert [-p for p in be.positions(pv)] == got, f"step {i}"
+        be.commit(st, rnd, accepted)
+        if accepted:
+            be.update(ref, *be.kv(nxt, nxt + accepted))
+        nxt += accepted
+        assert live.offset == ref.offset == nxt, f"step {i}"
+        assert be.meta(live) == be.meta(ref), f"step {i}"
+        lv, rv = be.view(live, window), be.view(ref, window)
+        assert be.positions(lv[0]) == be.positions(rv[0]), f"step {i}"
+        assert [-p for p in be.positions(lv[1])] == be.positions(rv[0]), f"step {i}"
+
+
 SIMPLE_CASES = [
+    case_long_random_schedule,
     case_ring_untouched_before_commit,
     case_write_through_restored_by_rollback,
     case_presentation_equals_live_write_path,
