@@ -1,4 +1,7 @@
-// Chunked-prefill attention tile on the matrix cores (gfx950, v_mfma_f32_16x16x32_f16).
+// Chunked-prefill attention tile on the matrix cores (gfx950, v_mfma_f32_16x16x32_f16) for
+// quantized caches; full-precision caches take the double-buffered kernel of
+// kvhip_attend_prefill_fp.hip (the BITS == 0 paths below are what that kernel grew out of and
+// are no longer instantiated).
 //
 // Many query rows per kv head (r = Hq/Hkv heads times L new tokens).  One workgroup
 // (4 wavefronts) owns 128 query rows of one (batch, kv-head) pair -- 32 per wavefront
@@ -29,6 +32,8 @@ union Op8 {
 };
 
 constexpr int BN = 32;    // key slots per tile
+
+
 constexpr float LOG2E = 1.4426950408889634f;
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -51,6 +56,7 @@ prefill_kernel(AttendArgs a, int nsplit) {
     __shared__ __attribute__((aligned(16))) _Float16 Ks[BN * KS];
     __shared__ __attribute__((aligned(16))) _Float16 Vs[D * VS];
     __shared__ int rows_s[BN];
+    __shared__ int tile_full_s;
     __shared__ float sb_s[Q ? BN * 2 * (D / 32) : 1];  // V (scale, bias) per token and group
 
     const Store &st = a.st;
@@ -118,6 +124,26 @@ prefill_kernel(AttendArgs a, int nsplit) {
             if (a.mask.window > 0) tile_lo = max(0, (a.mask.offset + l_min - a.mask.window + 1) / BN);
         }
         tile_hi = min(tile_hi, (a.T + BN - 1) / BN);
+    }
+
+    // presented rows [keep_lo, keep_hi] are seen by every query row of this workgroup: a key
+    // tile made only of such rows needs no per-element test (flag set while staging)
+    int keep_lo = 0, keep_hi = -1;
+    if (MM != 2) {
+        keep_hi = a.T - 1;
+        if (MM == 1) {
+            const int i_first = blockIdx.x * BM, i_last = min(R, i_first + BM) - 1;
+            const bool spans = (i_first / a.L) != (i_last / a.L);
+            const int l_min = spans ? 0 : i_first % a.L, l_max = spans ? a.L - 1 : i_last % a.L;
+            if (sym.mode == KVHIP_MASK_CAUSAL) {
+                keep_hi = a.T - a.L + l_min;
+            } else {
+                keep_lo = sym.pad_b;
+                keep_hi = min(sym.offset + l_min, sym.len_b - 1);
+                if (sym.window > 0) keep_lo = max(keep_lo, sym.offset + l_max - sym.window + 1);
+            }
+            keep_hi = min(keep_hi, a.T - 1);
+        }
     }
 
     // ---- optional split of the key range over blockIdx.z (small grids): each part leaves an
@@ -209,6 +235,10 @@ prefill_kernel(AttendArgs a, int nsplit) {
     };
     auto stage_k = [&]() {  // K, row indices and (quantized) the V scale/bias table
         if (tid < BN) rows_s[tid] = row_reg;
+        if (wave == 0) {
+            const bool full = __all(lane >= BN || (row_reg >= keep_lo && row_reg <= keep_hi));
+            if (lane == 0) tile_full_s = full;
+        }
         if constexpr (!Q) {
             _Float16 *dst = Ks + kt * KS + kpart * (D / 8);
 #pragma unroll
@@ -306,8 +336,11 @@ prefill_kernel(AttendArgs a, int nsplit) {
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
             for (int i = 0; i < 4; ++i) trow[mt][i] = rows_s[16 * mt + 4 * jj + i];
+        const bool tile_full = tile_full_s != 0;
 
         // ---- online softmax per query column; P^T stays in place as the PV B operand ------
+        // Tiles every query row of the workgroup sees completely (all slots live rows, inside
+        // the mask for every row) skip the per-element tests.
         Op8 pb[QT];
 #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
@@ -318,45 +351,52 @@ prefill_kernel(AttendArgs a, int nsplit) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     float s_ = Q ? round_dt<DT>(sacc[qt][mt][i]) : sacc[qt][mt][i] * a.scale;
-                    const int row = trow[mt][i];
-                    if (row >= 0 && q_ok[qt]) {
-                        if constexpr (MM == 1) {
-                            if (!sym_mask_keep(sym, q_l[qt], row)) s_ = Q ? fill : -INFINITY;
-                        } else if constexpr (MM == 2) {
-                            float add;
-                            const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
-                            if (Q) {
-                                if (!keep) s_ = fill;
-                                else if (a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
-                            } else {
-                                s_ = keep ? s_ + add : -INFINITY;
+                    if (MM == 2 || !tile_full) {  // workgroup-uniform
+                        const int row = trow[mt][i];
+                        if (row >= 0 && q_ok[qt]) {
+                            if constexpr (MM == 1) {
+                                if (!sym_mask_keep(sym, q_l[qt], row)) s_ = Q ? fill : -INFINITY;
+                            } else if constexpr (MM == 2) {
+                                float add;
+                                const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
+                                if (Q) {
+                                    if (!keep) s_ = fill;
+                                    else if (a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
+                                } else {
+                                    s_ = keep ? s_ + add : -INFINITY;
+                                }
                             }
+                        } else {
+                            s_ = -INFINITY;
                         }
-                    } else {
-                        s_ = -INFINITY;
                     }
                     sc[mt][i] = s_;
                     tmax = fmaxf(tmax, s_);
                 }
             tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-            const float mn = fmaxf(m_run[qt], tmax);
-            const float alpha = (mn == -INFINITY) ? 1.f : exp2_fast((m_run[qt] - mn) * LOG2E);
-            m_run[qt] = mn;
+            // rescale the accumulators only when some row's maximum rose (rare after the first tiles)
+            if (__any(tmax > m_run[qt])) {
+                const float mn = fmaxf(m_run[qt], tmax);
+                const float alpha = (mn == -INFINITY) ? 1.f : exp2_fast((m_run[qt] - mn) * LOG2E);
+                m_run[qt] = mn;
+                l_run[qt] *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) oacc[qt][dt][i] *= alpha;
+            }
+            const float mu = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt];
             float psum = 0.f;
             float p[2][4];
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    p[mt][i] = (sc[mt][i] == -INFINITY) ? 0.f : exp2_fast((sc[mt][i] - mn) * LOG2E);
+                    p[mt][i] = exp2_fast((sc[mt][i] - mu) * LOG2E);  // exp2(-inf) = 0 for excluded keys
                     psum += p[mt][i];
                 }
-            l_run[qt] = l_run[qt] * alpha + psum;
-#pragma unroll
-            for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) oacc[qt][dt][i] *= alpha;
+            l_run[qt] += psum;
             pb[qt].u[0] = h2_bits(p[0][0], p[0][1]);
             pb[qt].u[1] = h2_bits(p[0][2], p[0][3]);
             pb[qt].u[2] = h2_bits(p[1][0], p[1][1]);
@@ -421,11 +461,18 @@ bool attend_prefill_supported(const AttendArgs &a) {
     return (a.Hq / a.Hkv) * a.L > 16;
 }
 
+// 128 query rows per workgroup reuse each staged tile twice as often as 64; 64 rows are
+// used when that would leave the grid too small to fill 256 CUs twice over.
+static bool prefill_wide(const AttendArgs &a) {
+    const int R = (a.Hq / a.Hkv) * a.L;
+    return (size_t)((R + 127) / 128) * a.st.BH >= 512 && a.st.Dk <= 128;
+}
+
 // Key-range parts per query block: only when the grid would leave most CUs without a
 // second workgroup, and only while the partials stay small.
 static int prefill_splits(const AttendArgs &a) {
     const int R = (a.Hq / a.Hkv) * a.L;
-    const bool wide = (size_t)((R + 127) / 128) * a.st.BH >= 512 && a.st.Dk <= 128;
+    const bool wide = prefill_wide(a);
     const size_t wgs = (size_t)((R + (wide ? 127 : 63)) / (wide ? 128 : 64)) * a.st.BH;
     int n = (int)(768 / (wgs ? wgs : 1));
     const int tiles = (a.slots + BN - 1) / BN;
@@ -447,7 +494,7 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
     const int R = (a.Hq / a.Hkv) * a.L;
     // 128 query rows per workgroup reuse each staged tile twice as often; 64 rows are used
     // when that would leave the grid too small to fill 256 CUs twice over
-    const bool wide = (size_t)((R + 127) / 128) * st.BH >= 512 && st.Dk <= 128;
+    const bool wide = prefill_wide(a);
     const int bm = wide ? 128 : 64;
     const int nsplit = prefill_splits(a);
     dim3 grid((R + bm - 1) / bm, st.BH, nsplit), block(256);
@@ -483,10 +530,13 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
     } while (0)
     if (st.bits == 4) PF_D(4);
     else if (st.bits == 8) PF_D(8);
-    else if (st.Dk == 64) PF_DT(0, 64);
-    else if (st.Dk == 128) PF_DT(0, 128);
-    else if (st.dtype == KVHIP_F16) PF(0, 256, 0, 1);
-    else PF(0, 256, 1, 1);
+    else {
+        // full-precision caches have their own double-buffered kernel
+        profile_mark(s, true);
+        hipError_t e = launch_attend_prefill_fp(a, nsplit, wide, s);
+        profile_mark(s, false);
+        if (e != hipSuccess) return e;
+    }
 #undef PF_D
 #undef PF_DT
 #undef PF_QT

@@ -1,0 +1,376 @@
+// Chunked-prefill attention for full-precision caches (fp16 / bf16) on the matrix cores
+// (gfx950, v_mfma_f32_16x16x32_f16 / _bf16).
+//
+// One workgroup (4 wavefronts) owns 64 (QT = 1) or 128 (QT = 2) query rows of one
+// (batch, kv-head) pair and walks the cached keys in tiles of 32 slots:
+//   S^T   = K . Q^T      A = K rows from LDS in the cache's own dtype (no conversion),
+//                        B = query rows held in registers
+//   out^T += V^T . P^T   A = V^T rows from LDS as fp16 (bf16 is converted while staging),
+//                        B = the fp16 probabilities exactly where the S^T accumulators left
+//                        them, so P never moves between lanes
+// K/V tiles are double-buffered in LDS: while a tile is contracted, the next one (already in
+// registers) is written to the other buffer and the one after that is requested from global
+// memory, with a single barrier per tile.  Global reads and LDS writes of a tile are
+// chunk-interleaved over the 256 threads (consecutive lanes, consecutive 16 bytes), LDS rows
+// are padded so that both the writes and the operand reads are bank-conflict free.
+// The online softmax rescales the accumulators only when a row maximum rises, and key tiles
+// that every query row of the workgroup sees completely skip all mask tests.
+#include "kvhip_mask.hpp"
+
+namespace kvhip {
+
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef __bf16 b8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+union Op8 {
+    h8 h;
+    b8 b;
+    u4 v;
+};
+
+constexpr int BN = 32;  // key slots per tile
+constexpr float LOG2E = 1.4426950408889634f;
+
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ uint32_t rn_h2(float lo, float hi) {  // round to nearest even
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
+}
+// two bf16 (one dword) -> two fp16, exact for every bf16 inside the fp16 range
+__device__ __forceinline__ uint32_t bf2_to_h2(uint32_t w) {
+    return rn_h2(__uint_as_float(w << 16), __uint_as_float(w & 0xffff0000u));
+}
+
+template <int DT> __device__ __forceinline__ f4 mfma_qk(const Op8 &a, const Op8 &b, f4 c) {
+    if constexpr (DT == 0) return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, c, 0, 0, 0);
+}
+
+// D = 256 runs 64 query rows per workgroup only: 128 rows need the accumulator registers of
+// a whole SIMD lane (one wavefront per SIMD), which measured slower (0.34 ms against 0.29 ms
+// for a 512 x 4607 chunk at B4, 8 query heads).
+template <int D, int DT, bool IDENT, int QT, int MM>
+__global__ void __launch_bounds__(256, 2)
+prefill_fp_kernel(AttendArgs a, int nsplit) {
+    constexpr int BM = 64 * QT;
+    constexpr int KS = D + 8;     // 16-bit elements per K row in LDS
+    constexpr int VS = BN + 8;    // halves per V^T row in LDS (80 bytes: 16-byte aligned rows)
+    constexpr int S = D / 32;     // contraction steps over the head dim
+    constexpr int NDT = D / 16;   // 16-row tiles of out^T
+    constexpr int NC = D / 64;    // 16-byte chunks per thread, for K and for V
+    __shared__ __attribute__((aligned(16))) uint16_t Ks[2][BN * KS];
+    __shared__ __attribute__((aligned(16))) _Float16 Vs[2][D * VS];
+    __shared__ int rows_s[2][BN];
+    __shared__ int full_s[2];
+
+    const Store &st = a.st;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int n = lane & 15, jj = lane >> 4;
+    const int bh = blockIdx.y;
+    const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
+    const int r = a.Hq / a.Hkv;
+    const int R = r * a.L;
+    const int row0 = blockIdx.x * BM + wave * 16 * QT;  // first query row of this wavefront
+    const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
+
+    // ---- query operands: B of S^T = K . Q^T; lane (n, jj) holds q[row][32 s + 8 jj ..] raw ----
+    Op8 qop[QT][S];
+    int q_l[QT], q_h[QT];
+    bool q_ok[QT];
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        const int i = row0 + 16 * qt + n;
+        q_ok[qt] = i < R;
+        const int rep = q_ok[qt] ? i / a.L : 0;
+        q_l[qt] = q_ok[qt] ? i - rep * a.L : 0;
+        q_h[qt] = hk * r + rep;
+        const u4 *qp = reinterpret_cast<const u4 *>(
+            reinterpret_cast<const uint16_t *>(a.q) + ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D + 8 * jj);
+#pragma unroll
+        for (int s = 0; s < S; ++s) qop[qt][s].v = q_ok[qt] ? qp[4 * s] : u4{0, 0, 0, 0};
+    }
+
+    f4 oacc[QT][NDT];
+    float m_run[QT], l_run[QT];
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        m_run[qt] = -INFINITY;
+        l_run[qt] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) oacc[qt][dt] = f4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // ---- key tiles this workgroup has to visit, and the rows all of its queries keep ---------
+    int tile_lo = 0, tile_hi = (a.slots + BN - 1) / BN;
+    int keep_lo = 0, keep_hi = -1;
+    {
+        const int i_first = blockIdx.x * BM, i_last = min(R, i_first + BM) - 1;
+        const bool spans = (i_first / a.L) != (i_last / a.L);
+        const int l_min = spans ? 0 : i_first % a.L, l_max = spans ? a.L - 1 : i_last % a.L;
+        if (MM != 2) {
+            keep_hi = a.T - 1;
+            if (MM == 1) {
+                if (sym.mode == KVHIP_MASK_CAUSAL) {
+                    keep_hi = a.T - a.L + l_min;
+                } else {
+                    keep_lo = sym.pad_b;
+                    keep_hi = min(sym.offset + l_min, sym.len_b - 1);
+                    if (sym.window > 0) keep_lo = max(keep_lo, sym.offset + l_max - sym.window + 1);
+                }
+                keep_hi = min(keep_hi, a.T - 1);
+            }
+        }
+        if (IDENT) {  // slots are presented rows: tiles outside a symbolic mask are skipped
+            if (a.mask.mode == KVHIP_MASK_CAUSAL) {
+                tile_hi = min(tile_hi, (a.T - a.L + l_max) / BN + 1);
+            } else if (a.mask.mode == KVHIP_MASK_WINDOW) {
+                tile_hi = min(tile_hi, (a.mask.offset + l_max) / BN + 1);
+                if (a.mask.window > 0) tile_lo = max(0, (a.mask.offset + l_min - a.mask.window + 1) / BN);
+            }
+            tile_hi = min(tile_hi, (a.T + BN - 1) / BN);
+        }
+    }
+    // optional split of the key range over blockIdx.z (small grids): each part leaves an
+    // unnormalised partial per query row, merged by the decode path's combine kernel
+    const int split = blockIdx.z;
+    if (nsplit > 1) {
+        const int span = (tile_hi - tile_lo + nsplit - 1) / nsplit;
+        tile_lo = tile_lo + split * span;
+        tile_hi = min(tile_hi, tile_lo + span);
+    }
+
+    // ---- staging ------------------------------------------------------------------------
+    // chunk c = e * 256 + tid.  K: row c / (D/8), 16-byte column c % (D/8).  V: head-dim row
+    // c / 4, 16-byte quarter c % 4 of the 32 tokens of this tile.
+    u4 kreg[NC], vreg[NC];
+    int row_reg = -1;
+    auto fetch = [&](int tile) __attribute__((always_inline)) {
+        const int slot0 = tile * BN;
+        if (tid < BN) {
+            const int slot = slot0 + tid;
+            int row;
+            if (IDENT) row = slot;
+            else row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
+            row_reg = (row >= 0 && row < a.T) ? row : -1;
+        }
+        const char *kbase = k_row_ptr(st, bh, slot0);
+        const char *vbase = v_cell_ptr(st, bh, slot0) + v_row_off(st, slot0, 0) + ((slot0 & 32) ? 64 : 0);
+#pragma unroll
+        for (int e = 0; e < NC; ++e) {
+            const int c = e * 256 + tid;
+            kreg[e] = *reinterpret_cast<const u4 *>(kbase + (size_t)(c / (D / 8)) * st.k_row + (c % (D / 8)) * 16);
+            vreg[e] = *reinterpret_cast<const u4 *>(vbase + (size_t)(c >> 2) * (TILE * 2) + (c & 3) * 16);
+        }
+    };
+    auto stage = [&](int buf) __attribute__((always_inline)) {
+        if (tid < BN) rows_s[buf][tid] = row_reg;
+        if (wave == 0) {
+            const bool full = __all(lane >= BN || (row_reg >= keep_lo && row_reg <= keep_hi));
+            if (lane == 0) full_s[buf] = full;
+        }
+#pragma unroll
+        for (int e = 0; e < NC; ++e) {
+            const int c = e * 256 + tid;
+            *reinterpret_cast<u4 *>(&Ks[buf][(c / (D / 8)) * KS + (c % (D / 8)) * 8]) = kreg[e];
+            u4 v = vreg[e];
+            if (DT == 1) v = u4{bf2_to_h2(v.x), bf2_to_h2(v.y), bf2_to_h2(v.z), bf2_to_h2(v.w)};
+            *reinterpret_cast<u4 *>(&Vs[buf][(c >> 2) * VS + (c & 3) * 8]) = v;
+        }
+    };
+
+    if (tile_lo < tile_hi) {
+        fetch(tile_lo);
+        stage(0);
+        if (tile_lo + 1 < tile_hi) fetch(tile_lo + 1);
+    }
+    __syncthreads();
+    for (int tile = tile_lo; tile < tile_hi; ++tile) {
+        const int cur = (tile - tile_lo) & 1;
+        // the tile fetched during the previous iteration goes to the other buffer (last read
+        // one barrier ago); the tile after it is requested now and has this whole iteration
+        if (tile + 1 < tile_hi) stage(cur ^ 1);
+        if (tile + 2 < tile_hi) fetch(tile + 2);
+
+        // ---- S^T = K . Q^T: acc[qt][mt] rows = tokens 16 mt + 4 jj + i, column = query n -----
+        f4 sacc[QT][2];
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt) sacc[qt][mt] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+            Op8 ka[S];
+#pragma unroll
+            for (int s = 0; s < S; ++s)
+                ka[s].v = *reinterpret_cast<const u4 *>(&Ks[cur][(16 * mt + n) * KS + 32 * s + 8 * jj]);
+#pragma unroll
+            for (int s = 0; s < S; ++s)
+#pragma unroll
+                for (int qt = 0; qt < QT; ++qt) sacc[qt][mt] = mfma_qk<DT>(ka[s], qop[qt][s], sacc[qt][mt]);
+        }
+        const bool tile_full = full_s[cur] != 0;
+        int trow[2][4];
+        if (MM == 2 || !tile_full) {
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) trow[mt][i] = rows_s[cur][16 * mt + 4 * jj + i];
+        }
+
+        // ---- online softmax per query column; P^T stays in place as the PV B operand ------
+        Op8 pb[QT];
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+            float sc[2][4];
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float s_ = sacc[qt][mt][i] * a.scale;
+                    if (MM == 2 || !tile_full) {  // workgroup-uniform
+                        const int row = trow[mt][i];
+                        if (row >= 0 && q_ok[qt]) {
+                            if constexpr (MM == 1) {
+                                if (!sym_mask_keep(sym, q_l[qt], row)) s_ = -INFINITY;
+                            } else if constexpr (MM == 2) {
+                                float add;
+                                const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
+                                s_ = keep ? s_ + add : -INFINITY;
+                            }
+                        } else {
+                            s_ = -INFINITY;
+                        }
+                    }
+                    sc[mt][i] = s_;
+                    tmax = fmaxf(tmax, s_);
+                }
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+            if (__any(tmax > m_run[qt])) {  // rare after the first tiles
+                const float mn = fmaxf(m_run[qt], tmax);
+                const float alpha = (mn == -INFINITY) ? 1.f : exp2_fast((m_run[qt] - mn) * LOG2E);
+                m_run[qt] = mn;
+                l_run[qt] *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) oacc[qt][dt][i] *= alpha;
+            }
+            const float mu = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt];
+            float psum = 0.f;
+            float p[2][4];
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    p[mt][i] = exp2_fast((sc[mt][i] - mu) * LOG2E);  // exp2(-inf) = 0 for excluded keys
+                    psum += p[mt][i];
+                }
+            l_run[qt] += psum;
+            pb[qt].v = u4{rn_h2(p[0][0], p[0][1]), rn_h2(p[0][2], p[0][3]), rn_h2(p[1][0], p[1][1]), rn_h2(p[1][2], p[1][3])};
+        }
+
+        // ---- out^T += V^T . P^T: A = V^T rows (tokens 4jj..4jj+3 and 16+4jj..) from LDS -------
+#pragma unroll
+        for (int d0 = 0; d0 < NDT; d0 += 4) {
+            Op8 va[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const _Float16 *vrow = &Vs[cur][(16 * (d0 + x) + n) * VS];
+                const u2 lo = *reinterpret_cast<const u2 *>(vrow + 4 * jj);
+                const u2 hi = *reinterpret_cast<const u2 *>(vrow + 16 + 4 * jj);
+                va[x].v = u4{lo.x, lo.y, hi.x, hi.y};
+            }
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+#pragma unroll
+                for (int qt = 0; qt < QT; ++qt)
+                    oacc[qt][d0 + x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[x].h, pb[qt].h, oacc[qt][d0 + x], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // ---- normalise and store: lane (n, jj) holds out[q = n][d = 16 dt + 4 jj + i] ------------
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+        float l = l_run[qt];
+        l += __shfl_xor(l, 16);
+        l += __shfl_xor(l, 32);
+        if (!q_ok[qt]) continue;
+        if (nsplit > 1) {
+            const int i = row0 + 16 * qt + n;
+            float *part = a.workspace + (((size_t)bh * nsplit + split) * R + i) * (D + 2);
+#pragma unroll
+            for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<f4 *>(part + 16 * dt + 4 * jj) = oacc[qt][dt];
+            if (jj == 0) {
+                part[D] = m_run[qt];
+                part[D + 1] = l;
+            }
+            continue;
+        }
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        const size_t ooff = ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+            const float o0 = oacc[qt][dt][0] * inv, o1 = oacc[qt][dt][1] * inv;
+            const float o2 = oacc[qt][dt][2] * inv, o3 = oacc[qt][dt][3] * inv;
+            uint2 w;
+            if (DT == 0) {
+                w.x = rn_h2(o0, o1);
+                w.y = rn_h2(o2, o3);
+            } else {
+                w.x = (uint32_t)Elem<1>::bits(o0) | ((uint32_t)Elem<1>::bits(o1) << 16);
+                w.y = (uint32_t)Elem<1>::bits(o2) | ((uint32_t)Elem<1>::bits(o3) << 16);
+            }
+            *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(a.out) + ooff + 16 * dt + 4 * jj) = w;
+        }
+    }
+}
+
+}  // namespace
+
+hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, hipStream_t s) {
+    const Store &st = a.st;
+    const int R = (a.Hq / a.Hkv) * a.L;
+    const int bm = wide ? 128 : 64;
+    dim3 grid((R + bm - 1) / bm, st.BH, nsplit), block(256);
+    const bool ident = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
+    const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
+#define PF_M(D, DT, QT, MM)                                                                                   \
+    do {                                                                                                      \
+        if (ident) hipLaunchKernelGGL((prefill_fp_kernel<D, DT, true, QT, MM>), grid, block, 0, s, a, nsplit);  \
+        else hipLaunchKernelGGL((prefill_fp_kernel<D, DT, false, QT, MM>), grid, block, 0, s, a, nsplit);       \
+    } while (0)
+#define PF(D, DT, QT)                        \
+    do {                                     \
+        if (mm == 0) PF_M(D, DT, QT, 0);     \
+        else if (mm == 1) PF_M(D, DT, QT, 1); \
+        else PF_M(D, DT, QT, 2);             \
+    } while (0)
+#define PF_QT(D, DT)                 \
+    do {                             \
+        if (wide) PF(D, DT, 2);      \
+        else PF(D, DT, 1);           \
+    } while (0)
+#define PF_DT(D)                                  \
+    do {                                          \
+        if (st.dtype == KVHIP_F16) PF_QT(D, 0);   \
+        else PF_QT(D, 1);                         \
+    } while (0)
+    if (st.Dk == 64) PF_DT(64);
+    else if (st.Dk == 128) PF_DT(128);
+    else if (st.dtype == KVHIP_F16) PF(256, 0, 1);
+    else PF(256, 1, 1);
+#undef PF_DT
+#undef PF_QT
+#undef PF
+#undef PF_M
+    return hipGetLastError();
+}
+
+}  // namespace kvhip
