@@ -57,7 +57,8 @@ __global__ void __launch_bounds__(256, 2)
 prefill_fp_kernel(AttendArgs a, int nsplit) {
     constexpr int BM = 64 * QT;
     constexpr int KS = D + 8;     // 16-bit elements per K row in LDS
-    constexpr int VS = BN + 8;    // halves per V^T row in LDS (80 bytes: 16-byte aligned rows)
+    constexpr int VS = BN + 4;    // halves per V^T row in LDS: 18 dwords, so the 16 rows an operand
+                                  // read touches fall in distinct banks
     constexpr int S = D / 32;     // contraction steps over the head dim
     constexpr int NDT = D / 16;   // 16-row tiles of out^T
     constexpr int NC = D / 64;    // 16-byte chunks per thread, for K and for V
@@ -178,7 +179,9 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             *reinterpret_cast<u4 *>(&Ks[buf][(c / (D / 8)) * KS + (c % (D / 8)) * 8]) = kreg[e];
             u4 v = vreg[e];
             if (DT == 1) v = u4{bf2_to_h2(v.x), bf2_to_h2(v.y), bf2_to_h2(v.z), bf2_to_h2(v.w)};
-            *reinterpret_cast<u4 *>(&Vs[buf][(c >> 2) * VS + (c & 3) * 8]) = v;
+            u2 *vd = reinterpret_cast<u2 *>(&Vs[buf][(c >> 2) * VS + (c & 3) * 8]);  // rows are 8-byte aligned
+            vd[0] = u2{v.x, v.y};
+            vd[1] = u2{v.z, v.w};
         }
     };
 
