@@ -223,8 +223,11 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     // the bias term; built from the same registers: the 16 steps of one operand pair lie in
     // one group (group sizes are multiples of 64), so a lane sums its 4 elements, the 16
     // lane groups are added up by shuffles and the four rows are read out of their quad.
+    // (Built by a lambda that the main loop calls after it has requested its first tile, so the
+    // first K/V loads are in flight while the queries are fetched and reduced.)
     Op qa[RG][NQA];
     float qsum[RG][G][4];
+    auto load_queries = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) {
         const int i = 4 * rg + qi;
@@ -258,6 +261,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 qsum[rg][g][ii] = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), ii));
         }
     }
+    };
 
     // ---- running state ---------------------------------------------------------------
     // m_use = m_run, or 0 while m_run is still -inf, so exp2((s - m_use) log2 e) needs no guard
@@ -522,6 +526,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         if constexpr (PREFETCH) {
             T bufA, bufB;
             load_tile(bufA);
+            load_queries();
             for (int done = 0;;) {
                 load_tile(bufB);
                 compute_tile(bufA);
@@ -533,6 +538,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         } else {
             T buf;
             load_k(buf);
+            load_queries();
             for (int done = 0; done < my_tiles; ++done) {
                 load_v(buf);
                 compute_qk_softmax(buf);
