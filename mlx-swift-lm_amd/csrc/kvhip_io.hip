@@ -91,24 +91,39 @@ append_quant_kernel(Store st, const char *keys, const char *values, int L, int s
     const int hi = min(slot0 + n, tile * TILE + TILE);
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    for (int slot = lo + wave; slot < hi; slot += 4) {
-        const int l = src0 + (slot - slot0);
-        const char *krow = keys + ((size_t)bh * L + l) * st.Dk * st.es;
-        const char *vrow = values + ((size_t)bh * L + l) * st.Dv * st.es;
-        quantize_row_wave<DT, BITS>(krow, st.Dk, st.gs, lane,
-                                    reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot))),
-                                    nullptr, const_cast<char *>(ksb_row_ptr(st, bh, slot)), nullptr, nullptr);
-        quantize_row_wave<DT, BITS>(vrow, st.Dv, st.gs, lane, nullptr, vcodes + (slot & (TILE - 1)) * st.Dv,
-                                    const_cast<char *>(vsb_row_ptr(st, bh, slot)), nullptr, nullptr);
-    }
-    __syncthreads();
-    char *cell = const_cast<char *>(v_cell_ptr(st, bh, lo));
     constexpr int TPW = 32 / BITS;          // tokens per word
     constexpr int WPR = TILE / TPW;         // words per tile row
     const int t_lo = lo & (TILE - 1), t_hi = t_lo + (hi - lo);
-    for (int u = threadIdx.x; u < st.Dv * WPR; u += blockDim.x) {
-        const int d = u / WPR, w = u - d * WPR;
-        if ((w + 1) * TPW <= t_lo || w * TPW >= t_hi) continue;
+    // the words of a V tile row this append touches, and this thread's first merge item:
+    // its old word is requested now, so a single-token append does not wait for it later
+    const int w_lo = t_lo / TPW, nw = (t_hi - 1) / TPW - w_lo + 1;
+    const int items = st.Dv * nw;
+    char *cell = const_cast<char *>(v_cell_ptr(st, bh, lo));
+    auto word_ptr = [&](int u) -> uint32_t * {
+        const int d = u / nw, w = w_lo + (u - d * nw);
+        return reinterpret_cast<uint32_t *>(cell + v_row_off(st, lo, d)) + w;
+    };
+    const bool partial = (t_lo % TPW) != 0 || (t_hi % TPW) != 0;  // some word keeps old tokens
+    uint32_t old0 = 0;
+    if (partial && (int)threadIdx.x < items) old0 = *word_ptr(threadIdx.x);
+    // (row, K or V) pairs go round the four wavefronts, so one new token uses two of them
+    for (int item = wave; item < 2 * (hi - lo); item += 4) {
+        const int slot = lo + (item >> 1);
+        const int l = src0 + (slot - slot0);
+        if ((item & 1) == 0) {
+            const char *krow = keys + ((size_t)bh * L + l) * st.Dk * st.es;
+            quantize_row_wave<DT, BITS>(krow, st.Dk, st.gs, lane,
+                                        reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot))),
+                                        nullptr, const_cast<char *>(ksb_row_ptr(st, bh, slot)), nullptr, nullptr);
+        } else {
+            const char *vrow = values + ((size_t)bh * L + l) * st.Dv * st.es;
+            quantize_row_wave<DT, BITS>(vrow, st.Dv, st.gs, lane, nullptr, vcodes + (slot & (TILE - 1)) * st.Dv,
+                                        const_cast<char *>(vsb_row_ptr(st, bh, slot)), nullptr, nullptr);
+        }
+    }
+    __syncthreads();
+    for (int u = threadIdx.x; u < items; u += blockDim.x) {
+        const int d = u / nw, w = w_lo + (u - d * nw);
         uint32_t nbits = 0, mbits = 0;
         for (int tt = 0; tt < TPW; ++tt) {
             const int t = w * TPW + tt;
@@ -118,8 +133,13 @@ append_quant_kernel(Store st, const char *keys, const char *values, int L, int s
                 mbits |= ((1u << BITS) - 1u) << bp;
             }
         }
-        uint32_t *p = reinterpret_cast<uint32_t *>(cell + v_row_off(st, lo, d)) + w;
-        *p = (mbits == 0xffffffffu) ? nbits : ((*p & ~mbits) | nbits);
+        uint32_t *p = word_ptr(u);
+        if (mbits == 0xffffffffu) {
+            *p = nbits;
+        } else {
+            const uint32_t old = (u == (int)threadIdx.x) ? old0 : *p;
+            *p = (old & ~mbits) | nbits;
+        }
     }
 }
 
