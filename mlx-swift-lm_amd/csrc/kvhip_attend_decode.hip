@@ -198,8 +198,11 @@ template <int BITS, int D, int G> struct TileRegs {
 // bounds preloaded: no memory access in the loop), 2 array masks (loads in the loop, which
 // force conservative waits on the prefetch).  Slots map to presented rows one to one: only
 // RotatingKVCache remaps slots, and it is never quantized.
-template <int BITS, int D, int GS, int DT, int RG, int MM>
-__global__ void __launch_bounds__(WAVES * 64, 2)
+// NW = wavefronts per workgroup: 4 (two workgroups per CU), or 8 when that lets one
+// workgroup take the whole sequence of its (batch, kv-head) pair -- then the output rows are
+// normalised and written here and no partial goes through memory.
+template <int BITS, int D, int GS, int DT, int RG, int MM, int NW>
+__global__ void __launch_bounds__(NW * 64, NW == 4 ? 2 : 1)
 decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     using GEO = Geo<BITS>;
     constexpr int G = D / GS;      // quantization groups per row (1 or 2)
@@ -216,7 +219,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     const int r = a.Hq / a.Hkv;
     const int R = r * a.L;
 
-    __shared__ float cbuf[WAVES][RR][D + 2];
+    __shared__ float cbuf[NW][RR][D + 2];
 
     // ---- query operands: lane (blk, qi) holds row qi's 4 elements of step 16 x + blk ----
     // qsum[rg][g][i] = sum over group g of the (rounded, fp16-held) query row 4 rg + i, for
@@ -292,7 +295,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         const int t_lo = max(0, vis_lo) >> 6, t_hi = min(tiles_total, (min(vis_hi, a.T - 1) >> 6) + 1);
         // tiles_per_wg == 0: divide this batch row's own visible range over the spans
         const int per = tiles_per_wg > 0 ? tiles_per_wg
-                                         : (max(t_hi - t_lo, 1) + nsplit * WAVES - 1) / (nsplit * WAVES) * WAVES;
+                                         : (max(t_hi - t_lo, 1) + nsplit * NW - 1) / (nsplit * NW) * NW;
         tile_begin = t_lo + split * per;  // spans past t_hi are empty
         tile_end = min(t_hi, tile_begin + per);
     }
@@ -306,12 +309,14 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 
     constexpr int VROW = T::VW * 4;  // bytes of one V tile row
 
-    // This wavefront takes tiles tile0, tile0 + 4, ...: always the same tile of
-    // successive pages, so its four plane pointers advance by one page cell stride.
+    // This wavefront takes tiles tile0, tile0 + NW, ...: always the same tile of
+    // successive pages (4 tiles each), so its four plane pointers advance by NW / 4 page
+    // cell strides.
     const int tile0 = tile_begin + wave;
-    const int my_tiles = tile0 < tile_end ? (tile_end - tile0 + WAVES - 1) / WAVES : 0;
-    const size_t k_step = (size_t)st.BH * st.k_cell, v_step = (size_t)st.BH * st.v_cell;
-    const size_t ksb_step = (size_t)st.BH * st.ksb_cell, vsb_step = (size_t)st.BH * st.vsb_cell;
+    const int my_tiles = tile0 < tile_end ? (tile_end - tile0 + NW - 1) / NW : 0;
+    constexpr int PSTEP = NW / 4;  // pages per step
+    const size_t k_step = (size_t)st.BH * st.k_cell * PSTEP, v_step = (size_t)st.BH * st.v_cell * PSTEP;
+    const size_t ksb_step = (size_t)st.BH * st.ksb_cell * PSTEP, vsb_step = (size_t)st.BH * st.vsb_cell * PSTEP;
     const int page0 = tile0 >> 2, tip = tile0 & 3;  // 4 tiles per page
     const char *kp = st.k + ((size_t)page0 * st.BH + bh) * st.k_cell + (size_t)tip * TILE * st.k_row;
     const char *vp = st.v + ((size_t)page0 * st.BH + bh) * st.v_cell + (size_t)tip * D * VROW;
@@ -352,8 +357,8 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         if (k_loaded < my_tiles) {  // wave-uniform: step to the same tile of the next page
             kp += k_step;
             ksp += ksb_step;
-            slot_next += PAGE;
-            base_next += PAGE;
+            slot_next += PAGE * PSTEP;
+            base_next += PAGE * PSTEP;
         }
     };
     auto load_v = [&](T &t) {
@@ -571,20 +576,39 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         }
     }
     __syncthreads();
-    // ---- merge the 4 wavefronts, write the span's partial ------------------------------
+    // ---- merge the wavefronts; a single span writes the output rows, several leave partials
+    if (nsplit == 1) {
+        for (int idx = threadIdx.x; idx < R * D; idx += NW * 64) {
+            const int i = idx / D, c = idx - i * D;
+            float mx = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) mx = fmaxf(mx, cbuf[w][i][D]);
+            float v = 0.f, l = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                const float mw = cbuf[w][i][D];
+                const float wgt = (mw == -INFINITY) ? 0.f : fast_exp2((mw - mx) * LOG2E);
+                v += wgt * cbuf[w][i][c];
+                l += wgt * cbuf[w][i][D + 1];
+            }
+            const int rep = i / a.L, lq = i - rep * a.L;
+            Elem<DT>::store(a.out, ((size_t)(b * a.Hq + hk * r + rep) * a.L + lq) * D + c, l > 0.f ? v / l : 0.f);
+        }
+        return;
+    }
     float *part = a.workspace + ((size_t)bh * nsplit + split) * RR * (D + 2);
-    for (int idx = threadIdx.x; idx < RR * (D + 2); idx += WAVES * 64) {
+    for (int idx = threadIdx.x; idx < RR * (D + 2); idx += NW * 64) {
         const int i = idx / (D + 2), c = idx - i * (D + 2);
         float mx = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, cbuf[w][i][D]);
+        for (int w = 0; w < NW; ++w) mx = fmaxf(mx, cbuf[w][i][D]);
         float v;
         if (c == D) {
             v = mx;
         } else {
             v = 0.f;
 #pragma unroll
-            for (int w = 0; w < WAVES; ++w) {
+            for (int w = 0; w < NW; ++w) {
                 const float mw = cbuf[w][i][D];
                 const float wgt = (mw == -INFINITY) ? 0.f : fast_exp2((mw - mx) * LOG2E);
                 v += wgt * cbuf[w][i][c];
@@ -884,7 +908,7 @@ combine_kernel(AttendArgs a, int nsplit, int rr) {
 }
 
 struct Plan {
-    int tiles_total, tiles_per_wg, nsplit, rg;
+    int tiles_total, tiles_per_wg, nsplit, rg, nw;
 };
 
 Plan plan_for(const AttendArgs &a) {
@@ -908,8 +932,17 @@ Plan plan_for(const AttendArgs &a) {
     // row's visible range divided among them in the kernel (all workgroups stay resident
     // and none is empty; measured faster than equal-sized spans with more of them for the
     // long rows)
-    if (a.mask.mode == KVHIP_MASK_WINDOW && (a.mask.left_pad || a.mask.lengths) && !getenv("KVHIP_DECODE_TILES"))
+    p.nw = WAVES;
+    if (a.mask.mode == KVHIP_MASK_WINDOW && (a.mask.left_pad || a.mask.lengths) && !getenv("KVHIP_DECODE_TILES")) {
         p.tiles_per_wg = 0;
+    } else if (a.st.bits != 0 && p.nsplit == 2 && p.rg <= 2 && a.mask.mode != KVHIP_MASK_ARRAY &&
+               !getenv("KVHIP_DECODE_TILES")) {
+        // two spans of 4 wavefronts per pair become one workgroup of 8: same wavefronts per CU,
+        // but the merge stays on chip and the kernel writes the output itself
+        p.nw = 2 * WAVES;
+        p.nsplit = 1;
+        p.tiles_per_wg = (p.tiles_total + p.nw - 1) / p.nw * p.nw;
+    }
     return p;
 }
 
@@ -983,7 +1016,7 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
     AttendArgs a = a_in;
     const Plan p = plan_for(a);
     const Store &st = a.st;
-    dim3 grid(p.nsplit, st.BH), block(WAVES * 64);
+    dim3 grid(p.nsplit, st.BH), block(WAVES * 64);  // the quantized kernel sets its own block size
     const int R = (a.Hq / a.Hkv) * a.L;
     if (st.bits != 0 && p.rg == 4 && a.mask.mode == KVHIP_MASK_NONE) {
         // the 16-row unmasked variants need more registers than the index-mask ones (which
@@ -995,20 +1028,27 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
         a.mask.left_pad = nullptr;
     }
     const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
+#define DEC_K(BITS, D, GS, DT, RG, MM, NW)                                                                \
+    hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG, MM, NW>), grid, dim3(NW * 64), 0, s, a,        \
+                       p.tiles_total, p.tiles_per_wg, p.nsplit)
 #define DEC(BITS, D, GS, DT, RG)                                                                          \
     do {                                                                                                  \
         profile_mark(s, true);                                                                            \
-        if (mm == 0)                                                                                      \
-            hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG, 0>), grid, block, 0, s, a,             \
-                               p.tiles_total, p.tiles_per_wg, p.nsplit);                                  \
-        else if (mm == 1)                                                                                 \
-            hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG, 1>), grid, block, 0, s, a,             \
-                               p.tiles_total, p.tiles_per_wg, p.nsplit);                                  \
-        else                                                                                              \
-            hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG, 2>), grid, block, 0, s, a,             \
-                               p.tiles_total, p.tiles_per_wg, p.nsplit);                                  \
+        if (p.nw == 2 * WAVES) {                                                                          \
+            if constexpr (RG <= 2) {                                                                      \
+                if (mm == 0) DEC_K(BITS, D, GS, DT, RG, 0, 2 * WAVES);                                    \
+                else DEC_K(BITS, D, GS, DT, RG, 1, 2 * WAVES);                                            \
+            }                                                                                             \
+        } else if (mm == 0) {                                                                             \
+            DEC_K(BITS, D, GS, DT, RG, 0, WAVES);                                                         \
+        } else if (mm == 1) {                                                                             \
+            DEC_K(BITS, D, GS, DT, RG, 1, WAVES);                                                         \
+        } else {                                                                                          \
+            DEC_K(BITS, D, GS, DT, RG, 2, WAVES);                                                         \
+        }                                                                                                 \
         profile_mark(s, false);                                                                           \
-        hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG);  \
+        if (p.nsplit > 1)                                                                                 \
+            hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG); \
     } while (0)
 #define DEC_RG(BITS, D, GS, DT)                       \
     do {                                              \
@@ -1069,6 +1109,7 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
 #undef DEC_DT
 #undef DEC_RG
 #undef DEC
+#undef DEC_K
     return hipGetLastError();
 }
 

@@ -92,7 +92,6 @@ append_quant_kernel(Store st, const char *keys, const char *values, int L, int s
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     constexpr int TPW = 32 / BITS;          // tokens per word
-    constexpr int WPR = TILE / TPW;         // words per tile row
     const int t_lo = lo & (TILE - 1), t_hi = t_lo + (hi - lo);
     // the words of a V tile row this append touches, and this thread's first merge item:
     // its old word is requested now, so a single-token append does not wait for it later
