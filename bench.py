@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes moved per launch of the decode kernel divided by its algorithmic bytes, from two
 # rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a
 # plain 1 GiB copy; summary in profiles/decode_kernel_q4_d128_cfg3.md
-MEASURED_TRAFFIC_RATIO = 1.0033
+MEASURED_TRAFFIC_RATIO = 1.0024
 ROW_BYTES = 144  # per cached token and kv head: K and V codes 2*64 B + 2*2 groups*(scale+bias)*2 B
 
 
@@ -48,7 +48,7 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=2, help="decode steps timed on the CPU baseline (0 = skip)")
     ap.add_argument("--workload", default="cfg3", choices=["cfg3", "cfg2", "cfg4", "cfg5"],
                     help="cfg3 (default) is the configuration the metric is quoted on; the others are the "
-                         "remaining BASELINE.json configs, measured for DESIGN.md")
+                         "remaining BASELINE.json configs (reported as one JSON object each)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy 4 times (reference point for rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -57,7 +57,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus above 1 is not supported "
-              "(the path shards over batch / KV heads without exchange, see DESIGN.md)", file=sys.stderr)
+              "(the path shards over batch and KV heads without any exchange between devices)", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np
