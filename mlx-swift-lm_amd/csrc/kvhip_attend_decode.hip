@@ -886,6 +886,8 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 template <int D, int DT>
 __global__ void __launch_bounds__(D)
 combine_kernel(AttendArgs a, int nsplit, int rr) {
+    __shared__ float w_s[512];  // weight of each span for this row (nsplit <= 512)
+    __shared__ float red_s[4];
     const int i = blockIdx.x, bh = blockIdx.y;
     const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
     const int r = a.Hq / a.Hkv;
@@ -893,16 +895,42 @@ combine_kernel(AttendArgs a, int nsplit, int rr) {
     const size_t sstride = (size_t)rr * (D + 2);
     const float *part = a.workspace + (size_t)bh * nsplit * sstride + (size_t)i * (D + 2);
     const int d = threadIdx.x;
-    float mx = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, part[s * sstride + D]);
-    float num = 0.f, den = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-        const float *p = part + s * sstride;
-        const float mw = p[D];
-        const float w = (mw == -INFINITY) ? 0.f : fast_exp2((mw - mx) * LOG2E);
-        num += w * p[d];
-        den += w * p[D + 1];
+    // every span's (max, sum) in one parallel round of loads, reduced through LDS
+    float mloc = -INFINITY;
+    for (int s = d; s < nsplit; s += D) {
+        const float m = part[s * sstride + D];
+        w_s[s] = m;
+        mloc = fmaxf(mloc, m);
     }
+    mloc = wave_max(mloc);
+    if ((d & 63) == 0) red_s[d >> 6] = mloc;
+    __syncthreads();
+    float mx = red_s[0];
+#pragma unroll
+    for (int w = 1; w < D / 64; ++w) mx = fmaxf(mx, red_s[w]);
+    __syncthreads();
+    float dloc = 0.f;
+    for (int s = d; s < nsplit; s += D) {
+        const float m = w_s[s];
+        const float w = (m == -INFINITY) ? 0.f : fast_exp2((m - mx) * LOG2E);
+        w_s[s] = w;
+        dloc += w * part[s * sstride + D + 1];
+    }
+    dloc = wave_sum(dloc);
+    if ((d & 63) == 0) red_s[d >> 6] = dloc;
+    __syncthreads();
+    float den = red_s[0];
+#pragma unroll
+    for (int w = 1; w < D / 64; ++w) den += red_s[w];
+    // the column sums: independent loads, issued several at a time
+    float num = 0.f;
+    int s = 0;
+    for (; s + 4 <= nsplit; s += 4) {
+        const float p0 = part[(s + 0) * sstride + d], p1 = part[(s + 1) * sstride + d];
+        const float p2 = part[(s + 2) * sstride + d], p3 = part[(s + 3) * sstride + d];
+        num += w_s[s] * p0 + w_s[s + 1] * p1 + w_s[s + 2] * p2 + w_s[s + 3] * p3;
+    }
+    for (; s < nsplit; ++s) num += w_s[s] * part[s * sstride + d];
     const float o = den > 0.f ? num / den : 0.f;
     Elem<DT>::store(a.out, ((size_t)(b * a.Hq + hk * r + rep) * a.L + l) * D + d, o);
 }
@@ -926,6 +954,7 @@ Plan plan_for(const AttendArgs &a) {
     if (const char *e = getenv("KVHIP_DECODE_TILES")) per = atoi(e);
     per = per < WAVES ? WAVES : per;
     per = (per + WAVES - 1) / WAVES * WAVES;
+    while ((p.tiles_total + per - 1) / per > 512) per *= 2;  // the merge kernel holds 512 span weights
     p.tiles_per_wg = per;
     p.nsplit = (p.tiles_total + per - 1) / per;
     // ragged batches (per-batch bounds): the same number of spans for every batch row, each
