@@ -357,6 +357,30 @@ def trim_prompt_cache(caches, num_tokens):
     return caches[0].trim(num_tokens)
 
 
+def resolve_affine_scheme(scheme):
+    """`resolveAffineScheme` (KVCache.swift:2455-2461): (bits, group size) or None."""
+    return {"affine4": (4, 64), "affine8": (8, 64)}.get(scheme)
+
+
+def maybe_affine_quantize_kv_cache(caches, bits, group_size, compression_start):
+    """`maybeAffineQuantizeKVCache` (KVCache.swift:2500-2520): every `KVCacheSimple` whose offset
+    has passed `compression_start` is replaced, in place in the list, by its quantized form (one
+    bulk quantize kernel on the device); a cache whose head dims fit no supported group size
+    stays as it is.  Returns False while some cache is still waiting for the threshold."""
+    awaits = False
+    for i, c in enumerate(caches):
+        if type(c) is not KVCacheSimple:
+            continue
+        if not c.offset > compression_start:
+            awaits = True
+            continue
+        try:
+            caches[i] = c.to_quantized(group_size, bits)
+        except L.KVHipError:
+            pass
+    return not awaits
+
+
 def affine_quantize(w, group_size=64, bits=4):
     """`MLX.quantized(w, groupSize:, bits:)` on the device: (wq int32-as-u32, scales, biases)."""
     L.init()

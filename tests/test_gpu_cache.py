@@ -147,6 +147,35 @@ def test_simple_cache_update_fetch_state(dtype):
     assert all(torch.equal(a, b) for a, b in zip(fresh.state, st))
 
 
+def test_dynamic_conversion_at_compression_start():
+    """`maybeAffineQuantizeKVCache` (KVCache.swift:2500-2520): simple caches past the threshold
+    become quantized caches holding the same rows (bit-exact with the oracle's bulk quantize);
+    rings, already quantized caches and heads no group size divides stay as they are."""
+    rng = np.random.default_rng(4)
+    dtype = torch.float16
+    k, kd = randn(rng, (1, 2, 40, 64), dtype)
+    v, vd = randn(rng, (1, 2, 40, 64), dtype)
+    long_, short, ring, odd = kvhip.KVCacheSimple(), kvhip.KVCacheSimple(), kvhip.RotatingKVCache(64), kvhip.KVCacheSimple()
+    long_.update(kd, vd, fetch=False)
+    short.update(kd[:, :, :8].contiguous(), vd[:, :, :8].contiguous(), fetch=False)
+    ring.update(kd, vd, fetch=False)
+    _, k5 = randn(rng, (1, 1, 40, 5), dtype)
+    odd.update(k5, k5, fetch=False)
+    already = kvhip.QuantizedKVCache(64, 8)
+    caches = [long_, short, ring, odd, already]
+    assert kvhip.resolve_affine_scheme("affine4") == (4, 64) and kvhip.resolve_affine_scheme("turbo4") is None
+    done = kvhip.maybe_affine_quantize_kv_cache(caches, 4, 64, 16)
+    assert done is False                      # `short` still waits for the threshold
+    assert isinstance(caches[0], kvhip.QuantizedKVCache) and caches[0].offset == 40
+    assert caches[1] is short and caches[2] is ring and caches[3] is odd and caches[4] is already
+    o = O.KVCacheSimple("float16")
+    o.update(k, v)
+    check_quantized_state(caches[0], o.to_quantized(64, 4), dtype)
+    short.update(kd[:, :, 8:20].contiguous(), vd[:, :, 8:20].contiguous(), fetch=False)
+    assert kvhip.maybe_affine_quantize_kv_cache(caches, 4, 64, 16) is True
+    assert isinstance(caches[1], kvhip.QuantizedKVCache) and caches[1].offset == 20
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 def test_simple_to_quantized_and_back(dtype):
     rng = np.random.default_rng(9)
