@@ -647,24 +647,24 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     __shared__ float cbuf[WAVES][RR][D + 2];
 
     // query operands: lane (blk, qi) holds row qi's elements 4*(16 x + blk) .. +3, unscaled
+    // (fetched by the main loop after it has requested its first two pieces)
     Op qa[RG][NP];
+    auto load_queries = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int rg = 0; rg < RG; ++rg) {
-        const int i = 4 * rg + qi;
-        const int rep = i / a.L, l = i - rep * a.L;
-        const size_t qoff = ((size_t)(b * a.Hq + hk * r + rep) * a.L + l) * D;
+        for (int rg = 0; rg < RG; ++rg) {
+            const int i = 4 * rg + qi;
+            const int rep = i / a.L, l = i - rep * a.L;
+            const size_t qoff = ((size_t)(b * a.Hq + hk * r + rep) * a.L + l) * D;
 #pragma unroll
-        for (int x = 0; x < NP; ++x) {
-            uint32_t w0 = 0, w1 = 0;
-            if (i < R) {
-                const uint16_t *qp = reinterpret_cast<const uint16_t *>(a.q) + qoff + 4 * (16 * x + blk);
-                w0 = (uint32_t)qp[0] | ((uint32_t)qp[1] << 16);
-                w1 = (uint32_t)qp[2] | ((uint32_t)qp[3] << 16);
+            for (int x = 0; x < NP; ++x) {
+                uint2 w = make_uint2(0, 0);
+                if (i < R)
+                    w = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(a.q) + qoff + 4 * (16 * x + blk));
+                qa[rg][x].u[0] = w.x;
+                qa[rg][x].u[1] = w.y;
             }
-            qa[rg][x].u[0] = w0;
-            qa[rg][x].u[1] = w1;
         }
-    }
+    };
 
     float m_run[RG][4], l_part[RG][4];
     f4 oacc[RG][NP];
@@ -731,6 +731,7 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     if (my_tiles > 0) {
         load_k(buf_of(0), 0);
         if (NP > 1) load_k(buf_of(1), 1); else load_v(buf_of(1), 0);
+        load_queries();
         for (int done = 0; done < my_tiles; ++done) {
             int row;
             if (IDENT) row = slot_cur;
@@ -948,7 +949,9 @@ Plan plan_for(const AttendArgs &a) {
     // Spans are sized so that all workgroups are resident at once (2 per CU): every
     // wavefront streams for the whole kernel and no second scheduling round leaves CUs
     // idle.  A span is a multiple of WAVES tiles so each wavefront gets the same share.
-    int want = (256 * 2) / BH;
+    // (the full-precision kernel, whose tiles are 4x larger, measured faster with one
+    // workgroup per CU: 46 us against 52 us at 8192 tokens, B8, 8 kv heads, D 128)
+    int want = (a.st.bits != 0 ? 256 * 2 : 256) / BH;
     if (want < 1) want = 1;
     int per = (p.tiles_total + want - 1) / want;
     if (const char *e = getenv("KVHIP_DECODE_TILES")) per = atoi(e);
