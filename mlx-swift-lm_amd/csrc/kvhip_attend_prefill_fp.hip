@@ -77,6 +77,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     const int R = r * a.L;
     const int row0 = blockIdx.x * BM + wave * 16 * QT;  // first query row of this wavefront
     const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
+    const float sl2 = a.scale * LOG2E;
 
     // ---- query operands: B of S^T = K . Q^T; lane (n, jj) holds q[row][32 s + 8 jj ..] raw ----
     Op8 qop[QT][S];
@@ -225,38 +226,41 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         }
 
         // ---- online softmax per query column; P^T stays in place as the PV B operand ------
+        // Scores stay in the log2 domain: x = s * (scale * log2 e), p = exp2(x - m).  The running
+        // maximum m of a query is the same in the four lanes that share it; a tile raises it only
+        // if some lane's own maximum exceeds it, so the common tile needs no cross-lane traffic.
         Op8 pb[QT];
 #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
-            float sc[2][4];
+            float x[2][4];
             float tmax = -INFINITY;
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float s_ = sacc[qt][mt][i] * a.scale;
+                    float x_ = sacc[qt][mt][i] * sl2;
                     if (MM == 2 || !tile_full) {  // workgroup-uniform
                         const int row = trow[mt][i];
                         if (row >= 0 && q_ok[qt]) {
                             if constexpr (MM == 1) {
-                                if (!sym_mask_keep(sym, q_l[qt], row)) s_ = -INFINITY;
+                                if (!sym_mask_keep(sym, q_l[qt], row)) x_ = -INFINITY;
                             } else if constexpr (MM == 2) {
                                 float add;
                                 const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
-                                s_ = keep ? s_ + add : -INFINITY;
+                                x_ = keep ? x_ + add * LOG2E : -INFINITY;
                             }
                         } else {
-                            s_ = -INFINITY;
+                            x_ = -INFINITY;
                         }
                     }
-                    sc[mt][i] = s_;
-                    tmax = fmaxf(tmax, s_);
+                    x[mt][i] = x_;
+                    tmax = fmaxf(tmax, x_);
                 }
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
             if (__any(tmax > m_run[qt])) {  // rare after the first tiles
+                tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+                tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
                 const float mn = fmaxf(m_run[qt], tmax);
-                const float alpha = (mn == -INFINITY) ? 1.f : exp2_fast((m_run[qt] - mn) * LOG2E);
+                const float alpha = (mn == -INFINITY) ? 1.f : exp2_fast(m_run[qt] - mn);
                 m_run[qt] = mn;
                 l_run[qt] *= alpha;
 #pragma unroll
@@ -271,7 +275,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    p[mt][i] = exp2_fast((sc[mt][i] - mu) * LOG2E);  // exp2(-inf) = 0 for excluded keys
+                    p[mt][i] = exp2_fast(x[mt][i] - mu);  // exp2(-inf) = 0 for excluded keys
                     psum += p[mt][i];
                 }
             l_run[qt] += psum;
@@ -311,7 +315,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<f4 *>(part + 16 * dt + 4 * jj) = oacc[qt][dt];
             if (jj == 0) {
-                part[D] = m_run[qt];
+                part[D] = m_run[qt] * 0.6931471805599453f;  // back from the log2 domain
                 part[D + 1] = l;
             }
             continue;
