@@ -44,6 +44,8 @@ __device__ __forceinline__ uint32_t bf2_to_h2(uint32_t w) {
     return rn_h2(__uint_as_float(w << 16), __uint_as_float(w & 0xffff0000u));
 }
 
+__device__ __forceinline__ int st_BH(const AttendArgs &a) { return a.st.BH; }
+
 template <int DT> __device__ __forceinline__ f4 mfma_qk(const Op8 &a, const Op8 &b, f4 c) {
     if constexpr (DT == 0) return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, c, 0, 0, 0);
     else return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, c, 0, 0, 0);
@@ -71,11 +73,32 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, jj = lane >> 4;
-    const int bh = blockIdx.y;
-    const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
+    // Workgroups go to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  All
+    // query blocks of one (batch, kv-head) pair re-read that pair's K and V, so they are given
+    // ids of the same residue: a pair's tiles then stay hot in one L2 instead of missing in all.
     const int r = a.Hq / a.Hkv;
     const int R = r * a.L;
-    const int row0 = blockIdx.x * BM + wave * 16 * QT;  // first query row of this wavefront
+    const int nblk = (R + BM - 1) / BM;
+    int blk_x, bh, split;
+    {
+        const int id = blockIdx.x;
+        const int BH = st_BH(a);
+        if ((BH & 7) == 0) {
+            const int xcd = id & 7, j = id >> 3;
+            const int per_pair = nblk * nsplit;
+            const int h_local = j / per_pair, rem = j - h_local * per_pair;
+            bh = h_local * 8 + xcd;
+            split = rem / nblk;
+            blk_x = rem - split * nblk;
+        } else {
+            blk_x = id % nblk;
+            const int t = id / nblk;
+            bh = t % BH;
+            split = t / BH;
+        }
+    }
+    const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
+    const int row0 = blk_x * BM + wave * 16 * QT;  // first query row of this wavefront
     const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
     const float sl2 = a.scale * LOG2E;
 
@@ -110,7 +133,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     int tile_lo = 0, tile_hi = (a.slots + BN - 1) / BN;
     int keep_lo = 0, keep_hi = -1;
     {
-        const int i_first = blockIdx.x * BM, i_last = min(R, i_first + BM) - 1;
+        const int i_first = blk_x * BM, i_last = min(R, i_first + BM) - 1;
         const bool spans = (i_first / a.L) != (i_last / a.L);
         const int l_min = spans ? 0 : i_first % a.L, l_max = spans ? a.L - 1 : i_last % a.L;
         if (MM != 2) {
@@ -136,9 +159,8 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             tile_hi = min(tile_hi, (a.T + BN - 1) / BN);
         }
     }
-    // optional split of the key range over blockIdx.z (small grids): each part leaves an
+    // optional split of the key range (small grids): each part leaves an
     // unnormalised partial per query row, merged by the decode path's combine kernel
-    const int split = blockIdx.z;
     if (nsplit > 1) {
         const int span = (tile_hi - tile_lo + nsplit - 1) / nsplit;
         tile_lo = tile_lo + split * span;
@@ -345,7 +367,7 @@ hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, 
     const Store &st = a.st;
     const int R = (a.Hq / a.Hkv) * a.L;
     const int bm = wide ? 128 : 64;
-    dim3 grid((R + bm - 1) / bm, st.BH, nsplit), block(256);
+    dim3 grid((unsigned)((R + bm - 1) / bm) * st.BH * nsplit), block(256);  // linear: the kernel maps ids to tiles
     const bool ident = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
     const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
 #define PF_M(D, DT, QT, MM)                                                                                   \
