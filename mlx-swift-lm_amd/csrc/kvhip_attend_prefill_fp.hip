@@ -170,37 +170,46 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     // ---- staging ------------------------------------------------------------------------
     // chunk c = e * 256 + tid.  K: row c / (D/8), 16-byte column c % (D/8).  V: head-dim row
     // c / 4, 16-byte quarter c % 4 of the 32 tokens of this tile.
-    u4 kreg[NC], vreg[NC];
-    int row_reg = -1;
-    auto fetch = [&](int tile) __attribute__((always_inline)) {
+    // Up to D = 128 two register sets alternate, so a tile is requested two iterations before
+    // it is written to LDS and three before it is contracted; D = 256 has registers for one set
+    // (one iteration less of lead).
+    constexpr bool DEEP = D <= 128;
+    constexpr int LEAD = DEEP ? 3 : 2;
+    struct Stg {
+        u4 k[NC], v[NC];
+        int row;
+    };
+    Stg setA, setB;
+    setA.row = setB.row = -1;
+    auto fetch = [&](int tile, Stg &g) __attribute__((always_inline)) {
         const int slot0 = tile * BN;
         if (tid < BN) {
             const int slot = slot0 + tid;
             int row;
             if (IDENT) row = slot;
             else row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
-            row_reg = (row >= 0 && row < a.T) ? row : -1;
+            g.row = (row >= 0 && row < a.T) ? row : -1;
         }
         const char *kbase = k_row_ptr(st, bh, slot0);
         const char *vbase = v_cell_ptr(st, bh, slot0) + v_row_off(st, slot0, 0) + ((slot0 & 32) ? 64 : 0);
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
             const int c = e * 256 + tid;
-            kreg[e] = *reinterpret_cast<const u4 *>(kbase + (size_t)(c / (D / 8)) * st.k_row + (c % (D / 8)) * 16);
-            vreg[e] = *reinterpret_cast<const u4 *>(vbase + (size_t)(c >> 2) * (TILE * 2) + (c & 3) * 16);
+            g.k[e] = *reinterpret_cast<const u4 *>(kbase + (size_t)(c / (D / 8)) * st.k_row + (c % (D / 8)) * 16);
+            g.v[e] = *reinterpret_cast<const u4 *>(vbase + (size_t)(c >> 2) * (TILE * 2) + (c & 3) * 16);
         }
     };
-    auto stage = [&](int buf) __attribute__((always_inline)) {
-        if (tid < BN) rows_s[buf][tid] = row_reg;
+    auto stage = [&](int buf, const Stg &g) __attribute__((always_inline)) {
+        if (tid < BN) rows_s[buf][tid] = g.row;
         if (wave == 0) {
-            const bool full = __all(lane >= BN || (row_reg >= keep_lo && row_reg <= keep_hi));
+            const bool full = __all(lane >= BN || (g.row >= keep_lo && g.row <= keep_hi));
             if (lane == 0) full_s[buf] = full;
         }
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
             const int c = e * 256 + tid;
-            *reinterpret_cast<u4 *>(&Ks[buf][(c / (D / 8)) * KS + (c % (D / 8)) * 8]) = kreg[e];
-            u4 v = vreg[e];
+            *reinterpret_cast<u4 *>(&Ks[buf][(c / (D / 8)) * KS + (c % (D / 8)) * 8]) = g.k[e];
+            u4 v = g.v[e];
             if (DT == 1) v = u4{bf2_to_h2(v.x), bf2_to_h2(v.y), bf2_to_h2(v.z), bf2_to_h2(v.w)};
             u2 *vd = reinterpret_cast<u2 *>(&Vs[buf][(c >> 2) * VS + (c & 3) * 8]);  // rows are 8-byte aligned
             vd[0] = u2{v.x, v.y};
@@ -209,17 +218,18 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     };
 
     if (tile_lo < tile_hi) {
-        fetch(tile_lo);
-        stage(0);
-        if (tile_lo + 1 < tile_hi) fetch(tile_lo + 1);
+        fetch(tile_lo, setA);
+        stage(0, setA);
+        if (tile_lo + 1 < tile_hi) fetch(tile_lo + 1, setA);
+        if (DEEP && tile_lo + 2 < tile_hi) fetch(tile_lo + 2, setB);
     }
     __syncthreads();
-    for (int tile = tile_lo; tile < tile_hi; ++tile) {
-        const int cur = (tile - tile_lo) & 1;
-        // the tile fetched during the previous iteration goes to the other buffer (last read
-        // one barrier ago); the tile after it is requested now and has this whole iteration
-        if (tile + 1 < tile_hi) stage(cur ^ 1);
-        if (tile + 2 < tile_hi) fetch(tile + 2);
+    // one tile: `cur` is the LDS buffer that holds it, `g` the register set that holds the next one
+    auto step = [&](int tile, int cur, Stg &g) __attribute__((always_inline)) {
+        // the tile fetched two iterations ago goes to the other buffer (last read one barrier
+        // ago); its registers are then free for the tile three ahead
+        if (tile + 1 < tile_hi) stage(cur ^ 1, g);
+        if (tile + LEAD < tile_hi) fetch(tile + LEAD, g);
 
         // ---- S^T = K . Q^T: acc[qt][mt] rows = tokens 16 mt + 4 jj + i, column = query n -----
         f4 sacc[QT][2];
@@ -322,6 +332,10 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                     oacc[qt][d0 + x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[x].h, pb[qt].h, oacc[qt][d0 + x], 0, 0, 0);
         }
         __syncthreads();
+    };
+    for (int tile = tile_lo; tile < tile_hi; tile += 2) {
+        step(tile, 0, setA);
+        if (tile + 1 < tile_hi) step(tile + 1, 1, DEEP ? setB : setA);
     }
 
     // ---- normalise and store: lane (n, jj) holds out[q = n][d = 16 dt + 4 jj + i] ------------
