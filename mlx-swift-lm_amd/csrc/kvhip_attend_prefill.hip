@@ -63,11 +63,32 @@ prefill_kernel(AttendArgs a, int nsplit) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int n = lane & 15, jj = lane >> 4;
-    const int bh = blockIdx.y;
-    const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
+    // Linear workgroup ids go to the 8 XCDs round-robin and each XCD has its own L2: all query
+    // blocks of one (batch, kv-head) pair get ids of the same residue, so the pair's K/V tiles
+    // stay hot in one L2.
     const int r = a.Hq / a.Hkv;
     const int R = r * a.L;
-    const int row0 = blockIdx.x * BM + wave * 16 * QT;  // first query row of this wavefront
+    const int nblk = (R + BM - 1) / BM;
+    int blk_x, bh, split;
+    {
+        const int id = blockIdx.x;
+        const int BH = a.st.BH;
+        if ((BH & 7) == 0) {
+            const int xcd = id & 7, j = id >> 3;
+            const int per_pair = nblk * nsplit;
+            const int h_local = j / per_pair, rem = j - h_local * per_pair;
+            bh = h_local * 8 + xcd;
+            split = rem / nblk;
+            blk_x = rem - split * nblk;
+        } else {
+            blk_x = id % nblk;
+            const int t = id / nblk;
+            bh = t % BH;
+            split = t / BH;
+        }
+    }
+    const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
+    const int row0 = blk_x * BM + wave * 16 * QT;  // first query row of this wavefront
     const float fill = finfo_min_dt(DT);
     const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
 
@@ -114,7 +135,7 @@ prefill_kernel(AttendArgs a, int nsplit) {
     // ---- visible slot range for symbolic masks (only when slots are presented rows) -------
     int tile_lo = 0, tile_hi = (a.slots + BN - 1) / BN;
     if (IDENT) {
-        const int i_first = blockIdx.x * BM, i_last = min(R, i_first + BM) - 1;
+        const int i_first = blk_x * BM, i_last = min(R, i_first + BM) - 1;
         const bool spans = (i_first / a.L) != (i_last / a.L);
         const int l_min = spans ? 0 : i_first % a.L, l_max = spans ? a.L - 1 : i_last % a.L;
         if (a.mask.mode == KVHIP_MASK_CAUSAL) {
@@ -132,7 +153,7 @@ prefill_kernel(AttendArgs a, int nsplit) {
     if (MM != 2) {
         keep_hi = a.T - 1;
         if (MM == 1) {
-            const int i_first = blockIdx.x * BM, i_last = min(R, i_first + BM) - 1;
+            const int i_first = blk_x * BM, i_last = min(R, i_first + BM) - 1;
             const bool spans = (i_first / a.L) != (i_last / a.L);
             const int l_min = spans ? 0 : i_first % a.L, l_max = spans ? a.L - 1 : i_last % a.L;
             if (sym.mode == KVHIP_MASK_CAUSAL) {
@@ -146,9 +167,8 @@ prefill_kernel(AttendArgs a, int nsplit) {
         }
     }
 
-    // ---- optional split of the key range over blockIdx.z (small grids): each part leaves an
+    // ---- optional split of the key range (small grids): each part leaves an
     // unnormalised partial per query row, merged by the decode path's combine kernel
-    const int split = blockIdx.z;
     if (nsplit > 1) {
         const int span = (tile_hi - tile_lo + nsplit - 1) / nsplit;
         tile_lo = tile_lo + split * span;
@@ -497,7 +517,7 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
     const bool wide = prefill_wide(a);
     const int bm = wide ? 128 : 64;
     const int nsplit = prefill_splits(a);
-    dim3 grid((R + bm - 1) / bm, st.BH, nsplit), block(256);
+    dim3 grid((unsigned)((R + bm - 1) / bm) * st.BH * nsplit), block(256);  // linear: the kernel maps ids to tiles
     const bool ident = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
     const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
 #define PF_M(BITS, D, DT, QT, MM)                                                                         \
