@@ -292,7 +292,11 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         // visible tile, so a ragged batch gets workgroups in proportion to each length
         int vis_lo, vis_hi;
         sym_mask_row_range(sym, vis_lo, vis_hi);
-        const int t_lo = max(0, vis_lo) >> 6, t_hi = min(tiles_total, (min(vis_hi, a.T - 1) >> 6) + 1);
+        int t_lo = max(0, vis_lo) >> 6, t_hi = min(tiles_total, (min(vis_hi, a.T - 1) >> 6) + 1);
+        if (sym_mask_some_row_empty(sym)) {  // a fully masked row averages over every key
+            t_lo = 0;
+            t_hi = tiles_total;
+        }
         // tiles_per_wg == 0: divide this batch row's own visible range over the spans
         const int per = tiles_per_wg > 0 ? tiles_per_wg
                                          : (max(t_hi - t_lo, 1) + nsplit * NW - 1) / (nsplit * NW) * NW;

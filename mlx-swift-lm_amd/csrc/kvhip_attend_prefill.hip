@@ -145,6 +145,10 @@ prefill_kernel(AttendArgs a, int nsplit) {
             if (a.mask.window > 0) tile_lo = max(0, (a.mask.offset + l_min - a.mask.window + 1) / BN);
         }
         tile_hi = min(tile_hi, (a.T + BN - 1) / BN);
+        if (Q && sym_mask_some_row_empty(sym)) {  // a fully masked row averages over every key
+            tile_lo = 0;
+            tile_hi = (a.slots + BN - 1) / BN;
+        }
     }
 
     // presented rows [keep_lo, keep_hi] are seen by every query row of this workgroup: a key

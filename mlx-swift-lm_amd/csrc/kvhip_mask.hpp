@@ -69,6 +69,23 @@ __device__ __forceinline__ void sym_mask_row_range(const SymMask &s, int &lo, in
     if (s.window > 0) lo = max(lo, s.offset - s.window + 1);
 }
 
+// Whether some query position l in [0, L) sees no key row at all.  The quantized path fills
+// masked scores with finfo.min instead of dropping them (KVCache.swift:2396-2447), so such a
+// row attends uniformly over ALL presented keys and no key tile may be skipped for it.
+__device__ __forceinline__ bool sym_mask_some_row_empty(const SymMask &s) {
+    if (s.mode == KVHIP_MASK_CAUSAL) return s.T - s.L < 0;
+    // per position l the kept rows are [max(pad, offset + l - window + 1), min(offset + l, len - 1)]:
+    // the width is concave in l, so it is smallest at one of the two ends
+    for (int e = 0; e < 2; ++e) {
+        const int l = e ? s.L - 1 : 0;
+        int lo = s.pad_b;
+        const int hi = min(s.offset + l, min(s.len_b, s.T) - 1);
+        if (s.window > 0) lo = max(lo, s.offset + l - s.window + 1);
+        if (lo > hi) return true;
+    }
+    return false;
+}
+
 // Inclusive range of key rows EVERY query position l in [0, L) sees (empty if lo > hi).
 __device__ __forceinline__ void sym_mask_full_range(const SymMask &s, int &lo, int &hi) {
     if (s.mode == KVHIP_MASK_CAUSAL) {

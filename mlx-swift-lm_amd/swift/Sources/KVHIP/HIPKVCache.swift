@@ -198,6 +198,60 @@ public final class HIPRotatingKVCache: HIPKVCache {
     }
 }
 
+/// A `HIPRotatingKVCache` presented with uncommitted rows appended: the counterpart of
+/// `RotatingStagedKVCache` (RotatingStagedKVCache.swift:12-132) and what
+/// `RotatingRoundStrategy.presented` (KVCacheRound.swift:128-161) hands the model.  It shares
+/// the live ring's handle: staged rows sit in spare slots of the ring's page store, attention
+/// reads window ++ staged in place, and the ring does not move until `commit(retaining:)`.
+public final class HIPRotatingStagedKVCache {
+    public let live: HIPRotatingKVCache
+    private var open = true
+
+    public init(live: HIPRotatingKVCache) {
+        self.live = live
+        must(kvhip_cache_stage_begin(live.handle))
+    }
+
+    public var stagedCount: Int { open ? Int(kvhip_cache_stage_count(live.handle)) : 0 }
+    public var offset: Int { live.offset + stagedCount }
+    public var maxSize: Int? { live.maxSize }
+
+    /// Stages the rows and returns the trailing window of the ring followed by everything staged.
+    public func update<A: HIPArray>(keys: A, values: A) -> (A, A) { live.update(keys: keys, values: values) }
+
+    /// The fused form: stage, then attend over window ++ staged without exporting it.
+    public func attend<A: HIPArray>(queries: A, keys: A, values: A, scale: Float, mask: HIPMask) -> A {
+        live.attend(queries: queries, keys: keys, values: values, scale: scale, mask: mask)
+    }
+
+    /// The live cache's own mask (RotatingStagedKVCache.swift:49-58).
+    public func makeMask(n: Int, windowSize: Int?, returnArray: Bool) -> kvhip_mask_plan_t {
+        live.makeMask(n: n, windowSize: windowSize, returnArray: returnArray)
+    }
+
+    /// `stagedArrays` (RotatingStagedKVCache.swift:27-30), for a restore point's replay.
+    public func stagedArrays<A: HIPArray>(like: A) -> (A, A)? {
+        let n = stagedCount
+        guard n > 0 else { return nil }
+        let s = like.shape
+        let k = A.empty([s[0], s[1], n, s[3]], dtype: like.kvhipDType)
+        let v = A.empty([s[0], s[1], n, s[3]], dtype: like.kvhipDType)
+        must(kvhip_cache_stage_fetch(live.handle, k.devicePointer, v.devicePointer, live.stream))
+        return (k, v)
+    }
+
+    /// `commit(retaining:)` (RotatingStagedKVCache.swift:62-76); retaining 0 is a rollback.
+    public func commit(retaining: Int) {
+        guard open else { return }
+        open = false
+        must(kvhip_cache_stage_commit(live.handle, Int64(retaining), live.stream))
+    }
+
+    // round-scoped: not trimmable, not copyable, not restorable (RotatingStagedKVCache.swift:93-125)
+    public var isTrimmable: Bool { false }
+    @discardableResult public func trim(_ n: Int) -> Int { 0 }
+}
+
 public final class HIPQuantizedKVCache: HIPKVCache {
     public init(groupSize: Int = 64, bits: Int = 8) {
         super.init(kind: KVHIP_KIND_QUANTIZED, groupSize: groupSize, bits: bits)
