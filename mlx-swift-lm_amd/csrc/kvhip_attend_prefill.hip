@@ -1,12 +1,11 @@
 // Chunked-prefill attention tile on the matrix cores (gfx950, v_mfma_f32_16x16x32_f16) for
-// quantized caches; full-precision caches take the double-buffered kernel of
-// kvhip_attend_prefill_fp.hip (the BITS == 0 paths below are what that kernel grew out of and
-// are no longer instantiated).
+// quantized caches (full-precision caches take the kernel of kvhip_attend_prefill_fp.hip),
+// and the launcher of both.
 //
 // Many query rows per kv head (r = Hq/Hkv heads times L new tokens).  One workgroup
 // (4 wavefronts) owns 128 query rows of one (batch, kv-head) pair -- 32 per wavefront
 // -- and walks the cached keys in tiles of 32 physical slots.  A tile is staged once
-// per workgroup in LDS as fp16 (packed codes are dequantised here, bf16 is converted),
+// per workgroup in LDS as fp16 (the packed codes are dequantised here),
 // K as [token][d] and V as [d][token], which is how the page layout already stores
 // them; the dense contractions then run as
 //   S^T   = K . Q^T      A = K rows from LDS, B = query rows held in registers
@@ -47,7 +46,7 @@ __device__ __forceinline__ uint32_t h2_bits(float lo, float hi) { return (uint32
 template <int BITS, int D, int DT, bool IDENT, int QT, int MM>
 __global__ void __launch_bounds__(256, 2)
 prefill_kernel(AttendArgs a, int nsplit) {
-    constexpr bool Q = BITS != 0;
+    static_assert(BITS == 4 || BITS == 8, "quantized caches only");
     constexpr int BM = 64 * QT;
     constexpr int KS = D + 8;    // halves per K row in LDS (padded against bank conflicts)
     constexpr int VS = BN + 4;   // halves per V^T row in LDS
@@ -57,7 +56,7 @@ prefill_kernel(AttendArgs a, int nsplit) {
     __shared__ __attribute__((aligned(16))) _Float16 Vs[D * VS];
     __shared__ int rows_s[BN];
     __shared__ int tile_full_s;
-    __shared__ float sb_s[Q ? BN * 2 * (D / 32) : 1];  // V (scale, bias) per token and group
+    __shared__ float sb_s[BN * 2 * (D / 32)];  // V (scale, bias) per token and group
 
     const Store &st = a.st;
     const int tid = threadIdx.x;
@@ -112,10 +111,8 @@ prefill_kernel(AttendArgs a, int nsplit) {
                 if (q_ok[qt]) {
                     v0 = Elem<DT>::load(a.q, qoff + 32 * s + 8 * jj + 2 * w);
                     v1 = Elem<DT>::load(a.q, qoff + 32 * s + 8 * jj + 2 * w + 1);
-                    if (Q) {
-                        v0 = round_dt<DT>(v0 * a.scale);
-                        v1 = round_dt<DT>(v1 * a.scale);
-                    }
+                    v0 = round_dt<DT>(v0 * a.scale);  // the reference rounds q * scale to T
+                    v1 = round_dt<DT>(v1 * a.scale);
                 }
                 qop[qt][s].u[w] = h2_bits(v0, v1);
             }
@@ -145,7 +142,7 @@ prefill_kernel(AttendArgs a, int nsplit) {
             if (a.mask.window > 0) tile_lo = max(0, (a.mask.offset + l_min - a.mask.window + 1) / BN);
         }
         tile_hi = min(tile_hi, (a.T + BN - 1) / BN);
-        if (Q && sym_mask_some_row_empty(sym)) {  // a fully masked row averages over every key
+        if (sym_mask_some_row_empty(sym)) {  // a fully masked row averages over every key
             tile_lo = 0;
             tile_hi = (a.slots + BN - 1) / BN;
         }
@@ -181,15 +178,12 @@ prefill_kernel(AttendArgs a, int nsplit) {
 
     // ---- staging: a tile is fetched from global memory into registers one iteration ahead
     // (in flight while the current tile is contracted), then converted and written to LDS.
-    constexpr int BB = Q ? BITS : 4;
-    constexpr int KU = Q ? 1 : D / 64;            // uint4 per thread for K (fp); quantized: words below
-    constexpr int KQW = (D / 8) * BB / 32;        // quantized: packed words per thread for K (D/8 codes)
-    constexpr int VQW = 16 * BB / 32;             // quantized: packed words per thread and column for V
+    constexpr int BB = BITS;
+    constexpr int KQW = (D / 8) * BB / 32;        // packed words per thread for K (D/8 codes)
+    constexpr int VQW = 16 * BB / 32;             // packed words per thread and column for V
     constexpr int VCOLS = (2 * D + 255) / 256;    // (column, half) items per thread for V
-    uint4 kreg[Q ? 1 : KU];
-    uint4 vreg[Q ? 1 : 2 * VCOLS];
-    uint32_t kq[Q ? KQW : 1], vq[Q ? VCOLS * VQW : 1], ksb_raw = 0;
-    uint32_t vsb_raw[Q ? D / 32 : 1];
+    uint32_t kq[KQW], vq[VCOLS * VQW], ksb_raw = 0;
+    uint32_t vsb_raw[D / 32];
     int row_reg = -1;
     const int kt = tid >> 3, kpart = tid & 7;     // K: 8 threads per token row
 
@@ -203,46 +197,30 @@ prefill_kernel(AttendArgs a, int nsplit) {
             row_reg = (row >= 0 && row < a.T) ? row : -1;
         }
         const char *cell = v_cell_ptr(st, bh, slot0);
-        if constexpr (!Q) {
-            const uint4 *src = reinterpret_cast<const uint4 *>(k_row_ptr(st, bh, slot0 + kt)) + kpart * KU;
+        const uint32_t *w = reinterpret_cast<const uint32_t *>(k_row_ptr(st, bh, slot0 + kt)) + kpart * KQW;
 #pragma unroll
-            for (int e = 0; e < KU; ++e) kreg[e] = src[e];
-            const int half = (slot0 & 32) ? 1 : 0;
+        for (int e = 0; e < KQW; ++e) kq[e] = w[e];
+        // the D/8 codes of this thread lie in one group (group sizes are >= 32 >= D/8)
+        const int g = (kpart * (D / 8)) / st.gs;
+        ksb_raw = reinterpret_cast<const uint32_t *>(ksb_row_ptr(st, bh, slot0 + kt))[g];
+        if (tid < BN) {
+            const uint32_t *sb = reinterpret_cast<const uint32_t *>(vsb_row_ptr(st, bh, slot0 + tid));
 #pragma unroll
-            for (int ci = 0; ci < VCOLS; ++ci) {
-                const int c = tid + 256 * ci;
-                if (c < 2 * D) {
-                    const int d = c >> 1, part = c & 1;
-                    const uint4 *vs = reinterpret_cast<const uint4 *>(cell + v_row_off(st, slot0, d) + half * 64 + part * 32);
-                    vreg[2 * ci] = vs[0];
-                    vreg[2 * ci + 1] = vs[1];
-                }
-            }
-        } else {
-            const uint32_t *w = reinterpret_cast<const uint32_t *>(k_row_ptr(st, bh, slot0 + kt)) + kpart * KQW;
+            for (int gg = 0; gg < D / 32; ++gg)
+                if (gg < D / st.gs) vsb_raw[gg] = sb[gg];
+        }
+        const int tbase = slot0 & 32;
 #pragma unroll
-            for (int e = 0; e < KQW; ++e) kq[e] = w[e];
-            // the D/8 codes of this thread lie in one group (group sizes are >= 32 >= D/8)
-            const int g = (kpart * (D / 8)) / st.gs;
-            ksb_raw = reinterpret_cast<const uint32_t *>(ksb_row_ptr(st, bh, slot0 + kt))[g];
-            if (tid < BN) {
-                const uint32_t *sb = reinterpret_cast<const uint32_t *>(vsb_row_ptr(st, bh, slot0 + tid));
+        for (int ci = 0; ci < VCOLS; ++ci) {
+            const int c = tid + 256 * ci;
+            if (c < 2 * D) {
+                const int d = c >> 1, part = c & 1;
+                const uint32_t *vw = reinterpret_cast<const uint32_t *>(cell + v_row_off(st, slot0, d)) + (tbase + part * 16) * BB / 32;
 #pragma unroll
-                for (int gg = 0; gg < D / 32; ++gg)
-                    if (gg < D / st.gs) vsb_raw[gg] = sb[gg];
-            }
-            const int tbase = slot0 & 32;
-#pragma unroll
-            for (int ci = 0; ci < VCOLS; ++ci) {
-                const int c = tid + 256 * ci;
-                if (c < 2 * D) {
-                    const int d = c >> 1, part = c & 1;
-                    const uint32_t *vw = reinterpret_cast<const uint32_t *>(cell + v_row_off(st, slot0, d)) + (tbase + part * 16) * BB / 32;
-#pragma unroll
-                    for (int e = 0; e < VQW; ++e) vq[ci * VQW + e] = vw[e];
-                }
+                for (int e = 0; e < VQW; ++e) vq[ci * VQW + e] = vw[e];
             }
         }
+    
     };
     auto sb_pair = [&](uint32_t raw, float &sc, float &bi) {  // (scale, bias) of a 16-bit dtype
         if (DT == 0) {
@@ -253,48 +231,35 @@ prefill_kernel(AttendArgs a, int nsplit) {
             bi = __uint_as_float(raw & 0xffff0000u);
         }
     };
-    auto to_h2 = [&](uint32_t w) -> uint32_t {  // two cache-dtype elements -> two fp16
-        if (DT == 1) return h2_bits(__uint_as_float(w << 16), __uint_as_float(w & 0xffff0000u));
-        return w;
-    };
     auto stage_k = [&]() {  // K, row indices and (quantized) the V scale/bias table
         if (tid < BN) rows_s[tid] = row_reg;
         if (wave == 0) {
             const bool full = __all(lane >= BN || (row_reg >= keep_lo && row_reg <= keep_hi));
             if (lane == 0) tile_full_s = full;
         }
-        if constexpr (!Q) {
-            _Float16 *dst = Ks + kt * KS + kpart * (D / 8);
+        constexpr int per = 32 / BB;
+        float sc, bi;
+        sb_pair(ksb_raw, sc, bi);
+        _Float16 *dst = Ks + kt * KS + kpart * (D / 8);
 #pragma unroll
-            for (int e = 0; e < KU; ++e) {
-                uint4 r_ = kreg[e];
-                r_.x = to_h2(r_.x); r_.y = to_h2(r_.y); r_.z = to_h2(r_.z); r_.w = to_h2(r_.w);
-                *reinterpret_cast<uint4 *>(dst + 8 * e) = r_;
+        for (int e = 0; e < KQW; ++e)
+#pragma unroll
+            for (int x = 0; x < per; x += 2) {
+                const float c0 = (float)((kq[e] >> (x * BB)) & ((1u << BB) - 1u));
+                const float c1 = (float)((kq[e] >> ((x + 1) * BB)) & ((1u << BB) - 1u));
+                *reinterpret_cast<uint32_t *>(dst + e * per + x) = h2_bits(sc * c0 + bi, sc * c1 + bi);
             }
-        } else {
-            constexpr int per = 32 / BB;
-            float sc, bi;
-            sb_pair(ksb_raw, sc, bi);
-            _Float16 *dst = Ks + kt * KS + kpart * (D / 8);
+        if (tid < BN) {
 #pragma unroll
-            for (int e = 0; e < KQW; ++e)
-#pragma unroll
-                for (int x = 0; x < per; x += 2) {
-                    const float c0 = (float)((kq[e] >> (x * BB)) & ((1u << BB) - 1u));
-                    const float c1 = (float)((kq[e] >> ((x + 1) * BB)) & ((1u << BB) - 1u));
-                    *reinterpret_cast<uint32_t *>(dst + e * per + x) = h2_bits(sc * c0 + bi, sc * c1 + bi);
+            for (int gg = 0; gg < D / 32; ++gg)
+                if (gg < D / st.gs) {
+                    float s2, b2;
+                    sb_pair(vsb_raw[gg], s2, b2);
+                    sb_s[(tid * 2) * (D / 32) + gg] = s2;
+                    sb_s[(tid * 2 + 1) * (D / 32) + gg] = b2;
                 }
-            if (tid < BN) {
-#pragma unroll
-                for (int gg = 0; gg < D / 32; ++gg)
-                    if (gg < D / st.gs) {
-                        float s2, b2;
-                        sb_pair(vsb_raw[gg], s2, b2);
-                        sb_s[(tid * 2) * (D / 32) + gg] = s2;
-                        sb_s[(tid * 2 + 1) * (D / 32) + gg] = b2;
-                    }
-            }
         }
+    
     };
     auto stage_v = [&]() {
 #pragma unroll
@@ -303,27 +268,19 @@ prefill_kernel(AttendArgs a, int nsplit) {
             if (c < 2 * D) {
                 const int d = c >> 1, part = c & 1;
                 _Float16 *dst = Vs + d * VS + part * 16;
-                if constexpr (!Q) {
+                const int g = d / st.gs;
+                // token tt of the 16 sits at code position p(tt) of its word (V tile order)
 #pragma unroll
-                    for (int e = 0; e < 2; ++e) {
-                        const uint4 r_ = vreg[2 * ci + e];
-                        *reinterpret_cast<uint2 *>(dst + 8 * e) = make_uint2(to_h2(r_.x), to_h2(r_.y));
-                        *reinterpret_cast<uint2 *>(dst + 8 * e + 4) = make_uint2(to_h2(r_.z), to_h2(r_.w));
-                    }
-                } else {
-                    const int g = d / st.gs;
-                    // token tt of the 16 sits at code position p(tt) of its word (V tile order)
-#pragma unroll
-                    for (int tt = 0; tt < 16; tt += 2) {
-                        const int bp0 = v_bitpos<BB>(tt), bp1 = v_bitpos<BB>(tt + 1);
-                        const float c0 = (float)((vq[ci * VQW + (bp0 >> 5)] >> (bp0 & 31)) & ((1u << BB) - 1u));
-                        const float c1 = (float)((vq[ci * VQW + (bp1 >> 5)] >> (bp1 & 31)) & ((1u << BB) - 1u));
-                        const int t0 = part * 16 + tt;
-                        const float v0 = sb_s[(t0 * 2) * (D / 32) + g] * c0 + sb_s[(t0 * 2 + 1) * (D / 32) + g];
-                        const float v1 = sb_s[((t0 + 1) * 2) * (D / 32) + g] * c1 + sb_s[((t0 + 1) * 2 + 1) * (D / 32) + g];
-                        *reinterpret_cast<uint32_t *>(dst + tt) = h2_bits(v0, v1);
-                    }
+                for (int tt = 0; tt < 16; tt += 2) {
+                    const int bp0 = v_bitpos<BB>(tt), bp1 = v_bitpos<BB>(tt + 1);
+                    const float c0 = (float)((vq[ci * VQW + (bp0 >> 5)] >> (bp0 & 31)) & ((1u << BB) - 1u));
+                    const float c1 = (float)((vq[ci * VQW + (bp1 >> 5)] >> (bp1 & 31)) & ((1u << BB) - 1u));
+                    const int t0 = part * 16 + tt;
+                    const float v0 = sb_s[(t0 * 2) * (D / 32) + g] * c0 + sb_s[(t0 * 2 + 1) * (D / 32) + g];
+                    const float v1 = sb_s[((t0 + 1) * 2) * (D / 32) + g] * c1 + sb_s[((t0 + 1) * 2 + 1) * (D / 32) + g];
+                    *reinterpret_cast<uint32_t *>(dst + tt) = h2_bits(v0, v1);
                 }
+            
             }
         }
     };
@@ -332,7 +289,7 @@ prefill_kernel(AttendArgs a, int nsplit) {
     for (int tile = tile_lo; tile < tile_hi; ++tile) {
         if (tile > tile_lo) __syncthreads();  // everyone is done reading the previous tile
         stage_k();
-        if constexpr (Q) __syncthreads();     // the V dequantisation reads the scale/bias table
+        __syncthreads();  // the V dequantisation reads the scale/bias table
         stage_v();
         __syncthreads();
         if (tile + 1 < tile_hi) fetch(tile + 1);
@@ -374,21 +331,17 @@ prefill_kernel(AttendArgs a, int nsplit) {
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float s_ = Q ? round_dt<DT>(sacc[qt][mt][i]) : sacc[qt][mt][i] * a.scale;
+                    float s_ = round_dt<DT>(sacc[qt][mt][i]);
                     if (MM == 2 || !tile_full) {  // workgroup-uniform
                         const int row = trow[mt][i];
                         if (row >= 0 && q_ok[qt]) {
                             if constexpr (MM == 1) {
-                                if (!sym_mask_keep(sym, q_l[qt], row)) s_ = Q ? fill : -INFINITY;
+                                if (!sym_mask_keep(sym, q_l[qt], row)) s_ = fill;
                             } else if constexpr (MM == 2) {
                                 float add;
                                 const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
-                                if (Q) {
-                                    if (!keep) s_ = fill;
-                                    else if (a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
-                                } else {
-                                    s_ = keep ? s_ + add : -INFINITY;
-                                }
+                                if (!keep) s_ = fill;
+                                else if (a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
                             }
                         } else {
                             s_ = -INFINITY;
