@@ -1098,6 +1098,15 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
         else if (p.rg == 2) DEC(BITS, D, GS, DT, 2);  \
         else DEC(BITS, D, GS, DT, 4);                 \
     } while (0)
+    if (st.bits != 0 && p.rg == 4 && !getenv("KVHIP_NO_DECODE16")) {
+        // 9..16 rows per kv head fill the 16x16x32 instruction: its own kernel
+        profile_mark(s, true);
+        hipError_t e = launch_attend_decode16(a_in, p.tiles_total, p.tiles_per_wg, p.nsplit, s);
+        profile_mark(s, false);
+        if (e != hipSuccess) return e;
+        if (p.nsplit > 1) return launch_combine(a_in, p.nsplit, 16, s);
+        return hipSuccess;
+    }
 #define DEC_DT(BITS, D, GS)                                \
     do {                                                   \
         if (st.dtype == KVHIP_F16) DEC_RG(BITS, D, GS, 0); \

@@ -1,0 +1,473 @@
+// Split-sequence attention for quantized caches with 9..16 query rows per kv head (the
+// speculative-verify shape: 4 new tokens at a GQA ratio of 4) on v_mfma_f32_16x16x32_f16.
+//
+// With 16 rows the 16x16x32 instruction is filled exactly, at a quarter of the matrix-core
+// time the 4-row broadcast contraction of kvhip_attend_decode.hip needs for the same rows.
+// Same decomposition otherwise: a workgroup (4 wavefronts) owns a span of 64-token tiles of one
+// (batch, kv-head) pair, a wavefront takes every 4th tile, the partials (max, sum, out[D]) of
+// the spans are merged by the combine kernel.
+//
+//   S^T = K . Q^T    A: lane (n, jj) holds 8 codes of the K row of token tok(tb, n), block tb of
+//                    four; B: lane (n, jj) holds the same 8 head-dim positions of query row n.
+//                    C: lane (n, jj) receives the scores of row n for tokens tok(tb, 4 jj + i).
+//   out^T += V^T P^T A: lane (n, jj) holds 8 tokens of head-dim row 16 db + n of the transposed
+//                    V tile; B: the probabilities of row n for the same 8 tokens, which are
+//                    exactly what the C registers of two score blocks hold: P never moves.
+//
+// The freedom in both contractions is the order of the contracted index, which only has to agree
+// between A and B.  It is chosen so that every operand is a run of whole packed words:
+//   * head dim: a quantization group of GS codes is cut in four lane segments (jj) of GS/4
+//     codes; step h of the group takes codes 8 h .. 8 h + 7 of each segment, so one instruction
+//     stays inside one group and the group's scale can be applied to its accumulator;
+//   * tokens: tok(tb, m) = 16 (m / 4) + 4 tb + m % 4, so lane group jj scores tokens
+//     16 jj .. 16 jj + 15 and the 8 probabilities it feeds to step u of PV belong to tokens
+//     16 jj + 8 u .. + 7 -- one (4-bit) or two (8-bit) whole words of a V tile row.
+// Codes become operands as in the 4-row kernel: a masked word is a pair of fp16 subnormals
+// code * 2^-24 (high nibbles * 2^-20, compensated by 1/16 on the other operand).
+#include "kvhip_mask.hpp"
+
+namespace kvhip {
+
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+union Op8 {
+    h8 h;
+    u4 v;
+};
+
+constexpr int WAVES = 4;
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float TWO24 = 16777216.0f;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
+}
+template <int DT> __device__ __forceinline__ void sb_pair(uint32_t raw, float &sc, float &bi) {
+    if (DT == 0) {
+        sc = (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+        bi = (float)__builtin_bit_cast(_Float16, (uint16_t)(raw >> 16));
+    } else {
+        sc = __uint_as_float(raw << 16);
+        bi = __uint_as_float(raw & 0xffff0000u);
+    }
+}
+
+// 8 codes -> one 8-element operand.  4 bit: one word, element order (c0,c4,c1,c5,c2,c6,c3,c7),
+// registers 1 and 3 hold high nibbles (x16).  8 bit: two words, order (c0,c2,c1,c3,c4,c6,c5,c7).
+template <int BITS> struct Codes;
+template <> struct Codes<4> {
+    static constexpr int WORDS = 1;
+    static __device__ __forceinline__ Op8 unpack(const uint32_t *w) {
+        Op8 o;
+        const uint32_t w8 = w[0] >> 8;
+        o.v = u4{w[0] & 0x000f000fu, w[0] & 0x00f000f0u, w8 & 0x000f000fu, w8 & 0x00f000f0u};
+        return o;
+    }
+};
+template <> struct Codes<8> {
+    static constexpr int WORDS = 2;
+    static __device__ __forceinline__ Op8 unpack(const uint32_t *w) {
+        Op8 o;
+        o.v = u4{w[0] & 0x00ff00ffu, (w[0] >> 8) & 0x00ff00ffu, w[1] & 0x00ff00ffu, (w[1] >> 8) & 0x00ff00ffu};
+        return o;
+    }
+};
+// operand position p (0..7) -> which of the 8 codes it holds, and whether it is a high nibble
+template <int BITS> __device__ __forceinline__ constexpr int code_of(int p) {
+    if (BITS == 4) return 2 * (p >> 2) + ((p >> 1) & 1) + 4 * (p & 1);  // (0,4,1,5,2,6,3,7)
+    return 4 * (p >> 2) + ((p >> 1) & 1) + 2 * (p & 1);                  // (0,2,1,3,4,6,5,7)
+}
+template <int BITS> __device__ __forceinline__ constexpr bool hi_of(int p) { return BITS == 4 && ((p >> 1) & 1); }
+
+// MM: 0 no mask, 1 index-only mask (causal / window with per-batch bounds), 2 array mask.
+template <int BITS, int D, int GS, int DT, int MM>
+__global__ void __launch_bounds__(WAVES * 64, 2)
+decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
+    using CD = Codes<BITS>;
+    constexpr int G = D / GS;                    // quantization groups per row
+    constexpr int SPG = GS / 32;                 // contraction steps per group
+    constexpr int KWL = GS * BITS / 8 / 16;      // words per lane, group and K row (segment of GS/4 codes)
+    constexpr int NDB = D / 16;                  // 16-row blocks of out^T
+    constexpr int VWL = 16 * BITS / 32;          // words per lane and V row: its 16 tokens
+    constexpr int VROW = 64 * BITS / 8;          // bytes of one V tile row
+    constexpr int RR = 16;
+    const Store &st = a.st;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n = lane & 15, jj = lane >> 4;
+    const int bh = blockIdx.y, split = blockIdx.x;
+    const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
+    const int r = a.Hq / a.Hkv;
+    const int R = r * a.L;
+
+    __shared__ float cbuf[WAVES][RR][D + 2];
+
+    // ---- span of this workgroup (as in the 4-row kernel) -----------------------------------
+    const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
+    int tile_begin = split * tiles_per_wg;
+    int tile_end = min(tiles_total, tile_begin + tiles_per_wg);
+    if constexpr (MM == 1) {
+        int vis_lo, vis_hi;
+        sym_mask_row_range(sym, vis_lo, vis_hi);
+        int t_lo = max(0, vis_lo) >> 6, t_hi = min(tiles_total, (min(vis_hi, a.T - 1) >> 6) + 1);
+        if (sym_mask_some_row_empty(sym)) {  // a fully masked row averages over every key
+            t_lo = 0;
+            t_hi = tiles_total;
+        }
+        const int per = tiles_per_wg > 0 ? tiles_per_wg
+                                         : (max(t_hi - t_lo, 1) + nsplit * WAVES - 1) / (nsplit * WAVES) * WAVES;
+        tile_begin = t_lo + split * per;
+        tile_end = min(t_hi, tile_begin + per);
+    }
+    const int tile0 = tile_begin + wave;
+    const int my_tiles = tile0 < tile_end ? (tile_end - tile0 + WAVES - 1) / WAVES : 0;
+    int full_lo = 0, full_hi = a.T - 1;  // rows every query row keeps
+    if constexpr (MM == 1) {
+        sym_mask_full_range(sym, full_lo, full_hi);
+        full_hi = min(full_hi, a.T - 1);
+    }
+    const int row_l = n % a.L, row_rep = n / a.L;  // this lane's query row n = (head rep, position l)
+    const bool row_ok = n < R;
+
+    // ---- per-lane addresses inside a tile; tiles of one wavefront are a page apart -----------
+    // K block tb, lane (n, jj): row of token tok(tb, n) = 16 (n / 4) + 4 tb + n % 4, segment jj
+    const size_t k_step = (size_t)st.BH * st.k_cell, v_step = (size_t)st.BH * st.v_cell;
+    const size_t ksb_step = (size_t)st.BH * st.ksb_cell, vsb_step = (size_t)st.BH * st.vsb_cell;
+    const int page0 = tile0 >> 2, tip = tile0 & 3;
+    const char *kp = st.k + ((size_t)page0 * st.BH + bh) * st.k_cell + (size_t)tip * TILE * st.k_row
+                     + (size_t)(16 * (n >> 2) + (n & 3)) * st.k_row + jj * (KWL * 4);
+    const char *vp = st.v + ((size_t)page0 * st.BH + bh) * st.v_cell + (size_t)tip * D * VROW
+                     + (size_t)n * VROW + jj * (VWL * 4);
+    // (scale, bias) pairs of this lane group's 16 tokens, 16 jj .. 16 jj + 15
+    const char *ksp = st.ksb + ((size_t)page0 * st.BH + bh) * st.ksb_cell + (size_t)(tip * TILE + 16 * jj) * st.ksb_row;
+    const char *vsp = st.vsb + ((size_t)page0 * st.BH + bh) * st.vsb_cell + (size_t)(tip * TILE + 16 * jj) * st.vsb_row;
+    int base_next = tile0 * TILE;
+
+    struct Tile {
+        uint32_t k[4][G][KWL];
+        uint32_t v[NDB][VWL];
+        uint32_t ksb[16][G], vsb[16][G];  // raw (scale, bias) pairs per token of the lane group
+        int base;                          // first slot of the tile
+    };
+
+    int k_loaded = 0, v_loaded = 0;
+    auto load_k = [&](Tile &t) __attribute__((always_inline)) {
+#pragma unroll
+        for (int tb = 0; tb < 4; ++tb)
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const char *p = kp + (size_t)(4 * tb) * st.k_row + g * (GS * BITS / 8);
+                if constexpr (KWL == 2) {
+                    const u2 w = *reinterpret_cast<const u2 *>(p);
+                    t.k[tb][g][0] = w.x; t.k[tb][g][1] = w.y;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < KWL / 4; ++e) {
+                        const u4 w = reinterpret_cast<const u4 *>(p)[e];
+                        t.k[tb][g][4 * e] = w.x; t.k[tb][g][4 * e + 1] = w.y;
+                        t.k[tb][g][4 * e + 2] = w.z; t.k[tb][g][4 * e + 3] = w.w;
+                    }
+                }
+            }
+        // 16 tokens x G pairs of 4 bytes: contiguous rows of G * 4 bytes
+#pragma unroll
+        for (int e = 0; e < 16 * G / 4; ++e) {
+            const u4 w = reinterpret_cast<const u4 *>(ksp)[e];
+            (&t.ksb[0][0])[4 * e] = w.x; (&t.ksb[0][0])[4 * e + 1] = w.y;
+            (&t.ksb[0][0])[4 * e + 2] = w.z; (&t.ksb[0][0])[4 * e + 3] = w.w;
+        }
+        t.base = base_next;
+        ++k_loaded;
+        if (k_loaded < my_tiles) {  // wave-uniform: the same tile of the next page
+            kp += k_step;
+            ksp += ksb_step;
+            base_next += PAGE;
+        }
+    };
+    auto load_v = [&](Tile &t) __attribute__((always_inline)) {
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+            const char *p = vp + (size_t)(16 * db) * VROW;
+            if constexpr (VWL == 2) {
+                const u2 w = *reinterpret_cast<const u2 *>(p);
+                t.v[db][0] = w.x; t.v[db][1] = w.y;
+            } else {
+                const u4 w = *reinterpret_cast<const u4 *>(p);
+                t.v[db][0] = w.x; t.v[db][1] = w.y; t.v[db][2] = w.z; t.v[db][3] = w.w;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 16 * G / 4; ++e) {
+            const u4 w = reinterpret_cast<const u4 *>(vsp)[e];
+            (&t.vsb[0][0])[4 * e] = w.x; (&t.vsb[0][0])[4 * e + 1] = w.y;
+            (&t.vsb[0][0])[4 * e + 2] = w.z; (&t.vsb[0][0])[4 * e + 3] = w.w;
+        }
+        ++v_loaded;
+        if (v_loaded < my_tiles) {
+            vp += v_step;
+            vsp += vsb_step;
+        }
+    };
+
+    // ---- query operands (B of S^T) and the group sums of each query row ------------------------
+    Op8 qb[G][SPG];
+    float qsum[G];
+    auto load_queries = [&]() __attribute__((always_inline)) {
+        const size_t qoff = ((size_t)(b * a.Hq + hk * r + row_rep) * a.L + row_l) * D;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            float part = 0.f;
+#pragma unroll
+            for (int h = 0; h < SPG; ++h) {
+                float qv[8];
+#pragma unroll
+                for (int p = 0; p < 8; ++p) {
+                    const int d = GS * g + (GS / 4) * jj + 8 * h + code_of<BITS>(p);
+                    float v = 0.f;
+                    if (row_ok) v = (float)(_Float16)round_dt<DT>(Elem<DT>::load(a.q, qoff + d) * a.scale);
+                    part += v;
+                    qv[p] = hi_of<BITS>(p) ? v * 0.0625f : v;
+                }
+                qb[g][h].v = u4{pack_h2(qv[0], qv[1]), pack_h2(qv[2], qv[3]), pack_h2(qv[4], qv[5]), pack_h2(qv[6], qv[7])};
+            }
+            part += __shfl_xor(part, 16);
+            part += __shfl_xor(part, 32);
+            qsum[g] = part;
+        }
+    };
+
+    // ---- running state: lane (n, jj) carries row n; m is equal in the four lanes of a row -------
+    float m_run = -INFINITY, l_part = 0.f, bacc[G];
+    f4 oacc[NDB];
+#pragma unroll
+    for (int g = 0; g < G; ++g) bacc[g] = 0.f;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) oacc[db] = f4{0.f, 0.f, 0.f, 0.f};
+    const float fill = finfo_min_dt(DT);
+
+    Op8 pb[G][2];  // probabilities of the tile in flight: per group (pre-scaled by V's scale), step u
+
+    auto compute_qk_softmax = [&](const Tile &t) __attribute__((always_inline)) {
+        // ---- S^T blocks --------------------------------------------------------------------
+        f4 sacc[4][G];
+#pragma unroll
+        for (int tb = 0; tb < 4; ++tb)
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                sacc[tb][g] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int h = 0; h < SPG; ++h) {
+                    const Op8 ka = CD::unpack(&t.k[tb][g][h * CD::WORDS]);
+                    sacc[tb][g] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka.h, qb[g][h].h, sacc[tb][g], 0, 0, 0);
+                }
+            }
+        // ---- scores of row n for this lane group's 16 tokens: local token 4 tb + i ---------------
+        const bool edge = MM == 2 || t.base < full_lo || t.base + (TILE - 1) > full_hi;  // wave-uniform
+        float x[16];
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int tb = 0; tb < 4; ++tb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int tl = 4 * tb + i;
+                float s_ = 0.f;
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    float sc, bi;
+                    sb_pair<DT>(t.ksb[tl][g], sc, bi);
+                    s_ = __builtin_fmaf(bi, qsum[g], s_);
+                    s_ = __builtin_fmaf(sc * TWO24, sacc[tb][g][i], s_);
+                }
+                s_ = round_dt<DT>(s_);
+                if (edge) {
+                    const int row = t.base + 16 * jj + tl;  // slots are presented rows
+                    if (row < a.T) {
+                        if constexpr (MM == 1) {
+                            if (!sym_mask_keep(sym, row_l, row)) s_ = fill;
+                        } else if constexpr (MM == 2) {
+                            if (row_ok) {
+                                float add;
+                                const bool keep = mask_keep(a.mask, b, hk * r + row_rep, row_l, row, a.L, a.T, add);
+                                if (!keep) s_ = fill;
+                                else if (a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
+                            }
+                        }
+                    } else {
+                        s_ = -INFINITY;
+                    }
+                }
+                x[tl] = s_;
+                tmax = fmaxf(tmax, s_);
+            }
+        // raise the row maximum only when some lane's own maximum exceeds it (rare after the
+        // first tiles); it stays equal in the four lanes of a row
+        if (__any(tmax > m_run)) {
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+            const float mn = fmaxf(m_run, tmax);
+            const float alpha = (mn == -INFINITY) ? 1.f : fast_exp2((m_run - mn) * LOG2E);
+            m_run = mn;
+            l_part *= alpha;
+#pragma unroll
+            for (int g = 0; g < G; ++g) bacc[g] *= alpha;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) oacc[db][i] *= alpha;
+        }
+        const float mu = (m_run == -INFINITY) ? 0.f : m_run;
+        float pv[G][16];
+#pragma unroll
+        for (int tl = 0; tl < 16; ++tl) {
+            const float p = fast_exp2((x[tl] - mu) * LOG2E);  // exp2(-inf) = 0 for dead slots
+            l_part += p;
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                float sc, bi;
+                sb_pair<DT>(t.vsb[tl][g], sc, bi);
+                bacc[g] = __builtin_fmaf(p, bi, bacc[g]);
+                // step u = tl / 8 holds tokens 8 u .. 8 u + 7; positions 2, 3, 6, 7 of a 4-bit
+                // operand meet high nibbles
+                pv[g][tl] = p * (hi_of<BITS>(tl & 7) ? sc * 0.0625f : sc);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+                pb[g][u].v = u4{pack_h2(pv[g][8 * u], pv[g][8 * u + 1]), pack_h2(pv[g][8 * u + 2], pv[g][8 * u + 3]),
+                                pack_h2(pv[g][8 * u + 4], pv[g][8 * u + 5]), pack_h2(pv[g][8 * u + 6], pv[g][8 * u + 7])};
+    };
+
+    auto compute_pv = [&](const Tile &t) __attribute__((always_inline)) {
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+            constexpr int dummy = 0;
+            (void)dummy;
+            const int g = (16 * db) / GS;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const Op8 va = CD::unpack(&t.v[db][u * CD::WORDS]);
+                oacc[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va.h, (g == 0 ? pb[0][u] : pb[G - 1][u]).h, oacc[db], 0, 0, 0);
+            }
+        }
+    };
+
+    // one buffer with the halves skewed: V of a tile is requested before its scores, K of the
+    // next tile before its PV
+    if (my_tiles > 0) {
+        Tile buf;
+        load_k(buf);
+        load_queries();
+        for (int done = 0; done < my_tiles; ++done) {
+            load_v(buf);
+            compute_qk_softmax(buf);
+            load_k(buf);
+            compute_pv(buf);
+        }
+    } else {
+#pragma unroll
+        for (int g = 0; g < G; ++g) qsum[g] = 0.f;
+    }
+
+    // ---- wavefront partial -> LDS: lane (n, jj) holds out^T[d = 16 db + 4 jj + i][row n] ---------
+    l_part += __shfl_xor(l_part, 16);
+    l_part += __shfl_xor(l_part, 32);
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        bacc[g] += __shfl_xor(bacc[g], 16);
+        bacc[g] += __shfl_xor(bacc[g], 32);
+    }
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+        const int g = (16 * db) / GS;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            cbuf[wave][n][16 * db + 4 * jj + i] = oacc[db][i] * TWO24 + (g == 0 ? bacc[0] : bacc[G - 1]);
+    }
+    if (jj == 0) {
+        cbuf[wave][n][D] = m_run;
+        cbuf[wave][n][D + 1] = l_part;
+    }
+    __syncthreads();
+    // ---- merge the 4 wavefronts; a single span writes the output rows, several leave partials ---
+    if (nsplit == 1) {
+        for (int idx = threadIdx.x; idx < R * D; idx += WAVES * 64) {
+            const int i = idx / D, c = idx - i * D;
+            float mx = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, cbuf[w][i][D]);
+            float v = 0.f, l = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) {
+                const float mw = cbuf[w][i][D];
+                const float wgt = (mw == -INFINITY) ? 0.f : fast_exp2((mw - mx) * LOG2E);
+                v += wgt * cbuf[w][i][c];
+                l += wgt * cbuf[w][i][D + 1];
+            }
+            const int rep = i / a.L, lq = i - rep * a.L;
+            Elem<DT>::store(a.out, ((size_t)(b * a.Hq + hk * r + rep) * a.L + lq) * D + c, l > 0.f ? v / l : 0.f);
+        }
+        return;
+    }
+    float *part = a.workspace + ((size_t)bh * nsplit + split) * RR * (D + 2);
+    for (int idx = threadIdx.x; idx < RR * (D + 2); idx += WAVES * 64) {
+        const int i = idx / (D + 2), c = idx - i * (D + 2);
+        float mx = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, cbuf[w][i][D]);
+        float v;
+        if (c == D) {
+            v = mx;
+        } else {
+            v = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) {
+                const float mw = cbuf[w][i][D];
+                const float wgt = (mw == -INFINITY) ? 0.f : fast_exp2((mw - mx) * LOG2E);
+                v += wgt * cbuf[w][i][c];
+            }
+        }
+        part[idx] = v;
+    }
+}
+
+}  // namespace
+
+// Launches the 16-row kernel for the plan the caller made (spans as for the 4-row kernel with
+// 4 wavefronts); the caller merges the partials when nsplit > 1.
+hipError_t launch_attend_decode16(const AttendArgs &a, int tiles_total, int tiles_per_wg, int nsplit, hipStream_t s) {
+    const Store &st = a.st;
+    dim3 grid(nsplit, st.BH), block(WAVES * 64);
+    const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
+#define D16_M(BITS, D, GS, DT)                                                                                  \
+    do {                                                                                                        \
+        if (mm == 0) hipLaunchKernelGGL((decode16_kernel<BITS, D, GS, DT, 0>), grid, block, 0, s, a, tiles_total, tiles_per_wg, nsplit); \
+        else if (mm == 1) hipLaunchKernelGGL((decode16_kernel<BITS, D, GS, DT, 1>), grid, block, 0, s, a, tiles_total, tiles_per_wg, nsplit); \
+        else hipLaunchKernelGGL((decode16_kernel<BITS, D, GS, DT, 2>), grid, block, 0, s, a, tiles_total, tiles_per_wg, nsplit); \
+    } while (0)
+#define D16_DT(BITS, D, GS)                             \
+    do {                                                \
+        if (st.dtype == KVHIP_F16) D16_M(BITS, D, GS, 0); \
+        else D16_M(BITS, D, GS, 1);                     \
+    } while (0)
+#define D16_Q(BITS)                                     \
+    do {                                                \
+        if (st.Dk == 64) D16_DT(BITS, 64, 64);          \
+        else if (st.gs == 64) D16_DT(BITS, 128, 64);    \
+        else D16_DT(BITS, 128, 128);                    \
+    } while (0)
+    if (st.bits == 4) D16_Q(4);
+    else D16_Q(8);
+#undef D16_Q
+#undef D16_DT
+#undef D16_M
+    return hipGetLastError();
+}
+
+}  // namespace kvhip

@@ -180,6 +180,7 @@ size_t attend_prefill_workspace(const AttendArgs &a);
 // (out[D] unnormalised, running max, running sum), and write the normalised rows to a.out.
 hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s);
 hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s);
+hipError_t launch_attend_decode16(const AttendArgs &a, int tiles_total, int tiles_per_wg, int nsplit, hipStream_t s);
 hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, hipStream_t s);
 // Event bracket around the dominant kernel while profiling is enabled.
 void profile_enable(bool on);
