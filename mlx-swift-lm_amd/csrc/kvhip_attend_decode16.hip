@@ -47,14 +47,14 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
     return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
 }
-template <int DT> __device__ __forceinline__ void sb_pair(uint32_t raw, float &sc, float &bi) {
-    if (DT == 0) {
-        sc = (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
-        bi = (float)__builtin_bit_cast(_Float16, (uint16_t)(raw >> 16));
-    } else {
-        sc = __uint_as_float(raw << 16);
-        bi = __uint_as_float(raw & 0xffff0000u);
-    }
+// scale / bias of a raw (scale, bias) pair; for fp16 the widening folds into the consuming fma
+template <int DT> __device__ __forceinline__ float sb_scale(uint32_t raw) {
+    if (DT == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+    return __uint_as_float(raw << 16);
+}
+template <int DT> __device__ __forceinline__ float sb_bias(uint32_t raw) {
+    if (DT == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)(raw >> 16));
+    return __uint_as_float(raw & 0xffff0000u);
 }
 
 // 8 codes -> one 8-element operand.  4 bit: one word, element order (c0,c4,c1,c5,c2,c6,c3,c7),
@@ -218,7 +218,16 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     Op8 qb[G][SPG];
     float qsum[G];
     auto load_queries = [&]() __attribute__((always_inline)) {
-        const size_t qoff = ((size_t)(b * a.Hq + hk * r + row_rep) * a.L + row_l) * D;
+        // rows past R read row 0 (in bounds) and are zeroed: no branch around the loads, which
+        // are one 16-byte piece per contraction step
+        const int rep = row_ok ? row_rep : 0, lq = row_ok ? row_l : 0;
+        const uint16_t *qrow = reinterpret_cast<const uint16_t *>(a.q) + ((size_t)(b * a.Hq + hk * r + rep) * a.L + lq) * D;
+        u4 raw[G][SPG];
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int h = 0; h < SPG; ++h)
+                raw[g][h] = *reinterpret_cast<const u4 *>(qrow + GS * g + (GS / 4) * jj + 8 * h);
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             float part = 0.f;
@@ -227,9 +236,11 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 float qv[8];
 #pragma unroll
                 for (int p = 0; p < 8; ++p) {
-                    const int d = GS * g + (GS / 4) * jj + 8 * h + code_of<BITS>(p);
-                    float v = 0.f;
-                    if (row_ok) v = (float)(_Float16)round_dt<DT>(Elem<DT>::load(a.q, qoff + d) * a.scale);
+                    const int c = code_of<BITS>(p);  // element c of the 8 this step contracts
+                    const uint32_t w = raw[g][h][c >> 1];
+                    const uint16_t bits16 = (c & 1) ? (uint16_t)(w >> 16) : (uint16_t)w;
+                    const float e = DT == 0 ? (float)__builtin_bit_cast(_Float16, bits16) : __uint_as_float((uint32_t)bits16 << 16);
+                    const float v = row_ok ? (float)(_Float16)round_dt<DT>(e * a.scale) : 0.f;
                     part += v;
                     qv[p] = hi_of<BITS>(p) ? v * 0.0625f : v;
                 }
@@ -267,9 +278,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 }
             }
         // ---- scores of row n for this lane group's 16 tokens: local token 4 tb + i ---------------
-        const bool edge = MM == 2 || t.base < full_lo || t.base + (TILE - 1) > full_hi;  // wave-uniform
         float x[16];
-        float tmax = -INFINITY;
 #pragma unroll
         for (int tb = 0; tb < 4; ++tb)
 #pragma unroll
@@ -278,32 +287,37 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 float s_ = 0.f;
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
-                    float sc, bi;
-                    sb_pair<DT>(t.ksb[tl][g], sc, bi);
-                    s_ = __builtin_fmaf(bi, qsum[g], s_);
-                    s_ = __builtin_fmaf(sc * TWO24, sacc[tb][g][i], s_);
+                    const float s24 = sacc[tb][g][i] * TWO24;
+                    s_ = __builtin_fmaf(sb_bias<DT>(t.ksb[tl][g]), qsum[g], s_);
+                    s_ = __builtin_fmaf(sb_scale<DT>(t.ksb[tl][g]), s24, s_);
                 }
-                s_ = round_dt<DT>(s_);
-                if (edge) {
-                    const int row = t.base + 16 * jj + tl;  // slots are presented rows
-                    if (row < a.T) {
-                        if constexpr (MM == 1) {
-                            if (!sym_mask_keep(sym, row_l, row)) s_ = fill;
-                        } else if constexpr (MM == 2) {
-                            if (row_ok) {
-                                float add;
-                                const bool keep = mask_keep(a.mask, b, hk * r + row_rep, row_l, row, a.L, a.T, add);
-                                if (!keep) s_ = fill;
-                                else if (a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
-                            }
+                x[tl] = round_dt<DT>(s_);
+            }
+        if (MM == 2 || t.base < full_lo || t.base + (TILE - 1) > full_hi) {  // wave-uniform: edge tile
+#pragma unroll
+            for (int tl = 0; tl < 16; ++tl) {
+                const int row = t.base + 16 * jj + tl;  // slots are presented rows
+                float s_ = x[tl];
+                if (row < a.T) {
+                    if constexpr (MM == 1) {
+                        if (!sym_mask_keep(sym, row_l, row)) s_ = fill;
+                    } else if constexpr (MM == 2) {
+                        if (row_ok) {
+                            float add;
+                            const bool keep = mask_keep(a.mask, b, hk * r + row_rep, row_l, row, a.L, a.T, add);
+                            if (!keep) s_ = fill;
+                            else if (a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
                         }
-                    } else {
-                        s_ = -INFINITY;
                     }
+                } else {
+                    s_ = -INFINITY;
                 }
                 x[tl] = s_;
-                tmax = fmaxf(tmax, s_);
             }
+        }
+        float tmax = x[0];
+#pragma unroll
+        for (int tl = 1; tl < 16; ++tl) tmax = fmaxf(tmax, x[tl]);
         // raise the row maximum only when some lane's own maximum exceeds it (rare after the
         // first tiles); it stays equal in the four lanes of a row
         if (__any(tmax > m_run)) {
@@ -326,14 +340,12 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         for (int tl = 0; tl < 16; ++tl) {
             const float p = fast_exp2((x[tl] - mu) * LOG2E);  // exp2(-inf) = 0 for dead slots
             l_part += p;
+            // positions 2, 3, 6, 7 of a 4-bit operand meet high nibbles (x16)
+            const float ps = hi_of<BITS>(tl & 7) ? p * 0.0625f : p;
 #pragma unroll
             for (int g = 0; g < G; ++g) {
-                float sc, bi;
-                sb_pair<DT>(t.vsb[tl][g], sc, bi);
-                bacc[g] = __builtin_fmaf(p, bi, bacc[g]);
-                // step u = tl / 8 holds tokens 8 u .. 8 u + 7; positions 2, 3, 6, 7 of a 4-bit
-                // operand meet high nibbles
-                pv[g][tl] = p * (hi_of<BITS>(tl & 7) ? sc * 0.0625f : sc);
+                bacc[g] = __builtin_fmaf(p, sb_bias<DT>(t.vsb[tl][g]), bacc[g]);
+                pv[g][tl] = ps * sb_scale<DT>(t.vsb[tl][g]);
             }
         }
 #pragma unroll
