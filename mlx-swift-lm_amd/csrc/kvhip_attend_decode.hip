@@ -971,7 +971,7 @@ Plan plan_for(const AttendArgs &a) {
     p.nw = WAVES;
     if (a.mask.mode == KVHIP_MASK_WINDOW && (a.mask.left_pad || a.mask.lengths) && !getenv("KVHIP_DECODE_TILES")) {
         p.tiles_per_wg = 0;
-    } else if (a.st.bits != 0 && p.nsplit >= 2 && want <= 4 && p.rg <= 2 && a.mask.mode != KVHIP_MASK_ARRAY &&
+    } else if (a.st.bits != 0 && p.nsplit >= 2 && want <= 4 && p.rg == 1 && a.mask.mode != KVHIP_MASK_ARRAY &&
                !getenv("KVHIP_DECODE_TILES")) {
         // 128 pairs or more: workgroups of 8 wavefronts, one per CU -- the same wavefronts per CU
         // with half the spans.  With 256 pairs a workgroup takes its pair's whole sequence: the
@@ -1049,26 +1049,24 @@ bool attend_decode_supported(const AttendArgs &a) {
     return false;
 }
 
+// 5..16 rows per kv head of a quantized cache go to the 16x16x32 kernel
+// (kvhip_attend_decode16.hip), which always carries 16 rows: measured faster than the 4-row
+// broadcast contraction from 8 rows up (B16, 8 kv heads, 8192 tokens: 37 us against 43 us at
+// 8 rows, 36 us against 87 us at 16).
+static bool use_decode16(const AttendArgs &a, const Plan &p) { return a.st.bits != 0 && p.rg >= 2; }
+
 size_t attend_decode_workspace(const AttendArgs &a) {
     const Plan p = plan_for(a);
-    return (size_t)a.st.BH * p.nsplit * 4 * p.rg * (a.st.Dk + 2) * sizeof(float);
+    const int rows = use_decode16(a, p) ? 16 : 4 * p.rg;
+    return (size_t)a.st.BH * p.nsplit * rows * (a.st.Dk + 2) * sizeof(float);
 }
 
 hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
-    AttendArgs a = a_in;
+    const AttendArgs &a = a_in;
     const Plan p = plan_for(a);
     const Store &st = a.st;
     dim3 grid(p.nsplit, st.BH), block(WAVES * 64);  // the quantized kernel sets its own block size
     const int R = (a.Hq / a.Hkv) * a.L;
-    if (st.bits != 0 && p.rg == 4 && a.mask.mode == KVHIP_MASK_NONE) {
-        // the 16-row unmasked variants need more registers than the index-mask ones (which
-        // the compiler schedules tighter); an all-visible window is the same computation
-        a.mask.mode = KVHIP_MASK_WINDOW;
-        a.mask.offset = 1 << 30;
-        a.mask.window = 0;
-        a.mask.lengths = nullptr;
-        a.mask.left_pad = nullptr;
-    }
     const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
 #define DEC_K(BITS, D, GS, DT, RG, MM, NW)                                                                \
     hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG, MM, NW>), grid, dim3(NW * 64), 0, s, a,        \
@@ -1077,10 +1075,8 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
     do {                                                                                                  \
         profile_mark(s, true);                                                                            \
         if (p.nw == 2 * WAVES) {                                                                          \
-            if constexpr (RG <= 2) {                                                                      \
-                if (mm == 0) DEC_K(BITS, D, GS, DT, RG, 0, 2 * WAVES);                                    \
-                else DEC_K(BITS, D, GS, DT, RG, 1, 2 * WAVES);                                            \
-            }                                                                                             \
+            if (mm == 0) DEC_K(BITS, D, GS, DT, RG, 0, 2 * WAVES);                                        \
+            else DEC_K(BITS, D, GS, DT, RG, 1, 2 * WAVES);                                                \
         } else if (mm == 0) {                                                                             \
             DEC_K(BITS, D, GS, DT, RG, 0, WAVES);                                                         \
         } else if (mm == 1) {                                                                             \
@@ -1092,14 +1088,8 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
         if (p.nsplit > 1)                                                                                 \
             hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG); \
     } while (0)
-#define DEC_RG(BITS, D, GS, DT)                       \
-    do {                                              \
-        if (p.rg == 1) DEC(BITS, D, GS, DT, 1);       \
-        else if (p.rg == 2) DEC(BITS, D, GS, DT, 2);  \
-        else DEC(BITS, D, GS, DT, 4);                 \
-    } while (0)
-    if (st.bits != 0 && p.rg == 4 && !getenv("KVHIP_NO_DECODE16")) {
-        // 9..16 rows per kv head fill the 16x16x32 instruction: its own kernel
+#define DEC_RG(BITS, D, GS, DT) DEC(BITS, D, GS, DT, 1) /* more rows: the 16-row kernel above */
+    if (use_decode16(a_in, p)) {
         profile_mark(s, true);
         hipError_t e = launch_attend_decode16(a_in, p.tiles_total, p.tiles_per_wg, p.nsplit, s);
         profile_mark(s, false);
