@@ -34,6 +34,7 @@ constexpr int BN = 32;    // key slots per tile
 
 
 constexpr float LOG2E = 1.4426950408889634f;
+constexpr float RAISE = 5.545177444479562f;  // 8 ln 2
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ uint16_t h_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
@@ -352,8 +353,10 @@ prefill_kernel(AttendArgs a, int nsplit) {
                 }
             tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-            // rescale the accumulators only when some row's maximum rose (rare after the first tiles)
-            if (__any(tmax > m_run[qt])) {
+            // m_run is a reference value rather than the exact running maximum: it is raised (to the
+            // maximum seen) only when a score exceeds it by more than RAISE, so p stays below
+            // e^RAISE = 256 and the accumulators are rescaled a handful of times per query
+            if (__any(tmax > m_run[qt] + RAISE)) {
                 const float mn = fmaxf(m_run[qt], tmax);
                 const float alpha = (mn == -INFINITY) ? 1.f : exp2_fast((m_run[qt] - mn) * LOG2E);
                 m_run[qt] = mn;

@@ -34,6 +34,7 @@ union Op8 {
 
 constexpr int BN = 32;  // key slots per tile
 constexpr float LOG2E = 1.4426950408889634f;
+constexpr float RAISE = 8.f;  // log2 units
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ uint32_t rn_h2(float lo, float hi) {  // round to nearest even
@@ -258,9 +259,12 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         }
 
         // ---- online softmax per query column; P^T stays in place as the PV B operand ------
-        // Scores stay in the log2 domain: x = s * (scale * log2 e), p = exp2(x - m).  The running
-        // maximum m of a query is the same in the four lanes that share it; a tile raises it only
-        // if some lane's own maximum exceeds it, so the common tile needs no cross-lane traffic.
+        // Scores stay in the log2 domain: x = s * (scale * log2 e), p = exp2(x - m).  m is a reference
+        // value rather than the exact running maximum: it is the same in the four lanes that share a
+        // query and is raised (to the maximum seen) only when a score exceeds it by more than RAISE,
+        // so p stays below 2^RAISE (exact in fp16, whose relative precision does not depend on
+        // magnitude) and the accumulators are rescaled a handful of times per query, not on every
+        // tile that happens to hold a new maximum.
         Op8 pb[QT];
 #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
@@ -288,7 +292,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                     x[mt][i] = x_;
                     tmax = fmaxf(tmax, x_);
                 }
-            if (__any(tmax > m_run[qt])) {  // rare after the first tiles
+            if (__any(tmax > m_run[qt] + RAISE)) {  // a handful of times per query
                 tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
                 tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
                 const float mn = fmaxf(m_run[qt], tmax);
