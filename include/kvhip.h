@@ -171,6 +171,39 @@ kvhip_status kvhip_cache_update(kvhip_cache *cache, const void *keys, const void
                                 int32_t Hkv, int32_t L, int32_t Dk, int32_t Dv, int32_t dtype,
                                 void *stream);
 
+/* ---- rotary positions on the way in ----------------------------------------- */
+/*
+ * The rotary embedding a model applies to queries and keys immediately before the cache
+ * write (`applyRotaryPosition(rope, to:, offset: cache?.ropeOffset)`, Llama.swift:58-60,
+ * RoPEApplication.swift:62-74; the layers call `MLXFast.RoPE(x, dimensions:, traditional:,
+ * base:, scale:, offset:, freqs:)`, RoPEUtils.swift:139-156, SuScaledRoPE.swift:49-70).
+ * The first `dims` elements of each head rotate: pairs (2i, 2i+1) when `traditional`, else
+ * (i, i + dims/2); pair i of the row at position p turns by p * scale * base^(-2i/dims), or by
+ * p * scale / freqs[i] when `freqs` (a device array of dims/2 floats) is given.  Angles and
+ * products are float32, the result is rounded once to the array's dtype.
+ */
+typedef struct kvhip_rope {
+    int32_t dims;
+    int32_t traditional;
+    float base;
+    float scale;
+    const float *freqs; /* device, or NULL */
+} kvhip_rope;
+
+/* out = rope(x) for x [B,H,L,D]; row l sits at position offset + l, or batch_offsets[b] + l
+ * when batch_offsets (device, [B]: `RoPEOffset.batch`, RoPEApplication.swift:13-23) is given.
+ * out may be x. */
+kvhip_status kvhip_rope_apply(const kvhip_rope *rope, const void *x, void *out, int32_t B, int32_t H,
+                              int32_t L, int32_t D, int32_t dtype, int64_t offset,
+                              const int32_t *batch_offsets, void *stream);
+
+/* `kvhip_cache_update` with the keys rotated inside the append / quantize-on-append kernel
+ * (no rotated copy of the keys is written).  Positions start at the cache's `ropeOffset`:
+ * its offset before this write (plus the staged rows of an open round), or batch_offsets[b]. */
+kvhip_status kvhip_cache_update_rope(kvhip_cache *cache, const kvhip_rope *rope, const int32_t *batch_offsets,
+                                     const void *keys, const void *values, int32_t B, int32_t Hkv,
+                                     int32_t L, int32_t Dk, int32_t Dv, int32_t dtype, void *stream);
+
 /* The arrays the last `update` returned: dst_keys [B,Hkv,P,Dk], dst_values
  * [B,Hkv,P,Dv], P = kvhip_cache_presented_length.  Not for quantized caches. */
 kvhip_status kvhip_cache_fetch(const kvhip_cache *cache, void *dst_keys, void *dst_values, void *stream);

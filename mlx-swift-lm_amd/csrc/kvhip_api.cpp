@@ -74,6 +74,7 @@ struct kvhip_cache {
     int64_t presented_live = 0;       // `presented` of the live ring when the round opened
     void *stage_tmp_k = nullptr, *stage_tmp_v = nullptr;  // dense copy of the rows a commit keeps
     size_t stage_tmp_rows = 0;
+    const RopeDev *rope = nullptr;  // set for the duration of one update_rope call
     // scratch for attention
     float *ws = nullptr;
     size_t ws_bytes = 0;
@@ -294,9 +295,9 @@ kvhip_status write_rows(kvhip_cache *c, const void *keys, const void *values, in
     const RunList rl = runs_of(slots, n);
     for (size_t i = 0; i < rl.size(); ++i) {
         if (c->kind == KVHIP_KIND_QUANTIZED)
-            KV_HIP(launch_append_quant(c->st, keys, values, L, src0 + rl.row0[i], rl.phys0[i], rl.len[i], stream));
+            KV_HIP(launch_append_quant(c->st, keys, values, L, src0 + rl.row0[i], rl.phys0[i], rl.len[i], stream, c->rope));
         else
-            KV_HIP(launch_append_fp(c->st, keys, values, L, src0 + rl.row0[i], rl.phys0[i], rl.len[i], stream));
+            KV_HIP(launch_append_fp(c->st, keys, values, L, src0 + rl.row0[i], rl.phys0[i], rl.len[i], stream, c->rope));
     }
     return KVHIP_OK;
 }
@@ -352,8 +353,8 @@ kvhip_status update_simple(kvhip_cache *c, const void *k, const void *v, int L, 
     }
     KV_TRY(ensure_slots(c, prev + L, stream));
     c->offset += L;
-    if (c->kind == KVHIP_KIND_QUANTIZED) KV_HIP(launch_append_quant(c->st, k, v, L, 0, (int)prev, L, stream));
-    else KV_HIP(launch_append_fp(c->st, k, v, L, 0, (int)prev, L, stream));
+    if (c->kind == KVHIP_KIND_QUANTIZED) KV_HIP(launch_append_quant(c->st, k, v, L, 0, (int)prev, L, stream, c->rope));
+    else KV_HIP(launch_append_fp(c->st, k, v, L, 0, (int)prev, L, stream, c->rope));
     c->presented = c->offset;
     return KVHIP_OK;
 }
@@ -380,7 +381,7 @@ kvhip_status update_rotating(kvhip_cache *c, const void *k, const void *v, int L
             return fail(KVHIP_ERR_STATE, "RotatingKVCache write cursor lies outside its buffer");
         KV_TRY(ring_compact_if_needed(c, stream));
         const int32_t slot = c->rows[(size_t)c->idx];
-        KV_HIP(launch_append_fp(c->st, k, v, 1, 0, slot, 1, stream));
+        KV_HIP(launch_append_fp(c->st, k, v, 1, 0, slot, 1, stream, c->rope));
         c->offset += 1;
         c->idx += 1;
         c->presented = c->offset < M ? c->offset : c->ref_len;
@@ -627,6 +628,53 @@ kvhip_status kvhip_cache_update(kvhip_cache *c, const void *keys, const void *va
     if (c->staging) return stage_update(c, keys, values, L, S(stream));
     if (c->kind == KVHIP_KIND_ROTATING) return update_rotating(c, keys, values, L, S(stream));
     return update_simple(c, keys, values, L, S(stream));
+}
+
+namespace {
+// host description -> device description; `H` heads per batch row of the rotated array
+kvhip_status rope_dev(const kvhip_rope *rope, int D, int H, int64_t pos0, const int32_t *batch_pos, RopeDev &r) {
+    if (!rope) return fail(KVHIP_ERR_INVALID_ARG, "null rope description");
+    if (rope->dims <= 0 || (rope->dims & 1) || rope->dims > D)
+        return fail(KVHIP_ERR_INVALID_ARG, "rope dims must be even and at most the head dim");
+    if (!rope->freqs && !(rope->base > 0.f)) return fail(KVHIP_ERR_INVALID_ARG, "rope base must be positive");
+    r.dims = rope->dims;
+    r.traditional = rope->traditional ? 1 : 0;
+    r.scale = rope->scale;
+    r.log_base_over_half = rope->freqs ? 0. : log((double)rope->base) / (double)(rope->dims / 2);
+    r.freqs = rope->freqs;
+    r.pos0 = (int32_t)pos0;
+    r.batch_pos = batch_pos;
+    r.H = H;
+    return KVHIP_OK;
+}
+}  // namespace
+
+kvhip_status kvhip_rope_apply(const kvhip_rope *rope, const void *x, void *out, int32_t B, int32_t H,
+                              int32_t L, int32_t D, int32_t dtype, int64_t offset,
+                              const int32_t *batch_offsets, void *stream) {
+    if (!x || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (B <= 0 || H <= 0 || L <= 0 || D <= 0 || D > 1024) return fail(KVHIP_ERR_INVALID_ARG, "shape out of range");
+    if (dtype != KVHIP_F16 && dtype != KVHIP_BF16 && dtype != KVHIP_F32)
+        return fail(KVHIP_ERR_INVALID_ARG, "rope needs a floating-point dtype");
+    RopeDev r;
+    KV_TRY(rope_dev(rope, D, H, offset, batch_offsets, r));
+    KV_HIP(launch_rope_apply(r, x, out, B, H, L, D, dtype, S(stream)));
+    return KVHIP_OK;
+}
+
+kvhip_status kvhip_cache_update_rope(kvhip_cache *c, const kvhip_rope *rope, const int32_t *batch_offsets,
+                                     const void *keys, const void *values, int32_t B, int32_t Hkv, int32_t L,
+                                     int32_t Dk, int32_t Dv, int32_t dtype, void *stream) {
+    if (!c) return fail(KVHIP_ERR_INVALID_ARG, "null cache");
+    RopeDev r;
+    // `ropeOffset` is read before the write (Llama.swift:58-62); the staged wrapper's offset
+    // counts its staged rows (RotatingStagedKVCache.swift:33-37)
+    const int64_t pos0 = c->offset + (c->staging ? (int64_t)c->staged.size() : 0);
+    KV_TRY(rope_dev(rope, Dk, Hkv, pos0, batch_offsets, r));
+    c->rope = &r;
+    const kvhip_status st = kvhip_cache_update(c, keys, values, B, Hkv, L, Dk, Dv, dtype, stream);
+    c->rope = nullptr;
+    return st;
 }
 
 kvhip_status kvhip_cache_fetch(const kvhip_cache *c, void *dk, void *dv, void *stream) {

@@ -128,12 +128,29 @@ __device__ __forceinline__ int row_to_slot(const Runs &r, int row) {
 }
 #endif
 
+// Rotary position embedding applied to rows on their way into a kernel: row l of a
+// [B, H, L, D] array sits at position pos0 + l (or batch_pos[b] + l).
+struct RopeDev {
+    int32_t dims = 0;          // leading head-dim elements that rotate (even); 0 = off
+    int32_t traditional = 0;   // 1: pairs (2i, 2i+1); 0: pairs (i, i + dims/2)
+    float scale = 1.f;         // position scale
+    double log_base_over_half = 0.;  // log(base) / (dims/2): pair i turns by position * exp(-i * this)
+    const float *freqs = nullptr;    // optional [dims/2]: pair i turns by position / freqs[i]
+    int32_t pos0 = 0;
+    const int32_t *batch_pos = nullptr;  // optional [B] (device)
+    int32_t H = 1;             // heads per batch row of the array being rotated
+};
+
 // ---- kernel launchers (defined in the .hip files) ---------------------------
-// New rows src[l] for l in [src0, src0+n) go to physical slots [slot0, slot0+n).
+// New rows src[l] for l in [src0, src0+n) go to physical slots [slot0, slot0+n); with `rope`
+// the K rows are rotated (and rounded to the cache dtype) on the way in.
 hipError_t launch_append_fp(const Store &st, const void *keys, const void *values, int L, int src0,
-                            int slot0, int n, hipStream_t s);
+                            int slot0, int n, hipStream_t s, const RopeDev *rope = nullptr);
 hipError_t launch_append_quant(const Store &st, const void *keys, const void *values, int L, int src0,
-                               int slot0, int n, hipStream_t s);
+                               int slot0, int n, hipStream_t s, const RopeDev *rope = nullptr);
+// out = rope(x) for x [B, H, L, D] of `dtype` (out may alias x)
+hipError_t launch_rope_apply(const RopeDev &rope, const void *x, void *out, int B, int H, int L, int D,
+                             int dtype, hipStream_t s);
 // Copy rows [row_begin, row_begin+count) of `runs` out to dense [BH, dst_rows, D] arrays whose
 // row 0 corresponds to row dst_row0 of `runs`.  Either destination may be NULL.
 hipError_t launch_export_fp(const Store &st, const Runs &runs, int row_begin, int count, int dst_row0,

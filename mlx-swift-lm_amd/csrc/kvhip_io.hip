@@ -7,6 +7,55 @@ namespace kvhip {
 
 namespace {
 
+// Element d of a row at position `pos` after the rotary embedding, rounded to the row's dtype
+// (what the reference hands to the cache: `applyRotaryPosition` runs before `update`,
+// Llama.swift:58-62).  The angle is the float32 product of position * scale and the inverse
+// frequency exp(-i * log(base) / half), or 1 / freqs[i].
+template <int DT>
+__device__ __forceinline__ float rope_elem(const RopeDev &r, const void *row, int d, int pos) {
+    const float x = Elem<DT>::load(row, d);
+    if (d >= r.dims) return x;
+    const int half = r.dims >> 1;
+    int i, partner;
+    bool first;
+    if (r.traditional) {
+        i = d >> 1;
+        partner = d ^ 1;
+        first = (d & 1) == 0;
+    } else {
+        first = d < half;
+        i = first ? d : d - half;
+        partner = first ? d + half : d - half;
+    }
+    // the inverse frequency is formed in double and rounded once, so that it does not depend on
+    // one exp implementation's last float32 bit (a position of 10^5 turns one such bit into 10^-2 rad)
+    const float inv = r.freqs ? 1.0f / r.freqs[i] : (float)exp(-(double)i * r.log_base_over_half);
+    const float theta = ((float)pos * r.scale) * inv;
+    float sn, cs;
+    sincosf(theta, &sn, &cs);
+    const float y = Elem<DT>::load(row, partner);
+    const float v = first ? x * cs - y * sn : y * sn + x * cs;
+    return round_dt<DT>(v);
+}
+__device__ __forceinline__ int rope_pos(const RopeDev &r, int bh, int l) {
+    return (r.batch_pos ? r.batch_pos[bh / r.H] : r.pos0) + l;
+}
+
+// grid (L, B*H): one row per workgroup
+template <int DT>
+__global__ void rope_apply_kernel(RopeDev r, const char *x, char *out, int L, int D) {
+    const int bh = blockIdx.y, l = blockIdx.x;
+    const size_t off = ((size_t)bh * L + l) * D * (DT == 2 ? 4 : 2);
+    const int pos = rope_pos(r, bh, l);
+    // every element is read (with its partner) before any is written: out may alias x
+    float v[4];
+    int cnt = 0;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) v[cnt++] = rope_elem<DT>(r, x + off, d, pos);
+    __syncthreads();
+    cnt = 0;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) Elem<DT>::store(out + off, d, v[cnt++]);
+}
+
 // One wavefront quantizes one row of D elements.  Optional outputs:
 //   k_words   packed codes in MLX order (D*BITS/32 words)
 //   code_out  one byte per element (for the transposed V assembly)
@@ -15,7 +64,8 @@ namespace {
 template <int DT, int BITS>
 __device__ __forceinline__ void quantize_row_wave(const void *src, int D, int gs, int lane,
                                                   uint32_t *k_words, uint8_t *code_out, void *sb_row,
-                                                  void *scales, void *biases) {
+                                                  void *scales, void *biases, const RopeDev *rope = nullptr,
+                                                  int pos = 0) {
     const float nb = (float)((1 << BITS) - 1);
     const int K = gs > 64 ? gs / 64 : 1;
     const int width = gs < 64 ? gs : 64;
@@ -26,7 +76,7 @@ __device__ __forceinline__ void quantize_row_wave(const void *src, int D, int gs
         for (int k = 0; k < K; ++k) {
             const int d = base + k * 64 + lane;
             if (d < D) {
-                w[k] = Elem<DT>::load(src, d);
+                w[k] = rope ? rope_elem<DT>(*rope, src, d, pos) : Elem<DT>::load(src, d);
                 mn = fminf(mn, w[k]);
                 mx = fmaxf(mx, w[k]);
             }
@@ -62,7 +112,7 @@ __device__ __forceinline__ void quantize_row_wave(const void *src, int D, int gs
 // grid (rows, BH): K rows copied in natural order, V elements scattered into octets.
 template <int ES>
 __global__ void append_fp_kernel(Store st, const char *keys, const char *values, int L, int src0,
-                                 int slot0) {
+                                 int slot0, RopeDev rope) {
     const int bh = blockIdx.y;
     const int i = blockIdx.x;
     const int slot = slot0 + i;
@@ -70,7 +120,16 @@ __global__ void append_fp_kernel(Store st, const char *keys, const char *values,
     using E = typename std::conditional<ES == 2, uint16_t, uint32_t>::type;
     const E *ks = reinterpret_cast<const E *>(keys) + ((size_t)bh * L + l) * st.Dk;
     E *kd = reinterpret_cast<E *>(const_cast<char *>(k_row_ptr(st, bh, slot)));
-    for (int d = threadIdx.x; d < st.Dk; d += blockDim.x) kd[d] = ks[d];
+    if (rope.dims > 0) {
+        const int pos = rope_pos(rope, bh, l);
+        for (int d = threadIdx.x; d < st.Dk; d += blockDim.x) {
+            if (ES == 4) Elem<2>::store(kd, d, rope_elem<2>(rope, ks, d, pos));
+            else if (st.dtype == KVHIP_F16) Elem<0>::store(kd, d, rope_elem<0>(rope, ks, d, pos));
+            else Elem<1>::store(kd, d, rope_elem<1>(rope, ks, d, pos));
+        }
+    } else {
+        for (int d = threadIdx.x; d < st.Dk; d += blockDim.x) kd[d] = ks[d];
+    }
     const E *vs = reinterpret_cast<const E *>(values) + ((size_t)bh * L + l) * st.Dv;
     char *vc = const_cast<char *>(v_cell_ptr(st, bh, slot));
     const int t = slot & (TILE - 1);
@@ -83,7 +142,8 @@ __global__ void append_fp_kernel(Store st, const char *keys, const char *values,
 // tile rows, touching only the token positions this append writes.
 template <int DT, int BITS>
 __global__ void __launch_bounds__(256)
-append_quant_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, int n) {
+append_quant_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, int n,
+                    RopeDev rope) {
     extern __shared__ uint8_t vcodes[];  // [64][Dv]
     const int bh = blockIdx.y;
     const int tile = (slot0 >> 6) + blockIdx.x;
@@ -113,7 +173,8 @@ append_quant_kernel(Store st, const char *keys, const char *values, int L, int s
             const char *krow = keys + ((size_t)bh * L + l) * st.Dk * st.es;
             quantize_row_wave<DT, BITS>(krow, st.Dk, st.gs, lane,
                                         reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot))),
-                                        nullptr, const_cast<char *>(ksb_row_ptr(st, bh, slot)), nullptr, nullptr);
+                                        nullptr, const_cast<char *>(ksb_row_ptr(st, bh, slot)), nullptr, nullptr,
+                                        rope.dims > 0 ? &rope : nullptr, rope_pos(rope, bh, l));
         } else {
             const char *vrow = values + ((size_t)bh * L + l) * st.Dv * st.es;
             quantize_row_wave<DT, BITS>(vrow, st.Dv, st.gs, lane, nullptr, vcodes + (slot & (TILE - 1)) * st.Dv,
@@ -337,25 +398,37 @@ __global__ void mask_materialize_kernel(kvhip_mask_plan_t p, uint8_t *dst) {
     } while (0)
 
 hipError_t launch_append_fp(const Store &st, const void *keys, const void *values, int L, int src0,
-                            int slot0, int n, hipStream_t s) {
+                            int slot0, int n, hipStream_t s, const RopeDev *rope) {
     if (n <= 0) return hipSuccess;
     dim3 grid(n, st.BH), block(128);
+    const RopeDev r = rope ? *rope : RopeDev();
     if (st.es == 2)
-        hipLaunchKernelGGL(append_fp_kernel<2>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, src0, slot0);
+        hipLaunchKernelGGL(append_fp_kernel<2>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, src0, slot0, r);
     else
-        hipLaunchKernelGGL(append_fp_kernel<4>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, src0, slot0);
+        hipLaunchKernelGGL(append_fp_kernel<4>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, src0, slot0, r);
+    return hipGetLastError();
+}
+
+hipError_t launch_rope_apply(const RopeDev &rope, const void *x, void *out, int B, int H, int L, int D,
+                             int dtype, hipStream_t s) {
+    if ((size_t)B * H * L == 0) return hipSuccess;
+    dim3 grid(L, B * H), block(D <= 64 ? 64 : (D <= 128 ? 128 : 256));  // at most 4 elements per thread up to D = 1024
+    if (dtype == KVHIP_F16) hipLaunchKernelGGL(rope_apply_kernel<0>, grid, block, 0, s, rope, (const char *)x, (char *)out, L, D);
+    else if (dtype == KVHIP_BF16) hipLaunchKernelGGL(rope_apply_kernel<1>, grid, block, 0, s, rope, (const char *)x, (char *)out, L, D);
+    else hipLaunchKernelGGL(rope_apply_kernel<2>, grid, block, 0, s, rope, (const char *)x, (char *)out, L, D);
     return hipGetLastError();
 }
 
 hipError_t launch_append_quant(const Store &st, const void *keys, const void *values, int L, int src0,
-                               int slot0, int n, hipStream_t s) {
+                               int slot0, int n, hipStream_t s, const RopeDev *rope) {
     if (n <= 0) return hipSuccess;
+    const RopeDev r = rope ? *rope : RopeDev();
     const int ntile = ((slot0 + n - 1) >> 6) - (slot0 >> 6) + 1;
     dim3 grid(ntile, st.BH), block(256);
     const size_t lds = (size_t)TILE * st.Dv;
 #define CALL(DT, BITS)                                                                           \
     hipLaunchKernelGGL((append_quant_kernel<DT, BITS>), grid, block, lds, s, st, (const char *)keys, \
-                       (const char *)values, L, src0, slot0, n)
+                       (const char *)values, L, src0, slot0, n, r)
     KV_DISPATCH_DT_BITS(st.dtype, st.bits, CALL);
 #undef CALL
     return hipGetLastError();

@@ -35,6 +35,11 @@ class Mask(C.Structure):
                 ("lengths", C.c_void_p), ("left_pad", C.c_void_p)]
 
 
+class Rope(C.Structure):
+    _fields_ = [("dims", C.c_int32), ("traditional", C.c_int32), ("base", C.c_float), ("scale", C.c_float),
+                ("freqs", C.c_void_p)]
+
+
 class MaskPlan(C.Structure):
     _fields_ = [("mode", C.c_int32), ("rows", C.c_int32), ("cols", C.c_int32),
                 ("offset", C.c_int32), ("window", C.c_int32), ("rolled", C.c_int32),
@@ -67,6 +72,8 @@ SIGNATURES = {
     "kvhip_cache_trim": (_I64, [_P, _I64]),
     "kvhip_cache_set_offset": (_I32, [_P, _I64]),
     "kvhip_cache_update": (_I32, [_P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I32, _P]),
+    "kvhip_rope_apply": (_I32, [C.POINTER(Rope), _P, _P, _I32, _I32, _I32, _I32, _I32, _I64, _P, _P]),
+    "kvhip_cache_update_rope": (_I32, [_P, C.POINTER(Rope), _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I32, _P]),
     "kvhip_cache_fetch": (_I32, [_P, _P, _P, _P]),
     "kvhip_cache_attend": (_I32, [_P, _P, _I32, _I32, _I32, _I32, _F, C.POINTER(Mask), _P, _P]),
     "kvhip_cache_update_attend": (_I32, [_P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F,

@@ -115,6 +115,11 @@ class _Cache:
         L.check(self._lib.kvhip_cache_set_offset(self._h, int(v)))
 
     @property
+    def rope_offset(self):
+        """`ropeOffset` (KVCache.swift:190): `.scalar(offset)`, read before the write."""
+        return self.offset
+
+    @property
     def max_size(self):
         v = self._lib.kvhip_cache_max_size(self._h)
         return None if v < 0 else v
@@ -151,6 +156,21 @@ class _Cache:
         L.check(self._lib.kvhip_cache_update(self._h, _ptr(keys), _ptr(values), B, H, Lq, Dk,
                                              values.shape[3], _DT[keys.dtype], _stream()))
         self._note_shape(keys, values)
+
+    def update_rope(self, rope, keys, values, batch_offsets=None):
+        """`update` / `updateQuantized` of keys that still need their rotary embedding: the
+        rotation runs inside the append kernel, at positions starting from this cache's
+        `ropeOffset` (its offset before the write) or from `batch_offsets` [B] (int32)."""
+        assert keys.is_cuda and values.is_cuda and keys.dtype == values.dtype
+        keys, values = keys.contiguous(), values.contiguous()
+        B, H, Lq, Dk = keys.shape
+        r, keep = rope.to_c()
+        bo = None if batch_offsets is None else batch_offsets.to(device="cuda", dtype=torch.int32).contiguous()
+        L.check(self._lib.kvhip_cache_update_rope(self._h, C.byref(r), _ptr(bo) if bo is not None else None,
+                                                  _ptr(keys), _ptr(values), B, H, Lq, Dk, values.shape[3],
+                                                  _DT[keys.dtype], _stream()))
+        self._note_shape(keys, values)
+        del keep
 
     def attend(self, queries, scale, mask=None):
         """Attention of `queries` [B,Hq,L,D] over what the cache presents."""

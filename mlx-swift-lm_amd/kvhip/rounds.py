@@ -48,12 +48,20 @@ class RotatingStagedKVCache:
         return self.live.offset + self.staged_count
 
     @property
+    def rope_offset(self):
+        return self.offset
+
+    @property
     def max_size(self):
         return self.live.max_size
 
     @property
     def presented_length(self):
         return self.live.presented_length
+
+    def update_rope(self, rope, keys, values, batch_offsets=None):
+        self._require_open()
+        return self.live.update_rope(rope, keys, values, batch_offsets)
 
     def update(self, keys, values, fetch=True):
         """Stages the rows; returns trailing window ++ staged (:41-47, :78-91)."""

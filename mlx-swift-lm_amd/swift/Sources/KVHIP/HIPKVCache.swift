@@ -130,6 +130,26 @@ public class HIPKVCache {
         return out
     }
 
+    /// An attention layer's `applyRotaryPosition(rope, to: keys, offset: cache.ropeOffset)` followed by
+    /// the cache write (Llama.swift:58-62), with the rotation inside the append kernel.  `rope` carries
+    /// the layer's `dimensions`, `traditional`, `base`, `scale` and optional `freqs`.
+    public func updateRotating<A: HIPArray>(rope: kvhip_rope, keys: A, values: A, batchOffsets: UnsafePointer<Int32>? = nil) {
+        var r = rope
+        let k = keys.shape, v = values.shape
+        must(kvhip_cache_update_rope(handle, &r, batchOffsets, keys.devicePointer, values.devicePointer, Int32(k[0]),
+                                     Int32(k[1]), Int32(k[2]), Int32(k[3]), Int32(v[3]), keys.kvhipDType, stream))
+    }
+
+    /// `applyRotaryPosition(rope, to: queries, offset:)` (RoPEApplication.swift:62-74) on the device.
+    public func rotate<A: HIPArray>(rope: kvhip_rope, _ x: A, offset: Int) -> A {
+        var r = rope
+        let s = x.shape
+        let out = A.empty(s, dtype: x.kvhipDType)
+        must(kvhip_rope_apply(&r, x.devicePointer, out.devicePointer, Int32(s[0]), Int32(s[1]), Int32(s[2]),
+                              Int32(s[3]), x.kvhipDType, Int64(offset), nil, stream))
+        return out
+    }
+
     func appendOnly<A: HIPArray>(keys: A, values: A) {
         let k = keys.shape, v = values.shape
         must(kvhip_cache_update(handle, keys.devicePointer, values.devicePointer, Int32(k[0]), Int32(k[1]),
