@@ -83,12 +83,23 @@ def main():
     total = ctx + args.warmup + args.steps + 8
     cache.reserve(nb, HKV, D, D, torch.float16, total)
     chunk = 2048
+    pf_events = []
     for t0 in range(0, ctx, chunk):
         n = min(chunk, ctx - t0)
         k = (torch.randn(nb, HKV, n, D, generator=g, device=dev) * ch).to(torch.float16)
         v = (torch.randn(nb, HKV, n, D, generator=g, device=dev) * ch).to(torch.float16)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
         cache.update_quantized(k, v, fetch=False)
+        e1.record()
+        pf_events.append((e0, e1, n))
     del k, v
+    torch.cuda.synchronize()
+    # quantize-on-append of the prompt: reads the new fp16 rows, writes codes + scale/bias pairs
+    # (the median chunk: the first one also loads the code object)
+    pf_ms = sorted(a.elapsed_time(b) for a, b, _ in pf_events)[len(pf_events) // 2]
+    pf_rows = sorted(n for _, _, n in pf_events)[len(pf_events) // 2]
+    pf_bytes = nb * HKV * pf_rows * (2 * D * 2 + ROW_BYTES)
     nsteps = args.warmup + args.steps
     qs = torch.randn(nsteps, nb, HQ, 1, D, generator=g, device=dev).to(torch.float16)
     ks = (torch.randn(nsteps, nb, HKV, 1, D, generator=g, device=dev) * ch).to(torch.float16)
@@ -166,6 +177,8 @@ def main():
                                f"batch {nb}, context {ctx}+, quantize-on-append + fused dequant-SDPA, one layer",
                    "batch": nb, "context_first": int(t_first), "context_last": int(t_last)},
         "roofline": roofline, "cpu_baseline": cpu, "parity": parity,
+        "prefill_append": {"rows": pf_rows, "ms": round(pf_ms, 3), "GB/s": round(pf_bytes / (pf_ms * 1e-3) / 1e9, 1),
+                           "note": "quantize-on-append of one prompt chunk (median of the 2048-row chunks), HIP events; bytes = fp16 rows read + codes and scale/bias pairs written"},
         "hbm_gbs_whole_step": round(alg_bytes / (ms_per_step * 1e-3) / 1e9, 1),
     }
     print(json.dumps(line))

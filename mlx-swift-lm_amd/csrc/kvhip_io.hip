@@ -203,6 +203,201 @@ append_quant_kernel(Store st, const char *keys, const char *values, int L, int s
     }
 }
 
+// ---- whole 64-token tiles (prompt-sized appends) -----------------------------------------
+// The per-row kernels above fetch one element per lane and wait for every row in turn; for
+// many rows that is bound by load latency.  Here a workgroup takes one whole tile of one
+// (batch, kv-head): every thread first requests all of its 16-byte chunks of the 64 new K and
+// V rows, then quantizes / copies eight elements at a time.  Values, rounding and the
+// rotation are those of the per-row kernels (the same element functions).
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+
+template <int DT>
+__device__ __forceinline__ void unpack8(const u4v &raw, const void *row, int d0, const RopeDev &rope, int pos,
+                                        float (&w)[8]) {
+    if (rope.dims > 0 && d0 < rope.dims) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) w[j] = rope_elem<DT>(rope, row, d0 + j, pos);
+        return;
+    }
+    const uint32_t u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (DT == 0) {
+            w[2 * j] = __half2float(__ushort_as_half((unsigned short)(u[j] & 0xffffu)));
+            w[2 * j + 1] = __half2float(__ushort_as_half((unsigned short)(u[j] >> 16)));
+        } else {
+            w[2 * j] = __uint_as_float(u[j] << 16);
+            w[2 * j + 1] = __uint_as_float(u[j] & 0xffff0000u);
+        }
+    }
+}
+
+// Quantize the eight elements a thread holds; `gl` adjacent lanes share a group.
+template <int BITS>
+__device__ __forceinline__ void quantize8(const float (&w)[8], int gl, float &scale, float &bias, uint32_t (&code)[8]) {
+    const float nb = (float)((1 << BITS) - 1);
+    float mn = w[0], mx = w[0];
+#pragma unroll
+    for (int j = 1; j < 8; ++j) {
+        mn = fminf(mn, w[j]);
+        mx = fmaxf(mx, w[j]);
+    }
+    group_minmax(mn, mx, gl);
+    affine_params(mn, mx, nb, scale, bias);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) code[j] = affine_code(w[j], scale, bias, nb);
+}
+
+// grid (whole tiles, BH), 256 threads; slot0 is a multiple of 64; 16-bit dtypes, Dk == Dv == 32 NC
+template <int DT, int BITS, int NC>
+__global__ void __launch_bounds__(256)
+append_quant_tile_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, RopeDev rope) {
+    constexpr int D = 32 * NC;
+    constexpr int TPR = D / 8;   // threads per row
+    constexpr int VP = D + 8;    // byte pitch of a token's V codes in LDS
+    __shared__ __attribute__((aligned(8))) uint8_t vcodes[TILE * VP];
+    const int bh = blockIdx.y;
+    const int slot_t = slot0 + blockIdx.x * TILE;
+    const int l_t = src0 + blockIdx.x * TILE;
+    const int gl = st.gs / 8;
+    const char *kbase = keys + ((size_t)bh * L + l_t) * D * 2;
+    const char *vbase = values + ((size_t)bh * L + l_t) * D * 2;
+    u4v kraw[NC], vraw[NC];
+#pragma unroll
+    for (int e = 0; e < NC; ++e) {
+        const int c = e * 256 + threadIdx.x;
+        kraw[e] = *reinterpret_cast<const u4v *>(kbase + (size_t)c * 16);
+        vraw[e] = *reinterpret_cast<const u4v *>(vbase + (size_t)c * 16);
+    }
+#pragma unroll
+    for (int e = 0; e < NC; ++e) {
+        const int c = e * 256 + threadIdx.x;
+        const int r = c / TPR, d0 = (c - r * TPR) * 8;
+        const int slot = slot_t + r;
+        float w[8], scale, bias;
+        uint32_t code[8];
+        // ---- K: packed words in natural order ------------------------------------------------
+        unpack8<DT>(kraw[e], kbase + (size_t)r * D * 2, d0, rope, rope_pos(rope, bh, l_t + r), w);
+        quantize8<BITS>(w, gl, scale, bias, code);
+        uint32_t *kw = reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot)));
+        if (BITS == 4) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) word |= code[j] << (4 * j);
+            kw[d0 / 8] = word;
+        } else {
+            const uint32_t lo = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
+            const uint32_t hi = code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24);
+            *reinterpret_cast<uint2 *>(kw + d0 / 4) = make_uint2(lo, hi);
+        }
+        if ((d0 % st.gs) == 0) {
+            char *sb = const_cast<char *>(ksb_row_ptr(st, bh, slot));
+            Elem<DT>::store(sb, 2 * (d0 / st.gs), scale);
+            Elem<DT>::store(sb, 2 * (d0 / st.gs) + 1, bias);
+        }
+        // ---- V: codes as bytes, transposed below ------------------------------------------------
+        unpack8<DT>(vraw[e], vbase + (size_t)r * D * 2, d0, RopeDev(), 0, w);
+        quantize8<BITS>(w, gl, scale, bias, code);
+        *reinterpret_cast<uint2 *>(&vcodes[r * VP + d0]) =
+            make_uint2(code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24),
+                       code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24));
+        if ((d0 % st.gs) == 0) {
+            char *sb = const_cast<char *>(vsb_row_ptr(st, bh, slot));
+            Elem<DT>::store(sb, 2 * (d0 / st.gs), scale);
+            Elem<DT>::store(sb, 2 * (d0 / st.gs) + 1, bias);
+        }
+    }
+    __syncthreads();
+    // each thread assembles 16 bytes (4 words) of one transposed row; consecutive threads
+    // continue the same row, so the tile rows are written contiguously
+    constexpr int TPW = 32 / BITS;        // tokens per word
+    constexpr int CPR = TILE / TPW / 4;   // 16-byte chunks per row
+    char *cell = const_cast<char *>(v_cell_ptr(st, bh, slot_t)) + v_row_off(st, slot_t, 0);
+    for (int c = threadIdx.x; c < D * CPR; c += 256) {
+        const int d = c / CPR, q = c - d * CPR;
+        uint32_t out[4];
+#pragma unroll
+        for (int wi = 0; wi < 4; ++wi) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int tt = 0; tt < TPW; ++tt) {
+                const int t = (4 * q + wi) * TPW + tt;
+                word |= (uint32_t)vcodes[t * VP + d] << (v_bitpos<BITS>(t) & 31);
+            }
+            out[wi] = word;
+        }
+        *reinterpret_cast<u4v *>(cell + (size_t)d * (TILE * BITS / 8) + 16 * q) = u4v{out[0], out[1], out[2], out[3]};
+    }
+}
+
+// grid (whole tiles, BH), 256 threads; 16-bit dtypes, Dk == Dv == 32 NC
+template <int NC>
+__global__ void __launch_bounds__(256)
+append_fp_tile_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, RopeDev rope) {
+    constexpr int D = 32 * NC;
+    constexpr int TPR = D / 8;
+    constexpr int VPW = D / 2 + 1;  // dword pitch of a token's V row in LDS (odd: column reads spread over banks)
+    __shared__ uint32_t vt[TILE * VPW];
+    const int bh = blockIdx.y;
+    const int slot_t = slot0 + blockIdx.x * TILE;
+    const int l_t = src0 + blockIdx.x * TILE;
+    const char *kbase = keys + ((size_t)bh * L + l_t) * D * 2;
+    const char *vbase = values + ((size_t)bh * L + l_t) * D * 2;
+    u4v kraw[NC], vraw[NC];
+#pragma unroll
+    for (int e = 0; e < NC; ++e) {
+        const int c = e * 256 + threadIdx.x;
+        kraw[e] = *reinterpret_cast<const u4v *>(kbase + (size_t)c * 16);
+        vraw[e] = *reinterpret_cast<const u4v *>(vbase + (size_t)c * 16);
+    }
+#pragma unroll
+    for (int e = 0; e < NC; ++e) {
+        const int c = e * 256 + threadIdx.x;
+        const int r = c / TPR, d0 = (c - r * TPR) * 8;
+        u4v k = kraw[e];
+        if (rope.dims > 0 && d0 < rope.dims) {
+            const int pos = rope_pos(rope, bh, l_t + r);
+            const char *row = kbase + (size_t)r * D * 2;
+            uint32_t u[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                uint16_t lo, hi;
+                if (st.dtype == KVHIP_F16) {
+                    lo = __half_as_ushort(__float2half_rn(rope_elem<0>(rope, row, d0 + 2 * j, pos)));
+                    hi = __half_as_ushort(__float2half_rn(rope_elem<0>(rope, row, d0 + 2 * j + 1, pos)));
+                } else {
+                    lo = Elem<1>::bits(rope_elem<1>(rope, row, d0 + 2 * j, pos));
+                    hi = Elem<1>::bits(rope_elem<1>(rope, row, d0 + 2 * j + 1, pos));
+                }
+                u[j] = (uint32_t)lo | ((uint32_t)hi << 16);
+            }
+            k = u4v{u[0], u[1], u[2], u[3]};
+        }
+        *reinterpret_cast<u4v *>(const_cast<char *>(k_row_ptr(st, bh, slot_t + r)) + d0 * 2) = k;
+        uint32_t *vrow = &vt[r * VPW + d0 / 2];
+        vrow[0] = vraw[e].x;
+        vrow[1] = vraw[e].y;
+        vrow[2] = vraw[e].z;
+        vrow[3] = vraw[e].w;
+    }
+    __syncthreads();
+    // transposed rows: thread (d, c8) gathers tokens 8 c8 .. 8 c8 + 7 of column d; consecutive
+    // threads continue the same 128-byte row
+    char *cell = const_cast<char *>(v_cell_ptr(st, bh, slot_t)) + v_row_off(st, slot_t, 0);
+    const uint16_t *vt16 = reinterpret_cast<const uint16_t *>(vt);
+    for (int c = threadIdx.x; c < D * 8; c += 256) {
+        const int d = c >> 3, c8 = c & 7;
+        uint32_t out[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t lo = vt16[(8 * c8 + 2 * j) * (2 * VPW) + d];
+            const uint32_t hi = vt16[(8 * c8 + 2 * j + 1) * (2 * VPW) + d];
+            out[j] = lo | (hi << 16);
+        }
+        *reinterpret_cast<u4v *>(cell + (size_t)d * (TILE * 2) + 16 * c8) = u4v{out[0], out[1], out[2], out[3]};
+    }
+}
+
 template <int ES>
 __global__ void export_fp_kernel(Store st, Runs runs, int row_begin, int dst_row0, int nrows, char *dst_k, char *dst_v) {
     const int bh = blockIdx.y;
@@ -397,16 +592,47 @@ __global__ void mask_materialize_kernel(kvhip_mask_plan_t p, uint8_t *dst) {
         else { if ((DTV) == 0) { CALL(0, 2); } else if ((DTV) == 1) { CALL(1, 2); } else { CALL(2, 2); } } \
     } while (0)
 
-hipError_t launch_append_fp(const Store &st, const void *keys, const void *values, int L, int src0,
-                            int slot0, int n, hipStream_t s, const RopeDev *rope) {
+namespace {
+hipError_t launch_append_fp_rows(const Store &st, const void *keys, const void *values, int L, int src0,
+                                 int slot0, int n, hipStream_t s, const RopeDev &r) {
     if (n <= 0) return hipSuccess;
     dim3 grid(n, st.BH), block(128);
-    const RopeDev r = rope ? *rope : RopeDev();
     if (st.es == 2)
         hipLaunchKernelGGL(append_fp_kernel<2>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, src0, slot0, r);
     else
         hipLaunchKernelGGL(append_fp_kernel<4>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, src0, slot0, r);
     return hipGetLastError();
+}
+// slots [slot0, slot0 + n) as: rows up to the next tile boundary, whole tiles, remaining rows
+struct TileSplit {
+    int head, tiles, tail;
+};
+TileSplit tile_split(int slot0, int n) {
+    TileSplit t{0, 0, 0};
+    t.head = std::min(n, (TILE - (slot0 & (TILE - 1))) & (TILE - 1));
+    t.tiles = (n - t.head) / TILE;
+    t.tail = n - t.head - t.tiles * TILE;
+    return t;
+}
+}  // namespace
+
+hipError_t launch_append_fp(const Store &st, const void *keys, const void *values, int L, int src0,
+                            int slot0, int n, hipStream_t s, const RopeDev *rope) {
+    if (n <= 0) return hipSuccess;
+    const RopeDev r = rope ? *rope : RopeDev();
+    const bool tiled = st.es == 2 && st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 128 || st.Dk == 256);
+    const TileSplit t = tile_split(slot0, n);
+    if (!tiled || t.tiles == 0) return launch_append_fp_rows(st, keys, values, L, src0, slot0, n, s, r);
+    hipError_t e = launch_append_fp_rows(st, keys, values, L, src0, slot0, t.head, s, r);
+    if (e != hipSuccess) return e;
+    dim3 grid(t.tiles, st.BH), block(256);
+    const int a0 = src0 + t.head, b0 = slot0 + t.head;
+    if (st.Dk == 64) hipLaunchKernelGGL(append_fp_tile_kernel<2>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, a0, b0, r);
+    else if (st.Dk == 128) hipLaunchKernelGGL(append_fp_tile_kernel<4>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, a0, b0, r);
+    else hipLaunchKernelGGL(append_fp_tile_kernel<8>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, a0, b0, r);
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    return launch_append_fp_rows(st, keys, values, L, a0 + t.tiles * TILE, b0 + t.tiles * TILE, t.tail, s, r);
 }
 
 hipError_t launch_rope_apply(const RopeDev &rope, const void *x, void *out, int B, int H, int L, int D,
@@ -419,10 +645,10 @@ hipError_t launch_rope_apply(const RopeDev &rope, const void *x, void *out, int 
     return hipGetLastError();
 }
 
-hipError_t launch_append_quant(const Store &st, const void *keys, const void *values, int L, int src0,
-                               int slot0, int n, hipStream_t s, const RopeDev *rope) {
+namespace {
+hipError_t launch_append_quant_rows(const Store &st, const void *keys, const void *values, int L, int src0,
+                                    int slot0, int n, hipStream_t s, const RopeDev &r) {
     if (n <= 0) return hipSuccess;
-    const RopeDev r = rope ? *rope : RopeDev();
     const int ntile = ((slot0 + n - 1) >> 6) - (slot0 >> 6) + 1;
     dim3 grid(ntile, st.BH), block(256);
     const size_t lds = (size_t)TILE * st.Dv;
@@ -432,6 +658,40 @@ hipError_t launch_append_quant(const Store &st, const void *keys, const void *va
     KV_DISPATCH_DT_BITS(st.dtype, st.bits, CALL);
 #undef CALL
     return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_append_quant(const Store &st, const void *keys, const void *values, int L, int src0,
+                               int slot0, int n, hipStream_t s, const RopeDev *rope) {
+    if (n <= 0) return hipSuccess;
+    const RopeDev r = rope ? *rope : RopeDev();
+    const bool tiled = st.es == 2 && st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 128 || st.Dk == 256) &&
+                       (st.bits == 4 || st.bits == 8) && (st.gs == 32 || st.gs == 64 || st.gs == 128);
+    const TileSplit t = tile_split(slot0, n);
+    if (!tiled || t.tiles == 0) return launch_append_quant_rows(st, keys, values, L, src0, slot0, n, s, r);
+    hipError_t e = launch_append_quant_rows(st, keys, values, L, src0, slot0, t.head, s, r);
+    if (e != hipSuccess) return e;
+    dim3 grid(t.tiles, st.BH), block(256);
+    const int a0 = src0 + t.head, b0 = slot0 + t.head;
+#define TILE_CALL(DT, BITS, NC)                                                                      \
+    hipLaunchKernelGGL((append_quant_tile_kernel<DT, BITS, NC>), grid, block, 0, s, st, (const char *)keys, \
+                       (const char *)values, L, a0, b0, r)
+#define TILE_NC(DT, BITS)                              \
+    do {                                               \
+        if (st.Dk == 64) TILE_CALL(DT, BITS, 2);       \
+        else if (st.Dk == 128) TILE_CALL(DT, BITS, 4); \
+        else TILE_CALL(DT, BITS, 8);                   \
+    } while (0)
+    if (st.dtype == KVHIP_F16) {
+        if (st.bits == 4) TILE_NC(0, 4); else TILE_NC(0, 8);
+    } else {
+        if (st.bits == 4) TILE_NC(1, 4); else TILE_NC(1, 8);
+    }
+#undef TILE_NC
+#undef TILE_CALL
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    return launch_append_quant_rows(st, keys, values, L, a0 + t.tiles * TILE, b0 + t.tiles * TILE, t.tail, s, r);
 }
 
 hipError_t launch_export_fp(const Store &st, const Runs &runs, int row_begin, int count, int dst_row0,

@@ -147,6 +147,23 @@ def test_simple_cache_update_fetch_state(dtype):
     assert all(torch.equal(a, b) for a, b in zip(fresh.state, st))
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_simple_cache_prompt_sized_appends(dtype, D):
+    """Appends that cover whole 64-token tiles take the tile kernel (head rows, tiles, tail rows)."""
+    rng = np.random.default_rng(21)
+    B, H = 2, 3
+    c = kvhip.KVCacheSimple()
+    o = O.KVCacheSimple(NAME[dtype])
+    for L, trim in [(37, 0), (200, 5), (64, 0), (1, 0), (459, 3), (128, 0)]:
+        k, kd = randn(rng, (B, H, L, D), dtype)
+        v, vd = randn(rng, (B, H, L, D), dtype)
+        gk, gv = c.update(kd, vd)
+        ok, ov = o.update(k, v)
+        assert np.array_equal(np32(gk), ok) and np.array_equal(np32(gv), ov)
+        assert c.trim(trim) == o.trim(trim)
+
+
 def test_dynamic_conversion_at_compression_start():
     """`maybeAffineQuantizeKVCache` (KVCache.swift:2500-2520): simple caches past the threshold
     become quantized caches holding the same rows (bit-exact with the oracle's bulk quantize);

@@ -99,13 +99,31 @@ def test_fused_append_equals_rotate_then_append_simple_and_ring(dtype):
             assert torch.equal(fk, pk) and torch.equal(fv, pv)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("traditional", [False, True])
+def test_fused_prompt_sized_append_equals_rotate_then_append(dtype, traditional):
+    """Whole-tile appends rotate inside the tile kernel."""
+    rng = np.random.default_rng(7)
+    rope = kvhip.RoPE(128, traditional=traditional, base=500000.0)
+    fused, plain = kvhip.KVCacheSimple(), kvhip.KVCacheSimple()
+    for Lq in (5, 200, 130):
+        _, k = randn(rng, (2, 2, Lq, 128), dtype)
+        _, v = randn(rng, (2, 2, Lq, 128), dtype)
+        off = plain.offset
+        fused.update_rope(rope, k, v)
+        plain.update(kvhip.apply_rotary_position(rope, k, off), v, fetch=False)
+    fk, fv = fused.fetch()
+    pk, pv = plain.fetch()
+    assert torch.equal(fk, pk) and torch.equal(fv, pv)
+
+
 @pytest.mark.parametrize("bits,gs", [(4, 64), (8, 32)])
 def test_fused_quantize_on_append_equals_rotate_then_append(bits, gs):
     rng = np.random.default_rng(3)
     dtype = torch.float16
     rope = kvhip.RoPE(96, traditional=True, base=1e6)          # partial rotation of a 128-wide head
     fused, plain = kvhip.QuantizedKVCache(gs, bits), kvhip.QuantizedKVCache(gs, bits)
-    for Lq in (70, 1, 1, 3):
+    for Lq in (70, 1, 1, 3, 190):
         _, k = randn(rng, (2, 2, Lq, 128), dtype)
         _, v = randn(rng, (2, 2, Lq, 128), dtype)
         off = plain.offset
@@ -114,7 +132,7 @@ def test_fused_quantize_on_append_equals_rotate_then_append(bits, gs):
     for a, b in zip(fused.state, plain.state):
         assert torch.equal(a, b)
     # and the codes are what the restatement gives for the rotated keys (bit-exact quantizer)
-    assert fused.offset == 75
+    assert fused.offset == 265
 
 
 def test_layer_sequence_against_the_restatement():
