@@ -101,7 +101,15 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
     const int row0 = blk_x * BM + wave * 16 * QT;  // first query row of this wavefront
     const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
-    const float sl2 = a.scale * LOG2E;
+    // Fast softmax (fp16 caches up to D = 128; D = 256 has no registers to spare, and bf16 keeps its
+    // float32 denominators): scores enter as exp2(s * sl2 - m) with sl2 >= 0 -- a negative scale
+    // flips the sign of the query operands instead (exact), a zero one becomes a vanishing positive
+    // factor -- so that the maximum can be taken on the raw scores and the scale folded into one
+    // multiply-add; the denominators ride on the matrix cores (lacc = ones . P^T sums the same
+    // rounded probabilities the numerator uses; all 16 rows of the block hold the same sums).
+    constexpr bool LM = D <= 128 && DT == 0;
+    const bool flip = LM && a.scale < 0.f;
+    const float sl2 = LM ? fmaxf(fabsf(a.scale) * LOG2E, 1e-30f) : a.scale * LOG2E;
 
     // ---- query operands: B of S^T = K . Q^T; lane (n, jj) holds q[row][32 s + 8 jj ..] raw ----
     Op8 qop[QT][S];
@@ -117,15 +125,23 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         const u4 *qp = reinterpret_cast<const u4 *>(
             reinterpret_cast<const uint16_t *>(a.q) + ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D + 8 * jj);
 #pragma unroll
-        for (int s = 0; s < S; ++s) qop[qt][s].v = q_ok[qt] ? qp[4 * s] : u4{0, 0, 0, 0};
+        for (int s = 0; s < S; ++s) {
+            u4 w = q_ok[qt] ? qp[4 * s] : u4{0, 0, 0, 0};
+            if (flip) w ^= u4{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
+            qop[qt][s].v = w;
+        }
     }
 
     f4 oacc[QT][NDT];
     float m_run[QT], l_run[QT];
+    f4 lacc[LM ? QT : 1];
+    Op8 ones;
+    ones.v = u4{0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
         m_run[qt] = -INFINITY;
         l_run[qt] = 0.f;
+        if (LM) lacc[LM ? qt : 0] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) oacc[qt][dt] = f4{0.f, 0.f, 0.f, 0.f};
     }
@@ -225,6 +241,20 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         if (DEEP && tile_lo + 2 < tile_hi) fetch(tile_lo + 2, setB);
     }
     __syncthreads();
+    // (fast softmax) raise query block qt's reference maximum to what the tile holds and rescale
+    auto raise = [&](int qt, float tmax) __attribute__((always_inline)) {
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        const float mn = fmaxf(m_run[qt], tmax);
+        const float alpha = (mn == -INFINITY) ? 1.f : exp2_fast(m_run[qt] - mn);
+        m_run[qt] = mn;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) lacc[LM ? qt : 0][i] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) oacc[qt][dt][i] *= alpha;
+    };
     // one tile: `cur` is the LDS buffer that holds it, `g` the register set that holds the next one
     auto step = [&](int tile, int cur, Stg &g) __attribute__((always_inline)) {
         // the tile fetched two iterations ago goes to the other buffer (last read one barrier
@@ -268,6 +298,55 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         Op8 pb[QT];
 #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
+            if constexpr (LM) {
+                if (MM != 2 && tile_full) {
+                    // every key of the tile counts for every query
+                    float tmax = fmaxf(fmaxf(fmaxf(sacc[qt][0][0], sacc[qt][0][1]), fmaxf(sacc[qt][0][2], sacc[qt][0][3])),
+                                       fmaxf(fmaxf(sacc[qt][1][0], sacc[qt][1][1]), fmaxf(sacc[qt][1][2], sacc[qt][1][3])));
+                    tmax *= sl2;
+                    if (__any(tmax > m_run[qt] + RAISE)) raise(qt, tmax);
+                    const float mu = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt];
+                    float p[2][4];
+#pragma unroll
+                    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) p[mt][i] = exp2_fast(__builtin_fmaf(sacc[qt][mt][i], sl2, -mu));
+                    pb[qt].v = u4{rn_h2(p[0][0], p[0][1]), rn_h2(p[0][2], p[0][3]), rn_h2(p[1][0], p[1][1]), rn_h2(p[1][2], p[1][3])};
+                } else {
+                    float x[2][4];
+                    float tmax = -INFINITY;
+#pragma unroll
+                    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            float x_ = sacc[qt][mt][i] * sl2;
+                            const int row = trow[mt][i];
+                            if (row >= 0 && q_ok[qt]) {
+                                if constexpr (MM == 1) {
+                                    if (!sym_mask_keep(sym, q_l[qt], row)) x_ = -INFINITY;
+                                } else if constexpr (MM == 2) {
+                                    float add;
+                                    const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
+                                    x_ = keep ? x_ + add * LOG2E : -INFINITY;
+                                }
+                            } else {
+                                x_ = -INFINITY;
+                            }
+                            x[mt][i] = x_;
+                            tmax = fmaxf(tmax, x_);
+                        }
+                    if (__any(tmax > m_run[qt] + RAISE)) raise(qt, tmax);
+                    const float mu = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt];
+                    float p[2][4];
+#pragma unroll
+                    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) p[mt][i] = exp2_fast(x[mt][i] - mu);  // exp2(-inf) = 0 for excluded keys
+                    pb[qt].v = u4{rn_h2(p[0][0], p[0][1]), rn_h2(p[0][2], p[0][3]), rn_h2(p[1][0], p[1][1]), rn_h2(p[1][2], p[1][3])};
+                }
+                lacc[LM ? qt : 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones.h, pb[qt].h, lacc[LM ? qt : 0], 0, 0, 0);
+                continue;
+            }
             float x[2][4];
             float tmax = -INFINITY;
 #pragma unroll
@@ -316,6 +395,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                 }
             l_run[qt] += psum;
             pb[qt].v = u4{rn_h2(p[0][0], p[0][1]), rn_h2(p[0][2], p[0][3]), rn_h2(p[1][0], p[1][1]), rn_h2(p[1][2], p[1][3])};
+        
         }
 
         // ---- out^T += V^T . P^T: A = V^T rows (tokens 4jj..4jj+3 and 16+4jj..) from LDS -------
@@ -346,8 +426,12 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
         float l = l_run[qt];
-        l += __shfl_xor(l, 16);
-        l += __shfl_xor(l, 32);
+        if constexpr (LM) {
+            l = lacc[LM ? qt : 0][0];
+        } else {
+            l += __shfl_xor(l, 16);
+            l += __shfl_xor(l, 32);
+        }
         if (!q_ok[qt]) continue;
         if (nsplit > 1) {
             const int i = row0 + 16 * qt + n;

@@ -31,9 +31,20 @@ class MaskMode:
     """`MLXFast.ScaledDotProductAttentionMaskMode`: .none / .causal / .array(mask),
     plus .window -- createCausalMask evaluated from indices inside the kernel."""
 
-    def __init__(self, mode, array=None, offset=0, window=0, lengths=None, left_pad=None):
-        self.mode, self.array = mode, array
+    def __init__(self, mode, array=None, offset=0, window=0, lengths=None, left_pad=None, plan=None):
+        self.mode, self._array, self._plan = mode, array, plan
         self.offset, self.window, self.lengths, self.left_pad = offset, window, lengths, left_pad
+
+    @property
+    def array(self):
+        """The boolean array of an `.array` mask; a mask planned by `make_mask` and evaluated from
+        indices builds it (on the device) only when somebody asks for it."""
+        if self._array is None and self._plan is not None:
+            p = self._plan
+            buf = torch.empty((p.rows, p.cols), dtype=torch.uint8, device="cuda")
+            L.check(L.load().kvhip_mask_materialize(C.byref(p), _ptr(buf), _stream()))
+            self._array = buf.bool()
+        return self._array
 
     @staticmethod
     def none():
@@ -208,7 +219,11 @@ class _Cache:
             return MaskMode.none()
         if p.mode == L.MASK_CAUSAL:
             return MaskMode.causal()
-        shape = (p.cols,) if p.rolled else (p.rows, p.cols)
+        if not p.rolled:
+            # createCausalMask(n, offset, windowSize) (KVCache.swift:253-275) is a function of the
+            # indices: the kernels evaluate it in place, and `.array` materialises it on demand
+            return MaskMode(L.MASK_WINDOW, offset=p.offset, window=p.window, plan=p)
+        shape = (p.cols,)
         buf = torch.empty(shape, dtype=torch.uint8, device="cuda")
         L.check(self._lib.kvhip_mask_materialize(C.byref(p), _ptr(buf), _stream()))
         return MaskMode.from_array(buf.bool())
