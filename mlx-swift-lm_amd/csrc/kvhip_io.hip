@@ -140,7 +140,8 @@ __global__ void append_fp_kernel(Store st, const char *keys, const char *values,
 // grid (64-token tiles touched, BH), 256 threads.  Each wavefront quantizes rows of
 // the tile; V codes are staged as bytes in LDS and then merged into the transposed
 // tile rows, touching only the token positions this append writes.
-template <int DT, int BITS>
+// (ROPE = false carries no rotation code: the single-token decode append stays as small as it was)
+template <int DT, int BITS, bool ROPE>
 __global__ void __launch_bounds__(256)
 append_quant_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, int n,
                     RopeDev rope) {
@@ -174,7 +175,7 @@ append_quant_kernel(Store st, const char *keys, const char *values, int L, int s
             quantize_row_wave<DT, BITS>(krow, st.Dk, st.gs, lane,
                                         reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot))),
                                         nullptr, const_cast<char *>(ksb_row_ptr(st, bh, slot)), nullptr, nullptr,
-                                        rope.dims > 0 ? &rope : nullptr, rope_pos(rope, bh, l));
+                                        ROPE ? &rope : nullptr, ROPE ? rope_pos(rope, bh, l) : 0);
         } else {
             const char *vrow = values + ((size_t)bh * L + l) * st.Dv * st.es;
             quantize_row_wave<DT, BITS>(vrow, st.Dv, st.gs, lane, nullptr, vcodes + (slot & (TILE - 1)) * st.Dv,
@@ -652,9 +653,15 @@ hipError_t launch_append_quant_rows(const Store &st, const void *keys, const voi
     const int ntile = ((slot0 + n - 1) >> 6) - (slot0 >> 6) + 1;
     dim3 grid(ntile, st.BH), block(256);
     const size_t lds = (size_t)TILE * st.Dv;
-#define CALL(DT, BITS)                                                                           \
-    hipLaunchKernelGGL((append_quant_kernel<DT, BITS>), grid, block, lds, s, st, (const char *)keys, \
-                       (const char *)values, L, src0, slot0, n, r)
+#define CALL(DT, BITS)                                                                                      \
+    do {                                                                                                    \
+        if (r.dims > 0)                                                                                     \
+            hipLaunchKernelGGL((append_quant_kernel<DT, BITS, true>), grid, block, lds, s, st, (const char *)keys,  \
+                               (const char *)values, L, src0, slot0, n, r);                                 \
+        else                                                                                                \
+            hipLaunchKernelGGL((append_quant_kernel<DT, BITS, false>), grid, block, lds, s, st, (const char *)keys, \
+                               (const char *)values, L, src0, slot0, n, r);                                 \
+    } while (0)
     KV_DISPATCH_DT_BITS(st.dtype, st.bits, CALL);
 #undef CALL
     return hipGetLastError();
