@@ -245,8 +245,24 @@ __device__ __forceinline__ void quantize8(const float (&w)[8], int gl, float &sc
     }
     group_minmax(mn, mx, gl);
     affine_params(mn, mx, nb, scale, bias);
+    // code = rint((w - bias) / scale), clamped.  The quotient is first formed with one exact
+    // reciprocal per thread: it lies within two float32 ulps of the correctly rounded quotient
+    // (|q| <= 2^BITS, so within 2^-19), which can only change the rounded integer when the quotient
+    // sits that close to a half-integer.  Those elements (about one in 10^4) are redone with the
+    // exact division, so the codes are the reference's bit for bit.
+    const float inv = __fdiv_rn(1.0f, scale);
+    bool near_tie = false;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) code[j] = affine_code(w[j], scale, bias, nb);
+    for (int j = 0; j < 8; ++j) {
+        const float r = __fmul_rn(__fsub_rn(w[j], bias), inv);
+        const float q = rintf(r);
+        near_tie = near_tie || (fabsf(r - q) > 0.4999f);
+        code[j] = (uint32_t)fminf(fmaxf(q, 0.0f), nb);
+    }
+    if (near_tie) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) code[j] = affine_code(w[j], scale, bias, nb);
+    }
 }
 
 // grid (whole tiles, BH), 256 threads; slot0 is a multiple of 64; 16-bit dtypes, Dk == Dv == 32 NC

@@ -99,6 +99,38 @@ def test_quantized_cache_append_trim_state(dtype, bits, gs, D):
     check_quantized_state(fresh, ocache2, dtype)
 
 
+@pytest.mark.parametrize("bits", [4, 8])
+def test_quantized_prompt_append_on_rounding_ties(bits):
+    """Whole-tile appends whose quotients (w - bias) / scale sit exactly on, and within a few ulps
+    of, half-integers: the codes must still be the restatement's (round-half-to-even of the
+    correctly rounded quotient)."""
+    rng = np.random.default_rng(31)
+    B, H, L, D, gs = 1, 2, 128, 128, 64
+    nb = (1 << bits) - 1
+    step = 0.125 if bits == 4 else 2.0 ** -7
+    k = (rng.integers(0, nb, size=(B, H, L, D)).astype(np.float32) + 0.5) * np.float32(step)   # exact ties
+    near = rng.random((B, H, L, D)) < 0.3
+    k = np.where(near, k * np.float32(1.0 + 2.0 ** -10), k).astype(np.float32)                  # one fp16 ulp off
+    k[..., 0::gs] = 0.0                       # pin every group's extrema: scale = step exactly
+    k[..., 1::gs] = nb * step
+    k = O.round_to(k, "float16")
+    kd = dev(k, torch.float16)
+    cache = kvhip.QuantizedKVCache(gs, bits)
+    ocache = O.QuantizedKVCache(gs, bits, "float16")
+    cache.update_quantized(kd, kd, fetch=False)
+    ocache.update_quantized(k, k)
+    check_quantized_state(cache, ocache, torch.float16)
+    # scales that are not powers of two: about two in 10^4 quotients land within 10^-4 of a
+    # half-integer by chance, so half a million elements hold about a hundred of them
+    L2 = 1920
+    k2 = rng.standard_normal((B, H, L2, D)).astype(np.float32) * (10.0 ** rng.uniform(-2, 2, size=(B, H, L2, 1))).astype(np.float32)
+    k2 = O.round_to(k2, "float16")
+    k2d = dev(k2, torch.float16)
+    cache.update_quantized(k2d, k2d, fetch=False)
+    ocache.update_quantized(k2, k2)
+    check_quantized_state(cache, ocache, torch.float16)
+
+
 def test_quantized_group_size_fallback_and_errors():
     # KVCacheTests.swift:477-501: QuantizedKVCache(64, 4) fed D=32 -> groupSize 32
     rng = np.random.default_rng(0)
