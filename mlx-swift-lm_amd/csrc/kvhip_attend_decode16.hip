@@ -293,7 +293,15 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 }
                 x[tl] = round_dt<DT>(s_);
             }
-        if (MM == 2 || t.base < full_lo || t.base + (TILE - 1) > full_hi) {  // wave-uniform: edge tile
+        if (MM == 2 && a.mask.dtype == KVHIP_BOOL && t.base + (TILE - 1) < a.T) {
+            // a boolean array over a whole tile: this lane's 16 tokens are 16 consecutive bytes of its
+            // query row
+            uint32_t mw[4] = {~0u, ~0u, ~0u, ~0u};
+            if (row_ok) mask_bool_words<4>(a.mask, b, hk * r + row_rep, row_l, t.base + 16 * jj, mw);
+#pragma unroll
+            for (int tl = 0; tl < 16; ++tl)
+                if (((mw[tl >> 2] >> (8 * (tl & 3))) & 0xffu) == 0u) x[tl] = fill;
+        } else if (MM == 2 || t.base < full_lo || t.base + (TILE - 1) > full_hi) {  // wave-uniform: edge tile
 #pragma unroll
             for (int tl = 0; tl < 16; ++tl) {
                 const int row = t.base + 16 * jj + tl;  // slots are presented rows

@@ -323,9 +323,27 @@ prefill_kernel(AttendArgs a, int nsplit) {
         // ---- online softmax per query column; P^T stays in place as the PV B operand ------
         // Tiles every query row of the workgroup sees completely (all slots live rows, inside
         // the mask for every row) skip the per-element tests.
+        // a boolean array mask is read four keys at a time where this lane's four rows are consecutive
+        [[maybe_unused]] bool vec_ok[2] = {false, false};
+        if constexpr (MM == 2) {
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+                vec_ok[mt] = a.mask.dtype == KVHIP_BOOL && trow[mt][0] >= 0 && trow[mt][3] == trow[mt][0] + 3 &&
+                             trow[mt][1] == trow[mt][0] + 1 && trow[mt][2] == trow[mt][0] + 2;
+        }
         Op8 pb[QT];
 #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
+            [[maybe_unused]] uint32_t mword[2] = {0u, 0u};
+            if constexpr (MM == 2) {
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt)
+                    if (vec_ok[mt] && q_ok[qt]) {
+                        uint32_t w[1];
+                        mask_bool_words<1>(a.mask, b, q_h[qt], q_l[qt], trow[mt][0], w);
+                        mword[mt] = w[0];
+                    }
+            }
             float sc[2][4];
             float tmax = -INFINITY;
 #pragma unroll
@@ -339,10 +357,14 @@ prefill_kernel(AttendArgs a, int nsplit) {
                             if constexpr (MM == 1) {
                                 if (!sym_mask_keep(sym, q_l[qt], row)) s_ = fill;
                             } else if constexpr (MM == 2) {
-                                float add;
-                                const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
-                                if (!keep) s_ = fill;
-                                else if (a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
+                                if (vec_ok[mt]) {
+                                    if (((mword[mt] >> (8 * i)) & 0xffu) == 0u) s_ = fill;
+                                } else {
+                                    float add;
+                                    const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
+                                    if (!keep) s_ = fill;
+                                    else if (a.mask.dtype != KVHIP_BOOL) s_ = round_dt<DT>(s_ + add);
+                                }
                             }
                         } else {
                             s_ = -INFINITY;

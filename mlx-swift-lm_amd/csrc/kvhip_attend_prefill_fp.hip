@@ -288,6 +288,15 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                 for (int i = 0; i < 4; ++i) trow[mt][i] = rows_s[cur][16 * mt + 4 * jj + i];
         }
 
+        // a boolean array mask is read four keys at a time where this lane's four rows are consecutive
+        [[maybe_unused]] bool vec_ok[2] = {false, false};
+        if constexpr (MM == 2) {
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+                vec_ok[mt] = a.mask.dtype == KVHIP_BOOL && trow[mt][0] >= 0 && trow[mt][3] == trow[mt][0] + 3 &&
+                             trow[mt][1] == trow[mt][0] + 1 && trow[mt][2] == trow[mt][0] + 2;
+        }
+
         // ---- online softmax per query column; P^T stays in place as the PV B operand ------
         // Scores stay in the log2 domain: x = s * (scale * log2 e), p = exp2(x - m).  m is a reference
         // value rather than the exact running maximum: it is the same in the four lanes that share a
@@ -298,6 +307,16 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         Op8 pb[QT];
 #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
+            [[maybe_unused]] uint32_t mword[2] = {0u, 0u};
+            if constexpr (MM == 2) {
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt)
+                    if (vec_ok[mt] && q_ok[qt]) {
+                        uint32_t w[1];
+                        mask_bool_words<1>(a.mask, b, q_h[qt], q_l[qt], trow[mt][0], w);
+                        mword[mt] = w[0];
+                    }
+            }
             if constexpr (LM) {
                 if (MM != 2 && tile_full) {
                     // every key of the tile counts for every query
@@ -325,9 +344,13 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                                 if constexpr (MM == 1) {
                                     if (!sym_mask_keep(sym, q_l[qt], row)) x_ = -INFINITY;
                                 } else if constexpr (MM == 2) {
-                                    float add;
-                                    const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
-                                    x_ = keep ? x_ + add * LOG2E : -INFINITY;
+                                    if (vec_ok[mt]) {
+                                        if (((mword[mt] >> (8 * i)) & 0xffu) == 0u) x_ = -INFINITY;
+                                    } else {
+                                        float add;
+                                        const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
+                                        x_ = keep ? x_ + add * LOG2E : -INFINITY;
+                                    }
                                 }
                             } else {
                                 x_ = -INFINITY;
@@ -360,9 +383,13 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                             if constexpr (MM == 1) {
                                 if (!sym_mask_keep(sym, q_l[qt], row)) x_ = -INFINITY;
                             } else if constexpr (MM == 2) {
-                                float add;
-                                const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
-                                x_ = keep ? x_ + add * LOG2E : -INFINITY;
+                                if (vec_ok[mt]) {
+                                    if (((mword[mt] >> (8 * i)) & 0xffu) == 0u) x_ = -INFINITY;
+                                } else {
+                                    float add;
+                                    const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
+                                    x_ = keep ? x_ + add * LOG2E : -INFINITY;
+                                }
                             }
                         } else {
                             x_ = -INFINITY;

@@ -33,6 +33,20 @@ __device__ __forceinline__ bool mask_keep(const MaskDev &m, int b, int hq, int l
     }
 }
 
+// 4 * W consecutive bytes of a boolean array mask: query row l of (b, hq), key rows j0 .. j0 + 4 W - 1
+// (all below T; the address need not be aligned: global loads take any byte address).  One
+// load in place of 4 W byte loads per lane.
+template <int W>
+__device__ __forceinline__ void mask_bool_words(const MaskDev &m, int b, int hq, int l, int j0, uint32_t (&w)[W]) {
+    const uint8_t *p = reinterpret_cast<const uint8_t *>(m.data) + (size_t)(b * m.sb + hq * m.sh + l * m.sl) + j0;
+    struct __attribute__((packed, aligned(1))) Raw {
+        uint32_t v[W];
+    };
+    const Raw raw = *reinterpret_cast<const Raw *>(p);
+#pragma unroll
+    for (int i = 0; i < W; ++i) w[i] = raw.v[i];
+}
+
 // Index-only masks (causal, window with optional per-batch bounds) with the per-batch
 // bounds already in registers: no memory access, so kernels can keep loads in flight.
 struct SymMask {

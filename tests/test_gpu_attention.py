@@ -160,6 +160,13 @@ def test_simple_cache_attention(policy, dtype, Dk, Dv, r):
         out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
         ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
         check(out, ref, f"L={Lq} {mode}")
+        if mode == "array":
+            # the same mask handed over as data (boolean, then additive), as unmodified model code does
+            out = c.attend(qd, scale, kvhip.MaskMode.from_array(mask.array))
+            check(out, ref, f"L={Lq} boolean array")
+            addm = torch.where(mask.array, 0.0, -30000.0).to(dtype if dtype != torch.float32 else torch.float32)
+            out = c.attend(qd, scale, kvhip.MaskMode.from_array(addm))
+            check(out, ref, f"L={Lq} additive array")
 
 
 def test_rotating_attention_past_wrap_matches_never_rotated_reference(policy):
@@ -203,6 +210,10 @@ def test_rotating_cfg4_reduced(policy, dtype):
         ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
         if i in (0, 7, 8, 9, 19):
             check(out, ref, f"chunk {i}")
+        if i in (8, 19) and om.mode == "array":
+            # ring rows in run order, the mask handed over as data
+            out = c.attend(qd, scale, kvhip.MaskMode.from_array(mask.array))
+            check(out, ref, f"chunk {i} boolean array")
     for i in range(40):
         k, kd = randn(rng, (B, Hkv, 1, D), dtype)
         v, vd = randn(rng, (B, Hkv, 1, D), dtype)
@@ -231,6 +242,10 @@ def test_cfg1_quantized_prefill_then_decode(policy):
     ref = CO.qsdpa(q, qk, qv, scale, "causal", 64, 8, "float16")
     check(out, ref, "prefill")
     assert kvhip.load().kvhip_last_attend_kernel() == (3 if policy == 0 else 0)  # MFMA prefill tile
+    # the same causal mask handed over as a boolean array
+    tri = torch.ones(512, 512, dtype=torch.bool, device="cuda").tril()
+    out = c.attend(qd, scale, kvhip.MaskMode.from_array(tri))
+    check(out, ref, "prefill, boolean array")
     for step in range(128):
         q, qd = randn(rng, (B, Hq, 1, D), dtype)
         k, kd = randn(rng, (B, Hkv, 1, D), dtype)
