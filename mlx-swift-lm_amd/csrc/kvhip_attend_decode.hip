@@ -865,6 +865,26 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         }
     }
     __syncthreads();
+    // a single span writes the output rows itself, several leave partials for the merge kernel
+    if (nsplit == 1) {
+        for (int idx = threadIdx.x; idx < R * D; idx += WAVES * 64) {
+            const int i = idx / D, c = idx - i * D;
+            float mx = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, cbuf[w][i][D]);
+            float v = 0.f, l = 0.f;
+#pragma unroll
+            for (int w = 0; w < WAVES; ++w) {
+                const float mw = cbuf[w][i][D];
+                const float wgt = (mw == -INFINITY) ? 0.f : fast_exp2((mw - mx) * LOG2E);
+                v += wgt * cbuf[w][i][c];
+                l += wgt * cbuf[w][i][D + 1];
+            }
+            const int rep = i / a.L, lq = i - rep * a.L;
+            Elem<DT>::store(a.out, ((size_t)(b * a.Hq + hk * r + rep) * a.L + lq) * D + c, l > 0.f ? v / l : 0.f);
+        }
+        return;
+    }
     float *part = a.workspace + ((size_t)bh * nsplit + split) * RR * (D + 2);
     for (int idx = threadIdx.x; idx < RR * (D + 2); idx += WAVES * 64) {
         const int i = idx / (D + 2), c = idx - i * (D + 2);
@@ -958,7 +978,9 @@ Plan plan_for(const AttendArgs &a) {
     int want = (a.st.bits != 0 ? 256 * 2 : 256) / BH;
     if (want < 1) want = 1;
     int per = (p.tiles_total + want - 1) / want;
-    if (const char *e = getenv("KVHIP_DECODE_TILES")) per = atoi(e);
+    // KVHIP_DECODE_TILES (read once) forces the span size in tiles: a measurement aid
+    static const int forced_tiles = getenv("KVHIP_DECODE_TILES") ? atoi(getenv("KVHIP_DECODE_TILES")) : 0;
+    if (forced_tiles > 0) per = forced_tiles;
     per = per < WAVES ? WAVES : per;
     per = (per + WAVES - 1) / WAVES * WAVES;
     while ((p.tiles_total + per - 1) / per > 512) per *= 2;  // the merge kernel holds 512 span weights
@@ -969,10 +991,10 @@ Plan plan_for(const AttendArgs &a) {
     // and none is empty; measured faster than equal-sized spans with more of them for the
     // long rows)
     p.nw = WAVES;
-    if (a.mask.mode == KVHIP_MASK_WINDOW && (a.mask.left_pad || a.mask.lengths) && !getenv("KVHIP_DECODE_TILES")) {
+    if (a.mask.mode == KVHIP_MASK_WINDOW && (a.mask.left_pad || a.mask.lengths) && forced_tiles <= 0) {
         p.tiles_per_wg = 0;
     } else if (a.st.bits != 0 && p.nsplit >= 2 && want <= 4 && p.rg == 1 && a.mask.mode != KVHIP_MASK_ARRAY &&
-               !getenv("KVHIP_DECODE_TILES")) {
+               forced_tiles <= 0) {
         // 128 pairs or more: workgroups of 8 wavefronts, one per CU -- the same wavefronts per CU
         // with half the spans.  With 256 pairs a workgroup takes its pair's whole sequence: the
         // merge stays on chip and the kernel writes the output itself (no partials, no second
@@ -1115,7 +1137,8 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
         hipLaunchKernelGGL((decode_fp_kernel<D, DT, RG, M, I>), grid, block, 0, s, a, p.tiles_total,      \
                            p.tiles_per_wg, p.nsplit);                                                     \
         profile_mark(s, false);                                                                           \
-        hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG);  \
+        if (p.nsplit > 1)                                                                                 \
+            hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG); \
     } while (0)
 #define FP_MI(D, DT, RG)                                          \
     do {                                                          \

@@ -49,6 +49,31 @@ def test_simple_decode_grow(dtype, D, Hq, Hkv):
     assert mx <= 1e-2 and mean <= 1e-3, (mx, mean)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,Hkv,T0", [(32, 8, 333), (64, 8, 70), (16, 8, 900)])
+def test_simple_decode_many_pairs(dtype, B, Hkv, T0):
+    """128 (batch, kv-head) pairs and more: with 256 a single span covers a pair's sequence and
+    the decode kernel writes the output rows itself, with fewer the merge kernel runs."""
+    rng = np.random.default_rng(B + T0)
+    D, r = 128, 4
+    name = NAME[dtype]
+    scale = 1.0 / np.sqrt(D)
+    c = kvhip.KVCacheSimple()
+    k, kd = randn(rng, (B, Hkv, T0, D), dtype)
+    v, vd = randn(rng, (B, Hkv, T0, D), dtype)
+    c.update(kd, vd, fetch=False)
+    for Lq, mask, om in ((1, kvhip.MaskMode.none(), None), (3, kvhip.MaskMode.causal(), "causal")):
+        kn, knd = randn(rng, (B, Hkv, Lq, D), dtype)
+        vn, vnd = randn(rng, (B, Hkv, Lq, D), dtype)
+        q, qd = randn(rng, (B, Hkv * r, Lq, D), dtype)
+        out = kvhip.attention_with_cache_update(qd, knd, vnd, c, scale, mask)
+        k, v = np.concatenate([k, kn], 2), np.concatenate([v, vn], 2)
+        ref = CO.sdpa(q, k, v, scale, om, name)
+        mx, mean = err_stats(np32(out), ref)
+        assert mx <= 1e-2 and mean <= 1e-3, (Lq, mx, mean)
+        assert kvhip.load().kvhip_last_attend_kernel() == 2  # matrix-core full-precision decode
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_rotating_decode_after_wrap(dtype):
     """Ring of 1024 (keep 4), D 256: chunked prefill wraps it, then single-token decode over
