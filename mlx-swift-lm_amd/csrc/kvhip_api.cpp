@@ -126,7 +126,8 @@ kvhip_status set_geometry(kvhip_cache *c, int B, int Hkv, int Dk, int Dv, int dt
         s.ksb_cell = s.ksb_row * PAGE;
         s.vsb_cell = s.vsb_row * PAGE;
     } else {
-        s.k_row = (uint32_t)(Dk * s.es);
+        // K rows are laid out in whole 16-byte chunks (the interleaved tile of kvhip_internal.hpp)
+        s.k_row = (uint32_t)((Dk * s.es + 15) / 16 * 16);
         s.k_cell = s.k_row * PAGE;
         s.v_cell = (uint32_t)(Dv * s.es) * PAGE;
     }

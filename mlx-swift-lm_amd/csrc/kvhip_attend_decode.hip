@@ -705,22 +705,31 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     constexpr int VROW = TILE * 2;  // bytes of one V tile row
     const char *kp = st.k + ((size_t)page0 * st.BH + bh) * st.k_cell + (size_t)tip * TILE * st.k_row;
     const char *vp = st.v + ((size_t)page0 * st.BH + bh) * st.v_cell + (size_t)tip * D * VROW;
-    const uint32_t k_lane = lane * st.k_row, v_lane = lane * VROW;
+    // chunk-interleaved tiles: chunk j of the lane's token (K) or column (V) sits 16 * lane bytes into
+    // a 1 KB (K) / 16 D byte (V) row of chunks, so every load below is contiguous across the wavefront
+    const uint32_t k_lane = lane * 16, v_lane = lane * 16;
     int slot_cur = tile0 * TILE + lane;
     int k_loaded = 0, v_loaded = 0;  // tiles whose K / V pieces have been requested
+    auto load_chunks = [&](uint32_t *buf, const char *p, size_t stride) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < PW / 4; ++j) {
+            const uint4 v = *reinterpret_cast<const uint4 *>(p + (size_t)j * stride);
+            buf[4 * j] = v.x; buf[4 * j + 1] = v.y; buf[4 * j + 2] = v.z; buf[4 * j + 3] = v.w;
+        }
+    };
 
     // piece x of the K row / V column set of the tile the respective pointer stands on;
     // after the last piece the pointer steps to this wavefront's next tile (clamped, so
     // the prefetch past the end stays unconditional and in bounds)
     auto load_k = [&](uint32_t *buf, int x) {
-        load_words<PW>(buf, kp + k_lane + x * (PW * 4));
+        load_chunks(buf, kp + k_lane + (size_t)x * (PW / 4) * (TILE * 16), TILE * 16);  // chunks 8x .. 8x+7 of the lane's token
         if (x == NP - 1) {
             ++k_loaded;
             if (k_loaded < my_tiles) kp += k_step;
         }
     };
     auto load_v = [&](uint32_t *buf, int x) {
-        load_words<PW>(buf, vp + v_lane + (size_t)x * 64 * VROW);
+        load_chunks(buf, vp + v_lane + (size_t)x * 64 * 16, (size_t)D * 16);  // the 8 token chunks of column 64x + lane
         if (x == NP - 1) {
             ++v_loaded;
             if (v_loaded < my_tiles) vp += v_step;

@@ -74,8 +74,8 @@ attend_generic_kernel(AttendArgs a, int slots_pad) {
                 }
                 s = round_dt<DT>(sum);
             } else {
-                const char *krow = k_row_ptr(st, bh, slot);
-                for (int d = 0; d < st.Dk; ++d) sum += qs[d] * Elem<DT>::load(krow, d);
+                const char *kc = k_cell_ptr(st, bh, slot);
+                for (int d = 0; d < st.Dk; ++d) sum += qs[d] * Elem<DT>::load(kc + kfp_off(st, slot, d), 0);
                 s = sum;
             }
             float add;
@@ -124,7 +124,7 @@ attend_generic_kernel(AttendArgs a, int slots_pad) {
                     const int g = d / st.gs;
                     v = Elem<DT>::load(sb, 2 * g) * (float)v_code_load<BB>(vrow, t) + Elem<DT>::load(sb, 2 * g + 1);
                 } else {
-                    v = Elem<DT>::load(vrow, t);
+                    v = Elem<DT>::load(v_cell_ptr(st, bh, slot) + vfp_off(st, slot, d), 0);
                 }
                 acc += w * v;
             }

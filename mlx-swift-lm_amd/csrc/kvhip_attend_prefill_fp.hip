@@ -185,8 +185,8 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     }
 
     // ---- staging ------------------------------------------------------------------------
-    // chunk c = e * 256 + tid.  K: row c / (D/8), 16-byte column c % (D/8).  V: head-dim row
-    // c / 4, 16-byte quarter c % 4 of the 32 tokens of this tile.
+    // chunk c = e * 256 + tid.  K: token c % 32 of the tile, 8-element chunk c / 32.  V: column
+    // c % D, 8-token chunk c / D of the 32 tokens of this tile.
     // Up to D = 128 two register sets alternate, so a tile is requested two iterations before
     // it is written to LDS and three before it is contracted; D = 256 has registers for one set
     // (one iteration less of lead).
@@ -207,13 +207,15 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             else row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
             g.row = (row >= 0 && row < a.T) ? row : -1;
         }
-        const char *kbase = k_row_ptr(st, bh, slot0);
-        const char *vbase = v_cell_ptr(st, bh, slot0) + v_row_off(st, slot0, 0) + ((slot0 & 32) ? 64 : 0);
+        // pages are interleaved in 16-byte chunks (K: [8-element chunk][token], V: [8-token chunk][column]):
+        // consecutive threads take consecutive tokens of one K chunk, consecutive columns of one V chunk
+        const char *kbase = k_cell_ptr(st, bh, slot0) + kfp_off(st, slot0, 0);
+        const char *vbase = v_cell_ptr(st, bh, slot0) + vfp_off(st, slot0, 0);
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
             const int c = e * 256 + tid;
-            g.k[e] = *reinterpret_cast<const u4 *>(kbase + (size_t)(c / (D / 8)) * st.k_row + (c % (D / 8)) * 16);
-            g.v[e] = *reinterpret_cast<const u4 *>(vbase + (size_t)(c >> 2) * (TILE * 2) + (c & 3) * 16);
+            g.k[e] = *reinterpret_cast<const u4 *>(kbase + (size_t)(c / BN) * (TILE * 16) + (c % BN) * 16);
+            g.v[e] = *reinterpret_cast<const u4 *>(vbase + (size_t)(c / D) * (D * 16) + (c % D) * 16);
         }
     };
     auto stage = [&](int buf, const Stg &g) __attribute__((always_inline)) {
@@ -225,10 +227,10 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
             const int c = e * 256 + tid;
-            *reinterpret_cast<u4 *>(&Ks[buf][(c / (D / 8)) * KS + (c % (D / 8)) * 8]) = g.k[e];
+            *reinterpret_cast<u4 *>(&Ks[buf][(c % BN) * KS + (c / BN) * 8]) = g.k[e];
             u4 v = g.v[e];
             if (DT == 1) v = u4{bf2_to_h2(v.x), bf2_to_h2(v.y), bf2_to_h2(v.z), bf2_to_h2(v.w)};
-            u2 *vd = reinterpret_cast<u2 *>(&Vs[buf][(c >> 2) * VS + (c & 3) * 8]);  // rows are 8-byte aligned
+            u2 *vd = reinterpret_cast<u2 *>(&Vs[buf][(c % D) * VS + (c / D) * 8]);  // rows are 8-byte aligned
             vd[0] = u2{v.x, v.y};
             vd[1] = u2{v.z, v.w};
         }

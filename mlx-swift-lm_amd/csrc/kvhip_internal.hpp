@@ -88,13 +88,30 @@ __device__ __forceinline__ const char *vsb_row_ptr(const Store &st, int bh, int 
 __device__ __forceinline__ const char *v_cell_ptr(const Store &st, int bh, int slot) {
     return st.v + ((size_t)(slot >> PAGE_SHIFT) * st.BH + bh) * st.v_cell;
 }
+// Full-precision pages are interleaved in 16-byte chunks inside every 64-token tile, so that a
+// wavefront whose lanes are the 64 tokens (K) or 64 adjacent columns (V) reads 1 KB contiguous
+// per load and is the only load to touch those cache lines:
+//   K tile: [chunk of 16/es elements][token 0..63][16 bytes]
+//   V tile: [chunk of 16/es tokens][column 0..Dv-1][16 bytes]
+// byte offset of element (slot, d) inside its (page, pair) cell:
+__device__ __forceinline__ size_t kfp_off(const Store &st, int slot, int d) {
+    const int t = slot & (PAGE - 1), epc = 16 / st.es;
+    return (size_t)(t >> 6) * ((size_t)TILE * st.k_row) + ((size_t)(d / epc) * TILE + (t & 63)) * 16 + (size_t)(d % epc) * st.es;
+}
+__device__ __forceinline__ size_t vfp_off(const Store &st, int slot, int d) {
+    const int t = slot & (PAGE - 1), epc = 16 / st.es, tk = t & 63;
+    return (size_t)(t >> 6) * ((size_t)TILE * st.Dv * st.es) + ((size_t)(tk / epc) * st.Dv + d) * 16 + (size_t)(tk % epc) * st.es;
+}
+__device__ __forceinline__ const char *k_cell_ptr(const Store &st, int bh, int slot) {
+    return st.k + ((size_t)(slot >> PAGE_SHIFT) * st.BH + bh) * st.k_cell;
+}
 // bit position of token t (0..63 inside its tile) within the V tile row of a column
 template <int BITS> __device__ __forceinline__ int v_bitpos(int t) {
     if (BITS == 4) return 32 * (t >> 3) + 4 * (((t & 7) >> 1) + 4 * (t & 1));
     if (BITS == 8) return 32 * (t >> 2) + 8 * (((t & 3) >> 1) + 2 * (t & 1));
     return 2 * t;  // BITS == 2
 }
-// byte offset, inside the page cell, of the V tile row (tile of `slot`, column d)
+// (quantized pages) byte offset, inside the page cell, of the V tile row (tile of `slot`, column d)
 __device__ __forceinline__ size_t v_row_off(const Store &st, int slot, int d) {
     const size_t row_bytes = st.bits ? (size_t)TILE * st.bits / 8 : (size_t)TILE * st.es;
     return ((size_t)((slot & (PAGE - 1)) >> 6) * st.Dv + d) * row_bytes;

@@ -109,7 +109,7 @@ __device__ __forceinline__ void quantize_row_wave(const void *src, int D, int gs
     }
 }
 
-// grid (rows, BH): K rows copied in natural order, V elements scattered into octets.
+// grid (rows, BH): one new row per workgroup, scattered into the chunk-interleaved tile.
 template <int ES>
 __global__ void append_fp_kernel(Store st, const char *keys, const char *values, int L, int src0,
                                  int slot0, RopeDev rope) {
@@ -119,22 +119,21 @@ __global__ void append_fp_kernel(Store st, const char *keys, const char *values,
     const int l = src0 + i;
     using E = typename std::conditional<ES == 2, uint16_t, uint32_t>::type;
     const E *ks = reinterpret_cast<const E *>(keys) + ((size_t)bh * L + l) * st.Dk;
-    E *kd = reinterpret_cast<E *>(const_cast<char *>(k_row_ptr(st, bh, slot)));
+    char *kc = const_cast<char *>(k_cell_ptr(st, bh, slot));
     if (rope.dims > 0) {
         const int pos = rope_pos(rope, bh, l);
         for (int d = threadIdx.x; d < st.Dk; d += blockDim.x) {
-            if (ES == 4) Elem<2>::store(kd, d, rope_elem<2>(rope, ks, d, pos));
-            else if (st.dtype == KVHIP_F16) Elem<0>::store(kd, d, rope_elem<0>(rope, ks, d, pos));
-            else Elem<1>::store(kd, d, rope_elem<1>(rope, ks, d, pos));
+            char *dst = kc + kfp_off(st, slot, d);
+            if (ES == 4) Elem<2>::store(dst, 0, rope_elem<2>(rope, ks, d, pos));
+            else if (st.dtype == KVHIP_F16) Elem<0>::store(dst, 0, rope_elem<0>(rope, ks, d, pos));
+            else Elem<1>::store(dst, 0, rope_elem<1>(rope, ks, d, pos));
         }
     } else {
-        for (int d = threadIdx.x; d < st.Dk; d += blockDim.x) kd[d] = ks[d];
+        for (int d = threadIdx.x; d < st.Dk; d += blockDim.x) *reinterpret_cast<E *>(kc + kfp_off(st, slot, d)) = ks[d];
     }
     const E *vs = reinterpret_cast<const E *>(values) + ((size_t)bh * L + l) * st.Dv;
     char *vc = const_cast<char *>(v_cell_ptr(st, bh, slot));
-    const int t = slot & (TILE - 1);
-    for (int d = threadIdx.x; d < st.Dv; d += blockDim.x)
-        reinterpret_cast<E *>(vc + v_row_off(st, slot, d))[t] = vs[d];
+    for (int d = threadIdx.x; d < st.Dv; d += blockDim.x) *reinterpret_cast<E *>(vc + vfp_off(st, slot, d)) = vs[d];
 }
 
 // grid (64-token tiles touched, BH), 256 threads.  Each wavefront quantizes rows of
@@ -390,7 +389,7 @@ append_fp_tile_kernel(Store st, const char *keys, const char *values, int L, int
             }
             k = u4v{u[0], u[1], u[2], u[3]};
         }
-        *reinterpret_cast<u4v *>(const_cast<char *>(k_row_ptr(st, bh, slot_t + r)) + d0 * 2) = k;
+        *reinterpret_cast<u4v *>(const_cast<char *>(k_cell_ptr(st, bh, slot_t)) + kfp_off(st, slot_t + r, d0)) = k;
         uint32_t *vrow = &vt[r * VPW + d0 / 2];
         vrow[0] = vraw[e].x;
         vrow[1] = vraw[e].y;
@@ -398,12 +397,12 @@ append_fp_tile_kernel(Store st, const char *keys, const char *values, int L, int
         vrow[3] = vraw[e].w;
     }
     __syncthreads();
-    // transposed rows: thread (d, c8) gathers tokens 8 c8 .. 8 c8 + 7 of column d; consecutive
-    // threads continue the same 128-byte row
-    char *cell = const_cast<char *>(v_cell_ptr(st, bh, slot_t)) + v_row_off(st, slot_t, 0);
+    // 8-token chunks of every column: thread (c8, d) gathers tokens 8 c8 .. 8 c8 + 7 of column d;
+    // consecutive threads take consecutive columns, so a chunk row is written contiguously
+    char *cell = const_cast<char *>(v_cell_ptr(st, bh, slot_t));
     const uint16_t *vt16 = reinterpret_cast<const uint16_t *>(vt);
     for (int c = threadIdx.x; c < D * 8; c += 256) {
-        const int d = c >> 3, c8 = c & 7;
+        const int c8 = c / D, d = c - c8 * D;
         uint32_t out[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -411,7 +410,7 @@ append_fp_tile_kernel(Store st, const char *keys, const char *values, int L, int
             const uint32_t hi = vt16[(8 * c8 + 2 * j + 1) * (2 * VPW) + d];
             out[j] = lo | (hi << 16);
         }
-        *reinterpret_cast<u4v *>(cell + (size_t)d * (TILE * 2) + 16 * c8) = u4v{out[0], out[1], out[2], out[3]};
+        *reinterpret_cast<u4v *>(cell + vfp_off(st, slot_t + 8 * c8, d)) = u4v{out[0], out[1], out[2], out[3]};
     }
 }
 
@@ -423,16 +422,15 @@ __global__ void export_fp_kernel(Store st, Runs runs, int row_begin, int dst_row
     if (slot < 0) return;
     using E = typename std::conditional<ES == 2, uint16_t, uint32_t>::type;
     if (dst_k) {
-        const E *ks = reinterpret_cast<const E *>(k_row_ptr(st, bh, slot));
+        const char *kc = k_cell_ptr(st, bh, slot);
         E *kd = reinterpret_cast<E *>(dst_k) + ((size_t)bh * nrows + i) * st.Dk;
-        for (int d = threadIdx.x; d < st.Dk; d += blockDim.x) kd[d] = ks[d];
+        for (int d = threadIdx.x; d < st.Dk; d += blockDim.x) kd[d] = *reinterpret_cast<const E *>(kc + kfp_off(st, slot, d));
     }
     if (dst_v) {
         const char *vc = v_cell_ptr(st, bh, slot);
         E *vd = reinterpret_cast<E *>(dst_v) + ((size_t)bh * nrows + i) * st.Dv;
-        const int t = slot & (TILE - 1);
         for (int d = threadIdx.x; d < st.Dv; d += blockDim.x)
-            vd[d] = reinterpret_cast<const E *>(vc + v_row_off(st, slot, d))[t];
+            vd[d] = *reinterpret_cast<const E *>(vc + vfp_off(st, slot, d));
     }
 }
 
@@ -442,13 +440,11 @@ __global__ void import_fp_kernel(Store st, const char *src_k, const char *src_v,
     const int slot = blockIdx.x;
     using E = typename std::conditional<ES == 2, uint16_t, uint32_t>::type;
     const E *ks = reinterpret_cast<const E *>(src_k) + ((size_t)bh * nrows + slot) * st.Dk;
-    E *kd = reinterpret_cast<E *>(const_cast<char *>(k_row_ptr(st, bh, slot)));
-    for (int d = threadIdx.x; d < st.Dk; d += blockDim.x) kd[d] = ks[d];
+    char *kc = const_cast<char *>(k_cell_ptr(st, bh, slot));
+    for (int d = threadIdx.x; d < st.Dk; d += blockDim.x) *reinterpret_cast<E *>(kc + kfp_off(st, slot, d)) = ks[d];
     const E *vs = reinterpret_cast<const E *>(src_v) + ((size_t)bh * nrows + slot) * st.Dv;
     char *vc = const_cast<char *>(v_cell_ptr(st, bh, slot));
-    const int t = slot & (TILE - 1);
-    for (int d = threadIdx.x; d < st.Dv; d += blockDim.x)
-        reinterpret_cast<E *>(vc + v_row_off(st, slot, d))[t] = vs[d];
+    for (int d = threadIdx.x; d < st.Dv; d += blockDim.x) *reinterpret_cast<E *>(vc + vfp_off(st, slot, d)) = vs[d];
 }
 
 template <int ES>
@@ -458,14 +454,14 @@ __global__ void compact_fp_kernel(Store src, Runs runs, Store dst, int nrows) {
     const int slot = row_to_slot(runs, i);
     if (slot < 0) return;
     using E = typename std::conditional<ES == 2, uint16_t, uint32_t>::type;
-    const E *ks = reinterpret_cast<const E *>(k_row_ptr(src, bh, slot));
-    E *kd = reinterpret_cast<E *>(const_cast<char *>(k_row_ptr(dst, bh, i)));
-    for (int d = threadIdx.x; d < src.Dk; d += blockDim.x) kd[d] = ks[d];
+    const char *ks = k_cell_ptr(src, bh, slot);
+    char *kd = const_cast<char *>(k_cell_ptr(dst, bh, i));
+    for (int d = threadIdx.x; d < src.Dk; d += blockDim.x)
+        *reinterpret_cast<E *>(kd + kfp_off(dst, i, d)) = *reinterpret_cast<const E *>(ks + kfp_off(src, slot, d));
     const char *vs = v_cell_ptr(src, bh, slot);
     char *vd = const_cast<char *>(v_cell_ptr(dst, bh, i));
-    const int ts = slot & (TILE - 1), td = i & (TILE - 1);
     for (int d = threadIdx.x; d < src.Dv; d += blockDim.x)
-        reinterpret_cast<E *>(vd + v_row_off(dst, i, d))[td] = reinterpret_cast<const E *>(vs + v_row_off(src, slot, d))[ts];
+        *reinterpret_cast<E *>(vd + vfp_off(dst, i, d)) = *reinterpret_cast<const E *>(vs + vfp_off(src, slot, d));
 }
 
 // which: 0 k.wq 1 k.scales 2 k.biases 3 v.wq 4 v.scales 5 v.biases; grid (nrows, BH)
