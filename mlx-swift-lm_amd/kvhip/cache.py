@@ -153,6 +153,22 @@ class _Cache:
     def trim(self, n):
         return self._lib.kvhip_cache_trim(self._h, int(n))
 
+    def prepare(self, lengths=None):
+        """`prepare(lengths:)` (KVCache.swift:96-99): a hook for batched caches; these three
+        kinds keep the protocol's empty default (:114-116)."""
+
+    def finalize(self):
+        """`finalize()` (KVCache.swift:102, default :118): nothing transient to clear."""
+
+    def inner_state(self):
+        """`innerState()` (KVCache.swift:400-402, :572-574, :939-948): the arrays `eval(cache)`
+        materialises.  The rows already live on the device; their export is `state`."""
+        return self.state
+
+    def eval(self):
+        """`eval(cache)` (LLMModel.swift:52-58): wait for the work enqueued on the current stream."""
+        L.check(self._lib.kvhip_sync(_stream()))
+
     def reserve(self, B, Hkv, Dk, Dv, dtype, tokens):
         L.check(self._lib.kvhip_cache_reserve(self._h, B, Hkv, Dk, Dv, _DT[dtype], int(tokens)))
 

@@ -57,6 +57,13 @@ public class HIPKVCache {
     public var isTrimmable: Bool { kvhip_cache_is_trimmable(handle, 0) != 0 }
     public func isTrimmable(after positions: Int) -> Bool { kvhip_cache_is_trimmable(handle, Int64(positions)) != 0 }
     @discardableResult public func trim(_ n: Int) -> Int { Int(kvhip_cache_trim(handle, Int64(n))) }
+    /// `ropeOffset` (KVCache.swift:190): `.scalar(offset)`, read before the write.
+    public var ropeOffset: Int { offset }
+    /// `prepare(lengths:)` / `finalize()` keep the protocol's empty defaults (KVCache.swift:114-118).
+    public func prepare(lengths: [Int]?) {}
+    public func finalize() {}
+    /// `eval(cache)` (LLMModel.swift:52-58): the rows are device-resident already; wait for the stream.
+    public func eval() { must(kvhip_sync(stream)) }
 
     public var metaState: [String] {
         get {

@@ -149,3 +149,17 @@ def test_growth_across_many_pages_keeps_every_row():
             assert np.array_equal(got, b), i
         else:
             assert np.array_equal(O.to_bits(got, name), O.to_bits(b, name)), i
+
+
+def test_protocol_hooks_with_empty_defaults():
+    """`prepare(lengths:)`, `finalize()`, `innerState()`, `ropeOffset` (KVCache.swift:46-120)."""
+    rng = np.random.default_rng(3)
+    for c in (kvhip.KVCacheSimple(), kvhip.RotatingKVCache(32), kvhip.QuantizedKVCache(64, 4)):
+        assert c.inner_state() == [] and c.rope_offset == 0
+        c.prepare(lengths=[3, 4])
+        _, k = randn(rng, (1, 2, 5, 64), torch.float16)
+        (c.update_quantized if isinstance(c, kvhip.QuantizedKVCache) else c.update)(k, k)
+        c.eval()
+        c.finalize()
+        assert c.rope_offset == c.offset == 5
+        assert [tuple(a.shape) for a in c.inner_state()] == [tuple(a.shape) for a in c.state]
