@@ -399,9 +399,27 @@ def resolved_kv_quantization_group_size(requested, key_head_dim, value_head_dim)
     return g or None
 
 
+def create_attention_mask(n, cache=None, window_size=None, return_array=False):
+    """`createAttentionMask(h:cache:windowSize:returnArray:)` (KVCache.swift:359-380) for `n` new
+    positions (`h.dim(1)`): the cache's own `makeMask` when there is one, else the cache-less rule."""
+    if cache is not None:
+        return cache.make_mask(n, window_size, return_array)
+    if n == 1:
+        return MaskMode.none()
+    if return_array or (window_size is not None and n > window_size):
+        plan = L.MaskPlan(mode=L.MASK_ARRAY, rows=n, cols=n, offset=0, window=int(window_size or 0))
+        return MaskMode(L.MASK_WINDOW, offset=0, window=int(window_size or 0), plan=plan)
+    return MaskMode.causal()
+
+
+def can_trim_prompt_cache(caches):
+    """`canTrimPromptCache` (KVCache.swift:2293-2295)."""
+    return all(c.is_trimmable for c in caches)
+
+
 def trim_prompt_cache(caches, num_tokens):
     """`trimPromptCache` (KVCache.swift:2302-2306)."""
-    if not caches or not all(c.is_trimmable for c in caches):
+    if not caches or not can_trim_prompt_cache(caches):
         return 0
     for c in caches[1:]:
         c.trim(num_tokens)

@@ -163,3 +163,21 @@ def test_protocol_hooks_with_empty_defaults():
         c.finalize()
         assert c.rope_offset == c.offset == 5
         assert [tuple(a.shape) for a in c.inner_state()] == [tuple(a.shape) for a in c.state]
+
+
+def test_create_attention_mask_with_and_without_a_cache():
+    """`createAttentionMask` (KVCache.swift:359-380): delegates to the cache, else the cache-less rule."""
+    assert kvhip.create_attention_mask(1).mode == L.MASK_NONE
+    assert kvhip.create_attention_mask(5).mode == L.MASK_CAUSAL
+    m = kvhip.create_attention_mask(5, window_size=3)
+    assert np.array_equal(m.array.cpu().numpy(), O.create_causal_mask(5, 0, 3))
+    m = kvhip.create_attention_mask(4, return_array=True)
+    assert np.array_equal(m.array.cpu().numpy(), O.create_causal_mask(4, 0, None))
+    c = kvhip.KVCacheSimple()
+    c.offset = 9
+    m = kvhip.create_attention_mask(3, c, window_size=2)
+    assert np.array_equal(m.array.cpu().numpy(), O.create_causal_mask(3, 9, 2))
+    r = kvhip.RotatingKVCache(8)
+    assert kvhip.can_trim_prompt_cache([c, r]) and kvhip.can_trim_prompt_cache([])
+    r.meta_state = ["0", "8", "256", "9", "1"]
+    assert not kvhip.can_trim_prompt_cache([c, r]) and kvhip.trim_prompt_cache([c, r], 2) == 0
