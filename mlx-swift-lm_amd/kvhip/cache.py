@@ -399,6 +399,37 @@ def resolved_kv_quantization_group_size(requested, key_head_dim, value_head_dim)
     return g or None
 
 
+class KVCacheConfigurationError(ValueError):
+    """`KVCacheConfigurationError` (KVCacheConfiguration.swift:256): an invalid capacity or window."""
+
+
+def make_attention_kv_cache(max_kv_size=None):
+    """`makeAttentionKVCache(parameters:)` (CacheConfiguration.swift:291-296) for the legacy
+    `maxKVSize` request: a ring of that capacity that keeps min(4, maxKVSize - 1) leading
+    tokens (KVCachePlan.swift:455-462), else an unbounded `KVCacheSimple`."""
+    if max_kv_size is None:
+        return KVCacheSimple()
+    if max_kv_size <= 0:
+        raise KVCacheConfigurationError(f"invalid KV cache capacity {max_kv_size}")
+    return RotatingKVCache(int(max_kv_size), keep=min(4, max(0, int(max_kv_size) - 1)))
+
+
+def make_sliding_window_kv_cache(window, max_kv_size=None):
+    """`makeSlidingWindowKVCache(parameters:window:)` (CacheConfiguration.swift:312-317): the
+    architecture's window capped by the legacy `maxKVSize`, no pinned prefix."""
+    if window <= 0:
+        raise KVCacheConfigurationError(f"invalid sliding window {window}")
+    if max_kv_size is not None and max_kv_size <= 0:
+        raise KVCacheConfigurationError(f"invalid KV cache capacity {max_kv_size}")
+    return RotatingKVCache(int(min(window, max_kv_size) if max_kv_size is not None else window))
+
+
+def make_prompt_cache(num_layers, max_kv_size=None):
+    """`makePromptCacheWithLayerCount(numLayers:maxKVSize:)` (KVCache.swift:2281-2290): one cache
+    per layer."""
+    return [make_attention_kv_cache(max_kv_size) for _ in range(num_layers)]
+
+
 def create_attention_mask(n, cache=None, window_size=None, return_array=False):
     """`createAttentionMask(h:cache:windowSize:returnArray:)` (KVCache.swift:359-380) for `n` new
     positions (`h.dim(1)`): the cache's own `makeMask` when there is one, else the cache-less rule."""

@@ -181,3 +181,22 @@ def test_create_attention_mask_with_and_without_a_cache():
     assert kvhip.can_trim_prompt_cache([c, r]) and kvhip.can_trim_prompt_cache([])
     r.meta_state = ["0", "8", "256", "9", "1"]
     assert not kvhip.can_trim_prompt_cache([c, r]) and kvhip.trim_prompt_cache([c, r], 2) == 0
+
+
+def test_cache_factories():
+    """`makeAttentionKVCache` / `makeSlidingWindowKVCache` / `makePromptCacheWithLayerCount`
+    (CacheConfiguration.swift:291-317, KVCache.swift:2281-2290) for the legacy `maxKVSize` request."""
+    assert isinstance(kvhip.make_attention_kv_cache(), kvhip.KVCacheSimple)
+    r = kvhip.make_attention_kv_cache(4096)
+    assert isinstance(r, kvhip.RotatingKVCache) and r.max_size == 4096 and r.meta_state[:2] == ["4", "4096"]
+    assert kvhip.make_attention_kv_cache(3).meta_state[:2] == ["2", "3"]      # keep = min(4, maxKVSize - 1)
+    assert kvhip.make_attention_kv_cache(1).meta_state[:2] == ["0", "1"]
+    w = kvhip.make_sliding_window_kv_cache(1024, max_kv_size=512)
+    assert w.max_size == 512 and w.meta_state[0] == "0"
+    assert kvhip.make_sliding_window_kv_cache(1024).max_size == 1024
+    for bad in (lambda: kvhip.make_attention_kv_cache(0), lambda: kvhip.make_sliding_window_kv_cache(0),
+                lambda: kvhip.make_sliding_window_kv_cache(8, max_kv_size=-1)):
+        with pytest.raises(kvhip.KVCacheConfigurationError):
+            bad()
+    caches = kvhip.make_prompt_cache(3, max_kv_size=64)
+    assert len(caches) == 3 and all(c.max_size == 64 for c in caches)
