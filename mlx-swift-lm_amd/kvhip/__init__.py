@@ -10,4 +10,5 @@ from .cache import (KVCacheSimple, MaskMode, QuantizedKVCache, RotatingKVCache, 
 from .rounds import (AppendOnlyRoundStrategy, KVCacheRound, KVCacheRoundCommit, KVCacheStorage,  # noqa: F401
                      RotatingRestorePoint, RotatingRoundStrategy, RotatingStagedKVCache)
 from .rope import RoPE, apply_rotary_position, attention_with_rope_and_cache_update  # noqa: F401
+from .prefill import PrefillParameters  # noqa: F401
 from .prompt_cache import KVCacheError, load_prompt_cache, save_prompt_cache  # noqa: F401
