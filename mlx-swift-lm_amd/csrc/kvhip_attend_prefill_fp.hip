@@ -26,6 +26,7 @@ typedef __bf16 b8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) uint32_t LDS_U32;
 union Op8 {
     h8 h;
     b8 b;
@@ -65,10 +66,30 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     constexpr int S = D / 32;     // contraction steps over the head dim
     constexpr int NDT = D / 16;   // 16-row tiles of out^T
     constexpr int NC = D / 64;    // 16-byte chunks per thread, for K and for V
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[2][BN * KS];
-    __shared__ __attribute__((aligned(16))) _Float16 Vs[2][D * VS];
-    __shared__ int rows_s[2][BN];
-    __shared__ int full_s[2];
+    // fp16 caches up to D = 128 move their tiles from global memory straight into LDS (no
+    // registers, no conversion, no LDS store instructions): two buffers, each the tile's 16-byte
+    // chunks in page order -- K [8-element chunk][token], V [8-token chunk][column] -- the other
+    // one filled while this one is contracted.  Everything else stages through registers into two
+    // padded buffers.
+    constexpr bool DMA = DT == 0 && D <= 128;
+    constexpr int NB = 2;
+    // (for these one array per buffer, K then V, selected by constants after inlining: the compiler
+    // follows loads into LDS per variable, and a read of one buffer then need not wait for the loads
+    // in flight into the other; the register-staged path keeps K and V in arrays of their own)
+    constexpr int KSZ = BN * D;  // 16-bit elements of a tile's K (and of its V)
+    __shared__ __attribute__((aligned(16))) uint16_t KV0[DMA ? 2 * KSZ : 8], KV1[DMA ? 2 * KSZ : 8];
+    __shared__ __attribute__((aligned(16))) uint16_t Kpad[2][DMA ? 8 : BN * KS];
+    __shared__ __attribute__((aligned(16))) _Float16 Vpad[2][DMA ? 8 : D * VS];
+    auto Ks = [&](int buf) __attribute__((always_inline)) -> uint16_t * {
+        if constexpr (DMA) return buf == 0 ? KV0 : KV1;
+        else return Kpad[buf];
+    };
+    auto Vs = [&](int buf) __attribute__((always_inline)) -> _Float16 * {
+        if constexpr (DMA) return reinterpret_cast<_Float16 *>(buf == 0 ? KV0 : KV1) + KSZ;
+        else return Vpad[buf];
+    };
+    __shared__ int rows_s[NB][BN];
+    __shared__ int full_s[NB];
 
     const Store &st = a.st;
     const int tid = threadIdx.x;
@@ -227,22 +248,61 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
             const int c = e * 256 + tid;
-            *reinterpret_cast<u4 *>(&Ks[buf][(c % BN) * KS + (c / BN) * 8]) = g.k[e];
+            *reinterpret_cast<u4 *>(&Ks(buf)[(c % BN) * KS + (c / BN) * 8]) = g.k[e];
             u4 v = g.v[e];
             if (DT == 1) v = u4{bf2_to_h2(v.x), bf2_to_h2(v.y), bf2_to_h2(v.z), bf2_to_h2(v.w)};
-            u2 *vd = reinterpret_cast<u2 *>(&Vs[buf][(c % D) * VS + (c / D) * 8]);  // rows are 8-byte aligned
+            u2 *vd = reinterpret_cast<u2 *>(&Vs(buf)[(c % D) * VS + (c / D) * 8]);  // rows are 8-byte aligned
             vd[0] = u2{v.x, v.y};
             vd[1] = u2{v.z, v.w};
         }
     };
 
-    if (tile_lo < tile_hi) {
-        fetch(tile_lo, setA);
-        stage(0, setA);
-        if (tile_lo + 1 < tile_hi) fetch(tile_lo + 1, setA);
-        if (DEEP && tile_lo + 2 < tile_hi) fetch(tile_lo + 2, setB);
+    // direct global -> LDS: lane i of a wavefront's load lands at the wavefront's LDS base + 16 i, so
+    // chunk c = e * 256 + tid goes to slot c of the buffer.  K slot (chunk cc, position pos) takes token
+    // 8 ((pos & 15) / 4) + 4 (pos / 16) + pos % 4, the order in which the S^T accumulators of one lane
+    // cover the eight tokens of one V chunk (so K operand reads are contiguous across lanes and
+    // P never moves); V slots are the page's own order.
+    [[maybe_unused]] auto dma = [&](int tile, int buf) __attribute__((always_inline)) {
+        const int slot0 = tile * BN;
+        if (tid < BN) {
+            const int slot = slot0 + tid;
+            int row;
+            if (IDENT) row = slot;
+            else row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
+            row = (row >= 0 && row < a.T) ? row : -1;
+            rows_s[buf][tid] = row;
+            const bool full = __all(row >= keep_lo && row <= keep_hi);  // the first 32 lanes of wavefront 0
+            if (tid == 0) full_s[buf] = full;
+        }
+        const char *kbase = k_cell_ptr(st, bh, slot0) + kfp_off(st, slot0, 0);
+        const char *vbase = v_cell_ptr(st, bh, slot0) + vfp_off(st, slot0, 0);
+#pragma unroll
+        for (int e = 0; e < NC; ++e) {
+            const int c = e * 256 + tid;
+            const int pos = c % BN;
+            const int tok = 8 * ((pos & 15) >> 2) + 4 * (pos >> 4) + (pos & 3);
+            const int cw = e * 256 + (tid & ~63);  // the wavefront's first slot
+            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t *>(kbase + (size_t)(c / BN) * (TILE * 16) + tok * 16),
+                                             (LDS_U32 *)(&Ks(buf)[cw * 8]), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t *>(vbase + (size_t)c * 16),
+                                             (LDS_U32 *)(&Vs(buf)[cw * 8]), 16, 0, 0);
+        }
+    };
+    // all but the `newer` most recent vector-memory operations of this wavefront have completed
+    [[maybe_unused]] auto wait_older = [&](auto N) __attribute__((always_inline)) {
+        constexpr int n = decltype(N)::value;
+        __builtin_amdgcn_s_waitcnt((n & 15) | ((n >> 4) << 14) | 0x0f70);  // vmcnt(n), others untouched
+    };
+
+    if constexpr (!DMA) {
+        if (tile_lo < tile_hi) {
+            fetch(tile_lo, setA);
+            stage(0, setA);
+            if (tile_lo + 1 < tile_hi) fetch(tile_lo + 1, setA);
+            if (DEEP && tile_lo + 2 < tile_hi) fetch(tile_lo + 2, setB);
+        }
+        __syncthreads();
     }
-    __syncthreads();
     // (fast softmax) raise query block qt's reference maximum to what the tile holds and rescale
     auto raise = [&](int qt, float tmax) __attribute__((always_inline)) {
         tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
@@ -261,8 +321,13 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     auto step = [&](int tile, int cur, Stg &g) __attribute__((always_inline)) {
         // the tile fetched two iterations ago goes to the other buffer (last read one barrier
         // ago); its registers are then free for the tile three ahead
-        if (tile + 1 < tile_hi) stage(cur ^ 1, g);
-        if (tile + LEAD < tile_hi) fetch(tile + LEAD, g);
+        if constexpr (DMA) {
+            // the other buffer was last read in the previous step, which ended with a barrier
+            if (tile + 1 < tile_hi) dma(tile + 1, cur ^ 1);
+        } else {
+            if (tile + 1 < tile_hi) stage(cur ^ 1, g);
+            if (tile + LEAD < tile_hi) fetch(tile + LEAD, g);
+        }
 
         // ---- S^T = K . Q^T: acc[qt][mt] rows = tokens 16 mt + 4 jj + i, column = query n -----
         f4 sacc[QT][2];
@@ -275,7 +340,8 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             Op8 ka[S];
 #pragma unroll
             for (int s = 0; s < S; ++s)
-                ka[s].v = *reinterpret_cast<const u4 *>(&Ks[cur][(16 * mt + n) * KS + 32 * s + 8 * jj]);
+                ka[s].v = DMA ? *reinterpret_cast<const u4 *>(&Ks(cur)[((4 * s + jj) * BN + 16 * mt + n) * 8])
+                              : *reinterpret_cast<const u4 *>(&Ks(cur)[(16 * mt + n) * KS + 32 * s + 8 * jj]);
 #pragma unroll
             for (int s = 0; s < S; ++s)
 #pragma unroll
@@ -287,7 +353,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) trow[mt][i] = rows_s[cur][16 * mt + 4 * jj + i];
+                for (int i = 0; i < 4; ++i) trow[mt][i] = rows_s[cur][DMA ? 8 * jj + 4 * mt + i : 16 * mt + 4 * jj + i];
         }
 
         // a boolean array mask is read four keys at a time where this lane's four rows are consecutive
@@ -433,10 +499,14 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             Op8 va[4];
 #pragma unroll
             for (int x = 0; x < 4; ++x) {
-                const _Float16 *vrow = &Vs[cur][(16 * (d0 + x) + n) * VS];
-                const u2 lo = *reinterpret_cast<const u2 *>(vrow + 4 * jj);
-                const u2 hi = *reinterpret_cast<const u2 *>(vrow + 16 + 4 * jj);
-                va[x].v = u4{lo.x, lo.y, hi.x, hi.y};
+                if constexpr (DMA) {  // tokens 8 jj .. 8 jj + 7 of column 16 (d0 + x) + n: one chunk
+                    va[x].v = *reinterpret_cast<const u4 *>(&Vs(cur)[(jj * D + 16 * (d0 + x) + n) * 8]);
+                } else {
+                    const _Float16 *vrow = &Vs(cur)[(16 * (d0 + x) + n) * VS];
+                    const u2 lo = *reinterpret_cast<const u2 *>(vrow + 4 * jj);
+                    const u2 hi = *reinterpret_cast<const u2 *>(vrow + 16 + 4 * jj);
+                    va[x].v = u4{lo.x, lo.y, hi.x, hi.y};
+                }
             }
 #pragma unroll
             for (int x = 0; x < 4; ++x)
@@ -444,11 +514,33 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                 for (int qt = 0; qt < QT; ++qt)
                     oacc[qt][d0 + x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[x].h, pb[qt].h, oacc[qt][d0 + x], 0, 0, 0);
         }
-        __syncthreads();
+        if constexpr (DMA) {
+            // Everything requested so far has to land before the barrier: the request made at the
+            // top of this step has had the whole step for it, so the wait is short, and an LDS read of
+            // the next step never meets a load in flight into its own buffer.  (Leaving the newest
+            // request in flight across the barrier, with a third buffer, gains nothing: the compiler
+            // cannot tell the buffers apart on every path and then makes LDS reads wait for all.)
+            wait_older(std::integral_constant<int, 0>{});
+            __syncthreads();
+        } else {
+            __syncthreads();
+        }
     };
-    for (int tile = tile_lo; tile < tile_hi; tile += 2) {
-        step(tile, 0, setA);
-        if (tile + 1 < tile_hi) step(tile + 1, 1, DEEP ? setB : setA);
+    if constexpr (DMA) {
+        if (tile_lo < tile_hi) dma(tile_lo, 0);
+        wait_older(std::integral_constant<int, 0>{});
+        __syncthreads();
+        // (unrolled by the two buffers, so that every LDS address is a constant plus the lane's)
+        for (int tile = tile_lo; tile < tile_hi; tile += 2) {
+            step(tile, 0, setA);
+            if (tile + 1 >= tile_hi) break;
+            step(tile + 1, 1, setA);
+        }
+    } else {
+        for (int tile = tile_lo; tile < tile_hi; tile += 2) {
+            step(tile, 0, setA);
+            if (tile + 1 < tile_hi) step(tile + 1, 1, DEEP ? setB : setA);
+        }
     }
 
     // ---- normalise and store: lane (n, jj) holds out[q = n][d = 16 dt + 4 jj + i] ------------
