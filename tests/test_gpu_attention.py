@@ -299,3 +299,88 @@ def test_cfg5_ragged_speculative_rollback_reduced(policy):
     for a, b in zip(c.state, o.get_state()):
         if a.dtype == torch.int32:
             assert np.array_equal(np32(a), b)
+
+
+@pytest.mark.parametrize("kind,Lq", [("q4", 1), ("q4", 4), ("q8", 2), ("fp16", 1), ("bf16", 3)])
+def test_ragged_batch_spans(policy, kind, Lq):
+    """Per-batch lengths and left padding far apart (1 .. 3000 rows visible): the decode kernels
+    divide each row's own visible range over the spans; every row must come out as under the
+    equivalent array mask (the oracle's)."""
+    rng = np.random.default_rng(11 + Lq)
+    B, Hq, Hkv, D = 7, 8, 2, 128
+    dtype = torch.bfloat16 if kind == "bf16" else torch.float16
+    name = NAME[dtype]
+    T0 = 3000 - Lq
+    if kind[0] == "q":
+        bits = int(kind[1])
+        c, o = kvhip.QuantizedKVCache(64, bits), O.QuantizedKVCache(64, bits, name)
+    else:
+        c, o = kvhip.KVCacheSimple(), O.KVCacheSimple(name)
+    k, kd = randn(rng, (B, Hkv, T0, D), dtype)
+    v, vd = randn(rng, (B, Hkv, T0, D), dtype)
+    if kind[0] == "q":
+        c.update_quantized(kd, vd, fetch=False)
+        o.update_quantized(k, v)
+    else:
+        c.update(kd, vd, fetch=False)
+        o.update(k, v)
+    scale = 1.0 / np.sqrt(D)
+    T = T0 + Lq
+    j = np.arange(T)[None, None, None, :]
+    causal = O.create_causal_mask(Lq, T - Lq)[None, None]
+    cases = {
+        "lengths": dict(lengths=np.array([T, 1, 1500, 64, T - 1, 65, 700], np.int32)),
+        "left_pad": dict(left_pad=np.array([0, T - Lq - 1, 1500, T - 64 - Lq, 1, 2047, 2300], np.int32)),
+        "both": dict(lengths=np.array([T, 900, 1500, T, 2100, 2500, T], np.int32),
+                     left_pad=np.array([0, 800, 0, 2900, 100, 2400, 2990], np.int32)),
+    }
+    kn, knd = randn(rng, (B, Hkv, Lq, D), dtype)
+    vn, vnd = randn(rng, (B, Hkv, Lq, D), dtype)
+    q, qd = randn(rng, (B, Hq, Lq, D), dtype)
+    first = True
+    for what, kw in cases.items():
+        m = np.broadcast_to(causal, (B, 1, Lq, T)).copy()
+        if "lengths" in kw:
+            m &= j < kw["lengths"][:, None, None, None]
+        if "left_pad" in kw:
+            m &= j >= kw["left_pad"][:, None, None, None]
+        mask = kvhip.MaskMode.window_mask(T - Lq, 0, **{a: torch.from_numpy(b) for a, b in kw.items()})
+        if first:
+            out = kvhip.attention_with_cache_update(qd, knd, vnd, c, scale, mask)
+            ref = O.attention_with_cache_update(q, kn, vn, o, scale, O.Mask("array", m), name)
+            first = False
+        else:
+            out = c.attend(qd, scale, mask)
+            if kind[0] == "q":
+                ref = CO.qsdpa(q, *o.get_quantized_state(), scale, m, 64, int(kind[1]), name)
+            else:
+                ref = CO.sdpa(q, o.keys[:, :, :T], o.values[:, :, :T], scale, m, name)
+        check(out, ref, f"{kind} L={Lq} {what}")
+        assert kvhip.load().kvhip_last_attend_kernel() == (0 if policy else (1 if kind[0] == "q" else 2))
+
+
+def test_ring_in_temporal_order_with_lengths(policy):
+    """A wrapped ring after a multi-token write is presented through a row map (temporal order);
+    per-batch lengths over the presented rows must bound each row's keys there too."""
+    rng = np.random.default_rng(5)
+    B, Hq, Hkv, D, M, Lq = 4, 8, 4, 128, 1024, 2
+    dtype, name = torch.float16, "float16"
+    c, o = kvhip.RotatingKVCache(M, keep=4), O.RotatingKVCache(M, keep=4)
+    k, kd = randn(rng, (B, Hkv, 700, D), dtype)
+    c.update(kd, kd.flip(-1), fetch=False)
+    o.update(k, k[..., ::-1].copy())
+    for _ in range(400):  # single-token writes wrap the ring
+        k, kd = randn(rng, (B, Hkv, 1, D), dtype)
+        c.update(kd, kd.flip(-1), fetch=False)
+        o.update(k, k[..., ::-1].copy())
+    k, kd = randn(rng, (B, Hkv, Lq, D), dtype)
+    c.update(kd, kd.flip(-1), fetch=False)
+    ok, ov = o.update(k, k[..., ::-1].copy())
+    T = ok.shape[2]
+    assert c.presented_length == T and c.idx == o.idx
+    q, qd = randn(rng, (B, Hq, Lq, D), dtype)
+    lengths = np.array([T, T - 100, 300, 77], np.int32)
+    m = O.create_causal_mask(Lq, T - Lq)[None, None] & (np.arange(T)[None, None, None, :] < lengths[:, None, None, None])
+    out = c.attend(qd, 1.0 / np.sqrt(D), kvhip.MaskMode.window_mask(T - Lq, 0, lengths=torch.from_numpy(lengths)))
+    ref = CO.sdpa(q, ok, ov, 1.0 / np.sqrt(D), m, name)
+    check(out, ref, "ring, temporal order, lengths")
