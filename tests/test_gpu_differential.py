@@ -1,0 +1,91 @@
+"""Seeded random sweep over cache kind x dtype x head size x query rows x presentation x mask:
+the library's own kernel choice against the generic kernel (which the other GPU tests pin to the
+oracle), on the same device cache.  Every case prints what it is before it runs."""
+import numpy as np
+import pytest
+import torch
+
+import kvhip
+from tests.util import np32
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS = 1e-2, 1e-3
+
+
+def _case(seed):
+    rng = np.random.default_rng(seed)
+    kind = rng.choice(["simple", "rotating", "quantized"])
+    dtype = [torch.float16, torch.bfloat16][rng.integers(2)]
+    D = int(rng.choice([64, 128, 256] if kind != "quantized" else [64, 128]))
+    B, Hkv, r = int(rng.integers(1, 6)), int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 4, 8]))
+    Lq = int(rng.choice([1, 1, 2, 4, 7, 33, 70]))
+    T0 = int(rng.choice([1, 63, 64, 65, 200, 257, 700, 1500, 2600]))
+    return rng, kind, dtype, D, B, Hkv, r, Lq, T0
+
+
+@pytest.mark.parametrize("seed", range(160))
+def test_auto_kernel_against_generic(seed):
+    rng, kind, dtype, D, B, Hkv, r, Lq, T0 = _case(seed)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+
+    def rand(*shape):
+        return torch.randn(*shape, generator=g, device="cuda").to(dtype)
+
+    if kind == "simple":
+        c = kvhip.KVCacheSimple()
+    elif kind == "rotating":
+        c = kvhip.RotatingKVCache(int(rng.choice([96, 300, 1024])), keep=int(rng.choice([0, 4])))
+    else:
+        c = kvhip.QuantizedKVCache(64, int(rng.choice([4, 8])))
+    upd = c.update_quantized if kind == "quantized" else c.update
+    upd(rand(B, Hkv, T0, D), rand(B, Hkv, T0, D), fetch=False)
+    for _ in range(int(rng.integers(0, 40)) if kind == "rotating" else 0):  # walk (and wrap) the ring
+        upd(rand(B, Hkv, 1, D), rand(B, Hkv, 1, D), fetch=False)
+    upd(rand(B, Hkv, Lq, D), rand(B, Hkv, Lq, D), fetch=False)
+    T = c.presented_length
+    Lq = min(Lq, T)
+    q = rand(B, Hkv * r, Lq, D)
+    which = rng.choice(["none", "causal", "window", "lengths", "left_pad", "bool", "additive"])
+    if which == "none":
+        mask = kvhip.MaskMode.none()
+    elif which == "causal":
+        mask = kvhip.MaskMode.causal()
+    elif which == "window":
+        mask = kvhip.MaskMode.window_mask(T - Lq, int(rng.integers(1, T + 2)))
+    elif which == "lengths":
+        lens = torch.from_numpy(rng.integers(1, T + 1, size=B).astype(np.int32))
+        mask = kvhip.MaskMode.window_mask(T - Lq, 0, lengths=lens)
+    elif which == "left_pad":
+        pad = torch.from_numpy(rng.integers(0, max(T - Lq, 1), size=B).astype(np.int32))
+        mask = kvhip.MaskMode.window_mask(T - Lq, int(rng.choice([0, 50])), left_pad=pad)
+    else:
+        shape = [(B, 1, Lq, T), (1, 1, Lq, T), (B, Hkv * r, Lq, T)][rng.integers(3)]
+        keep = rng.random(shape) < 0.7
+        keep[..., int(rng.integers(T))] = True  # no row without a key
+        if which == "bool":
+            mask = kvhip.MaskMode.from_array(torch.from_numpy(keep).cuda())
+        else:
+            add = np.where(keep, rng.standard_normal(shape).astype(np.float32), -np.inf)
+            mask = kvhip.MaskMode.from_array(torch.from_numpy(add).to(dtype).cuda())
+    scale = float(rng.choice([D ** -0.5, 0.05, -0.1]))
+    print(f"seed {seed}: {kind} {dtype} D{D} B{B} Hkv{Hkv} r{r} L{Lq} T{T} mask {which} scale {scale:.3f}", flush=True)
+    lib = kvhip.load()
+    try:
+        lib.kvhip_set_kernel_policy(1)
+        ref = np32(c.attend(q, scale, mask))
+        lib.kvhip_set_kernel_policy(0)
+        out = np32(c.attend(q, scale, mask))
+        chosen = lib.kvhip_last_attend_kernel()
+    finally:
+        lib.kvhip_set_kernel_policy(0)
+    assert np.isfinite(ref).all() and np.isfinite(out).all(), f"kernel {chosen}"
+    d = np.abs(out.astype(np.float64) - ref.astype(np.float64))
+    # One ulp of a 16-bit output at the largest magnitude may separate two correctly rounded results;
+    # with a handful of keys the outputs are as large as single V rows and, the probabilities being
+    # rounded to the cache's dtype before the second product (as the reference does), a good part
+    # of them round the other way: hence the quarter ulp on the mean.
+    ulp = float(np.abs(ref).max()) * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10)
+    assert d.max() <= max(MAX_ABS, ulp) and d.mean() <= max(MEAN_ABS, ulp / 4), \
+        f"kernel {chosen}: max-abs {d.max():.3e} mean-abs {d.mean():.3e}"
