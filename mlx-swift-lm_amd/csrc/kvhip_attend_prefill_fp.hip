@@ -27,6 +27,18 @@ typedef float f4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) uint32_t LDS_U32;
+
+// 16 bytes per lane from global memory straight into LDS: lane i's land at `lds_wave_base` + 16 i
+// (the base is the same for the whole wavefront).  Written as assembly, with the waits for it placed
+// by hand (s_waitcnt vmcnt): the compiler's own bookkeeping of such loads makes every LDS read that
+// follows one wait for all vector-memory operations in flight, register loads included, wherever it
+// cannot prove on every path which buffer the load fills.  Its waits for its own loads stay correct:
+// vector-memory operations complete in order, so an operation it does not count only makes a wait
+// stricter.
+__device__ __forceinline__ void load_to_lds(const void *src, const void *lds_wave_base) {
+    const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(LDS_U32 *)lds_wave_base);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(base) : "memory", "m0");
+}
 union Op8 {
     h8 h;
     b8 b;
@@ -60,32 +72,27 @@ template <int D, int DT, bool IDENT, int QT, int MM>
 __global__ void __launch_bounds__(256, 2)
 prefill_fp_kernel(AttendArgs a, int nsplit) {
     constexpr int BM = 64 * QT;
-    constexpr int KS = D + 8;     // 16-bit elements per K row in LDS
     constexpr int VS = BN + 4;    // halves per V^T row in LDS: 18 dwords, so the 16 rows an operand
                                   // read touches fall in distinct banks
     constexpr int S = D / 32;     // contraction steps over the head dim
     constexpr int NDT = D / 16;   // 16-row tiles of out^T
     constexpr int NC = D / 64;    // 16-byte chunks per thread, for K and for V
-    // fp16 caches up to D = 128 move their tiles from global memory straight into LDS (no
-    // registers, no conversion, no LDS store instructions): two buffers, each the tile's 16-byte
-    // chunks in page order -- K [8-element chunk][token], V [8-token chunk][column] -- the other
-    // one filled while this one is contracted.  Everything else stages through registers into two
-    // padded buffers.
-    constexpr bool DMA = DT == 0 && D <= 128;
+    // K tiles move from global memory straight into LDS (no registers, no LDS store instructions):
+    // two buffers, each the tile's 16-byte chunks in page order, [8-element chunk][token], the other
+    // one filled while this one is contracted.  fp16 caches up to D = 128 move V the same way,
+    // [8-token chunk][column]; otherwise V is staged through registers (bf16 is converted to fp16 on
+    // the way) into two padded buffers of V^T.
+    constexpr bool VDMA = DT == 0 && D <= 128;
     constexpr int NB = 2;
-    // (for these one array per buffer, K then V, selected by constants after inlining: the compiler
-    // follows loads into LDS per variable, and a read of one buffer then need not wait for the loads
-    // in flight into the other; the register-staged path keeps K and V in arrays of their own)
+    // (one array per buffer, K then V, selected by constants after inlining: the compiler follows
+    // loads into LDS per variable, and a read of one buffer then need not wait for the loads in
+    // flight into the other)
     constexpr int KSZ = BN * D;  // 16-bit elements of a tile's K (and of its V)
-    __shared__ __attribute__((aligned(16))) uint16_t KV0[DMA ? 2 * KSZ : 8], KV1[DMA ? 2 * KSZ : 8];
-    __shared__ __attribute__((aligned(16))) uint16_t Kpad[2][DMA ? 8 : BN * KS];
-    __shared__ __attribute__((aligned(16))) _Float16 Vpad[2][DMA ? 8 : D * VS];
-    auto Ks = [&](int buf) __attribute__((always_inline)) -> uint16_t * {
-        if constexpr (DMA) return buf == 0 ? KV0 : KV1;
-        else return Kpad[buf];
-    };
+    __shared__ __attribute__((aligned(16))) uint16_t KV0[VDMA ? 2 * KSZ : KSZ], KV1[VDMA ? 2 * KSZ : KSZ];
+    __shared__ __attribute__((aligned(16))) _Float16 Vpad[2][VDMA ? 8 : D * VS];
+    auto Ks = [&](int buf) __attribute__((always_inline)) -> uint16_t * { return buf == 0 ? KV0 : KV1; };
     auto Vs = [&](int buf) __attribute__((always_inline)) -> _Float16 * {
-        if constexpr (DMA) return reinterpret_cast<_Float16 *>(buf == 0 ? KV0 : KV1) + KSZ;
+        if constexpr (VDMA) return reinterpret_cast<_Float16 *>(buf == 0 ? KV0 : KV1) + KSZ;
         else return Vpad[buf];
     };
     __shared__ int rows_s[NB][BN];
@@ -206,49 +213,28 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     }
 
     // ---- staging ------------------------------------------------------------------------
-    // chunk c = e * 256 + tid.  K: token c % 32 of the tile, 8-element chunk c / 32.  V: column
+    // chunk c = e * 256 + tid.  K: slot c % 32 of the tile, 8-element chunk c / 32.  V: column
     // c % D, 8-token chunk c / D of the 32 tokens of this tile.
-    // Up to D = 128 two register sets alternate, so a tile is requested two iterations before
-    // it is written to LDS and three before it is contracted; D = 256 has registers for one set
-    // (one iteration less of lead).
-    constexpr bool DEEP = D <= 128;
-    constexpr int LEAD = DEEP ? 3 : 2;
+    // V through registers: a tile's V is requested one iteration before it is written to LDS and two
+    // before it is contracted.
+    constexpr int LEAD = 2;
     struct Stg {
-        u4 k[NC], v[NC];
-        int row;
+        u4 v[NC];
     };
-    Stg setA, setB;
-    setA.row = setB.row = -1;
-    auto fetch = [&](int tile, Stg &g) __attribute__((always_inline)) {
+    Stg setA;
+    [[maybe_unused]] auto fetch = [&](int tile, Stg &g) __attribute__((always_inline)) {
         const int slot0 = tile * BN;
-        if (tid < BN) {
-            const int slot = slot0 + tid;
-            int row;
-            if (IDENT) row = slot;
-            else row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
-            g.row = (row >= 0 && row < a.T) ? row : -1;
-        }
-        // pages are interleaved in 16-byte chunks (K: [8-element chunk][token], V: [8-token chunk][column]):
-        // consecutive threads take consecutive tokens of one K chunk, consecutive columns of one V chunk
-        const char *kbase = k_cell_ptr(st, bh, slot0) + kfp_off(st, slot0, 0);
         const char *vbase = v_cell_ptr(st, bh, slot0) + vfp_off(st, slot0, 0);
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
             const int c = e * 256 + tid;
-            g.k[e] = *reinterpret_cast<const u4 *>(kbase + (size_t)(c / BN) * (TILE * 16) + (c % BN) * 16);
             g.v[e] = *reinterpret_cast<const u4 *>(vbase + (size_t)(c / D) * (D * 16) + (c % D) * 16);
         }
     };
-    auto stage = [&](int buf, const Stg &g) __attribute__((always_inline)) {
-        if (tid < BN) rows_s[buf][tid] = g.row;
-        if (wave == 0) {
-            const bool full = __all(lane >= BN || (g.row >= keep_lo && g.row <= keep_hi));
-            if (lane == 0) full_s[buf] = full;
-        }
+    [[maybe_unused]] auto stage = [&](int buf, const Stg &g) __attribute__((always_inline)) {
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
             const int c = e * 256 + tid;
-            *reinterpret_cast<u4 *>(&Ks(buf)[(c % BN) * KS + (c / BN) * 8]) = g.k[e];
             u4 v = g.v[e];
             if (DT == 1) v = u4{bf2_to_h2(v.x), bf2_to_h2(v.y), bf2_to_h2(v.z), bf2_to_h2(v.w)};
             u2 *vd = reinterpret_cast<u2 *>(&Vs(buf)[(c % D) * VS + (c / D) * 8]);  // rows are 8-byte aligned
@@ -258,19 +244,21 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     };
 
     // direct global -> LDS: lane i of a wavefront's load lands at the wavefront's LDS base + 16 i, so
-    // chunk c = e * 256 + tid goes to slot c of the buffer.  K slot (chunk cc, position pos) takes token
-    // 8 ((pos & 15) / 4) + 4 (pos / 16) + pos % 4, the order in which the S^T accumulators of one lane
-    // cover the eight tokens of one V chunk (so K operand reads are contiguous across lanes and
-    // P never moves); V slots are the page's own order.
-    [[maybe_unused]] auto dma = [&](int tile, int buf) __attribute__((always_inline)) {
+    // chunk c = e * 256 + tid goes to slot c of the buffer.  With V loaded the same way, K slot
+    // (chunk cc, position pos) takes token 8 ((pos & 15) / 4) + 4 (pos / 16) + pos % 4, the order in
+    // which the S^T accumulators of one lane cover the eight tokens of one V chunk (so K operand
+    // reads are contiguous across lanes and P never moves), and V slots are the page's own order;
+    // with V^T staged through registers K slots are the tokens in order.
+    auto dma = [&](int tile, int buf) __attribute__((always_inline)) {
         const int slot0 = tile * BN;
         if (tid < BN) {
-            const int slot = slot0 + tid;
+            const int pos = tid;
+            const int slot = slot0 + (VDMA ? 8 * ((pos & 15) >> 2) + 4 * (pos >> 4) + (pos & 3) : pos);
             int row;
             if (IDENT) row = slot;
             else row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
             row = (row >= 0 && row < a.T) ? row : -1;
-            rows_s[buf][tid] = row;
+            rows_s[buf][tid] = row;  // the row of the token in K slot `tid`
             const bool full = __all(row >= keep_lo && row <= keep_hi);  // the first 32 lanes of wavefront 0
             if (tid == 0) full_s[buf] = full;
         }
@@ -280,29 +268,17 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         for (int e = 0; e < NC; ++e) {
             const int c = e * 256 + tid;
             const int pos = c % BN;
-            const int tok = 8 * ((pos & 15) >> 2) + 4 * (pos >> 4) + (pos & 3);
+            const int tok = VDMA ? 8 * ((pos & 15) >> 2) + 4 * (pos >> 4) + (pos & 3) : pos;
             const int cw = e * 256 + (tid & ~63);  // the wavefront's first slot
-            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t *>(kbase + (size_t)(c / BN) * (TILE * 16) + tok * 16),
-                                             (LDS_U32 *)(&Ks(buf)[cw * 8]), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t *>(vbase + (size_t)c * 16),
-                                             (LDS_U32 *)(&Vs(buf)[cw * 8]), 16, 0, 0);
+            load_to_lds(kbase + (size_t)(c / BN) * (TILE * 16) + tok * 16, &Ks(buf)[cw * 8]);
+            if constexpr (VDMA) load_to_lds(vbase + (size_t)c * 16, &Vs(buf)[cw * 8]);
         }
     };
     // all but the `newer` most recent vector-memory operations of this wavefront have completed
-    [[maybe_unused]] auto wait_older = [&](auto N) __attribute__((always_inline)) {
-        constexpr int n = decltype(N)::value;
-        __builtin_amdgcn_s_waitcnt((n & 15) | ((n >> 4) << 14) | 0x0f70);  // vmcnt(n), others untouched
+    auto wait_older = [&](auto N) __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(decltype(N)::value) : "memory");
     };
 
-    if constexpr (!DMA) {
-        if (tile_lo < tile_hi) {
-            fetch(tile_lo, setA);
-            stage(0, setA);
-            if (tile_lo + 1 < tile_hi) fetch(tile_lo + 1, setA);
-            if (DEEP && tile_lo + 2 < tile_hi) fetch(tile_lo + 2, setB);
-        }
-        __syncthreads();
-    }
     // (fast softmax) raise query block qt's reference maximum to what the tile holds and rescale
     auto raise = [&](int qt, float tmax) __attribute__((always_inline)) {
         tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
@@ -319,15 +295,15 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     };
     // one tile: `cur` is the LDS buffer that holds it, `g` the register set that holds the next one
     auto step = [&](int tile, int cur, Stg &g) __attribute__((always_inline)) {
-        // the tile fetched two iterations ago goes to the other buffer (last read one barrier
-        // ago); its registers are then free for the tile three ahead
-        if constexpr (DMA) {
-            // the other buffer was last read in the previous step, which ended with a barrier
-            if (tile + 1 < tile_hi) dma(tile + 1, cur ^ 1);
-        } else {
+        // The other buffers were last read in the previous step, which ended with a barrier.
+        // V^T first (the tile fetched in the previous step; its registers are then free for the tile
+        // after it), the K request last: the compiler's waits for those registers -- it does not
+        // count the K request -- must not meet it.
+        if constexpr (!VDMA) {
             if (tile + 1 < tile_hi) stage(cur ^ 1, g);
             if (tile + LEAD < tile_hi) fetch(tile + LEAD, g);
         }
+        if (tile + 1 < tile_hi) dma(tile + 1, cur ^ 1);
 
         // ---- S^T = K . Q^T: acc[qt][mt] rows = tokens 16 mt + 4 jj + i, column = query n -----
         f4 sacc[QT][2];
@@ -340,8 +316,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             Op8 ka[S];
 #pragma unroll
             for (int s = 0; s < S; ++s)
-                ka[s].v = DMA ? *reinterpret_cast<const u4 *>(&Ks(cur)[((4 * s + jj) * BN + 16 * mt + n) * 8])
-                              : *reinterpret_cast<const u4 *>(&Ks(cur)[(16 * mt + n) * KS + 32 * s + 8 * jj]);
+                ka[s].v = *reinterpret_cast<const u4 *>(&Ks(cur)[((4 * s + jj) * BN + 16 * mt + n) * 8]);
 #pragma unroll
             for (int s = 0; s < S; ++s)
 #pragma unroll
@@ -353,7 +328,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) trow[mt][i] = rows_s[cur][DMA ? 8 * jj + 4 * mt + i : 16 * mt + 4 * jj + i];
+                for (int i = 0; i < 4; ++i) trow[mt][i] = rows_s[cur][16 * mt + 4 * jj + i];  // by K slot
         }
 
         // a boolean array mask is read four keys at a time where this lane's four rows are consecutive
@@ -499,7 +474,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             Op8 va[4];
 #pragma unroll
             for (int x = 0; x < 4; ++x) {
-                if constexpr (DMA) {  // tokens 8 jj .. 8 jj + 7 of column 16 (d0 + x) + n: one chunk
+                if constexpr (VDMA) {  // tokens 8 jj .. 8 jj + 7 of column 16 (d0 + x) + n: one chunk
                     va[x].v = *reinterpret_cast<const u4 *>(&Vs(cur)[(jj * D + 16 * (d0 + x) + n) * 8]);
                 } else {
                     const _Float16 *vrow = &Vs(cur)[(16 * (d0 + x) + n) * VS];
@@ -514,33 +489,34 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                 for (int qt = 0; qt < QT; ++qt)
                     oacc[qt][d0 + x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[x].h, pb[qt].h, oacc[qt][d0 + x], 0, 0, 0);
         }
-        if constexpr (DMA) {
-            // Everything requested so far has to land before the barrier: the request made at the
-            // top of this step has had the whole step for it, so the wait is short, and an LDS read of
-            // the next step never meets a load in flight into its own buffer.  (Leaving the newest
-            // request in flight across the barrier, with a third buffer, gains nothing: the compiler
-            // cannot tell the buffers apart on every path and then makes LDS reads wait for all.)
-            wait_older(std::integral_constant<int, 0>{});
-            __syncthreads();
-        } else {
-            __syncthreads();
-        }
-    };
-    if constexpr (DMA) {
-        if (tile_lo < tile_hi) dma(tile_lo, 0);
+        // What was requested at the top of this step has to land before the barrier: it has had the
+        // whole step for it, so the wait is short, and an LDS read of the next step never meets a load
+        // in flight into its own buffer.  (Leaving the newest LDS request in flight across the
+        // barrier, with a third buffer, measured the same.)
+        // A plain barrier instead of __syncthreads(): nothing but LDS traffic (drained here) has to
+        // be ordered across it.
         wait_older(std::integral_constant<int, 0>{});
-        __syncthreads();
-        // (unrolled by the two buffers, so that every LDS address is a constant plus the lane's)
-        for (int tile = tile_lo; tile < tile_hi; tile += 2) {
-            step(tile, 0, setA);
-            if (tile + 1 >= tile_hi) break;
-            step(tile + 1, 1, setA);
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    };
+    if (tile_lo < tile_hi) {
+        dma(tile_lo, 0);
+        if constexpr (!VDMA) {
+            fetch(tile_lo, setA);
+            stage(0, setA);
+            if (tile_lo + 1 < tile_hi) fetch(tile_lo + 1, setA);
         }
-    } else {
-        for (int tile = tile_lo; tile < tile_hi; tile += 2) {
-            step(tile, 0, setA);
-            if (tile + 1 < tile_hi) step(tile + 1, 1, DEEP ? setB : setA);
-        }
+    }
+    wait_older(std::integral_constant<int, 0>{});
+    // (the same wait once more in a form the compiler's bookkeeping sees: it then knows that the
+    // query operands have arrived, and does not wait for them -- and with them for every load just
+    // issued -- inside the loop)
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), others untouched
+    __syncthreads();
+    // (unrolled by the two buffers, so that every LDS address is a constant plus the lane's)
+    for (int tile = tile_lo; tile < tile_hi; tile += 2) {
+        step(tile, 0, setA);
+        if (tile + 1 >= tile_hi) break;
+        step(tile + 1, 1, setA);
     }
 
     // ---- normalise and store: lane (n, jj) holds out[q = n][d = 16 dt + 4 jj + i] ------------
