@@ -79,10 +79,10 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     constexpr int NC = D / 64;    // 16-byte chunks per thread, for K and for V
     // K tiles move from global memory straight into LDS (no registers, no LDS store instructions):
     // two buffers, each the tile's 16-byte chunks in page order, [8-element chunk][token], the other
-    // one filled while this one is contracted.  fp16 caches up to D = 128 move V the same way,
-    // [8-token chunk][column]; otherwise V is staged through registers (bf16 is converted to fp16 on
-    // the way) into two padded buffers of V^T.
-    constexpr bool VDMA = DT == 0 && D <= 128;
+    // one filled while this one is contracted.  fp16 caches move V the same way, [8-token
+    // chunk][column]; bf16 V is staged through registers (converted to fp16 on the way) into two
+    // padded buffers of V^T.
+    constexpr bool VDMA = DT == 0;
     constexpr int NB = 2;
     // (one array per buffer, K then V, selected by constants after inlining: the compiler follows
     // loads into LDS per variable, and a read of one buffer then need not wait for the loads in
