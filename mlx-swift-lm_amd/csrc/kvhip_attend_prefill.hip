@@ -23,6 +23,7 @@ namespace {
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 union Op8 {
     h8 h;
     uint32_t u[4];
@@ -103,18 +104,22 @@ prefill_kernel(AttendArgs a, int nsplit) {
         const int rep = q_ok[qt] ? i / a.L : 0;
         q_l[qt] = q_ok[qt] ? i - rep * a.L : 0;
         q_h[qt] = hk * r + rep;
-        const size_t qoff = ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D;
+        // rows past R read row (rep 0, l 0), which is in bounds, and are zeroed: no branch around the
+        // loads, which are one 16-byte piece per contraction step, all in flight together
+        const u4 *qp = reinterpret_cast<const u4 *>(
+            reinterpret_cast<const uint16_t *>(a.q) + ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D + 8 * jj);
+        u4 raw[S];
+#pragma unroll
+        for (int s = 0; s < S; ++s) raw[s] = qp[4 * s];
 #pragma unroll
         for (int s = 0; s < S; ++s) {
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                float v0 = 0.f, v1 = 0.f;
-                if (q_ok[qt]) {
-                    v0 = Elem<DT>::load(a.q, qoff + 32 * s + 8 * jj + 2 * w);
-                    v1 = Elem<DT>::load(a.q, qoff + 32 * s + 8 * jj + 2 * w + 1);
-                    v0 = round_dt<DT>(v0 * a.scale);  // the reference rounds q * scale to T
-                    v1 = round_dt<DT>(v1 * a.scale);
-                }
+                const uint32_t pair = raw[s][w];
+                float v0 = DT == 0 ? (float)__builtin_bit_cast(_Float16, (uint16_t)pair) : __uint_as_float(pair << 16);
+                float v1 = DT == 0 ? (float)__builtin_bit_cast(_Float16, (uint16_t)(pair >> 16)) : __uint_as_float(pair & 0xffff0000u);
+                v0 = q_ok[qt] ? round_dt<DT>(v0 * a.scale) : 0.f;  // the reference rounds q * scale to T
+                v1 = q_ok[qt] ? round_dt<DT>(v1 * a.scale) : 0.f;
                 qop[qt][s].u[w] = h2_bits(v0, v1);
             }
         }
