@@ -13,7 +13,9 @@
  *  - Every pointer named `keys`, `values`, `queries`, `out`, `dst`, `src` or
  *    `data` is a DEVICE pointer to a dense row-major array; shapes are given in
  *    the comment of each function.  Inputs are borrowed for the duration of the
- *    call's enqueued work only.
+ *    call's enqueued work only.  The element type's own alignment suffices (a
+ *    contiguous view that starts anywhere inside an allocation is accepted);
+ *    16-byte aligned arrays are read at full width.
  *  - `stream` is a `hipStream_t` passed as `void *` (NULL = the default
  *    stream).  Device work is enqueued on it; host-side counters (`offset`,
  *    `idx`) advance when the call returns, as the reference's do while it

@@ -200,3 +200,42 @@ def test_cache_factories():
             bad()
     caches = kvhip.make_prompt_cache(3, max_kv_size=64)
     assert len(caches) == 3 and all(c.max_size == 64 for c in caches)
+
+
+@pytest.mark.parametrize("kind", ["simple", "quantized", "rotating"])
+@pytest.mark.parametrize("Lq", [1, 4, 40])
+def test_inputs_at_odd_element_offsets(kind, Lq):
+    """Keys, values and queries that start one element into an allocation (contiguous views, 2-byte
+    aligned only): same cache state and outputs, bit for bit, as from 256-byte aligned copies."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(3)
+    B, Hq, Hkv, D, T0 = 2, 8, 2, 128, 300
+    dtype = torch.float16
+
+    def odd(*shape):
+        n = int(np.prod(shape))
+        flat = torch.randn(n + 1, generator=g, device="cuda").to(dtype)
+        v = flat[1:].view(*shape)
+        assert v.data_ptr() % 4 == 2 and v.is_contiguous()
+        return v
+
+    def make():
+        if kind == "simple":
+            return kvhip.KVCacheSimple()
+        if kind == "rotating":
+            return kvhip.RotatingKVCache(256, keep=4)
+        return kvhip.QuantizedKVCache(64, 4)
+
+    k0, v0, k1, v1, q = odd(B, Hkv, T0, D), odd(B, Hkv, T0, D), odd(B, Hkv, Lq, D), odd(B, Hkv, Lq, D), odd(B, Hq, Lq, D)
+    outs, states = [], []
+    for aligned in (False, True):
+        f = (lambda t: t.clone()) if aligned else (lambda t: t)
+        c = make()
+        upd = c.update_quantized if kind == "quantized" else c.update
+        upd(f(k0), f(v0), fetch=False)
+        upd(f(k1), f(v1), fetch=False)
+        mask = kvhip.MaskMode.none() if Lq == 1 else kvhip.MaskMode.causal()
+        outs.append(c.attend(f(q), D ** -0.5, mask))
+        states.append([a.clone() for a in c.state])
+    assert torch.equal(outs[0], outs[1])
+    assert len(states[0]) == len(states[1]) and all(torch.equal(a, b) for a, b in zip(*states))
