@@ -742,9 +742,12 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     auto buf_of = [&](int n) -> uint32_t * { return (n & 1) ? bufB : bufA; };
 
     if (my_tiles > 0) {
+        // (the queries first: loads complete in order, and a wait for queries requested after the
+        // first pieces would be a wait for those pieces too -- in every iteration, the compiler
+        // placing one wait for all ways into the loop)
+        load_queries();
         load_k(buf_of(0), 0);
         if (NP > 1) load_k(buf_of(1), 1); else load_v(buf_of(1), 0);
-        load_queries();
         for (int done = 0; done < my_tiles; ++done) {
             int row;
             if (IDENT) row = slot_cur;
