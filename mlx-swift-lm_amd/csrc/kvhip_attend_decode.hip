@@ -234,21 +234,28 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) {
         const int i = 4 * rg + qi;
-        const int rep = i / a.L, l = i - rep * a.L;
+        // rows past R read row 0 (in bounds) and count as zero: no branch around the loads, which
+        // are then all in flight together instead of one after the other
+        const bool ok = i < R;
+        const int rep = ok ? i / a.L : 0, l = ok ? i - rep * a.L : 0;
         const size_t qoff = ((size_t)(b * a.Hq + hk * r + rep) * a.L + l) * D;
+        float raw[NQA][4];
+#pragma unroll
+        for (int x = 0; x < NQA; ++x) {
+            const int step = 16 * x + blk;
+            const int w = step / GEO::WSTEPS, h = step % GEO::WSTEPS;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) raw[x][k] = Elem<DT>::load(a.q, qoff + w * GEO::EPW + GEO::elem(h, k));
+        }
         float part[G];
 #pragma unroll
         for (int g = 0; g < G; ++g) part[g] = 0.f;
 #pragma unroll
         for (int x = 0; x < NQA; ++x) {
-            const int step = 16 * x + blk;
-            const int w = step / GEO::WSTEPS, h = step % GEO::WSTEPS;
             float qv[4];
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                const int d = w * GEO::EPW + GEO::elem(h, k);
-                float v = 0.f;
-                if (i < R) v = (float)(_Float16)round_dt<DT>(Elem<DT>::load(a.q, qoff + d) * a.scale);
+                const float v = ok ? (float)(_Float16)round_dt<DT>(raw[x][k] * a.scale) : 0.f;
                 part[(64 * x) / GS] += v;
                 qv[k] = GEO::hi(k) ? v * 0.0625f : v;
             }
