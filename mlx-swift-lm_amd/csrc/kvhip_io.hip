@@ -232,9 +232,35 @@ __device__ __forceinline__ void unpack8(const u4v &raw, const void *row, int d0,
     }
 }
 
-// Quantize the eight elements a thread holds; `gl` adjacent lanes share a group.
-template <int BITS>
-__device__ __forceinline__ void quantize8(const float (&w)[8], int gl, float &scale, float &bias, uint32_t (&code)[8]) {
+// v of the lane that the data-parallel-primitive control CTRL names (all lanes take part)
+template <int CTRL> __device__ __forceinline__ float dpp_lane(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v),
+                                                                 CTRL, 0xF, 0xF, false));
+}
+
+// Min/max over GL (4, 8 or 16) adjacent lanes without LDS round trips: two quad permutes, then
+// the mirror of each half row and of each row (the lanes of a quad, then of a half row, already
+// agree, so the mirrored lane holds the other half's result).  Minimum and maximum do not depend
+// on the order of the reduction, so the values are those of group_minmax.
+template <int GL> __device__ __forceinline__ void group_minmax_dpp(float &mn, float &mx) {
+    mn = fminf(mn, dpp_lane<0xB1>(mn));  // quad_perm [1,0,3,2]
+    mx = fmaxf(mx, dpp_lane<0xB1>(mx));
+    mn = fminf(mn, dpp_lane<0x4E>(mn));  // quad_perm [2,3,0,1]
+    mx = fmaxf(mx, dpp_lane<0x4E>(mx));
+    if constexpr (GL >= 8) {
+        mn = fminf(mn, dpp_lane<0x141>(mn));  // row_half_mirror
+        mx = fmaxf(mx, dpp_lane<0x141>(mx));
+    }
+    if constexpr (GL >= 16) {
+        mn = fminf(mn, dpp_lane<0x140>(mn));  // row_mirror
+        mx = fmaxf(mx, dpp_lane<0x140>(mx));
+    }
+}
+
+// Quantize the eight elements a thread holds; GL adjacent lanes share a group.  The codes come
+// back as integer-valued floats in [0, 2^BITS - 1].
+template <int BITS, int GL>
+__device__ __forceinline__ void quantize8(const float (&w)[8], float &scale, float &bias, float (&q)[8]) {
     const float nb = (float)((1 << BITS) - 1);
     float mn = w[0], mx = w[0];
 #pragma unroll
@@ -242,40 +268,61 @@ __device__ __forceinline__ void quantize8(const float (&w)[8], int gl, float &sc
         mn = fminf(mn, w[j]);
         mx = fmaxf(mx, w[j]);
     }
-    group_minmax(mn, mx, gl);
+    group_minmax_dpp<GL>(mn, mx);
     affine_params(mn, mx, nb, scale, bias);
-    // code = rint((w - bias) / scale), clamped.  The quotient is first formed with one exact
-    // reciprocal per thread: it lies within two float32 ulps of the correctly rounded quotient
-    // (|q| <= 2^BITS, so within 2^-19), which can only change the rounded integer when the quotient
-    // sits that close to a half-integer.  Those elements (about one in 10^4) are redone with the
-    // exact division, so the codes are the reference's bit for bit.
-    const float inv = __fdiv_rn(1.0f, scale);
-    bool near_tie = false;
+    // code = rint((w - bias) / scale), clamped.  The quotient is first formed with the hardware
+    // reciprocal (one ulp): product and reciprocal together put it within 2^-22 relative, so within
+    // 2^-14 absolute (|quotient| <= 2^8), of the correctly rounded quotient, which can only change
+    // the rounded integer when the quotient sits that close to a half-integer.  Those elements
+    // (about one in 10^4) are redone with the exact division, so the codes are the reference's
+    // bit for bit.
+    const float inv = __builtin_amdgcn_rcpf(scale);
+    float dev = 0.0f;  // largest distance of a quotient from its rounded integer
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const float r = __fmul_rn(__fsub_rn(w[j], bias), inv);
-        const float q = rintf(r);
-        near_tie = near_tie || (fabsf(r - q) > 0.4999f);
-        code[j] = (uint32_t)fminf(fmaxf(q, 0.0f), nb);
+        const float c = rintf(r);
+        dev = fmaxf(dev, fabsf(r - c));
+        q[j] = fminf(fmaxf(c, 0.0f), nb);
     }
-    if (near_tie) {
+    if (dev > 0.4999f) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) code[j] = affine_code(w[j], scale, bias, nb);
+        for (int j = 0; j < 8; ++j) q[j] = (float)affine_code(w[j], scale, bias, nb);
     }
 }
 
-// grid (whole tiles, BH), 256 threads; slot0 is a multiple of 64; 16-bit dtypes, Dk == Dv == 32 NC
-template <int DT, int BITS, int NC>
+// Four integer-valued floats in [0, 255] as the bytes of one word, first value lowest.
+__device__ __forceinline__ uint32_t pack_bytes(float a, float b, float c, float d) {
+    uint32_t w = __builtin_amdgcn_cvt_pk_u8_f32(a, 0, 0);
+    w = __builtin_amdgcn_cvt_pk_u8_f32(b, 1, w);
+    w = __builtin_amdgcn_cvt_pk_u8_f32(c, 2, w);
+    return __builtin_amdgcn_cvt_pk_u8_f32(d, 3, w);
+}
+// Four integer-valued floats in [0, 15] as the nibbles of a 16-bit value, first value lowest
+// (the sums stay below 2^16, so float32 arithmetic is exact).
+__device__ __forceinline__ uint32_t pack_nibbles(float a, float b, float c, float d) {
+    return (uint32_t)__builtin_fmaf(d, 4096.0f, __builtin_fmaf(c, 256.0f, __builtin_fmaf(b, 16.0f, a)));
+}
+// (scale, bias) of one group as the pair of 16-bit values the cache holds
+template <int DT> __device__ __forceinline__ uint32_t pack_scale_bias(float scale, float bias) {
+    if (DT == 0)
+        return (uint32_t)__half_as_ushort(__float2half_rn(scale)) | ((uint32_t)__half_as_ushort(__float2half_rn(bias)) << 16);
+    return (uint32_t)Elem<1>::bits(scale) | ((uint32_t)Elem<1>::bits(bias) << 16);
+}
+
+// grid (whole tiles, BH), 256 threads; slot0 is a multiple of 64; 16-bit dtypes, Dk == Dv == 32 NC;
+// GL = group size / 8 lanes share a quantization group; ROPE = false carries no rotation code
+template <int DT, int BITS, int NC, int GL, bool ROPE>
 __global__ void __launch_bounds__(256)
 append_quant_tile_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, RopeDev rope) {
     constexpr int D = 32 * NC;
+    constexpr int GS = 8 * GL;
     constexpr int TPR = D / 8;   // threads per row
     constexpr int VP = D + 8;    // byte pitch of a token's V codes in LDS
     __shared__ __attribute__((aligned(8))) uint8_t vcodes[TILE * VP];
     const int bh = blockIdx.y;
     const int slot_t = slot0 + blockIdx.x * TILE;
     const int l_t = src0 + blockIdx.x * TILE;
-    const int gl = st.gs / 8;
     const char *kbase = keys + ((size_t)bh * L + l_t) * D * 2;
     const char *vbase = values + ((size_t)bh * L + l_t) * D * 2;
     u4v kraw[NC], vraw[NC];
@@ -285,43 +332,35 @@ append_quant_tile_kernel(Store st, const char *keys, const char *values, int L, 
         kraw[e] = *reinterpret_cast<const u4v *>(kbase + (size_t)c * 16);
         vraw[e] = *reinterpret_cast<const u4v *>(vbase + (size_t)c * 16);
     }
+    const RopeDev no_rope;
 #pragma unroll
     for (int e = 0; e < NC; ++e) {
         const int c = e * 256 + threadIdx.x;
         const int r = c / TPR, d0 = (c - r * TPR) * 8;
         const int slot = slot_t + r;
-        float w[8], scale, bias;
-        uint32_t code[8];
+        float w[8], q[8], scale, bias;
         // ---- K: packed words in natural order ------------------------------------------------
-        unpack8<DT>(kraw[e], kbase + (size_t)r * D * 2, d0, rope, rope_pos(rope, bh, l_t + r), w);
-        quantize8<BITS>(w, gl, scale, bias, code);
+        if constexpr (ROPE) unpack8<DT>(kraw[e], kbase + (size_t)r * D * 2, d0, rope, rope_pos(rope, bh, l_t + r), w);
+        else unpack8<DT>(kraw[e], nullptr, d0, no_rope, 0, w);
+        quantize8<BITS, GL>(w, scale, bias, q);
         uint32_t *kw = reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot)));
         if (BITS == 4) {
-            uint32_t word = 0;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) word |= code[j] << (4 * j);
-            kw[d0 / 8] = word;
+            kw[d0 / 8] = pack_nibbles(q[0], q[1], q[2], q[3]) | (pack_nibbles(q[4], q[5], q[6], q[7]) << 16);
         } else {
-            const uint32_t lo = code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24);
-            const uint32_t hi = code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24);
-            *reinterpret_cast<uint2 *>(kw + d0 / 4) = make_uint2(lo, hi);
+            *reinterpret_cast<uint2 *>(kw + d0 / 4) =
+                make_uint2(pack_bytes(q[0], q[1], q[2], q[3]), pack_bytes(q[4], q[5], q[6], q[7]));
         }
-        if ((d0 % st.gs) == 0) {
-            char *sb = const_cast<char *>(ksb_row_ptr(st, bh, slot));
-            Elem<DT>::store(sb, 2 * (d0 / st.gs), scale);
-            Elem<DT>::store(sb, 2 * (d0 / st.gs) + 1, bias);
-        }
+        if ((d0 % GS) == 0)
+            reinterpret_cast<uint32_t *>(const_cast<char *>(ksb_row_ptr(st, bh, slot)))[d0 / GS] =
+                pack_scale_bias<DT>(scale, bias);
         // ---- V: codes as bytes, transposed below ------------------------------------------------
-        unpack8<DT>(vraw[e], vbase + (size_t)r * D * 2, d0, RopeDev(), 0, w);
-        quantize8<BITS>(w, gl, scale, bias, code);
+        unpack8<DT>(vraw[e], nullptr, d0, no_rope, 0, w);
+        quantize8<BITS, GL>(w, scale, bias, q);
         *reinterpret_cast<uint2 *>(&vcodes[r * VP + d0]) =
-            make_uint2(code[0] | (code[1] << 8) | (code[2] << 16) | (code[3] << 24),
-                       code[4] | (code[5] << 8) | (code[6] << 16) | (code[7] << 24));
-        if ((d0 % st.gs) == 0) {
-            char *sb = const_cast<char *>(vsb_row_ptr(st, bh, slot));
-            Elem<DT>::store(sb, 2 * (d0 / st.gs), scale);
-            Elem<DT>::store(sb, 2 * (d0 / st.gs) + 1, bias);
-        }
+            make_uint2(pack_bytes(q[0], q[1], q[2], q[3]), pack_bytes(q[4], q[5], q[6], q[7]));
+        if ((d0 % GS) == 0)
+            reinterpret_cast<uint32_t *>(const_cast<char *>(vsb_row_ptr(st, bh, slot)))[d0 / GS] =
+                pack_scale_bias<DT>(scale, bias);
     }
     __syncthreads();
     // each thread assembles 16 bytes (4 words) of one transposed row; consecutive threads
@@ -692,14 +731,25 @@ hipError_t launch_append_quant(const Store &st, const void *keys, const void *va
     if (e != hipSuccess) return e;
     dim3 grid(t.tiles, st.BH), block(256);
     const int a0 = src0 + t.head, b0 = slot0 + t.head;
-#define TILE_CALL(DT, BITS, NC)                                                                      \
-    hipLaunchKernelGGL((append_quant_tile_kernel<DT, BITS, NC>), grid, block, 0, s, st, (const char *)keys, \
+#define TILE_CALL(DT, BITS, NC, GL, RP)                                                                  \
+    hipLaunchKernelGGL((append_quant_tile_kernel<DT, BITS, NC, GL, RP>), grid, block, 0, s, st, (const char *)keys, \
                        (const char *)values, L, a0, b0, r)
+#define TILE_RP(DT, BITS, NC, GL)                           \
+    do {                                                    \
+        if (r.dims > 0) TILE_CALL(DT, BITS, NC, GL, true);  \
+        else TILE_CALL(DT, BITS, NC, GL, false);            \
+    } while (0)
+#define TILE_GL(DT, BITS, NC)                               \
+    do {                                                    \
+        if (st.gs == 32) TILE_RP(DT, BITS, NC, 4);          \
+        else if (st.gs == 64) TILE_RP(DT, BITS, NC, 8);     \
+        else TILE_RP(DT, BITS, NC, 16);                     \
+    } while (0)
 #define TILE_NC(DT, BITS)                              \
     do {                                               \
-        if (st.Dk == 64) TILE_CALL(DT, BITS, 2);       \
-        else if (st.Dk == 128) TILE_CALL(DT, BITS, 4); \
-        else TILE_CALL(DT, BITS, 8);                   \
+        if (st.Dk == 64) TILE_GL(DT, BITS, 2);         \
+        else if (st.Dk == 128) TILE_GL(DT, BITS, 4);   \
+        else TILE_GL(DT, BITS, 8);                     \
     } while (0)
     if (st.dtype == KVHIP_F16) {
         if (st.bits == 4) TILE_NC(0, 4); else TILE_NC(0, 8);
@@ -707,6 +757,8 @@ hipError_t launch_append_quant(const Store &st, const void *keys, const void *va
         if (st.bits == 4) TILE_NC(1, 4); else TILE_NC(1, 8);
     }
 #undef TILE_NC
+#undef TILE_GL
+#undef TILE_RP
 #undef TILE_CALL
     e = hipGetLastError();
     if (e != hipSuccess) return e;
