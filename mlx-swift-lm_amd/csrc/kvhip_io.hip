@@ -257,26 +257,16 @@ template <int GL> __device__ __forceinline__ void group_minmax_dpp(float &mn, fl
     }
 }
 
-// Quantize the eight elements a thread holds; GL adjacent lanes share a group.  The codes come
-// back as integer-valued floats in [0, 2^BITS - 1].
-template <int BITS, int GL>
-__device__ __forceinline__ void quantize8(const float (&w)[8], float &scale, float &bias, float (&q)[8]) {
+// Codes of the eight elements a thread holds, as integer-valued floats in [0, 2^BITS - 1], from
+// the parameters of their group; `inv` is the hardware reciprocal of `scale`.
+// code = rint((w - bias) / scale), clamped.  The quotient is first formed with the reciprocal
+// (one ulp): product and reciprocal together put it within 2^-22 relative, so within 2^-14
+// absolute (|quotient| <= 2^8), of the correctly rounded quotient, which can only change the
+// rounded integer when the quotient sits that close to a half-integer.  Those elements (about
+// one in 10^4) are redone with the exact division, so the codes are the reference's bit for bit.
+template <int BITS>
+__device__ __forceinline__ void codes8(const float (&w)[8], float scale, float bias, float inv, float (&q)[8]) {
     const float nb = (float)((1 << BITS) - 1);
-    float mn = w[0], mx = w[0];
-#pragma unroll
-    for (int j = 1; j < 8; ++j) {
-        mn = fminf(mn, w[j]);
-        mx = fmaxf(mx, w[j]);
-    }
-    group_minmax_dpp<GL>(mn, mx);
-    affine_params(mn, mx, nb, scale, bias);
-    // code = rint((w - bias) / scale), clamped.  The quotient is first formed with the hardware
-    // reciprocal (one ulp): product and reciprocal together put it within 2^-22 relative, so within
-    // 2^-14 absolute (|quotient| <= 2^8), of the correctly rounded quotient, which can only change
-    // the rounded integer when the quotient sits that close to a half-integer.  Those elements
-    // (about one in 10^4) are redone with the exact division, so the codes are the reference's
-    // bit for bit.
-    const float inv = __builtin_amdgcn_rcpf(scale);
     float dev = 0.0f;  // largest distance of a quotient from its rounded integer
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -289,6 +279,11 @@ __device__ __forceinline__ void quantize8(const float (&w)[8], float &scale, flo
 #pragma unroll
         for (int j = 0; j < 8; ++j) q[j] = (float)affine_code(w[j], scale, bias, nb);
     }
+}
+
+// `v` of the lane whose number is byte_addr / 4
+__device__ __forceinline__ float lane_value(int byte_addr, float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(byte_addr, __builtin_bit_cast(int, v)));
 }
 
 // Four integer-valued floats in [0, 255] as the bytes of one word, first value lowest.
@@ -311,7 +306,12 @@ template <int DT> __device__ __forceinline__ uint32_t pack_scale_bias(float scal
 }
 
 // grid (whole tiles, BH), 256 threads; slot0 is a multiple of 64; 16-bit dtypes, Dk == Dv == 32 NC;
-// GL = group size / 8 lanes share a quantization group; ROPE = false carries no rotation code
+// GL = group size / 8 lanes share a quantization group; ROPE = false carries no rotation code.
+// A thread holds 16-byte chunks of K and of V rows (a "chunk-instance" each), up to eight at a
+// time.  The extrema of every chunk-instance are reduced over the lanes of its group; then the
+// affine parameters -- four exact divisions, the costly part -- are worked out once per group
+// instead of once per lane: lane j of a group takes chunk-instance j (and j + GL, ...), writes
+// that group's (scale, bias) pair, and the other lanes fetch bias and reciprocal from it.
 template <int DT, int BITS, int NC, int GL, bool ROPE>
 __global__ void __launch_bounds__(256)
 append_quant_tile_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, RopeDev rope) {
@@ -319,6 +319,10 @@ append_quant_tile_kernel(Store st, const char *keys, const char *values, int L, 
     constexpr int GS = 8 * GL;
     constexpr int TPR = D / 8;   // threads per row
     constexpr int VP = D + 8;    // byte pitch of a token's V codes in LDS
+    constexpr int EB = NC < 4 ? NC : 4;    // chunks of K and of V per batch
+    constexpr int NI = 2 * EB;             // chunk-instances per batch: (chunk e0 + i / 2, K or V by i & 1)
+    constexpr int SH = GL < NI ? GL : NI;  // lanes of a group that work out parameters
+    constexpr int PER = NI / SH;           // chunk-instances per such lane
     __shared__ __attribute__((aligned(8))) uint8_t vcodes[TILE * VP];
     const int bh = blockIdx.y;
     const int slot_t = slot0 + blockIdx.x * TILE;
@@ -333,34 +337,82 @@ append_quant_tile_kernel(Store st, const char *keys, const char *values, int L, 
         vraw[e] = *reinterpret_cast<const u4v *>(vbase + (size_t)c * 16);
     }
     const RopeDev no_rope;
+    const float nb = (float)((1 << BITS) - 1);
+    const int lane = threadIdx.x & 63;
+    const int pos = lane & (GL - 1);            // place in the group
+    const int psel = pos & (SH - 1);
+    const int gbase4 = (lane & ~(GL - 1)) * 4;  // byte address (lane number x 4) of the group's first lane
+    const int r_t = threadIdx.x / TPR;          // row of this thread's chunk 0; chunk e lies 256 / TPR rows further
+    const int d0 = (threadIdx.x - r_t * TPR) * 8;
+    const int page_off = (slot_t & (PAGE - 1));
+    const size_t cell_idx = (size_t)(slot_t >> PAGE_SHIFT) * st.BH + bh;
 #pragma unroll
-    for (int e = 0; e < NC; ++e) {
-        const int c = e * 256 + threadIdx.x;
-        const int r = c / TPR, d0 = (c - r * TPR) * 8;
-        const int slot = slot_t + r;
-        float w[8], q[8], scale, bias;
-        // ---- K: packed words in natural order ------------------------------------------------
-        if constexpr (ROPE) unpack8<DT>(kraw[e], kbase + (size_t)r * D * 2, d0, rope, rope_pos(rope, bh, l_t + r), w);
-        else unpack8<DT>(kraw[e], nullptr, d0, no_rope, 0, w);
-        quantize8<BITS, GL>(w, scale, bias, q);
-        uint32_t *kw = reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot)));
-        if (BITS == 4) {
-            kw[d0 / 8] = pack_nibbles(q[0], q[1], q[2], q[3]) | (pack_nibbles(q[4], q[5], q[6], q[7]) << 16);
-        } else {
-            *reinterpret_cast<uint2 *>(kw + d0 / 4) =
-                make_uint2(pack_bytes(q[0], q[1], q[2], q[3]), pack_bytes(q[4], q[5], q[6], q[7]));
+    for (int e0 = 0; e0 < NC; e0 += EB) {
+        float w[NI][8], mn[NI], mx[NI];
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int e = e0 + i / 2;
+            if ((i & 1) == 0) {
+                const int r = r_t + e * (256 / TPR);
+                if constexpr (ROPE) unpack8<DT>(kraw[e], kbase + (size_t)r * D * 2, d0, rope, rope_pos(rope, bh, l_t + r), w[i]);
+                else unpack8<DT>(kraw[e], nullptr, d0, no_rope, 0, w[i]);
+            } else {
+                unpack8<DT>(vraw[e], nullptr, d0, no_rope, 0, w[i]);
+            }
+            float a = w[i][0], b = w[i][0];
+#pragma unroll
+            for (int j = 1; j < 8; ++j) {
+                a = fminf(a, w[i][j]);
+                b = fmaxf(b, w[i][j]);
+            }
+            group_minmax_dpp<GL>(a, b);
+            mn[i] = a;
+            mx[i] = b;
         }
-        if ((d0 % GS) == 0)
-            reinterpret_cast<uint32_t *>(const_cast<char *>(ksb_row_ptr(st, bh, slot)))[d0 / GS] =
-                pack_scale_bias<DT>(scale, bias);
-        // ---- V: codes as bytes, transposed below ------------------------------------------------
-        unpack8<DT>(vraw[e], nullptr, d0, no_rope, 0, w);
-        quantize8<BITS, GL>(w, scale, bias, q);
-        *reinterpret_cast<uint2 *>(&vcodes[r * VP + d0]) =
-            make_uint2(pack_bytes(q[0], q[1], q[2], q[3]), pack_bytes(q[4], q[5], q[6], q[7]));
-        if ((d0 % GS) == 0)
-            reinterpret_cast<uint32_t *>(const_cast<char *>(vsb_row_ptr(st, bh, slot)))[d0 / GS] =
-                pack_scale_bias<DT>(scale, bias);
+        float sc[PER], bi[PER], iv[PER];
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            float a = mn[k * SH], b = mx[k * SH];
+#pragma unroll
+            for (int j = 1; j < SH; ++j) {
+                a = psel == j ? mn[k * SH + j] : a;
+                b = psel == j ? mx[k * SH + j] : b;
+            }
+            affine_params(a, b, nb, sc[k], bi[k]);
+            iv[k] = __builtin_amdgcn_rcpf(sc[k]);
+            if (pos < SH) {
+                const int i = psel + k * SH;  // this lane's chunk-instance
+                const int row = page_off + r_t + (e0 + i / 2) * (256 / TPR);
+                char *sb = (i & 1) ? const_cast<char *>(st.vsb) + cell_idx * st.vsb_cell + (size_t)row * st.vsb_row
+                                   : const_cast<char *>(st.ksb) + cell_idx * st.ksb_cell + (size_t)row * st.ksb_row;
+                reinterpret_cast<uint32_t *>(sb)[d0 / GS] = pack_scale_bias<DT>(sc[k], bi[k]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int e = e0 + i / 2;
+            const int r = r_t + e * (256 / TPR);
+            const int src = gbase4 + (i % SH) * 4;
+            const float scale = lane_value(src, sc[i / SH]);
+            const float bias = lane_value(src, bi[i / SH]);
+            const float inv = lane_value(src, iv[i / SH]);
+            float q[8];
+            codes8<BITS>(w[i], scale, bias, inv, q);
+            if ((i & 1) == 0) {
+                // ---- K: packed words in natural order --------------------------------------------
+                uint32_t *kw = reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot_t + r)));
+                if (BITS == 4) {
+                    kw[d0 / 8] = pack_nibbles(q[0], q[1], q[2], q[3]) | (pack_nibbles(q[4], q[5], q[6], q[7]) << 16);
+                } else {
+                    *reinterpret_cast<uint2 *>(kw + d0 / 4) =
+                        make_uint2(pack_bytes(q[0], q[1], q[2], q[3]), pack_bytes(q[4], q[5], q[6], q[7]));
+                }
+            } else {
+                // ---- V: codes as bytes, transposed below -----------------------------------------
+                *reinterpret_cast<uint2 *>(&vcodes[r * VP + d0]) =
+                    make_uint2(pack_bytes(q[0], q[1], q[2], q[3]), pack_bytes(q[4], q[5], q[6], q[7]));
+            }
+        }
     }
     __syncthreads();
     // each thread assembles 16 bytes (4 words) of one transposed row; consecutive threads
@@ -724,7 +776,8 @@ hipError_t launch_append_quant(const Store &st, const void *keys, const void *va
     if (n <= 0) return hipSuccess;
     const RopeDev r = rope ? *rope : RopeDev();
     const bool tiled = st.es == 2 && st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 128 || st.Dk == 256) &&
-                       (st.bits == 4 || st.bits == 8) && (st.gs == 32 || st.gs == 64 || st.gs == 128);
+                       (st.bits == 4 || st.bits == 8) && (st.gs == 32 || st.gs == 64 || st.gs == 128) &&
+                       st.Dk % st.gs == 0;
     const TileSplit t = tile_split(slot0, n);
     if (!tiled || t.tiles == 0) return launch_append_quant_rows(st, keys, values, L, src0, slot0, n, s, r);
     hipError_t e = launch_append_quant_rows(st, keys, values, L, src0, slot0, t.head, s, r);
