@@ -131,6 +131,25 @@ def test_quantized_prompt_append_on_rounding_ties(bits):
     check_quantized_state(cache, ocache, torch.float16)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("D,gs", [(64, 32), (64, 64), (128, 32), (128, 64), (128, 128), (256, 32), (256, 64), (256, 128)])
+def test_quantized_prompt_append_every_tile_shape(dtype, bits, D, gs):
+    """Whole 64-token tiles for every head size and group size the tile quantizer is built for (how
+    many lanes share a group, and how many groups a lane works parameters out for, differ between
+    them), with a ragged head and tail around the tiles."""
+    rng = np.random.default_rng(D + gs + bits)
+    B, H = 2, 2
+    cache = kvhip.QuantizedKVCache(gs, bits)
+    ocache = O.QuantizedKVCache(gs, bits, NAME[dtype])
+    for L in (7, 210, 64):
+        k, kd = randn(rng, (B, H, L, D), dtype, 3.0)
+        v, vd = randn(rng, (B, H, L, D), dtype, 0.25)
+        cache.update_quantized(kd, vd, fetch=False)
+        ocache.update_quantized(k, v)
+        check_quantized_state(cache, ocache, dtype)
+
+
 def test_quantized_group_size_fallback_and_errors():
     # KVCacheTests.swift:477-501: QuantizedKVCache(64, 4) fed D=32 -> groupSize 32
     rng = np.random.default_rng(0)
