@@ -46,7 +46,7 @@ def main():
     ap.add_argument("--context", type=int, default=CTX)
     ap.add_argument("--batch", type=int, default=B)
     ap.add_argument("--cpu-steps", type=int, default=2, help="decode steps timed on the CPU baseline (0 = skip)")
-    ap.add_argument("--workload", default="cfg3", choices=["cfg3", "cfg2", "cfg4", "cfg5"],
+    ap.add_argument("--workload", default="cfg3", choices=["cfg3", "cfg1", "cfg2", "cfg4", "cfg5"],
                     help="cfg3 (default) is the configuration the metric is quoted on; the others are the "
                          "remaining BASELINE.json configs (reported as one JSON object each)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -166,7 +166,15 @@ def main():
                "sample": f"{args.cpu_steps} decode attention steps at B={nb}, T={t_last} "
                          f"(oracle/kv_oracle.c kvo_qsdpa, OpenMP; restated reference CPU path, not MLX)"}
         d = np.abs(gpu_last.astype(np.float64) - ref.astype(np.float64))
-        parity = {"max_abs": float(d.max()), "mean_abs": float(d.mean()), "vs": "oracle at full size, last step"}
+        # The oracle keeps the reference's rounding points (scores and probabilities rounded to
+        # float16); the kernel rounds the scores the same way but keeps the probabilities in float32.
+        # With this workload's peaked rows (one key holding more than half the weight, |V| up to 60) a
+        # handful of outputs differ by more than 1e-2 through that rounding alone, so the share of
+        # outputs inside the bound and a high quantile are reported beside the maximum.
+        parity = {"max_abs": float(d.max()), "mean_abs": float(d.mean()),
+                  "fraction_within_1e-2": float((d <= 1e-2).mean()),
+                  "quantile_0.9999_abs": float(np.quantile(d, 0.9999)),
+                  "vs": "oracle at full size, last step"}
 
     line = {
         "metric": "KV-attn decode tok/s + HBM GB/s (% of peak), Llama-3-8B shape 4-bit KV 32k",
@@ -194,7 +202,7 @@ def _timed(torch, fn, steps):
 
 
 def other_workload(args, torch, kvhip, L, dev):
-    """BASELINE.json configs[1], [3], [4] on synthetic data; returns one JSON-able dict."""
+    """BASELINE.json configs[0], [1], [3], [4] on synthetic data; returns one JSON-able dict."""
     import ctypes as C
     lib = kvhip.load()
     g = torch.Generator(device=dev)
@@ -204,6 +212,61 @@ def other_workload(args, torch, kvhip, L, dev):
         n, ms = C.c_int32(), C.c_double()
         L.check(lib.kvhip_profile_read(C.byref(n), C.byref(ms)))
         return ms.value / max(n.value, 1), n.value
+
+    if args.workload == "cfg1":
+        # the reference's own CPU-runnable case: B1, 16q/4kv, D64, fp16, 8-bit g64; prefill 512 under
+        # .causal, then 128 x (append one token + quantized SDPA).  Latency-bound (0.3 MB per step).
+        import numpy as np
+        from oracle import c_oracle as CO
+        from oracle import kv_oracle as O
+        Bn, Hq, Hkv, D = 1, 16, 4, 64
+        scale = 0.125
+        rng = np.random.default_rng(0)
+
+        def draw(shape):
+            a = O.round_to(rng.standard_normal(shape).astype(np.float32), "float16")
+            return a, torch.from_numpy(a).to(dev).to(torch.float16)
+
+        qp, qpd = draw((Bn, Hq, 512, D))
+        kp, kpd = draw((Bn, Hkv, 512, D))
+        vp, vpd = draw((Bn, Hkv, 512, D))
+        steps = [(draw((Bn, Hq, 1, D)), draw((Bn, Hkv, 1, D)), draw((Bn, Hkv, 1, D))) for _ in range(128)]
+
+        def run_gpu():
+            c = kvhip.QuantizedKVCache(64, 8)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            outs = [kvhip.attention_with_cache_update(qpd, kpd, vpd, c, scale, c.make_mask(512))]
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for (_, qd), (_, kd), (_, vd) in steps:
+                outs.append(kvhip.attention_with_cache_update(qd, kd, vd, c, scale, c.make_mask(1)))
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+            return outs, t1 - t0, t2 - t1
+
+        run_gpu()
+        outs, t_pf, t_dec = min((run_gpu() for _ in range(5)), key=lambda r: r[1] + r[2])
+        o = O.QuantizedKVCache(64, 8, "float16")
+        c0 = time.perf_counter()
+        qk, qv = o.update_quantized(kp, vp)
+        refs = [CO.qsdpa(qp, qk, qv, scale, "causal", 64, 8, "float16")]
+        c1 = time.perf_counter()
+        for (q, _), (k, _), (v, _) in steps:
+            qk, qv = o.update_quantized(k, v)
+            refs.append(CO.qsdpa(q, qk, qv, scale, None, 64, 8, "float16"))
+        c2 = time.perf_counter()
+        d = [np.abs(a.float().cpu().numpy().astype(np.float64) - r.astype(np.float64)) for a, r in zip(outs, refs)]
+        return {"workload": "configs[0]: QuantizedKVCache 8-bit g64, B1 16q/4kv D64 fp16, prefill 512 (.causal) + 128 "
+                            "decode steps of append + quantized SDPA",
+                "prefill_ms": round(t_pf * 1e3, 4), "decode_step_us": round(t_dec / 128 * 1e6, 2),
+                "decode_tokens_per_s": round(128 / t_dec, 1),
+                "cpu_baseline": {"prefill_ms": round((c1 - c0) * 1e3, 3), "decode_step_us": round((c2 - c1) / 128 * 1e6, 1),
+                                 "cores": CO.num_threads(), "kind": "port",
+                                 "sample": "the whole workload (numpy cache restatement + oracle/kv_oracle.c kvo_qsdpa); "
+                                           "restated reference CPU path, not MLX"},
+                "parity": {"max_abs": float(max(x.max() for x in d)),
+                           "mean_abs": float(np.mean([x.mean() for x in d])), "vs": "oracle, prefill and all 128 steps"}}
 
     if args.workload == "cfg2":
         # KVCacheSimple fp16 append + SDPA decode, B8, 32q/8kv, D128, grow to 8192 one token per step
