@@ -464,8 +464,8 @@ bool attend_prefill_supported(const AttendArgs &a) {
     if (s.Dk != s.Dv) return false;
     if (s.Dk != 64 && s.Dk != 128 && s.Dk != 256) return false;
     if (s.bits != 0 && s.bits != 4 && s.bits != 8) return false;
-    if (s.bits != 0 && (s.gs < 32 || s.Dk > 128)) return false;
-    return (a.Hq / a.Hkv) * a.L > 16;
+    if (s.bits != 0 && s.gs < 32) return false;
+    return true;  // 16 rows or fewer come here only when the decode kernels do not take the shape
 }
 
 // 128 query rows per workgroup reuse each staged tile twice as often as 64; 64 rows are
@@ -530,10 +530,12 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
         if (st.dtype == KVHIP_F16) PF_QT(BITS, D, 0); \
         else PF_QT(BITS, D, 1);                  \
     } while (0)
-#define PF_D(BITS)                               \
-    do {                                         \
-        if (st.Dk == 64) PF_DT(BITS, 64);        \
-        else PF_DT(BITS, 128);                   \
+#define PF_D(BITS)                                    \
+    do {                                              \
+        if (st.Dk == 64) PF_DT(BITS, 64);             \
+        else if (st.Dk == 128) PF_DT(BITS, 128);      \
+        else if (st.dtype == KVHIP_F16) PF(BITS, 256, 0, 1); /* 64 query rows per workgroup only */ \
+        else PF(BITS, 256, 1, 1);                     \
     } while (0)
     if (st.bits == 4) PF_D(4);
     else if (st.bits == 8) PF_D(8);

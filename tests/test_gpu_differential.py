@@ -89,3 +89,62 @@ def test_auto_kernel_against_generic(seed):
     ulp = float(np.abs(ref).max()) * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10)
     assert d.max() <= max(MAX_ABS, ulp) and d.mean() <= max(MEAN_ABS, ulp / 4), \
         f"kernel {chosen}: max-abs {d.max():.3e} mean-abs {d.mean():.3e}"
+
+
+@pytest.mark.parametrize("seed", range(72))
+def test_quantized_shapes_against_generic(seed):
+    """Quantized caches over head size x group size x bits x query rows (decode rows included: the
+    shapes the decode kernels do not take go to the prefill tile, not to the generic kernel)."""
+    rng = np.random.default_rng(1000 + seed)
+    D = [64, 128, 256][seed % 3]
+    gs = [32, 64, 128][(seed // 3) % 3]
+    if gs > D:
+        gs = 64
+    bits = [4, 8][(seed // 9) % 2]
+    dtype = [torch.float16, torch.bfloat16][(seed // 18) % 2]
+    B, Hkv, r = int(rng.integers(1, 4)), int(rng.choice([1, 2])), int(rng.choice([1, 4, 8]))
+    Lq = int(rng.choice([1, 1, 2, 4, 5, 40, 70]))
+    T0 = int(rng.choice([1, 31, 64, 200, 257, 700, 1300]))
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+
+    def rand(*shape):
+        return torch.randn(*shape, generator=g, device="cuda").to(dtype)
+
+    c = kvhip.QuantizedKVCache(gs, bits)
+    c.update_quantized(rand(B, Hkv, T0, D), rand(B, Hkv, T0, D), fetch=False)
+    c.update_quantized(rand(B, Hkv, Lq, D), rand(B, Hkv, Lq, D), fetch=False)
+    assert c.group_size == gs
+    T = c.offset
+    q = rand(B, Hkv * r, Lq, D)
+    which = rng.choice(["none", "causal", "left_pad", "bool"])
+    if which == "none":
+        mask = kvhip.MaskMode.none()
+    elif which == "causal":
+        mask = kvhip.MaskMode.causal()
+    elif which == "left_pad":
+        pad = torch.from_numpy(rng.integers(0, max(T - Lq, 1), size=B).astype(np.int32))
+        mask = kvhip.MaskMode.window_mask(T - Lq, 0, left_pad=pad)
+    else:
+        keep = rng.random((B, 1, Lq, T)) < 0.7
+        keep[..., int(rng.integers(T))] = True
+        mask = kvhip.MaskMode.from_array(torch.from_numpy(keep).cuda())
+    scale = D ** -0.5
+    print(f"seed {seed}: {dtype} D{D} g{gs} {bits}-bit B{B} Hkv{Hkv} r{r} L{Lq} T{T} mask {which}", flush=True)
+    lib = kvhip.load()
+    try:
+        lib.kvhip_set_kernel_policy(1)
+        ref = np32(c.attend(q, scale, mask))
+        lib.kvhip_set_kernel_policy(0)
+        out = np32(c.attend(q, scale, mask))
+        chosen = lib.kvhip_last_attend_kernel()
+    finally:
+        lib.kvhip_set_kernel_policy(0)
+    assert chosen != 0, "a quantized cache of a supported head size fell back to the generic kernel"
+    assert np.isfinite(ref).all() and np.isfinite(out).all(), f"kernel {chosen}"
+    d = np.abs(out.astype(np.float64) - ref.astype(np.float64))
+    # two results that each lie within one step of the 16-bit output type of the exact value may
+    # differ by two steps (the generic kernel also rounds the probabilities to that type)
+    ulp = float(np.abs(ref).max()) * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10)
+    assert d.max() <= max(MAX_ABS, 2 * ulp) and d.mean() <= max(MEAN_ABS, ulp / 4), \
+        f"kernel {chosen}: max-abs {d.max():.3e} mean-abs {d.mean():.3e}"
