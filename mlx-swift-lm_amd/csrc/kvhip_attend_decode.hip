@@ -205,7 +205,7 @@ template <int BITS, int D, int GS, int DT, int RG, int MM, int NW>
 __global__ void __launch_bounds__(NW * 64, NW == 4 ? 2 : 1)
 decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     using GEO = Geo<BITS>;
-    constexpr int G = D / GS;      // quantization groups per row (1 or 2)
+    constexpr int G = D / GS;      // quantization groups per row (1, 2 or 4)
     constexpr int NH = D / 64;     // 64-column halves of the output
     constexpr int NQA = D / 64;    // query operand register pairs (16 steps of 4 elements each)
     constexpr int RR = 4 * RG;     // query rows carried
@@ -483,27 +483,33 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                     for (int h = 0; h < NH; ++h) oacc[rg][h][i] *= alpha;
                 }
             }
-            uint32_t x[4];
+            constexpr int GP = (G + 1) / 2;  // groups travel through the transpose two to a register
+            uint32_t x[GP][4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 // exp2(-inf) = 0 covers dead lanes; m_use is finite even before any live token
                 const float p = fast_exp2((sc[i] - m_use[rg][i]) * LOG2E);
                 l_part[rg][i] += p;
-                float pv[2] = {0.f, 0.f};
+                float pv[2 * GP];
+                pv[2 * GP - 1] = 0.f;
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
                     bacc[rg][g][i] = __builtin_fmaf(p, t.vb[g], bacc[rg][g][i]);
                     pv[g] = p * vsf[g];
                 }
-                x[i] = pack_h2(pv[0], pv[1]);
+#pragma unroll
+                for (int j = 0; j < GP; ++j) x[j][i] = pack_h2(pv[2 * j], pv[2 * j + 1]);
             }
-            // lane (blk, i) now gets, in x[k], row i's value for token 4 blk + k
-            quad_transpose(x, lane);
-            pa[rg][0].u[0] = __builtin_amdgcn_perm(x[1], x[0], 0x05040100u);
-            pa[rg][0].u[1] = __builtin_amdgcn_perm(x[3], x[2], 0x05040100u);
-            if (G > 1) {
-                pa[rg][G - 1].u[0] = __builtin_amdgcn_perm(x[1], x[0], 0x07060302u);
-                pa[rg][G - 1].u[1] = __builtin_amdgcn_perm(x[3], x[2], 0x07060302u);
+            // lane (blk, i) now gets, in x[j][k], row i's value for token 4 blk + k
+#pragma unroll
+            for (int j = 0; j < GP; ++j) {
+                quad_transpose(x[j], lane);
+                pa[rg][2 * j].u[0] = __builtin_amdgcn_perm(x[j][1], x[j][0], 0x05040100u);
+                pa[rg][2 * j].u[1] = __builtin_amdgcn_perm(x[j][3], x[j][2], 0x05040100u);
+                if (2 * j + 1 < G) {
+                    pa[rg][2 * j + 1].u[0] = __builtin_amdgcn_perm(x[j][1], x[j][0], 0x07060302u);
+                    pa[rg][2 * j + 1].u[1] = __builtin_amdgcn_perm(x[j][3], x[j][2], 0x07060302u);
+                }
             }
         };
         static_for<RG>([&](auto RGC) { softmax_rg(RGC); });
@@ -537,7 +543,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     // tile of loads in flight ahead of the arithmetic.  The others run one buffer with the
     // halves skewed: V of a tile is requested before its QK^T and softmax, K of the next
     // tile before its PV, so each half has the other half's arithmetic to arrive in.
-    constexpr bool PREFETCH = (RG == 1 && !(BITS == 8 && D == 128)) || (BITS == 4 && (RG == 2 || D == 64));
+    constexpr bool PREFETCH = (RG == 1 && !(BITS == 8 && D >= 128)) || (BITS == 4 && D <= 128 && (RG == 2 || D == 64));
     if (my_tiles > 0) {
         if constexpr (PREFETCH) {
             T bufA, bufB;
@@ -1091,6 +1097,7 @@ bool attend_decode_supported(const AttendArgs &a) {
     if (s.bits != 4 && s.bits != 8) return false;
     if (s.Dk == 64) return s.gs == 64;
     if (s.Dk == 128) return s.gs == 64 || s.gs == 128;
+    if (s.Dk == 256) return R <= 4 && (s.gs == 64 || s.gs == 128);  // more rows: the prefill tile
     return false;
 }
 
@@ -1150,6 +1157,8 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
 #define DEC_Q(BITS)                                 \
     do {                                            \
         if (st.Dk == 64) DEC_DT(BITS, 64, 64);      \
+        else if (st.Dk == 256 && st.gs == 64) DEC_DT(BITS, 256, 64);  \
+        else if (st.Dk == 256) DEC_DT(BITS, 256, 128);                \
         else if (st.gs == 64) DEC_DT(BITS, 128, 64); \
         else DEC_DT(BITS, 128, 128);                \
     } while (0)

@@ -30,7 +30,17 @@ def policy(request):
 def check(out, ref, what=""):
     mx, mean = err_stats(np32(out), ref)
     assert np.isfinite(np32(out)).all(), what
-    assert mx <= MAX_ABS and mean <= MEAN_ABS, f"{what}: max-abs {mx:.3e} mean-abs {mean:.3e}"
+    tol = MAX_ABS
+    if out.dtype == torch.bfloat16:
+        # one step of bfloat16 is 2^-7 = 7.8e-3 from |x| = 1 on and 1.56e-2 from 2 on.  The oracle
+        # rounds the probabilities to bfloat16 (8 bits) as the reference's softmax does, the
+        # matrix-core kernels hold them with more bits, so an output may land one step away before
+        # the final rounding puts it another step away: two steps at the largest output (the mean
+        # bound is unchanged)
+        top = float(np.abs(ref).max())
+        if top >= 1.0:
+            tol = max(tol, 2.0 * 2.0 ** (np.floor(np.log2(top)) - 7))
+    assert mx <= tol and mean <= MEAN_ABS, f"{what}: max-abs {mx:.3e} mean-abs {mean:.3e}"
 
 
 def omask(mask, dtype):
@@ -44,7 +54,8 @@ def omask(mask, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("bits,gs,D", [(8, 64, 64), (4, 64, 128), (4, 32, 64), (2, 64, 128)])
+@pytest.mark.parametrize("bits,gs,D", [(8, 64, 64), (4, 64, 128), (4, 32, 64), (2, 64, 128), (4, 64, 256), (8, 128, 256),
+                                        (8, 32, 128)])
 @pytest.mark.parametrize("r", [1, 4])
 def test_quantized_attention_modes(policy, dtype, bits, gs, D, r):
     rng = np.random.default_rng(bits + D + r)
@@ -110,6 +121,31 @@ def test_quantized_decode_many_pairs(bits, D, gs, B, Hkv, T0):
     o.update_quantized(k, v)
     scale = 1.0 / np.sqrt(D)
     for Lq, mask, om in ((1, None, O.Mask.NONE), (2, kvhip.MaskMode.causal(), O.Mask.CAUSAL)):
+        k, kd = randn(rng, (B, Hkv, Lq, D), dtype)
+        v, vd = randn(rng, (B, Hkv, Lq, D), dtype)
+        q, qd = randn(rng, (B, Hkv * r, Lq, D), dtype)
+        out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
+        assert kvhip.load().kvhip_last_attend_kernel() == 1
+        ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
+        check(out, ref, f"L={Lq}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bits,gs", [(4, 64), (8, 64), (4, 128), (8, 128)])
+@pytest.mark.parametrize("B,Hkv,r,T0", [(16, 8, 2, 777), (32, 8, 4, 300), (3, 2, 1, 2100)])
+def test_quantized_decode_head_size_256(dtype, bits, gs, B, Hkv, r, T0):
+    """Head size 256 (four or two groups per row) on the matrix-core decode kernel: one token
+    without a mask, then as many tokens as still make four query rows per kv head under .causal."""
+    rng = np.random.default_rng(B + T0 + bits + gs)
+    name, D = NAME[dtype], 256
+    c = kvhip.QuantizedKVCache(gs, bits)
+    o = O.QuantizedKVCache(gs, bits, name)
+    k, kd = randn(rng, (B, Hkv, T0, D), dtype)
+    v, vd = randn(rng, (B, Hkv, T0, D), dtype)
+    c.update_quantized(kd, vd, fetch=False)
+    o.update_quantized(k, v)
+    scale = 1.0 / np.sqrt(D)
+    for Lq, mask, om in ((1, None, O.Mask.NONE), (4 // r, kvhip.MaskMode.causal(), O.Mask.CAUSAL)):
         k, kd = randn(rng, (B, Hkv, Lq, D), dtype)
         v, vd = randn(rng, (B, Hkv, Lq, D), dtype)
         q, qd = randn(rng, (B, Hkv * r, Lq, D), dtype)
