@@ -1092,7 +1092,10 @@ bool attend_decode_supported(const AttendArgs &a) {
     if (s.Dk != s.Dv) return false;
     const int R = (a.Hq / a.Hkv) * a.L;
     if (R > 16) return false;
-    if (s.bits == 0) return s.Dk == 64 || s.Dk == 128 || s.Dk == 256;
+    // full precision: more than 8 rows (4 at D = 256) are faster on the prefill tile than on further
+    // passes of the broadcast contraction (8192 keys, 8 kv heads: B16 D 128 16 rows 104 us against
+    // 164 us; B8 D 256 8 rows about 105 us against 133 us)
+    if (s.bits == 0) return (s.Dk == 64 || s.Dk == 128 || s.Dk == 256) && R <= (s.Dk == 256 ? 4 : 8);
     if (a.runs.n != 1 || a.runs.row0[0] != 0 || a.runs.phys0[0] != 0) return false;
     if (s.bits != 4 && s.bits != 8) return false;
     if (s.Dk == 64) return s.gs == 64;

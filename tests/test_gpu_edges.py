@@ -75,15 +75,17 @@ def test_lengths_around_tile_and_page_boundaries(T, quant):
         assert mx <= 1e-2 and mean <= 1e-3, (T, quant, Lq, mx, mean)
 
 
-def test_sixteen_query_rows_per_kv_head_is_the_decode_limit():
-    """r * L = 16 rows still run on the split-sequence kernels, 17 go to the prefill tile; both
-    agree with the oracle."""
+def test_query_rows_per_kv_head_at_the_decode_limit():
+    """Quantized caches: r * L = 16 rows still run on the split-sequence kernels, 17 go to the
+    prefill tile.  Full-precision caches: 8 rows still do, 9 go to the prefill tile (faster there).
+    All agree with the oracle."""
     rng = np.random.default_rng(3)
     dtype, name = torch.float16, "float16"
     B, Hkv, D, T0 = 1, 2, 128, 300
     lib = kvhip.load()
     for quant in (None, (64, 4)):
-        for r, Lq, family in ((16, 1, None), (4, 4, None), (1, 16, None), (1, 17, 3), (17, 1, 3)):
+        for r, Lq in ((16, 1), (4, 4), (1, 16), (1, 17), (17, 1), (8, 1), (2, 4), (1, 8), (9, 1), (3, 3)):
+            family = (1 if r * Lq <= 16 else 3) if quant else (2 if r * Lq <= 8 else 3)
             if quant:
                 c, o = kvhip.QuantizedKVCache(*quant), O.QuantizedKVCache(*quant, name)
             else:
@@ -98,7 +100,7 @@ def test_sixteen_query_rows_per_kv_head_is_the_decode_limit():
             mask, om = (None, O.Mask.NONE) if Lq == 1 else (kvhip.MaskMode.causal(), O.Mask.CAUSAL)
             out = kvhip.attention_with_cache_update(qd, kd, vd, c, D ** -0.5, mask)
             fam = lib.kvhip_last_attend_kernel()
-            assert fam == (family if family else (1 if quant else 2)), (quant, r, Lq, fam)
+            assert fam == family, (quant, r, Lq, fam)
             ref = O.attention_with_cache_update(q, k, v, o, D ** -0.5, om, name)
             mx, mean = err_stats(np32(out), ref)
             assert mx <= 1e-2 and mean <= 1e-3, (quant, r, Lq, mx, mean)
