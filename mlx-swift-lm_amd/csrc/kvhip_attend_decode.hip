@@ -209,6 +209,12 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     constexpr int NH = D / 64;     // 64-column halves of the output
     constexpr int NQA = D / 64;    // query operand register pairs (16 steps of 4 elements each)
     constexpr int RR = 4 * RG;     // query rows carried
+    // Group size 32: the 64 columns a PV instruction covers lie in two groups, and the probability
+    // operand (which carries the V scale) is the same for every lane.  Each V step is therefore
+    // issued twice, once with either group's operand, into two accumulators; lanes 0-31 keep the
+    // first, lanes 32-63 the second.
+    constexpr bool HALF = GS < 64;
+    constexpr int NO2 = HALF ? D / 64 : 1;  // second accumulators (one dummy when unused)
     using T = TileRegs<BITS, D, G>;
     const Store &st = a.st;
     const int lane = threadIdx.x & 63;
@@ -224,7 +230,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     // ---- query operands: lane (blk, qi) holds row qi's 4 elements of step 16 x + blk ----
     // qsum[rg][g][i] = sum over group g of the (rounded, fp16-held) query row 4 rg + i, for
     // the bias term; built from the same registers: the 16 steps of one operand pair lie in
-    // one group (group sizes are multiples of 64), so a lane sums its 4 elements, the 16
+    // one group (group sizes of 64 and more; with 32 the lane groups 0-7 and 8-15 feed two sums), so a lane sums its 4 elements, the 16
     // lane groups are added up by shuffles and the four rows are read out of their quad.
     // (Built by a lambda that the main loop calls after it has requested its first tile, so the
     // first K/V loads are in flight while the queries are fetched and reduced.)
@@ -256,7 +262,12 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const float v = ok ? (float)(_Float16)round_dt<DT>(raw[x][k] * a.scale) : 0.f;
-                part[(64 * x) / GS] += v;
+                if constexpr (HALF) {  // steps 16 x + blk: lane groups 0-7 are one group of 32, 8-15 the next
+                    part[2 * x] += blk < 8 ? v : 0.f;
+                    part[2 * x + 1] += blk < 8 ? 0.f : v;
+                } else {
+                    part[(64 * x) / GS] += v;
+                }
                 qv[k] = GEO::hi(k) ? v * 0.0625f : v;
             }
             qa[rg][x].u[0] = pack_h2(qv[0], qv[1]);
@@ -277,8 +288,11 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     // m_use = m_run, or 0 while m_run is still -inf, so exp2((s - m_use) log2 e) needs no guard
     float m_run[RG][4], m_use[RG][4], l_part[RG][4], bacc[RG][G][4];
     f4 oacc[RG][NH];
+    f4 oacc2[RG][NO2];
 #pragma unroll
     for (int rg = 0; rg < RG; ++rg) {
+#pragma unroll
+        for (int h = 0; h < NO2; ++h) oacc2[rg][h] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < 4; ++i) { m_run[rg][i] = -INFINITY; m_use[rg][i] = 0.f; l_part[rg][i] = 0.f; }
 #pragma unroll
@@ -481,6 +495,10 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                     for (int g = 0; g < G; ++g) bacc[rg][g][i] *= alpha;
 #pragma unroll
                     for (int h = 0; h < NH; ++h) oacc[rg][h][i] *= alpha;
+                    if constexpr (HALF) {
+#pragma unroll
+                        for (int h = 0; h < NH; ++h) oacc2[rg][h][i] *= alpha;
+                    }
                 }
             }
             constexpr int GP = (G + 1) / 2;  // groups travel through the transpose two to a register
@@ -519,7 +537,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     auto compute_pv = [&](const T &t) {
         static_for<NH>([&](auto HH) {
             constexpr int h = decltype(HH)::value;
-            constexpr int g = (64 * h) / GS;
+            constexpr int g = HALF ? 2 * h : (64 * h) / GS;
             static_for<T::VW>([&](auto W) {
                 constexpr int w = decltype(W)::value;
                 Op o[GEO::WSTEPS];
@@ -527,8 +545,11 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 static_for<GEO::WSTEPS>([&](auto S2) {
                     constexpr int s = w * GEO::WSTEPS + decltype(S2)::value;
 #pragma unroll
-                    for (int rg = 0; rg < RG; ++rg)
+                    for (int rg = 0; rg < RG; ++rg) {
                         oacc[rg][h] = mfma444<s>(pa[rg][g], o[decltype(S2)::value], oacc[rg][h]);
+                        if constexpr (HALF)
+                            oacc2[rg][h] = mfma444<s>(pa[rg][g + 1], o[decltype(S2)::value], oacc2[rg][h]);
+                    }
                 });
             });
         });
@@ -581,11 +602,17 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         }
 #pragma unroll
         for (int h = 0; h < NH; ++h) {
-            constexpr int dummy = 0;
-            (void)dummy;
-            const int g = (64 * h) / GS;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) cbuf[wave][4 * rg + i][64 * h + lane] = oacc[rg][h][i] * TWO24 + bacc[rg][g][i];
+            for (int i = 0; i < 4; ++i) {
+                float o_ = oacc[rg][h][i], b_ = bacc[rg][HALF ? 2 * h : (64 * h) / GS][i];
+                if constexpr (HALF) {
+                    if (lane >= 32) {
+                        o_ = oacc2[rg][h][i];
+                        b_ = bacc[rg][2 * h + 1][i];
+                    }
+                }
+                cbuf[wave][4 * rg + i][64 * h + lane] = o_ * TWO24 + b_;
+            }
         }
         if (lane < 4) {
             cbuf[wave][4 * rg + lane][D] = m_run[rg][lane];
@@ -1098,8 +1125,8 @@ bool attend_decode_supported(const AttendArgs &a) {
     if (s.bits == 0) return (s.Dk == 64 || s.Dk == 128 || s.Dk == 256) && R <= (s.Dk == 256 ? 4 : 8);
     if (a.runs.n != 1 || a.runs.row0[0] != 0 || a.runs.phys0[0] != 0) return false;
     if (s.bits != 4 && s.bits != 8) return false;
-    if (s.Dk == 64) return s.gs == 64;
-    if (s.Dk == 128) return s.gs == 64 || s.gs == 128;
+    if (s.Dk == 64) return R <= 4 ? (s.gs == 32 || s.gs == 64) : s.gs == 64;  // group 32: 4-row kernel only
+    if (s.Dk == 128) return R <= 4 ? (s.gs == 32 || s.gs == 64 || s.gs == 128) : (s.gs == 64 || s.gs == 128);
     if (s.Dk == 256) return R <= 4 && (s.gs == 64 || s.gs == 128);  // more rows: the prefill tile
     return false;
 }
@@ -1159,7 +1186,9 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
     } while (0)
 #define DEC_Q(BITS)                                 \
     do {                                            \
-        if (st.Dk == 64) DEC_DT(BITS, 64, 64);      \
+        if (st.Dk == 64 && st.gs == 32) DEC_DT(BITS, 64, 32);   \
+        else if (st.Dk == 128 && st.gs == 32) DEC_DT(BITS, 128, 32); \
+        else if (st.Dk == 64) DEC_DT(BITS, 64, 64); \
         else if (st.Dk == 256 && st.gs == 64) DEC_DT(BITS, 256, 64);  \
         else if (st.Dk == 256) DEC_DT(BITS, 256, 128);                \
         else if (st.gs == 64) DEC_DT(BITS, 128, 64); \
