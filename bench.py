@@ -29,13 +29,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "mlx-swift-lm_amd"))
 
-B, HQ, HKV, D, BITS, GS, CTX = 32, 32, 8, 128, 4, 64, 32768
+HQ, HKV = 32, 8  # configs[2]: batch 32, head size 128, 4-bit codes in groups of 64, context 32768 (defaults below)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes moved per launch of the decode kernel divided by its algorithmic bytes, from two
 # rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) scaled by what the same counters read for a
 # plain 1 GiB copy; summary in profiles/decode_kernel_q4_d128_cfg3.md
 MEASURED_TRAFFIC_RATIO = 1.0024
-ROW_BYTES = 144  # per cached token and kv head: K and V codes 2*64 B + 2*2 groups*(scale+bias)*2 B
 
 
 def main():
@@ -43,8 +42,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--context", type=int, default=CTX)
-    ap.add_argument("--batch", type=int, default=B)
+    ap.add_argument("--context", type=int, default=32768)
+    ap.add_argument("--batch", type=int, default=32)
+    ap.add_argument("--head-dim", type=int, default=128, help="head size of the cfg3-shaped run (64, 128, 256)")
+    ap.add_argument("--group-size", type=int, default=64, help="quantization group size (32, 64, 128)")
+    ap.add_argument("--bits", type=int, default=4, help="code width (4, 8)")
     ap.add_argument("--cpu-steps", type=int, default=2, help="decode steps timed on the CPU baseline (0 = skip)")
     ap.add_argument("--workload", default="cfg3", choices=["cfg3", "cfg1", "cfg2", "cfg4", "cfg5"],
                     help="cfg3 (default) is the configuration the metric is quoted on; the others are the "
@@ -75,6 +77,10 @@ def main():
         print(json.dumps(other_workload(args, torch, kvhip, L, dev)))
         return
     nb, ctx = args.batch, args.context
+    D, GS, BITS = args.head_dim, args.group_size, args.bits
+    # per cached token and kv head: K and V codes + (scale, bias) pairs of 2 x 2 bytes per group
+    ROW_BYTES = 2 * (D * BITS // 8 + (D // GS) * 4)
+    headline = (nb, ctx, D, GS, BITS) == (32, 32768, 128, 64, 4)
     g = torch.Generator(device=dev)
     g.manual_seed(0)
     ch = (10.0 ** (torch.rand(D, generator=g, device=dev) * 2 - 1)).to(torch.float32)
@@ -139,11 +145,11 @@ def main():
     if launches.value > 0:
         kernel_ms = kms.value / launches.value
         achieved = alg_bytes / (kernel_ms * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "kernel": "decode_kernel<4,128,64,f16>", "achieved": round(achieved, 1),
+        roofline = {"bound": "hbm", "kernel": f"decode_kernel<{BITS},{D},{GS},f16>", "achieved": round(achieved, 1),
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                     "kernel_ms": round(kernel_ms, 5), "algorithmic_bytes": int(alg_bytes),
                     "traffic": int(args.traffic_kib * 1024) if args.traffic_kib is not None
-                    else (int(alg_bytes * MEASURED_TRAFFIC_RATIO) if (nb, ctx) == (B, CTX) else None)}
+                    else (int(alg_bytes * MEASURED_TRAFFIC_RATIO) if headline else None)}
 
     # ---- CPU baseline + full-size parity sample ------------------------------------
     cpu = None
@@ -180,8 +186,9 @@ def main():
         "metric": "KV-attn decode tok/s + HBM GB/s (% of peak), Llama-3-8B shape 4-bit KV 32k",
         "value": round(tok_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16 (4-bit affine codes, fp32 accumulate)", "data": "synthetic",
-        "config": {"workload": "configs[2]: QuantizedKVCache 4-bit g64, 32q/8kv heads, head_dim 128, "
+        "dtype": f"f16 ({BITS}-bit affine codes, fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": ("configs[2]: " if headline else "configs[2]'s shape varied: ") +
+                               f"QuantizedKVCache {BITS}-bit g{GS}, 32q/8kv heads, head_dim {D}, "
                                f"batch {nb}, context {ctx}+, quantize-on-append + fused dequant-SDPA, one layer",
                    "batch": nb, "context_first": int(t_first), "context_last": int(t_last)},
         "roofline": roofline, "cpu_baseline": cpu, "parity": parity,
