@@ -959,10 +959,12 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     }
 }
 
-// grid (R, BH): merge the span partials of one query row and write the output row
+// grid (R, BH), D rounded up to whole wavefronts of threads: merge the span partials of one query
+// row and write the output row
 template <int D, int DT>
-__global__ void __launch_bounds__(D)
+__global__ void __launch_bounds__((D + 63) / 64 * 64)
 combine_kernel(AttendArgs a, int nsplit, int rr) {
+    constexpr int NT = (D + 63) / 64 * 64;
     __shared__ float w_s[512];  // weight of each span for this row (nsplit <= 512)
     __shared__ float red_s[4];
     const int i = blockIdx.x, bh = blockIdx.y;
@@ -971,34 +973,35 @@ combine_kernel(AttendArgs a, int nsplit, int rr) {
     const int rep = i / a.L, l = i - rep * a.L;
     const size_t sstride = (size_t)rr * (D + 2);
     const float *part = a.workspace + (size_t)bh * nsplit * sstride + (size_t)i * (D + 2);
-    const int d = threadIdx.x;
+    const int t = threadIdx.x;
+    const int d = t < D ? t : 0;  // threads past the last column read column 0 and write nothing
     // every span's (max, sum) in one parallel round of loads, reduced through LDS
     float mloc = -INFINITY;
-    for (int s = d; s < nsplit; s += D) {
+    for (int s = t; s < nsplit; s += NT) {
         const float m = part[s * sstride + D];
         w_s[s] = m;
         mloc = fmaxf(mloc, m);
     }
     mloc = wave_max(mloc);
-    if ((d & 63) == 0) red_s[d >> 6] = mloc;
+    if ((t & 63) == 0) red_s[t >> 6] = mloc;
     __syncthreads();
     float mx = red_s[0];
 #pragma unroll
-    for (int w = 1; w < D / 64; ++w) mx = fmaxf(mx, red_s[w]);
+    for (int w = 1; w < NT / 64; ++w) mx = fmaxf(mx, red_s[w]);
     __syncthreads();
     float dloc = 0.f;
-    for (int s = d; s < nsplit; s += D) {
+    for (int s = t; s < nsplit; s += NT) {
         const float m = w_s[s];
         const float w = (m == -INFINITY) ? 0.f : fast_exp2((m - mx) * LOG2E);
         w_s[s] = w;
         dloc += w * part[s * sstride + D + 1];
     }
     dloc = wave_sum(dloc);
-    if ((d & 63) == 0) red_s[d >> 6] = dloc;
+    if ((t & 63) == 0) red_s[t >> 6] = dloc;
     __syncthreads();
     float den = red_s[0];
 #pragma unroll
-    for (int w = 1; w < D / 64; ++w) den += red_s[w];
+    for (int w = 1; w < NT / 64; ++w) den += red_s[w];
     // the column sums: independent loads, issued several at a time
     float num = 0.f;
     int s = 0;
@@ -1009,7 +1012,7 @@ combine_kernel(AttendArgs a, int nsplit, int rr) {
     }
     for (; s < nsplit; ++s) num += w_s[s] * part[s * sstride + d];
     const float o = den > 0.f ? num / den : 0.f;
-    Elem<DT>::store(a.out, ((size_t)(b * a.Hq + hk * r + rep) * a.L + l) * D + d, o);
+    if (t < D) Elem<DT>::store(a.out, ((size_t)(b * a.Hq + hk * r + rep) * a.L + l) * D + d, o);
 }
 
 struct Plan {
@@ -1107,10 +1110,11 @@ hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t
     dim3 grid(R, a.st.BH);
 #define CMB(D)                                                                                       \
     do {                                                                                             \
-        if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL((combine_kernel<D, 0>), grid, dim3(D), 0, s, a, nsplit, rows); \
-        else hipLaunchKernelGGL((combine_kernel<D, 1>), grid, dim3(D), 0, s, a, nsplit, rows);       \
+        if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL((combine_kernel<D, 0>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows); \
+        else hipLaunchKernelGGL((combine_kernel<D, 1>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows);       \
     } while (0)
     if (a.st.Dk == 64) CMB(64);
+    else if (a.st.Dk == 96) CMB(96);
     else if (a.st.Dk == 128) CMB(128);
     else CMB(256);
 #undef CMB

@@ -76,7 +76,9 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                                   // read touches fall in distinct banks
     constexpr int S = D / 32;     // contraction steps over the head dim
     constexpr int NDT = D / 16;   // 16-row tiles of out^T
-    constexpr int NC = D / 64;    // 16-byte chunks per thread, for K and for V
+    constexpr int NC = (D + 63) / 64;  // rounds of 256 16-byte chunks, for K and for V
+    constexpr int CH = 4 * D;          // 16-byte chunks of a tile's K (and of its V); a multiple of 64
+    static_assert(D % 32 == 0, "the contraction takes 32 head-dim elements per step");
     // K tiles move from global memory straight into LDS (no registers, no LDS store instructions):
     // two buffers, each the tile's 16-byte chunks in page order, [8-element chunk][token], the other
     // one filled while this one is contracted.  fp16 caches move V the same way, [8-token
@@ -87,7 +89,11 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     // (one array per buffer, K then V, selected by constants after inlining: the compiler follows
     // loads into LDS per variable, and a read of one buffer then need not wait for the loads in
     // flight into the other)
-    constexpr int KSZ = BN * D;  // 16-bit elements of a tile's K (and of its V)
+    // 16-bit elements reserved for a tile's K (and for its V): whole rounds of 256 chunks.  With a head
+    // size that is not a multiple of 64 (96) the last round is partly empty: its wavefronts past the
+    // tile's last chunk repeat that chunk into the unused tail, so that every wavefront issues the same
+    // number of loads and the hand-placed waits below count alike in all of them.
+    constexpr int KSZ = NC * 256 * 8;
     __shared__ __attribute__((aligned(16))) uint16_t KV0[VDMA ? 2 * KSZ : KSZ], KV1[VDMA ? 2 * KSZ : KSZ];
     __shared__ __attribute__((aligned(16))) _Float16 Vpad[2][VDMA ? 8 : D * VS];
     auto Ks = [&](int buf) __attribute__((always_inline)) -> uint16_t * { return buf == 0 ? KV0 : KV1; };
@@ -227,7 +233,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         const char *vbase = v_cell_ptr(st, bh, slot0) + vfp_off(st, slot0, 0);
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
-            const int c = e * 256 + tid;
+            const int c = min(e * 256 + tid, CH - 1);
             g.v[e] = *reinterpret_cast<const u4 *>(vbase + (size_t)(c / D) * (D * 16) + (c % D) * 16);
         }
     };
@@ -235,6 +241,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
             const int c = e * 256 + tid;
+            if (c >= CH) continue;
             u4 v = g.v[e];
             if (DT == 1) v = u4{bf2_to_h2(v.x), bf2_to_h2(v.y), bf2_to_h2(v.z), bf2_to_h2(v.w)};
             u2 *vd = reinterpret_cast<u2 *>(&Vs(buf)[(c % D) * VS + (c / D) * 8]);  // rows are 8-byte aligned
@@ -266,7 +273,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         const char *vbase = v_cell_ptr(st, bh, slot0) + vfp_off(st, slot0, 0);
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
-            const int c = e * 256 + tid;
+            const int c = min(e * 256 + tid, CH - 1);
             const int pos = c % BN;
             const int tok = VDMA ? 8 * ((pos & 15) >> 2) + 4 * (pos >> 4) + (pos & 3) : pos;
             const int cw = e * 256 + (tid & ~63);  // the wavefront's first slot
@@ -591,6 +598,7 @@ hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, 
         else PF_QT(D, 1);                         \
     } while (0)
     if (st.Dk == 64) PF_DT(64);
+    else if (st.Dk == 96) PF_DT(96);
     else if (st.Dk == 128) PF_DT(128);
     else if (st.dtype == KVHIP_F16) PF(256, 0, 1);
     else PF(256, 1, 1);

@@ -175,7 +175,7 @@ def test_quantized_causal_close_to_full_precision(policy, r):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("Dk,Dv,r", [(128, 128, 4), (64, 32, 1), (256, 256, 2), (80, 80, 2)])
+@pytest.mark.parametrize("Dk,Dv,r", [(128, 128, 4), (64, 32, 1), (256, 256, 2), (80, 80, 2), (96, 96, 4), (96, 96, 1)])
 def test_simple_cache_attention(policy, dtype, Dk, Dv, r):
     rng = np.random.default_rng(Dk + r)
     B, Hkv = 2, 2
