@@ -724,7 +724,7 @@ hipError_t launch_append_fp(const Store &st, const void *keys, const void *value
                             int slot0, int n, hipStream_t s, const RopeDev *rope) {
     if (n <= 0) return hipSuccess;
     const RopeDev r = rope ? *rope : RopeDev();
-    const bool tiled = st.es == 2 && st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 128 || st.Dk == 256);
+    const bool tiled = st.es == 2 && st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 96 || st.Dk == 128 || st.Dk == 256);
     const TileSplit t = tile_split(slot0, n);
     if (!tiled || t.tiles == 0) return launch_append_fp_rows(st, keys, values, L, src0, slot0, n, s, r);
     hipError_t e = launch_append_fp_rows(st, keys, values, L, src0, slot0, t.head, s, r);
@@ -732,6 +732,7 @@ hipError_t launch_append_fp(const Store &st, const void *keys, const void *value
     dim3 grid(t.tiles, st.BH), block(256);
     const int a0 = src0 + t.head, b0 = slot0 + t.head;
     if (st.Dk == 64) hipLaunchKernelGGL(append_fp_tile_kernel<2>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, a0, b0, r);
+    else if (st.Dk == 96) hipLaunchKernelGGL(append_fp_tile_kernel<3>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, a0, b0, r);
     else if (st.Dk == 128) hipLaunchKernelGGL(append_fp_tile_kernel<4>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, a0, b0, r);
     else hipLaunchKernelGGL(append_fp_tile_kernel<8>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, a0, b0, r);
     e = hipGetLastError();

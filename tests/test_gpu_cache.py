@@ -199,7 +199,7 @@ def test_simple_cache_update_fetch_state(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("D", [64, 96, 128, 256])
 def test_simple_cache_prompt_sized_appends(dtype, D):
     """Appends that cover whole 64-token tiles take the tile kernel (head rows, tiles, tail rows)."""
     rng = np.random.default_rng(21)
