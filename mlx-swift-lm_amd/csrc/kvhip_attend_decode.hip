@@ -1114,6 +1114,7 @@ hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t
         else hipLaunchKernelGGL((combine_kernel<D, 1>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows);       \
     } while (0)
     if (a.st.Dk == 64) CMB(64);
+    else if (a.st.Dk == 80) CMB(80);
     else if (a.st.Dk == 96) CMB(96);
     else if (a.st.Dk == 128) CMB(128);
     else CMB(256);

@@ -462,8 +462,8 @@ bool attend_prefill_supported(const AttendArgs &a) {
     const Store &s = a.st;
     if (s.dtype != KVHIP_F16 && s.dtype != KVHIP_BF16) return false;
     if (s.Dk != s.Dv) return false;
-    // head size 96: full-precision caches only, every row count (no decode kernel is built for it)
-    if (s.Dk != 64 && s.Dk != 128 && s.Dk != 256 && !(s.Dk == 96 && s.bits == 0)) return false;
+    // head sizes 80 and 96: full-precision caches only, every row count (no decode kernel is built for them)
+    if (s.Dk != 64 && s.Dk != 128 && s.Dk != 256 && !((s.Dk == 80 || s.Dk == 96) && s.bits == 0)) return false;
     if (s.bits != 0 && s.bits != 4 && s.bits != 8) return false;
     if (s.bits != 0 && s.gs < 32) return false;
     return true;  // 16 rows or fewer come here only when the decode kernels do not take the shape

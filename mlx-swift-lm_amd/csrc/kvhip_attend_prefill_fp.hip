@@ -74,11 +74,15 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     constexpr int BM = 64 * QT;
     constexpr int VS = BN + 4;    // halves per V^T row in LDS: 18 dwords, so the 16 rows an operand
                                   // read touches fall in distinct banks
-    constexpr int S = D / 32;     // contraction steps over the head dim
+    constexpr int S = (D + 31) / 32;  // contraction steps over the head dim (the last one partly zero at D = 80)
     constexpr int NDT = D / 16;   // 16-row tiles of out^T
     constexpr int NC = (D + 63) / 64;  // rounds of 256 16-byte chunks, for K and for V
     constexpr int CH = 4 * D;          // 16-byte chunks of a tile's K (and of its V); a multiple of 64
-    static_assert(D % 32 == 0, "the contraction takes 32 head-dim elements per step");
+    static_assert(D % 16 == 0, "out^T is built from 16-row tiles");
+    // A head size that is not a multiple of 32 (80): the last contraction step reads K chunks past the
+    // row -- the unused tail that the repeated loads fill with finite values -- against query
+    // operands that are zero there.
+    static_assert(4 * S * BN <= ((D + 63) / 64) * 256, "the padded contraction stays inside the staged buffer");
     // K tiles move from global memory straight into LDS (no registers, no LDS store instructions):
     // two buffers, each the tile's 16-byte chunks in page order, [8-element chunk][token], the other
     // one filled while this one is contracted.  fp16 caches move V the same way, [8-token
@@ -90,7 +94,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     // loads into LDS per variable, and a read of one buffer then need not wait for the loads in
     // flight into the other)
     // 16-bit elements reserved for a tile's K (and for its V): whole rounds of 256 chunks.  With a head
-    // size that is not a multiple of 64 (96) the last round is partly empty: its wavefronts past the
+    // size that is not a multiple of 64 (80, 96) the last round is partly empty: its wavefronts past the
     // tile's last chunk repeat that chunk into the unused tail, so that every wavefront issues the same
     // number of loads and the hand-placed waits below count alike in all of them.
     constexpr int KSZ = NC * 256 * 8;
@@ -160,7 +164,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             reinterpret_cast<const uint16_t *>(a.q) + ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D + 8 * jj);
 #pragma unroll
         for (int s = 0; s < S; ++s) {
-            u4 w = q_ok[qt] ? qp[4 * s] : u4{0, 0, 0, 0};
+            u4 w = (q_ok[qt] && (D % 32 == 0 || 32 * s + 8 * jj < D)) ? qp[4 * s] : u4{0, 0, 0, 0};
             if (flip) w ^= u4{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
             qop[qt][s].v = w;
         }
@@ -598,6 +602,7 @@ hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, 
         else PF_QT(D, 1);                         \
     } while (0)
     if (st.Dk == 64) PF_DT(64);
+    else if (st.Dk == 80) PF_DT(80);
     else if (st.Dk == 96) PF_DT(96);
     else if (st.Dk == 128) PF_DT(128);
     else if (st.dtype == KVHIP_F16) PF(256, 0, 1);

@@ -19,7 +19,7 @@ def _case(seed):
     dtype = [torch.float16, torch.bfloat16][rng.integers(2)]
     D = int(rng.choice([64, 128, 256] if kind != "quantized" else [64, 128]))
     if kind != "quantized" and seed % 5 == 4:
-        D = 96  # full-precision caches of head size 96 run on the prefill tile at every row count
+        D = 96 if seed % 10 == 4 else 80  # these head sizes run on the prefill tile at every row count
     B, Hkv, r = int(rng.integers(1, 6)), int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 4, 8]))
     Lq = int(rng.choice([1, 1, 2, 4, 7, 33, 70]))
     T0 = int(rng.choice([1, 63, 64, 65, 200, 257, 700, 1500, 2600]))
