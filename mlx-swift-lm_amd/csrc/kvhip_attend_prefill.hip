@@ -185,13 +185,20 @@ prefill_kernel(AttendArgs a, int nsplit) {
     // ---- staging: a tile is fetched from global memory into registers one iteration ahead
     // (in flight while the current tile is contracted), then converted and written to LDS.
     constexpr int BB = BITS;
-    constexpr int KQW = (D / 8) * BB / 32;        // packed words per thread for K (D/8 codes)
+    // K: KT threads per token row, CPT codes each: 8 threads where that gives whole packed words
+    // (head sizes that are multiples of 64), 4 otherwise (96: 24 codes = 3 or 6 words, which may
+    // straddle two groups of 32)
+    constexpr int KT = (D % 64 == 0) ? 8 : 4;
+    constexpr int CPT = D / KT;
+    constexpr int KQW = CPT * BB / 32;            // packed words per thread for K
+    static_assert((CPT * BB) % 32 == 0, "a thread's K codes are whole packed words");
     constexpr int VQW = 16 * BB / 32;             // packed words per thread and column for V
     constexpr int VCOLS = (2 * D + 255) / 256;    // (column, half) items per thread for V
-    uint32_t kq[KQW], vq[VCOLS * VQW], ksb_raw = 0;
+    uint32_t kq[KQW], vq[VCOLS * VQW], ksb_raw = 0, ksb_raw_hi = 0;
     uint32_t vsb_raw[D / 32];
     int row_reg = -1;
-    const int kt = tid >> 3, kpart = tid & 7;     // K: 8 threads per token row
+    const int kt = tid / KT, kpart = tid % KT;
+    const bool k_on = KT == 8 || tid < BN * KT;   // with 4 threads per row the upper half has no K work
 
     auto fetch = [&](int tile) {
         const int slot0 = tile * BN;
@@ -203,12 +210,16 @@ prefill_kernel(AttendArgs a, int nsplit) {
             row_reg = (row >= 0 && row < a.T) ? row : -1;
         }
         const char *cell = v_cell_ptr(st, bh, slot0);
-        const uint32_t *w = reinterpret_cast<const uint32_t *>(k_row_ptr(st, bh, slot0 + kt)) + kpart * KQW;
+        if (k_on) {
+            const uint32_t *w = reinterpret_cast<const uint32_t *>(k_row_ptr(st, bh, slot0 + kt)) + kpart * KQW;
 #pragma unroll
-        for (int e = 0; e < KQW; ++e) kq[e] = w[e];
-        // the D/8 codes of this thread lie in one group (group sizes are >= 32 >= D/8)
-        const int g = (kpart * (D / 8)) / st.gs;
-        ksb_raw = reinterpret_cast<const uint32_t *>(ksb_row_ptr(st, bh, slot0 + kt))[g];
+            for (int e = 0; e < KQW; ++e) kq[e] = w[e];
+            // 8 threads per row: the D/8 codes of this thread lie in one group (group sizes are >= 32 >= D/8);
+            // 4 threads per row: in at most two, the first code's and the last code's
+            const uint32_t *sbp = reinterpret_cast<const uint32_t *>(ksb_row_ptr(st, bh, slot0 + kt));
+            ksb_raw = sbp[(kpart * CPT) / st.gs];
+            if constexpr (KT != 8) ksb_raw_hi = sbp[(kpart * CPT + CPT - 1) / st.gs];
+        }
         if (tid < BN) {
             const uint32_t *sb = reinterpret_cast<const uint32_t *>(vsb_row_ptr(st, bh, slot0 + tid));
 #pragma unroll
@@ -244,17 +255,32 @@ prefill_kernel(AttendArgs a, int nsplit) {
             if (lane == 0) tile_full_s = full;
         }
         constexpr int per = 32 / BB;
-        float sc, bi;
-        sb_pair(ksb_raw, sc, bi);
-        _Float16 *dst = Ks + kt * KS + kpart * (D / 8);
-#pragma unroll
-        for (int e = 0; e < KQW; ++e)
-#pragma unroll
-            for (int x = 0; x < per; x += 2) {
-                const float c0 = (float)((kq[e] >> (x * BB)) & ((1u << BB) - 1u));
-                const float c1 = (float)((kq[e] >> ((x + 1) * BB)) & ((1u << BB) - 1u));
-                *reinterpret_cast<uint32_t *>(dst + e * per + x) = h2_bits(sc * c0 + bi, sc * c1 + bi);
+        if (k_on) {
+            float sc, bi, sc_hi = 0.f, bi_hi = 0.f;
+            sb_pair(ksb_raw, sc, bi);
+            [[maybe_unused]] int g_lo = 0;
+            if constexpr (KT != 8) {
+                sb_pair(ksb_raw_hi, sc_hi, bi_hi);
+                g_lo = (kpart * CPT) / st.gs;
             }
+            _Float16 *dst = Ks + kt * KS + kpart * CPT;
+#pragma unroll
+            for (int e = 0; e < KQW; ++e) {
+                float s_ = sc, b_ = bi;
+                if constexpr (KT != 8) {  // a packed word lies in one group (32 is a multiple of the codes per word)
+                    if ((kpart * CPT + e * per) / st.gs != g_lo) {
+                        s_ = sc_hi;
+                        b_ = bi_hi;
+                    }
+                }
+#pragma unroll
+                for (int x = 0; x < per; x += 2) {
+                    const float c0 = (float)((kq[e] >> (x * BB)) & ((1u << BB) - 1u));
+                    const float c1 = (float)((kq[e] >> ((x + 1) * BB)) & ((1u << BB) - 1u));
+                    *reinterpret_cast<uint32_t *>(dst + e * per + x) = h2_bits(s_ * c0 + b_, s_ * c1 + b_);
+                }
+            }
+        }
         if (tid < BN) {
 #pragma unroll
             for (int gg = 0; gg < D / 32; ++gg)
@@ -462,8 +488,8 @@ bool attend_prefill_supported(const AttendArgs &a) {
     const Store &s = a.st;
     if (s.dtype != KVHIP_F16 && s.dtype != KVHIP_BF16) return false;
     if (s.Dk != s.Dv) return false;
-    // head sizes 80 and 96: full-precision caches only, every row count (no decode kernel is built for them)
-    if (s.Dk != 64 && s.Dk != 128 && s.Dk != 256 && !((s.Dk == 80 || s.Dk == 96) && s.bits == 0)) return false;
+    // head sizes 80 (full precision only) and 96: every row count (no decode kernel is built for them)
+    if (s.Dk != 64 && s.Dk != 128 && s.Dk != 256 && s.Dk != 96 && !(s.Dk == 80 && s.bits == 0)) return false;
     if (s.bits != 0 && s.bits != 4 && s.bits != 8) return false;
     if (s.bits != 0 && s.gs < 32) return false;
     return true;  // 16 rows or fewer come here only when the decode kernels do not take the shape
@@ -534,6 +560,7 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
 #define PF_D(BITS)                                    \
     do {                                              \
         if (st.Dk == 64) PF_DT(BITS, 64);             \
+        else if (st.Dk == 96) PF_DT(BITS, 96);        \
         else if (st.Dk == 128) PF_DT(BITS, 128);      \
         else if (st.dtype == KVHIP_F16) PF(BITS, 256, 0, 1); /* 64 query rows per workgroup only */ \
         else PF(BITS, 256, 1, 1);                     \
