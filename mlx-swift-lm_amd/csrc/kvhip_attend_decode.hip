@@ -1134,8 +1134,9 @@ bool attend_decode_supported(const AttendArgs &a) {
     if (s.bits == 0) return (s.Dk == 64 || s.Dk == 128 || s.Dk == 256) && R <= (s.Dk == 256 ? 4 : 8);
     if (a.runs.n != 1 || a.runs.row0[0] != 0 || a.runs.phys0[0] != 0) return false;
     if (s.bits != 4 && s.bits != 8) return false;
-    if (s.Dk == 64) return R <= 4 ? (s.gs == 32 || s.gs == 64) : s.gs == 64;  // group 32: 4-row kernel only
-    if (s.Dk == 128) return R <= 4 ? (s.gs == 32 || s.gs == 64 || s.gs == 128) : (s.gs == 64 || s.gs == 128);
+    if (s.Dk == 64) return s.gs == 32 || s.gs == 64;
+    // 5..16 rows of group size 32 at D = 128: the 16-row kernel is built for 4-bit codes only
+    if (s.Dk == 128) return s.gs == 64 || s.gs == 128 || (s.gs == 32 && (R <= 4 || s.bits == 4));
     if (s.Dk == 256) return R <= 4 && (s.gs == 64 || s.gs == 128);  // more rows: the prefill tile
     return false;
 }

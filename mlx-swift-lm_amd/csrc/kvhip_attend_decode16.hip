@@ -162,7 +162,9 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 const char *p = kp + (size_t)(4 * tb) * st.k_row + g * (GS * BITS / 8);
-                if constexpr (KWL == 2) {
+                if constexpr (KWL == 1) {
+                    t.k[tb][g][0] = *reinterpret_cast<const uint32_t *>(p);
+                } else if constexpr (KWL == 2) {
                     const u2 w = *reinterpret_cast<const u2 *>(p);
                     t.k[tb][g][0] = w.x; t.k[tb][g][1] = w.y;
                 } else {
@@ -367,13 +369,11 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     auto compute_pv = [&](const Tile &t) __attribute__((always_inline)) {
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
-            constexpr int dummy = 0;
-            (void)dummy;
-            const int g = (16 * db) / GS;
+            const int g = (16 * db) / GS;  // a constant once the loop is unrolled
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const Op8 va = CD::unpack(&t.v[db][u * CD::WORDS]);
-                oacc[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va.h, (g == 0 ? pb[0][u] : pb[G - 1][u]).h, oacc[db], 0, 0, 0);
+                oacc[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va.h, pb[g][u].h, oacc[db], 0, 0, 0);
             }
         }
     };
@@ -408,7 +408,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         const int g = (16 * db) / GS;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            cbuf[wave][n][16 * db + 4 * jj + i] = oacc[db][i] * TWO24 + (g == 0 ? bacc[0] : bacc[G - 1]);
+            cbuf[wave][n][16 * db + 4 * jj + i] = oacc[db][i] * TWO24 + bacc[g];
     }
     if (jj == 0) {
         cbuf[wave][n][D] = m_run;
@@ -478,11 +478,16 @@ hipError_t launch_attend_decode16(const AttendArgs &a, int tiles_total, int tile
     } while (0)
 #define D16_Q(BITS)                                     \
     do {                                                \
-        if (st.Dk == 64) D16_DT(BITS, 64, 64);          \
-        else if (st.gs == 64) D16_DT(BITS, 128, 64);    \
-        else D16_DT(BITS, 128, 128);                    \
+        if (st.Dk == 64 && st.gs == 32) D16_DT(BITS, 64, 32);        \
+        else if (st.Dk == 64) D16_DT(BITS, 64, 64);                  \
+        else if (st.gs == 64) D16_DT(BITS, 128, 64);                 \
+        else D16_DT(BITS, 128, 128);                                 \
     } while (0)
-    if (st.bits == 4) D16_Q(4);
+    // (group size 32 at D = 128 is built for 4-bit codes only: the 8-bit tile plus four groups of
+    // scale / bias registers no longer fits the register file; the caller sends that shape, and
+    // D = 256, whose partials exceed a workgroup's LDS, to the prefill tile)
+    if (st.bits == 4 && st.Dk == 128 && st.gs == 32) D16_DT(4, 128, 32);
+    else if (st.bits == 4) D16_Q(4);
     else D16_Q(8);
 #undef D16_Q
 #undef D16_DT

@@ -125,8 +125,9 @@ def test_quantized_decode_many_pairs(bits, D, gs, B, Hkv, T0):
         v, vd = randn(rng, (B, Hkv, Lq, D), dtype)
         q, qd = randn(rng, (B, Hkv * r, Lq, D), dtype)
         out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
-        # group size 32 is built into the 4-row decode kernel only; more rows take the prefill tile
-        assert kvhip.load().kvhip_last_attend_kernel() == (1 if gs != 32 or r * Lq <= 4 else 3)
+        # group size 32 with 8-bit codes at D = 128 is built into the 4-row decode kernel only; more
+        # rows of it take the prefill tile
+        assert kvhip.load().kvhip_last_attend_kernel() == (3 if (gs, bits, D) == (32, 8, 128) and r * Lq > 4 else 1)
         ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
         check(out, ref, f"L={Lq}")
 
