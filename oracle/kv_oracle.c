@@ -18,10 +18,13 @@
  * The arithmetic of these ops belongs to the third-party dependency
  * ml-explore/mlx-swift (0.31.6 ..< 0.32.0, Package.swift:64), which is not
  * part of the reference checkout; its published CPU algorithm is restated
- * here.  Exact code/scale/bias bits and the accumulation order inside
- * quantizedMM/softmax are therefore "parity unpinned" against MLX itself; they
- * are pinned against closed forms, invariants and the independent numpy
- * restatement in kv_oracle.py.
+ * here.  kvo_affine_quantize is pinned against that published loop by the
+ * hand-worked known answers of tests/quantizer_kats.py (and by closed forms,
+ * invariants and the independent numpy restatement in kv_oracle.py); against
+ * an output of MLX itself, which the reference does not hold, code / scale /
+ * bias bits stay "parity unpinned", and so does the accumulation order and
+ * dtype inside quantizedMM / softmax (softmax(precise: false) accumulates in T
+ * on MLX's CPU backend, in float32 here).
  *
  * Arrays are float32 holding values representable in the logical dtype T
  * (0 = float16, 1 = bfloat16, 2 = float32); kvo_round applies T's rounding

@@ -22,15 +22,26 @@ Parity status of each function
   metaState strings, mask mode choice, createCausalMask truth table,
   logicalView): fully specified by the Swift source and pinned by the
   integer known answers of the reference's own tests (tests/test_oracle_kat.py).
-* `affine_quantize` / `affine_dequantize` / `quantized_matmul` / softmax
-  rounding points: the arithmetic lives in the third-party dependency
-  ml-explore/mlx-swift (pinned 0.31.6 ..< 0.32.0, Package.swift:64 -> MLX
-  core, CPU backend), whose sources are absent from the reference checkout.
-  The published algorithm is restated; it is pinned by closed forms,
-  invariants and an independent scalar implementation (oracle/kv_oracle.c),
-  but NOT by an output of MLX itself: **parity unpinned** at the MLX boundary
-  for exact code/scale/bias bits and for accumulation order inside
-  quantizedMM / softmax.
+* `affine_quantize` / `affine_dequantize`: the arithmetic lives in the
+  third-party dependency ml-explore/mlx-swift (pinned 0.31.6 ..< 0.32.0,
+  Package.swift:64 -> MLX core, CPU backend: `quantize<T, U>` in
+  mlx/backend/cpu/quantized.cpp), whose sources are absent from the reference
+  checkout.  The published loop is restated; it is pinned by known answers
+  worked out by hand from that loop (tests/quantizer_kats.py: float32 scale
+  versus the stored T-rounded one, round-half-to-even for q0 and the codes, the
+  1e-7 floor on a non-constant group, the strict magnitude comparison, both
+  clamps), by closed forms, invariants and an independent scalar implementation
+  (oracle/kv_oracle.c).  No output of MLX itself is held by the reference for
+  packed codes or scale / bias bits, so against the MLX binary this stays
+  **parity unpinned**; against the published algorithm it is pinned.
+* `quantized_matmul` / `softmax_last` rounding points and accumulation order:
+  **parity unpinned** (tolerance-level only).  `softmax(precise: false)`, which
+  KVCache.swift:2416 calls, accumulates in the input dtype on MLX's CPU backend
+  (`softmax<T, AccT = T>`, mlx/backend/cpu/softmax.cpp); this oracle exponentiates
+  and sums in float32 and rounds the normalised probabilities to T once.  For
+  float16 / bfloat16 inputs that is the more accurate of the two and differs from
+  MLX's own output by about one unit in the last place of T per probability; the
+  attention bound (max-abs 1e-2, mean-abs 1e-3) is a tolerance, not a bit pattern.
 """
 
 from __future__ import annotations
@@ -188,7 +199,11 @@ def quantized_matmul(x, wq, scales, biases, transpose, group_size, bits, dtype):
 
 
 def softmax_last(x: np.ndarray, dtype: str) -> np.ndarray:
-    """`softmax(scores, axis: -1)` (KVCache.swift:2416): float32 inside, T out."""
+    """`softmax(scores, axis: -1)` (KVCache.swift:2416): float32 inside, T out.
+
+    MLX's CPU backend accumulates in T when `precise` is false (the default the
+    reference uses); accumulating in float32 here is a deliberate choice, stated in
+    the module header: tolerance-level parity only."""
     x = x.astype(np.float32)
     m = x.max(axis=-1, keepdims=True)
     e = np.exp(x - m, dtype=np.float32)

@@ -7,7 +7,9 @@ import torch
 
 import kvhip
 from oracle import kv_oracle as O
-from tests.util import NAME, bits_equal, dev, np32, randn
+from tests.util import NAME, TORCH, bits_equal, dev, np32, randn
+
+import quantizer_kats as QK
 
 pytestmark = pytest.mark.gpu
 
@@ -40,6 +42,38 @@ def test_affine_quantize_bit_exact(dtype, bits, gs):
     assert bits_equal(s, os_, dtype) and bits_equal(b, ob, dtype)
     deq = kvhip.affine_dequantize(wq, s, b, gs, bits)
     assert bits_equal(deq, O.affine_dequantize(owq, os_, ob, gs, bits, NAME[dtype]), dtype)
+
+
+@pytest.mark.parametrize("path", ["standalone", "append one row", "append whole tiles"])
+@pytest.mark.parametrize("gs", [32, 64])
+@pytest.mark.parametrize("case", QK.CASES, ids=[c["name"] for c in QK.CASES])
+def test_quantizers_on_hand_worked_known_answers(case, gs, path):
+    """The device quantizers (the standalone one, the per-row append kernel and the whole-tile
+    append kernel, whose quotient comes from the hardware reciprocal) against literals worked out by
+    hand from MLX's published CPU loop (tests/quantizer_kats.py) -- not against the oracle."""
+    dtype = TORCH[case["dtype"]]
+    bits, reps = case["bits"], gs // 32
+    row = np.asarray(QK.group_values(case) * reps + [0.0] * gs, np.float32)       # D = 2 * gs
+    rows = 1 if path != "append whole tiles" else 128
+    w = np.broadcast_to(row, (1, 1, rows, 2 * gs)).copy()
+    if path == "standalone":
+        wq, s, b = kvhip.affine_quantize(dev(w, dtype), gs, bits)
+    else:
+        cache = kvhip.QuantizedKVCache(gs, bits)
+        cache.update_quantized(dev(w, dtype), dev(w, dtype), fetch=False)
+        st = cache.state
+        for i in range(3):   # K and V planes hold the same rows (V through its transposed tile layout)
+            assert torch.equal(st[i], st[i + 3])
+        wq, s, b = st[0], st[1], st[2]
+    words = QK.packed_words(case) * reps
+    got_w = np32(wq).reshape(rows, -1)
+    sb = O.to_bits(np32(s), case["dtype"]).reshape(rows, 2)
+    bb = O.to_bits(np32(b), case["dtype"]).reshape(rows, 2)
+    for r in range(rows):
+        assert [int(x) for x in got_w[r, :len(words)]] == words, case["wrong"]
+        assert not got_w[r, len(words):].any()
+        assert int(sb[r, 0]) == case["scale_bits"] and int(bb[r, 0]) == case["bias_bits"], case["wrong"]
+        assert int(sb[r, 1]) == {"float16": 0x8002, "bfloat16": 0xB3D7}[case["dtype"]] and int(bb[r, 1]) == 0
 
 
 def check_quantized_state(cache, ocache, dtype):

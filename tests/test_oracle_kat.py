@@ -10,6 +10,8 @@ import pytest
 from oracle import kv_oracle as O
 from oracle import c_oracle as CO
 
+import quantizer_kats as QK
+
 
 def positioned_kv(lo, hi, head_dim=2):
     """positionedKV (KVCacheTests.swift:1282-1293): keys hold +p, values -p."""
@@ -309,6 +311,36 @@ def test_quantize_closed_forms(bits):
     wq, s, b = O.affine_quantize(-ramp - 1, gs, bits, "float32")
     assert np.all(s > 0) and np.all(b == -(nb + 1))
     assert np.array_equal(O.affine_dequantize(wq, s, b, gs, bits, "float32"), -ramp - 1)
+
+
+@pytest.mark.parametrize("impl", ["numpy", "c"])
+@pytest.mark.parametrize("gs", [32, 64])
+@pytest.mark.parametrize("case", QK.CASES, ids=[c["name"] for c in QK.CASES])
+def test_quantize_hand_worked_known_answers(case, gs, impl):
+    """Known answers worked out by hand from MLX's published CPU loop (`quantize<T, U>`,
+    mlx/backend/cpu/quantized.cpp, reached from KVCache.swift:1069-1070); the expected
+    codes, words and parameter bits are literals of tests/quantizer_kats.py, not outputs of
+    a restatement.  Each case separates the algorithm from one plausible misreading
+    (T-rounded scale for the codes, round-half-away, no 1e-7 floor, a non-strict
+    magnitude comparison).  With group size 64 the 32 values are repeated, which leaves
+    the extrema and so every expected value unchanged."""
+    q = O if impl == "numpy" else CO
+    reps = gs // 32
+    row = np.asarray(QK.group_values(case) * reps, np.float32)
+    assert np.array_equal(O.round_to(row, case["dtype"]), row), "case values must be exact in the dtype"
+    # two groups per row, the second one all zeros, so that group boundaries are exercised
+    w = np.concatenate([row, np.zeros(gs, np.float32)])[None]
+    wq, s, b = q.affine_quantize(w, gs, case["bits"], case["dtype"])
+    words = QK.packed_words(case) * reps
+    assert [int(x) for x in wq[0, :len(words)]] == words, case["wrong"]
+    assert [int(x) for x in O.unpack_codes(wq, case["bits"])[0, :32]] == QK.group_codes(case)
+    assert int(O.to_bits(s, case["dtype"])[0, 0]) == case["scale_bits"], case["wrong"]
+    assert int(O.to_bits(b, case["dtype"])[0, 0]) == case["bias_bits"], case["wrong"]
+    # the all-zero neighbour: codes 0, scale T(-1e-7), bias 0.  float32(1e-7) = 0x33D6BF95:
+    # float16 -> 1.68 * 2^-24 -> 2 * 2^-24; bfloat16 -> the low half 0xBF95 rounds 0x33D6 up
+    assert not wq[0, len(words):].any()
+    assert int(O.to_bits(s, case["dtype"])[0, 1]) == {"float16": 0x8002, "bfloat16": 0xB3D7}[case["dtype"]]
+    assert int(O.to_bits(b, case["dtype"])[0, 1]) == 0
 
 
 @pytest.mark.parametrize("bits,bytes_per_group", [(8, 68), (4, 36)])
