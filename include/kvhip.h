@@ -225,6 +225,25 @@ kvhip_status kvhip_cache_attend(kvhip_cache *cache, const void *queries, int32_t
                                 int32_t L, int32_t D, float scale, const kvhip_mask *mask, void *out,
                                 void *stream);
 
+/*
+ * kvhip_cache_attend for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments, same kernels and the same results as kvhip_cache_attend, but the
+ * kernels' scratch (the partial results of the sequence spans) lives in a fixed array of
+ * KVHIP_STATIC_SCRATCH_BYTES that every device the library was initialised on holds until the
+ * process ends, and the call makes no hipMalloc / hipFree.  A call that needs more scratch than
+ * that (the plain kernel on long sequences; every split-sequence decode shape fits) returns
+ * KVHIP_ERR_UNSUPPORTED and enqueues nothing.  Nothing in the array has to start from zero:
+ * each span writes its partial before the merge reads it.  All calls on one device share the
+ * array, so two calls whose device work can overlap (different streams, or a captured graph
+ * replayed beside eager calls) race; calls on one stream are ordered and safe.
+ * Requires kvhip_init on the current device.
+ */
+#define KVHIP_STATIC_SCRATCH_BYTES (16u << 20)
+kvhip_status kvhip_cache_attend_static(kvhip_cache *cache, const void *queries, int32_t B, int32_t Hq,
+                                       int32_t L, int32_t D, float scale, const kvhip_mask *mask,
+                                       void *out, void *stream);
+
 /* `attentionWithCacheUpdate` (AttentionUtils.swift:37-95): update, then attend. */
 kvhip_status kvhip_cache_update_attend(kvhip_cache *cache, const void *queries, const void *keys,
                                        const void *values, int32_t B, int32_t Hq, int32_t Hkv,

@@ -41,7 +41,17 @@ kvhip_status fail(kvhip_status code, const std::string &msg) {
 
 int elem_size(int dtype) { return dtype == KVHIP_F32 ? 4 : 2; }
 
+// Fixed scratch of kvhip_cache_attend_static: the span partials of the attention kernels when the
+// caller cannot allocate.  One copy per device, resident until the process ends.  In host code
+// the array's name is only a handle for hipGetSymbolAddress; every use of its memory goes through
+// the per-device address looked up in kvhip_init.
+constexpr size_t SCRATCH_BYTES = (size_t)KVHIP_STATIC_SCRATCH_BYTES;
+constexpr int MAX_DEVICES = 64;
+float *g_scratch_ptr[MAX_DEVICES] = {};
+
 }  // namespace
+
+static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
 
 struct kvhip_cache {
     int kind = 0;
@@ -503,6 +513,11 @@ kvhip_status kvhip_init(int32_t device) {
     KV_HIP(hipGetDeviceProperties(&prop, device));
     if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(KVHIP_ERR_NO_DEVICE, std::string("libkvhip is built for gfx950 only, found ") + prop.gcnArchName);
+    if (device < MAX_DEVICES && !g_scratch_ptr[device]) {
+        void *p = nullptr;
+        KV_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));  // this device's copy of the array
+        g_scratch_ptr[device] = static_cast<float *>(p);
+    }
     g_inited = true;
     return KVHIP_OK;
 }
@@ -692,8 +707,26 @@ kvhip_status kvhip_cache_fetch(const kvhip_cache *c, void *dk, void *dv, void *s
     return export_slots(c, ident.data(), c->presented, dk, dv, S(stream));
 }
 
-kvhip_status kvhip_cache_attend(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, int32_t L,
-                                int32_t D, float scale, const kvhip_mask *mask, void *out, void *stream) {
+namespace {
+// The cache's own workspace (grown with hipMalloc when a call needs more), or -- for callers that
+// cannot allocate -- a fixed one the call must fit into.
+kvhip_status bind_workspace(kvhip_cache *c, AttendArgs &a, size_t need, float *fixed, size_t fixed_bytes, hipStream_t s) {
+    if (fixed) {
+        if (need > fixed_bytes)
+            return fail(KVHIP_ERR_UNSUPPORTED, "this call needs " + std::to_string(need) + " bytes of scratch, more than the " +
+                                                   std::to_string(fixed_bytes) + " the allocation-free entry point holds");
+        a.workspace = fixed;
+        a.workspace_bytes = fixed_bytes;
+        return KVHIP_OK;
+    }
+    KV_TRY(ensure_ws(c, need, s));
+    a.workspace = c->ws;
+    a.workspace_bytes = c->ws_bytes;
+    return KVHIP_OK;
+}
+
+kvhip_status attend_impl(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, int32_t L, int32_t D, float scale,
+                         const kvhip_mask *mask, void *out, void *stream, float *fixed, size_t fixed_bytes) {
     if (!c || !q || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
     const bool staged_view = c->staging && !c->stage_view.empty();
     if (!c->has_geom || (!c->has_buffers && !staged_view) || c->presented <= 0)
@@ -736,25 +769,34 @@ kvhip_status kvhip_cache_attend(kvhip_cache *c, const void *q, int32_t B, int32_
     }
     hipStream_t s = S(stream);
     if (g_policy == 0 && attend_decode_supported(a)) {
-        KV_TRY(ensure_ws(c, attend_decode_workspace(a), s));
-        a.workspace = c->ws;
-        a.workspace_bytes = c->ws_bytes;
+        KV_TRY(bind_workspace(c, a, attend_decode_workspace(a), fixed, fixed_bytes, s));
         KV_HIP(launch_attend_decode(a, s));
         g_last_kernel = a.st.bits ? 1 : 2;
     } else if (g_policy == 0 && attend_prefill_supported(a)) {
-        KV_TRY(ensure_ws(c, attend_prefill_workspace(a), s));
-        a.workspace = c->ws;
-        a.workspace_bytes = c->ws_bytes;
+        KV_TRY(bind_workspace(c, a, attend_prefill_workspace(a), fixed, fixed_bytes, s));
         KV_HIP(launch_attend_prefill(a, s));
         g_last_kernel = 3;
     } else {
+        KV_TRY(bind_workspace(c, a, attend_generic_workspace(a), fixed, fixed_bytes, s));
         g_last_kernel = 0;
-        KV_TRY(ensure_ws(c, attend_generic_workspace(a), s));
-        a.workspace = c->ws;
-        a.workspace_bytes = c->ws_bytes;
         KV_HIP(launch_attend_generic(a, s));
     }
     return KVHIP_OK;
+}
+}  // namespace
+
+kvhip_status kvhip_cache_attend(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, int32_t L,
+                                int32_t D, float scale, const kvhip_mask *mask, void *out, void *stream) {
+    return attend_impl(c, q, B, Hq, L, D, scale, mask, out, stream, nullptr, 0);
+}
+
+kvhip_status kvhip_cache_attend_static(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, int32_t L,
+                                       int32_t D, float scale, const kvhip_mask *mask, void *out, void *stream) {
+    int dev = -1;
+    KV_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES || !g_scratch_ptr[dev])
+        return fail(KVHIP_ERR_STATE, "kvhip_init has not run on the current device");
+    return attend_impl(c, q, B, Hq, L, D, scale, mask, out, stream, g_scratch_ptr[dev], SCRATCH_BYTES);
 }
 
 kvhip_status kvhip_cache_update_attend(kvhip_cache *c, const void *q, const void *k, const void *v,

@@ -76,6 +76,7 @@ SIGNATURES = {
     "kvhip_cache_update_rope": (_I32, [_P, C.POINTER(Rope), _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I32, _P]),
     "kvhip_cache_fetch": (_I32, [_P, _P, _P, _P]),
     "kvhip_cache_attend": (_I32, [_P, _P, _I32, _I32, _I32, _I32, _F, C.POINTER(Mask), _P, _P]),
+    "kvhip_cache_attend_static": (_I32, [_P, _P, _I32, _I32, _I32, _I32, _F, C.POINTER(Mask), _P, _P]),
     "kvhip_cache_update_attend": (_I32, [_P, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F,
                                          C.POINTER(Mask), _P, _P]),
     "kvhip_cache_mask_plan": (_I32, [_P, _I32, _I32, _I32, C.POINTER(MaskPlan)]),

@@ -199,22 +199,35 @@ class _Cache:
         self._note_shape(keys, values)
         del keep
 
-    def attend(self, queries, scale, mask=None):
-        """Attention of `queries` [B,Hq,L,D] over what the cache presents."""
+    def _check_query_dtype(self, q, k=None):
+        # the C entry points carry no dtype for queries / out: they are read as the cache's dtype
+        want = k.dtype if k is not None else (self._shape[4] if self._shape else q.dtype)
+        if q.dtype != want or (k is not None and self._shape and k.dtype != self._shape[4]):
+            raise TypeError(f"queries are {q.dtype}, keys {k.dtype if k is not None else want}, "
+                            f"the cache holds {self._shape[4] if self._shape else want}")
+
+    def attend(self, queries, scale, mask=None, out=None, static_scratch=False):
+        """Attention of `queries` [B,Hq,L,D] over what the cache presents.  With `static_scratch` the
+        call goes through the allocation-free entry point (`kvhip_cache_attend_static`); pass `out`
+        too if the caller must not allocate at all."""
         q = queries.contiguous()
+        self._check_query_dtype(q)
         B, Hq, Lq, D = q.shape
         Dv = self._shape[3]
-        out = torch.empty((B, Hq, Lq, Dv), dtype=q.dtype, device=q.device)
+        if out is None:
+            out = torch.empty((B, Hq, Lq, Dv), dtype=q.dtype, device=q.device)
+        assert out.is_contiguous() and tuple(out.shape) == (B, Hq, Lq, Dv) and out.dtype == q.dtype
         mask = mask or MaskMode.none()
         m, keep = mask.to_c(B, Hq, Lq)
-        L.check(self._lib.kvhip_cache_attend(self._h, _ptr(q), B, Hq, Lq, D, float(scale), C.byref(m),
-                                             _ptr(out), _stream()))
+        fn = self._lib.kvhip_cache_attend_static if static_scratch else self._lib.kvhip_cache_attend
+        L.check(fn(self._h, _ptr(q), B, Hq, Lq, D, float(scale), C.byref(m), _ptr(out), _stream()))
         del keep
         return out
 
     def update_attend(self, queries, keys, values, scale, mask=None):
         """`attentionWithCacheUpdate` for this cache (AttentionUtils.swift:37-95)."""
         q, k, v = queries.contiguous(), keys.contiguous(), values.contiguous()
+        self._check_query_dtype(q, k)
         B, Hq, Lq, D = q.shape
         H = k.shape[1]
         out = torch.empty((B, Hq, Lq, v.shape[3]), dtype=q.dtype, device=q.device)
