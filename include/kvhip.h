@@ -155,6 +155,9 @@ int32_t kvhip_cache_group_size(const kvhip_cache *cache);      /* QuantizedKVCac
 int32_t kvhip_cache_bits(const kvhip_cache *cache);            /* QuantizedKVCacheProtocol.bits */
 int64_t kvhip_cache_capacity(const kvhip_cache *cache);        /* row extent of the reference's buffers */
 int64_t kvhip_cache_presented_length(const kvhip_cache *cache);/* key extent `update` last returned */
+/* Rows the device pages allocated so far can hold (a multiple of 256).  No counterpart in the
+ * reference, whose `capacity` above is the extent of its arrays; for tests and measurements. */
+int64_t kvhip_cache_device_rows(const kvhip_cache *cache);
 int32_t kvhip_cache_is_trimmable(const kvhip_cache *cache, int64_t after_positions); /* isTrimmable(after:) */
 int64_t kvhip_cache_trim(kvhip_cache *cache, int64_t n);       /* trim(_:) -> positions trimmed */
 /* `offset` is a settable stored property in the reference (KVCache.swift:185;

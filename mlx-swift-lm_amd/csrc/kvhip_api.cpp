@@ -6,7 +6,9 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "kvhip_internal.hpp"
@@ -33,6 +35,15 @@ kvhip_status fail(kvhip_status code, const std::string &msg) {
         if (e_ != hipSuccess)                                                                \
             return fail(KVHIP_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(e_));   \
     } while (0)
+// the same, running `cleanup` before the early return
+#define KV_HIP_OR(expr, cleanup)                                                             \
+    do {                                                                                     \
+        hipError_t e_ = (expr);                                                              \
+        if (e_ != hipSuccess) {                                                              \
+            cleanup;                                                                         \
+            return fail(KVHIP_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(e_));   \
+        }                                                                                    \
+    } while (0)
 #define KV_TRY(expr)                         \
     do {                                     \
         kvhip_status s_ = (expr);            \
@@ -53,6 +64,12 @@ float *g_scratch_ptr[MAX_DEVICES] = {};
 
 static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
 
+// One device allocation backing a run of consecutive pages (all planes of those pages).
+struct Slab {
+    void *base = nullptr;
+    int64_t first_page = 0, pages = 0;
+};
+
 struct kvhip_cache {
     int kind = 0;
     // constructor arguments
@@ -70,8 +87,10 @@ struct kvhip_cache {
     // geometry, fixed by the first update / import / reserve
     bool has_geom = false;
     int B = 0, Hkv = 0;
-    Store st;
-    int64_t cap_pages = 0;
+    Store st;                  // st.pt = the page table in device memory
+    std::vector<Slab> slabs;   // the allocations behind the pages, in page order
+    int64_t cap_pages = 0;     // pages allocated (= page-table entries in use)
+    int64_t pt_cap = 0;        // entries the device page table has room for
     // rotating only: reference row -> physical slot, and slot occupancy
     std::vector<int32_t> rows;
     std::vector<uint8_t> used;
@@ -88,18 +107,84 @@ struct kvhip_cache {
     // scratch for attention
     float *ws = nullptr;
     size_t ws_bytes = 0;
+    // buffers replaced by larger ones while work that reads them may still be in flight: kept
+    // until the cache is freed (hipFree would wait for the whole device)
+    std::vector<void *> parked;
+    // the stream the cache's device work was last enqueued on: freeing the cache releases its
+    // memory behind that work instead of waiting for it
+    mutable hipStream_t last_stream = nullptr;
+    mutable bool used_stream = false;
 
     int64_t cap_slots() const { return cap_pages * PAGE; }
 };
 
 namespace {
 
-void free_store(Store &st) {
-    if (st.k) (void)hipFree(st.k);
-    if (st.v) (void)hipFree(st.v);
-    if (st.ksb) (void)hipFree(st.ksb);
-    if (st.vsb) (void)hipFree(st.vsb);
-    st.k = st.v = st.ksb = st.vsb = nullptr;
+// ---- page storage: slabs of pages behind a page table ------------------------------------------
+// Device buffers that work in flight may still read (page tables and page slabs that were
+// replaced) cannot be freed on the spot: hipFree waits for the whole device.  They are handed
+// over here and freed by the next call that is allowed to block (kvhip_sync, kvhip_cache_free,
+// kvhip_cache_reserve), each once an event recorded behind its last reader has completed.
+struct Retired {
+    hipEvent_t done;
+    std::vector<void *> ptrs;
+};
+std::mutex g_retired_mu;
+std::vector<Retired> g_retired;
+
+void retire(std::vector<void *> &&ptrs, hipStream_t stream) {
+    if (ptrs.empty()) return;
+    Retired r;
+    r.ptrs = std::move(ptrs);
+    if (hipEventCreateWithFlags(&r.done, hipEventDisableTiming) != hipSuccess || hipEventRecord(r.done, stream) != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipDeviceSynchronize();
+        for (void *p : r.ptrs) (void)hipFree(p);
+        return;
+    }
+    std::lock_guard<std::mutex> lock(g_retired_mu);
+    g_retired.push_back(std::move(r));
+}
+
+// Frees what has been retired and is no longer in use.  Blocks (hipFree does): never on the hot path.
+void reap_retired() {
+    std::lock_guard<std::mutex> lock(g_retired_mu);
+    for (size_t i = 0; i < g_retired.size();) {
+        if (hipEventQuery(g_retired[i].done) != hipSuccess) {
+            (void)hipGetLastError();
+            ++i;
+            continue;
+        }
+        for (void *p : g_retired[i].ptrs) (void)hipFree(p);
+        (void)hipEventDestroy(g_retired[i].done);
+        g_retired[i] = std::move(g_retired.back());
+        g_retired.pop_back();
+    }
+}
+
+// The same when `stream` has nothing in flight (then hipFree has little to wait for).
+void reap_if_idle(hipStream_t stream) {
+    if (hipStreamQuery(stream) == hipSuccess) reap_retired();
+    else (void)hipGetLastError();
+}
+
+size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+
+// Gives up the cache's pages and page table: freed at once when nothing in flight can read them
+// (`drained`), otherwise retired behind the work enqueued on `stream` so far.
+void drop_pages(kvhip_cache *c, hipStream_t stream, bool drained) {
+    std::vector<void *> ptrs;
+    for (const Slab &sl : c->slabs) ptrs.push_back(sl.base);
+    if (c->st.pt) ptrs.push_back(const_cast<PageEntry *>(c->st.pt));
+    c->slabs.clear();
+    c->st.pt = nullptr;
+    c->cap_pages = 0;
+    c->pt_cap = 0;
+    if (drained) {
+        for (void *p : ptrs) (void)hipFree(p);
+    } else {
+        retire(std::move(ptrs), stream);
+    }
 }
 
 kvhip_status set_geometry(kvhip_cache *c, int B, int Hkv, int Dk, int Dv, int dtype) {
@@ -145,49 +230,74 @@ kvhip_status set_geometry(kvhip_cache *c, int B, int Hkv, int Dk, int Dv, int dt
     return KVHIP_OK;
 }
 
-// Make room for `slots` physical slots.  Pages are appended; contents keep their place.
+// Make room for `slots` physical slots.  Pages are appended: one new allocation backs the new
+// pages, their entries are added to the page table by a small kernel on `stream`, and nothing
+// that was written moves or is copied.  hipMalloc does not wait for work in flight, so the call
+// only enqueues (the reference re-concatenates every buffer instead, KVCache.swift:419-435,
+// :704-728, :981-989).  When the page table itself is full, a larger one is allocated and the old
+// entries are copied into it on the stream (32 bytes per page); the old table is retired.
 kvhip_status ensure_slots(kvhip_cache *c, int64_t slots, hipStream_t stream, bool exact = false) {
     const int64_t need = (slots + PAGE - 1) / PAGE;
     if (need <= c->cap_pages) return KVHIP_OK;
     int64_t pages = need;
     if (!exact && c->cap_pages > 0) pages = std::max(need, c->cap_pages + (c->cap_pages + 1) / 2);
-    Store ns = c->st;
-    ns.k = ns.v = ns.ksb = ns.vsb = nullptr;
-    const size_t BH = c->st.BH;
-    struct P { char **dst; char *src; size_t cell; } planes[4] = {
-        {&ns.k, c->st.k, c->st.k_cell}, {&ns.v, c->st.v, c->st.v_cell},
-        {&ns.ksb, c->st.ksb, c->st.ksb_cell}, {&ns.vsb, c->st.vsb, c->st.vsb_cell}};
-    for (auto &p : planes) {
-        if (p.cell == 0) continue;
-        const size_t bytes = (size_t)pages * BH * p.cell;
-        hipError_t e = hipMalloc((void **)p.dst, bytes);
-        if (e != hipSuccess) {
-            free_store(ns);
-            return fail(KVHIP_ERR_HIP, std::string("hipMalloc of a cache plane failed: ") + hipGetErrorString(e));
-        }
-        const size_t old = (size_t)c->cap_pages * BH * p.cell;
-        if (old) KV_HIP(hipMemcpyAsync(*p.dst, p.src, old, hipMemcpyDeviceToDevice, stream));
-        // octet words are merged read-modify-write: start them from zero
-        KV_HIP(hipMemsetAsync(*p.dst + old, 0, bytes - old, stream));
+    if (pages > ((int64_t)1 << 22)) return fail(KVHIP_ERR_UNSUPPORTED, "cache longer than 2^30 rows");
+    const Store &st = c->st;
+    const size_t BH = st.BH;
+    if (pages > c->pt_cap) {
+        int64_t cap = std::max<int64_t>(c->pt_cap * 2, 64);
+        while (cap < pages) cap *= 2;
+        void *npt = nullptr;
+        KV_HIP(hipMalloc(&npt, (size_t)cap * sizeof(PageEntry)));
+        if (c->cap_pages > 0)
+            KV_HIP_OR(launch_copy_bytes(npt, st.pt, (size_t)c->cap_pages * sizeof(PageEntry), stream), (void)hipFree(npt));
+        if (st.pt) retire({const_cast<PageEntry *>(st.pt)}, stream);
+        c->st.pt = static_cast<PageEntry *>(npt);
+        c->pt_cap = cap;
     }
-    if (c->cap_pages > 0) KV_HIP(hipStreamSynchronize(stream));
-    free_store(c->st);
-    c->st = ns;
+    // one allocation for the new pages: [K cells | K pairs | V cells | V pairs], each part page-major
+    const int64_t add = pages - c->cap_pages;
+    const size_t stride[4] = {BH * st.k_cell, BH * st.v_cell, BH * st.ksb_cell, BH * st.vsb_cell};
+    const size_t part[4] = {align256(stride[0] * add), align256(stride[1] * add), align256(stride[2] * add), align256(stride[3] * add)};
+    const size_t bytes = part[0] + part[1] + part[2] + part[3];
+    void *base = nullptr;
+    hipError_t e = hipMalloc(&base, bytes);
+    if (e != hipSuccess) {  // memory of freed caches may still be waiting for its release: wait for it and retry
+        (void)hipGetLastError();
+        (void)hipDeviceSynchronize();
+        reap_retired();
+        e = hipMalloc(&base, bytes);
+    }
+    if (e != hipSuccess)
+        return fail(KVHIP_ERR_HIP, std::string("hipMalloc of ") + std::to_string(bytes) + " bytes of cache pages failed: " + hipGetErrorString(e));
+    // packed V words are merged read-modify-write: new pages start from zero
+    KV_HIP_OR(launch_fill_zero(base, bytes, stream), (void)hipFree(base));
+    PageEntry first;
+    char *p = static_cast<char *>(base);
+    first.k = p;
+    first.v = p + part[0];
+    first.ksb = st.ksb_cell ? p + part[0] + part[1] : nullptr;
+    first.vsb = st.vsb_cell ? p + part[0] + part[1] + part[2] : nullptr;
+    KV_HIP_OR(launch_set_pages(const_cast<PageEntry *>(st.pt), (int)c->cap_pages, (int)add, first, stride, stream), (void)hipFree(base));
+    Slab sl;
+    sl.base = base;
+    sl.first_page = c->cap_pages;
+    sl.pages = add;
+    c->slabs.push_back(sl);
     c->cap_pages = pages;
     if (c->kind == KVHIP_KIND_ROTATING) c->used.resize((size_t)c->cap_slots(), 0);
     return KVHIP_OK;
 }
 
-kvhip_status ensure_ws(kvhip_cache *c, size_t bytes, hipStream_t stream) {
+// Scratch of the attention kernels.  A larger one replaces it without waiting for the device:
+// the old buffer stays allocated until the cache is freed.
+kvhip_status ensure_ws(kvhip_cache *c, size_t bytes, hipStream_t) {
     if (bytes <= c->ws_bytes) return KVHIP_OK;
-    if (c->ws) {
-        KV_HIP(hipStreamSynchronize(stream));
-        (void)hipFree(c->ws);
-        c->ws = nullptr;
-        c->ws_bytes = 0;
-    }
-    const size_t want = bytes + bytes / 4;
-    KV_HIP(hipMalloc((void **)&c->ws, want));
+    const size_t want = std::max(bytes + bytes / 4, 2 * c->ws_bytes);
+    void *p = nullptr;
+    KV_HIP(hipMalloc(&p, want));
+    if (c->ws) c->parked.push_back(c->ws);
+    c->ws = static_cast<float *>(p);
     c->ws_bytes = want;
     return KVHIP_OK;
 }
@@ -320,22 +430,28 @@ kvhip_status compact_store(kvhip_cache *c, hipStream_t stream) {
     all.insert(all.end(), c->staged.begin(), c->staged.end());
     const RunList rl = runs_of(all.data(), (int64_t)all.size());
     kvhip_cache tmp;
-    tmp.kind = c->kind;
+    tmp.kind = KVHIP_KIND_SIMPLE;  // plain page store: no slot occupancy to size
     tmp.has_geom = true;
     tmp.B = c->B;
     tmp.Hkv = c->Hkv;
     tmp.st = c->st;
-    tmp.st.k = tmp.st.v = tmp.st.ksb = tmp.st.vsb = nullptr;
-    tmp.cap_pages = 0;
-    KV_TRY(ensure_slots(&tmp, c->cap_slots(), stream, true));
-    for (size_t first = 0; first < rl.size(); first += MAXRUNS) {
+    tmp.st.pt = nullptr;
+    kvhip_status st = ensure_slots(&tmp, c->cap_slots(), stream, true);
+    for (size_t first = 0; st == KVHIP_OK && first < rl.size(); first += MAXRUNS) {
         const size_t cnt = std::min((size_t)MAXRUNS, rl.size() - first);
-        KV_HIP(launch_compact_fp(c->st, pack_runs(rl, first, cnt), tmp.st, (int)all.size(), stream));
+        const hipError_t e = launch_compact_fp(c->st, pack_runs(rl, first, cnt), tmp.st, (int)all.size(), stream);
+        if (e != hipSuccess) st = fail(KVHIP_ERR_HIP, std::string("ring gather failed: ") + hipGetErrorString(e));
     }
-    KV_HIP(hipStreamSynchronize(stream));
-    free_store(c->st);
-    c->st = tmp.st;
-    tmp.st = Store();
+    if (st != KVHIP_OK) {
+        drop_pages(&tmp, stream, false);
+        return st;
+    }
+    // the old pages are retired behind the gather that reads them; the host does not wait
+    drop_pages(c, stream, false);
+    c->slabs.swap(tmp.slabs);
+    c->st.pt = tmp.st.pt;
+    c->cap_pages = tmp.cap_pages;
+    c->pt_cap = tmp.pt_cap;
     std::fill(c->used.begin(), c->used.end(), 0);
     for (size_t i = 0; i < all.size(); ++i) c->used[i] = 1;
     for (size_t i = 0; i < c->rows.size(); ++i) c->rows[i] = (int32_t)i;
@@ -355,17 +471,19 @@ kvhip_status ring_compact_if_needed(kvhip_cache *c, hipStream_t stream) {
 kvhip_status update_simple(kvhip_cache *c, const void *k, const void *v, int L, hipStream_t stream) {
     // KVCache.swift:404-447
     const int64_t prev = c->offset;
+    int64_t ref_len = c->ref_len;
     if (!c->has_buffers || prev + L > c->ref_len) {
         const int64_t n_steps = (c->step + L - 1) / c->step;
         const int64_t grow = n_steps * c->step;
-        if (c->has_buffers) c->ref_len = ((prev % c->step) != 0 ? prev : c->ref_len) + grow;
-        else c->ref_len = grow;
-        c->has_buffers = true;
+        ref_len = c->has_buffers ? ((prev % c->step) != 0 ? prev : c->ref_len) + grow : grow;
     }
     KV_TRY(ensure_slots(c, prev + L, stream));
-    c->offset += L;
     if (c->kind == KVHIP_KIND_QUANTIZED) KV_HIP(launch_append_quant(c->st, k, v, L, 0, (int)prev, L, stream, c->rope));
     else KV_HIP(launch_append_fp(c->st, k, v, L, 0, (int)prev, L, stream, c->rope));
+    // the host counters move only once the device work is enqueued
+    c->ref_len = ref_len;
+    c->has_buffers = true;
+    c->offset = prev + L;
     c->presented = c->offset;
     return KVHIP_OK;
 }
@@ -483,6 +601,12 @@ int64_t state_rows(const kvhip_cache *c) {
 }
 
 hipStream_t S(void *s) { return reinterpret_cast<hipStream_t>(s); }
+// the stream of a call that enqueues work reading or writing the cache's memory
+hipStream_t S(const kvhip_cache *c, void *s) {
+    c->last_stream = reinterpret_cast<hipStream_t>(s);
+    c->used_stream = true;
+    return c->last_stream;
+}
 
 kvhip_cache *new_cache_like(const kvhip_cache *c) {
     kvhip_cache *n = new kvhip_cache();
@@ -524,6 +648,7 @@ kvhip_status kvhip_init(int32_t device) {
 
 kvhip_status kvhip_sync(void *stream) {
     KV_HIP(hipStreamSynchronize(S(stream)));
+    reap_retired();
     return KVHIP_OK;
 }
 
@@ -566,11 +691,27 @@ kvhip_status kvhip_cache_create(const kvhip_config *cfg, kvhip_cache **out) {
 
 void kvhip_cache_free(kvhip_cache *c) {
     if (!c) return;
-    free_store(c->st);
-    if (c->ws) (void)hipFree(c->ws);
-    if (c->stage_tmp_k) (void)hipFree(c->stage_tmp_k);
-    if (c->stage_tmp_v) (void)hipFree(c->stage_tmp_v);
+    // Work that reads the cache may still be in flight on the stream it was last used on.  Its
+    // memory is handed to the retired list behind an event on that stream and released later,
+    // so that dropping a cache (a conversion replacing it, the end of a round) does not make the
+    // host wait for the device.
+    std::vector<void *> ptrs;
+    for (const Slab &sl : c->slabs) ptrs.push_back(sl.base);
+    if (c->st.pt) ptrs.push_back(const_cast<PageEntry *>(c->st.pt));
+    if (c->ws) ptrs.push_back(c->ws);
+    if (c->stage_tmp_k) ptrs.push_back(c->stage_tmp_k);
+    if (c->stage_tmp_v) ptrs.push_back(c->stage_tmp_v);
+    for (void *p : c->parked) ptrs.push_back(p);
+    const hipStream_t stream = c->last_stream;
+    const bool used = c->used_stream;
     delete c;
+    if (ptrs.empty()) return;
+    if (!used) {  // no device work ever touched it
+        for (void *p : ptrs) (void)hipFree(p);
+        return;
+    }
+    retire(std::move(ptrs), stream);
+    reap_if_idle(stream);
 }
 
 int64_t kvhip_cache_offset(const kvhip_cache *c) { return c ? c->offset : -1; }
@@ -580,6 +721,7 @@ int32_t kvhip_cache_group_size(const kvhip_cache *c) { return c ? c->gs : -1; }
 int32_t kvhip_cache_bits(const kvhip_cache *c) { return c ? c->bits : -1; }
 int64_t kvhip_cache_capacity(const kvhip_cache *c) { return c ? c->ref_len : -1; }
 int64_t kvhip_cache_presented_length(const kvhip_cache *c) { return c ? c->presented : -1; }
+int64_t kvhip_cache_device_rows(const kvhip_cache *c) { return c ? c->cap_slots() : -1; }
 
 int32_t kvhip_cache_is_trimmable(const kvhip_cache *c, int64_t after) {
     if (!c) return 0;
@@ -621,7 +763,12 @@ kvhip_status kvhip_cache_reserve(kvhip_cache *c, int32_t B, int32_t Hkv, int32_t
         c->gs = eff;
     }
     KV_TRY(set_geometry(c, B, Hkv, Dk, Dv, dtype));
-    return ensure_slots(c, tokens, nullptr, true);
+    reap_retired();
+    KV_TRY(ensure_slots(c, tokens, nullptr, true));
+    // the zero-fill of the new pages ran on the default stream: wait for it here, so that a
+    // first update on any other (non-blocking) stream is ordered after it
+    KV_HIP(hipStreamSynchronize(nullptr));
+    return KVHIP_OK;
 }
 
 kvhip_status kvhip_cache_update(kvhip_cache *c, const void *keys, const void *values, int32_t B,
@@ -641,9 +788,9 @@ kvhip_status kvhip_cache_update(kvhip_cache *c, const void *keys, const void *va
         }
     }
     KV_TRY(set_geometry(c, B, Hkv, Dk, Dv, dtype));
-    if (c->staging) return stage_update(c, keys, values, L, S(stream));
-    if (c->kind == KVHIP_KIND_ROTATING) return update_rotating(c, keys, values, L, S(stream));
-    return update_simple(c, keys, values, L, S(stream));
+    if (c->staging) return stage_update(c, keys, values, L, S(c, stream));
+    if (c->kind == KVHIP_KIND_ROTATING) return update_rotating(c, keys, values, L, S(c, stream));
+    return update_simple(c, keys, values, L, S(c, stream));
 }
 
 namespace {
@@ -698,13 +845,13 @@ kvhip_status kvhip_cache_fetch(const kvhip_cache *c, void *dk, void *dv, void *s
     if (c->kind == KVHIP_KIND_QUANTIZED)
         return fail(KVHIP_ERR_STATE, "`update` was called on `QuantizedKVCache`. Use `updateQuantized` instead.");
     if (c->staging && !c->stage_view.empty())
-        return export_slots(c, c->stage_view.data(), (int64_t)c->stage_view.size(), dk, dv, S(stream));
+        return export_slots(c, c->stage_view.data(), (int64_t)c->stage_view.size(), dk, dv, S(c, stream));
     if (!c->has_buffers) return fail(KVHIP_ERR_STATE, "cache is empty");
     if (c->kind == KVHIP_KIND_ROTATING)
-        return export_slots(c, c->rows.data(), c->presented, dk, dv, S(stream));
+        return export_slots(c, c->rows.data(), c->presented, dk, dv, S(c, stream));
     std::vector<int32_t> ident((size_t)c->presented);
     for (size_t i = 0; i < ident.size(); ++i) ident[i] = (int32_t)i;
-    return export_slots(c, ident.data(), c->presented, dk, dv, S(stream));
+    return export_slots(c, ident.data(), c->presented, dk, dv, S(c, stream));
 }
 
 namespace {
@@ -767,7 +914,7 @@ kvhip_status attend_impl(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, i
             m.left_pad = mask->left_pad;
         }
     }
-    hipStream_t s = S(stream);
+    hipStream_t s = S(c, stream);
     if (g_policy == 0 && attend_decode_supported(a)) {
         KV_TRY(bind_workspace(c, a, attend_decode_workspace(a), fixed, fixed_bytes, s));
         KV_HIP(launch_attend_decode(a, s));
@@ -901,7 +1048,7 @@ kvhip_status kvhip_cache_state_export(const kvhip_cache *c, int32_t i, void *dst
     const int64_t n = state_rows(c);
     if (n == 0) return KVHIP_OK;
     if (c->kind == KVHIP_KIND_QUANTIZED) {
-        KV_HIP(launch_export_quant(c->st, i, (int)n, dst, S(stream)));
+        KV_HIP(launch_export_quant(c->st, i, (int)n, dst, S(c, stream)));
         return KVHIP_OK;
     }
     std::vector<int32_t> ident;
@@ -911,7 +1058,7 @@ kvhip_status kvhip_cache_state_export(const kvhip_cache *c, int32_t i, void *dst
         for (size_t r = 0; r < ident.size(); ++r) ident[r] = (int32_t)r;
         slots = ident.data();
     }
-    return export_slots(c, slots, n, i == 0 ? dst : nullptr, i == 1 ? dst : nullptr, S(stream));
+    return export_slots(c, slots, n, i == 0 ? dst : nullptr, i == 1 ? dst : nullptr, S(c, stream));
 }
 
 kvhip_status kvhip_cache_state_import(kvhip_cache *c, int32_t count, const void *const *srcs,
@@ -943,16 +1090,23 @@ kvhip_status kvhip_cache_state_import(kvhip_cache *c, int32_t count, const void 
         Dv = (int)v0[3];
         dtype = dtypes[0];
     }
-    // a state setter replaces the buffers wholesale
-    free_store(c->st);
+    {   // refuse a bad geometry before anything the cache holds is given up
+        kvhip_cache probe;
+        probe.kind = c->kind;
+        probe.gs = c->gs;
+        probe.bits = c->bits;
+        KV_TRY(set_geometry(&probe, (int)B, (int)H, Dk, Dv, dtype));
+    }
+    // a state setter replaces the buffers wholesale (the old pages go once the work enqueued
+    // on this stream so far, which may still read them, has run)
+    drop_pages(c, S(c, stream), false);
     c->st = Store();
     c->has_geom = false;
-    c->cap_pages = 0;
     c->rows.clear();
     c->used.clear();
     c->cursor = 0;
     KV_TRY(set_geometry(c, (int)B, (int)H, Dk, Dv, dtype));
-    hipStream_t s = S(stream);
+    hipStream_t s = S(c, stream);
     KV_TRY(ensure_slots(c, std::max<int64_t>(n, 1), s, true));
     if (q) KV_HIP(launch_import_quant(c->st, srcs, (int)n, s));
     else KV_HIP(launch_import_fp(c->st, srcs[0], srcs[1], (int)n, s));
@@ -1051,7 +1205,7 @@ kvhip_status kvhip_cache_copy(const kvhip_cache *c, void *stream, kvhip_cache **
     if (!c || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
     if (c->staging)  // RotatingStagedKVCache.swift:123-125
         return fail(KVHIP_ERR_STATE, "RotatingStagedKVCache is round-scoped and cannot be copied");
-    hipStream_t s = S(stream);
+    hipStream_t s = S(c, stream);
     kvhip_cache *n = new_cache_like(c);
     const int64_t rows = state_rows(c);
     if (c->has_buffers) {
@@ -1062,12 +1216,7 @@ kvhip_status kvhip_cache_copy(const kvhip_cache *c, void *stream, kvhip_cache **
         if (st != KVHIP_OK) { kvhip_cache_free(n); return st; }
         if (c->kind == KVHIP_KIND_QUANTIZED) {
             const int64_t pages = (rows + PAGE - 1) / PAGE;
-            const size_t BH = c->st.BH;
-            const struct { char *d; const char *s; size_t cell; } pl[4] = {
-                {n->st.k, c->st.k, c->st.k_cell}, {n->st.v, c->st.v, c->st.v_cell},
-                {n->st.ksb, c->st.ksb, c->st.ksb_cell}, {n->st.vsb, c->st.vsb, c->st.vsb_cell}};
-            for (auto &p : pl)
-                if (pages) KV_HIP(hipMemcpyAsync(p.d, p.s, (size_t)pages * BH * p.cell, hipMemcpyDeviceToDevice, s));
+            KV_HIP_OR(launch_copy_pages(c->st, n->st, (int)pages, s), kvhip_cache_free(n));
         } else {
             std::vector<int32_t> ident;
             const int32_t *slots = c->rows.data();
@@ -1079,12 +1228,13 @@ kvhip_status kvhip_cache_copy(const kvhip_cache *c, void *stream, kvhip_cache **
             const RunList rl = runs_of(slots, rows);
             for (size_t first = 0; first < rl.size(); first += MAXRUNS) {
                 const size_t cnt = std::min((size_t)MAXRUNS, rl.size() - first);
-                KV_HIP(launch_compact_fp(c->st, pack_runs(rl, first, cnt), n->st, (int)rows, s));
+                KV_HIP_OR(launch_compact_fp(c->st, pack_runs(rl, first, cnt), n->st, (int)rows, s), kvhip_cache_free(n));
             }
         }
         n->has_buffers = true;
         n->ref_len = rows;
         n->presented = rows;
+        (void)S(n, stream);
         if (c->kind == KVHIP_KIND_ROTATING) {
             n->rows.resize((size_t)rows);
             for (int64_t r = 0; r < rows; ++r) {
@@ -1124,13 +1274,13 @@ int64_t kvhip_cache_stage_count(const kvhip_cache *c) { return c ? (int64_t)c->s
 kvhip_status kvhip_cache_stage_fetch(const kvhip_cache *c, void *dk, void *dv, void *stream) {
     if (!c) return fail(KVHIP_ERR_INVALID_ARG, "null cache");
     if (!c->staging || c->staged.empty()) return fail(KVHIP_ERR_STATE, "nothing is staged");
-    return export_slots(c, c->staged.data(), (int64_t)c->staged.size(), dk, dv, S(stream));
+    return export_slots(c, c->staged.data(), (int64_t)c->staged.size(), dk, dv, S(c, stream));
 }
 
 kvhip_status kvhip_cache_stage_commit(kvhip_cache *c, int64_t retaining, void *stream) {
     if (!c) return fail(KVHIP_ERR_INVALID_ARG, "null cache");
     if (!c->staging) return fail(KVHIP_ERR_STATE, "no staged round is open on this cache");
-    hipStream_t s = S(stream);
+    hipStream_t s = S(c, stream);
     // RotatingStagedKVCache.swift:62-76: the first `keep` staged rows go to the ring through
     // the normal write path, the rest are dropped.  The kept rows are first gathered into a
     // dense pair (a few rows), because the normal write path may reuse their slots.
@@ -1138,12 +1288,13 @@ kvhip_status kvhip_cache_stage_commit(kvhip_cache *c, int64_t retaining, void *s
     kvhip_status st = KVHIP_OK;
     if (keep > 0) {
         if ((size_t)keep > c->stage_tmp_rows) {
-            KV_HIP(hipStreamSynchronize(s));
-            if (c->stage_tmp_k) (void)hipFree(c->stage_tmp_k);
-            if (c->stage_tmp_v) (void)hipFree(c->stage_tmp_v);
+            // a larger pair replaces the old one, which an earlier commit's append may still read:
+            // it stays allocated until the cache is freed (no wait for the device here)
+            if (c->stage_tmp_k) c->parked.push_back(c->stage_tmp_k);
+            if (c->stage_tmp_v) c->parked.push_back(c->stage_tmp_v);
             c->stage_tmp_k = c->stage_tmp_v = nullptr;
             c->stage_tmp_rows = 0;
-            const size_t rows = (size_t)std::max<int64_t>(keep, 16);
+            const size_t rows = (size_t)std::max<int64_t>(2 * keep, 16);
             KV_HIP(hipMalloc(&c->stage_tmp_k, (size_t)c->st.BH * rows * c->st.Dk * c->st.es));
             KV_HIP(hipMalloc(&c->stage_tmp_v, (size_t)c->st.BH * rows * c->st.Dv * c->st.es));
             c->stage_tmp_rows = rows;
@@ -1168,7 +1319,7 @@ kvhip_status kvhip_cache_logical_view(const kvhip_cache *c, int64_t tail, int64_
     const std::vector<int32_t> ordered = logical_rows(c, tail);
     *out_rows = (int64_t)ordered.size();
     if ((dk || dv) && !ordered.empty())
-        return export_slots(c, ordered.data(), (int64_t)ordered.size(), dk, dv, S(stream));
+        return export_slots(c, ordered.data(), (int64_t)ordered.size(), dk, dv, S(c, stream));
     return KVHIP_OK;
 }
 
@@ -1181,7 +1332,7 @@ kvhip_status kvhip_cache_to_quantized(const kvhip_cache *c, int32_t group_size, 
     if (c->kind != KVHIP_KIND_SIMPLE) return fail(KVHIP_ERR_INVALID_ARG, "toQuantized belongs to KVCacheSimple");
     if (group_size <= 0) group_size = 64;
     if (bits <= 0) bits = 4;
-    hipStream_t s = S(stream);
+    hipStream_t s = S(c, stream);
     kvhip_config cfg{KVHIP_KIND_QUANTIZED, 0, 0, 0, group_size, bits};
     if (!c->has_buffers) {
         KV_TRY(kvhip_cache_create(&cfg, out));
@@ -1199,17 +1350,10 @@ kvhip_status kvhip_cache_to_quantized(const kvhip_cache *c, int32_t group_size, 
     kvhip_status st = set_geometry(n, c->B, c->Hkv, c->st.Dk, c->st.Dv, c->st.dtype);
     if (st == KVHIP_OK) st = ensure_slots(n, std::max<int64_t>(rows, 1), s, true);
     if (st != KVHIP_OK) { kvhip_cache_free(n); return st; }
-    if (rows > 0) {
-        void *tk = nullptr, *tv = nullptr;
-        const size_t bk = (size_t)c->st.BH * rows * c->st.Dk * c->st.es, bv = (size_t)c->st.BH * rows * c->st.Dv * c->st.es;
-        KV_HIP(hipMalloc(&tk, bk));
-        KV_HIP(hipMalloc(&tv, bv));
-        KV_HIP(launch_export_fp(c->st, identity_runs(rows), 0, (int)rows, 0, (int)rows, tk, tv, s));
-        KV_HIP(launch_append_quant(n->st, tk, tv, (int)rows, 0, 0, (int)rows, s));
-        KV_HIP(hipStreamSynchronize(s));
-        (void)hipFree(tk);
-        (void)hipFree(tv);
-    }
+    // one pass from the full-precision pages into the new cache's pages, enqueued on the stream
+    const int64_t have = std::min(rows, c->cap_slots());  // (an offset set past the buffers has no rows behind it)
+    if (have > 0) KV_HIP_OR(launch_requant_pages(c->st, n->st, (int)have, s), kvhip_cache_free(n));
+    (void)S(n, stream);
     n->has_buffers = true;
     n->ref_len = rows;  // the state setter keeps the arrays' extent
     n->presented = rows;
@@ -1221,7 +1365,7 @@ kvhip_status kvhip_cache_to_quantized(const kvhip_cache *c, int32_t group_size, 
 kvhip_status kvhip_cache_to_unquantized(const kvhip_cache *c, void *stream, kvhip_cache **out) {
     if (!c || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
     if (c->kind != KVHIP_KIND_QUANTIZED) return fail(KVHIP_ERR_INVALID_ARG, "toUnquantized belongs to QuantizedKVCache");
-    hipStream_t s = S(stream);
+    hipStream_t s = S(c, stream);
     kvhip_config cfg{KVHIP_KIND_SIMPLE, 0, 0, 0, 0, 0};
     kvhip_cache *n = nullptr;
     KV_TRY(kvhip_cache_create(&cfg, &n));
@@ -1232,24 +1376,8 @@ kvhip_status kvhip_cache_to_unquantized(const kvhip_cache *c, void *stream, kvhi
     kvhip_status st = set_geometry(n, c->B, c->Hkv, q.Dk, q.Dv, q.dtype);
     if (st == KVHIP_OK) st = ensure_slots(n, std::max<int64_t>(rows, 1), s, true);
     if (st != KVHIP_OK) { kvhip_cache_free(n); return st; }
-    if (rows > 0) {
-        const size_t R = (size_t)q.BH * rows;
-        void *buf[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
-        const size_t bytes[6] = {R * q.Dk * q.bits / 8, R * (q.Dk / q.gs) * q.es, R * (q.Dk / q.gs) * q.es,
-                                 R * q.Dv * q.bits / 8, R * (q.Dv / q.gs) * q.es, R * (q.Dv / q.gs) * q.es};
-        void *dk = nullptr, *dv = nullptr;
-        for (int i = 0; i < 6; ++i) KV_HIP(hipMalloc(&buf[i], bytes[i]));
-        KV_HIP(hipMalloc(&dk, R * q.Dk * q.es));
-        KV_HIP(hipMalloc(&dv, R * q.Dv * q.es));
-        for (int i = 0; i < 6; ++i) KV_HIP(launch_export_quant(q, i, (int)rows, buf[i], s));
-        KV_HIP(launch_affine_dequantize((const uint32_t *)buf[0], buf[1], buf[2], (int64_t)R, q.Dk, q.gs, q.bits, q.dtype, dk, s));
-        KV_HIP(launch_affine_dequantize((const uint32_t *)buf[3], buf[4], buf[5], (int64_t)R, q.Dv, q.gs, q.bits, q.dtype, dv, s));
-        KV_HIP(launch_import_fp(n->st, dk, dv, (int)rows, s));
-        KV_HIP(hipStreamSynchronize(s));
-        for (int i = 0; i < 6; ++i) (void)hipFree(buf[i]);
-        (void)hipFree(dk);
-        (void)hipFree(dv);
-    }
+    if (rows > 0) KV_HIP_OR(launch_dequant_pages(q, n->st, (int)rows, s), kvhip_cache_free(n));
+    (void)S(n, stream);
     n->has_buffers = true;
     n->ref_len = rows;
     n->presented = rows;

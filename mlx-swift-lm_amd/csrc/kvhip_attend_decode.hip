@@ -340,13 +340,18 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     const int tile0 = tile_begin + wave;
     const int my_tiles = tile0 < tile_end ? (tile_end - tile0 + NW - 1) / NW : 0;
     constexpr int PSTEP = NW / 4;  // pages per step
-    const size_t k_step = (size_t)st.BH * st.k_cell * PSTEP, v_step = (size_t)st.BH * st.v_cell * PSTEP;
-    const size_t ksb_step = (size_t)st.BH * st.ksb_cell * PSTEP, vsb_step = (size_t)st.BH * st.vsb_cell * PSTEP;
-    const int page0 = tile0 >> 2, tip = tile0 & 3;  // 4 tiles per page
-    const char *kp = st.k + ((size_t)page0 * st.BH + bh) * st.k_cell + (size_t)tip * TILE * st.k_row;
-    const char *vp = st.v + ((size_t)page0 * st.BH + bh) * st.v_cell + (size_t)tip * D * VROW;
-    const char *ksp = st.ksb + ((size_t)page0 * st.BH + bh) * st.ksb_cell + (size_t)tip * TILE * st.ksb_row;
-    const char *vsp = st.vsb + ((size_t)page0 * st.BH + bh) * st.vsb_cell + (size_t)tip * TILE * st.vsb_row;
+    // pages are found through the page table: one scalar load per plane pair and page; the
+    // offsets of this (b, kv-head)'s cell and of the tile inside it are the same in every page
+    const int tip = tile0 & 3;  // 4 tiles per page
+    int page_k = my_tiles > 0 ? tile0 >> 2 : 0, page_v = page_k;
+    const size_t k_off = (size_t)bh * st.k_cell + (size_t)tip * TILE * st.k_row;
+    const size_t v_off = (size_t)bh * st.v_cell + (size_t)tip * D * VROW;
+    const size_t ksb_off = (size_t)bh * st.ksb_cell + (size_t)tip * TILE * st.ksb_row;
+    const size_t vsb_off = (size_t)bh * st.vsb_cell + (size_t)tip * TILE * st.vsb_row;
+    const char *kp = st.pt[page_k].k + k_off;
+    const char *vp = st.pt[page_k].v + v_off;
+    const char *ksp = st.pt[page_k].ksb + ksb_off;
+    const char *vsp = st.pt[page_k].vsb + vsb_off;
     const uint32_t k_lane = lane * st.k_row, v_lane = lane * VROW;
     const uint32_t ksb_lane = lane * st.ksb_row, vsb_lane = lane * st.vsb_row;
     int slot_next = tile0 * TILE + lane;  // slot of this lane's token in the tile loaded next
@@ -380,8 +385,9 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         t.edge = base_next < full_lo || base_next + (TILE - 1) > full_hi;
         ++k_loaded;
         if (k_loaded < my_tiles) {  // wave-uniform: step to the same tile of the next page
-            kp += k_step;
-            ksp += ksb_step;
+            page_k += PSTEP;
+            kp = st.pt[page_k].k + k_off;
+            ksp = st.pt[page_k].ksb + ksb_off;
             slot_next += PAGE * PSTEP;
             base_next += PAGE * PSTEP;
         }
@@ -403,8 +409,9 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         }
         ++v_loaded;
         if (v_loaded < my_tiles) {
-            vp += v_step;
-            vsp += vsb_step;
+            page_v += PSTEP;
+            vp = st.pt[page_v].v + v_off;
+            vsp = st.pt[page_v].vsb + vsb_off;
         }
     };
     auto load_tile = [&](T &t) {
@@ -740,11 +747,14 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     }
     const int tile0 = tile_begin + wave;
     const int my_tiles = tile0 < tile_end ? (tile_end - tile0 + WAVES - 1) / WAVES : 0;
-    const size_t k_step = (size_t)st.BH * st.k_cell, v_step = (size_t)st.BH * st.v_cell;
-    const int page0 = tile0 >> 2, tip = tile0 & 3;
+    // a wavefront's tiles are a page apart: each is found through the page table (a scalar load)
+    const int tip = tile0 & 3;
+    int page_k = my_tiles > 0 ? tile0 >> 2 : 0, page_v = page_k;
     constexpr int VROW = TILE * 2;  // bytes of one V tile row
-    const char *kp = st.k + ((size_t)page0 * st.BH + bh) * st.k_cell + (size_t)tip * TILE * st.k_row;
-    const char *vp = st.v + ((size_t)page0 * st.BH + bh) * st.v_cell + (size_t)tip * D * VROW;
+    const size_t k_off = (size_t)bh * st.k_cell + (size_t)tip * TILE * st.k_row;
+    const size_t v_off = (size_t)bh * st.v_cell + (size_t)tip * D * VROW;
+    const char *kp = st.pt[page_k].k + k_off;
+    const char *vp = st.pt[page_k].v + v_off;
     // chunk-interleaved tiles: chunk j of the lane's token (K) or column (V) sits 16 * lane bytes into
     // a 1 KB (K) / 16 D byte (V) row of chunks, so every load below is contiguous across the wavefront
     const uint32_t k_lane = lane * 16, v_lane = lane * 16;
@@ -765,14 +775,14 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         load_chunks(buf, kp + k_lane + (size_t)x * (PW / 4) * (TILE * 16), TILE * 16);  // chunks 8x .. 8x+7 of the lane's token
         if (x == NP - 1) {
             ++k_loaded;
-            if (k_loaded < my_tiles) kp += k_step;
+            if (k_loaded < my_tiles) kp = st.pt[++page_k].k + k_off;
         }
     };
     auto load_v = [&](uint32_t *buf, int x) {
         load_chunks(buf, vp + v_lane + (size_t)x * 64 * 16, (size_t)D * 16);  // the 8 token chunks of column 64x + lane
         if (x == NP - 1) {
             ++v_loaded;
-            if (v_loaded < my_tiles) vp += v_step;
+            if (v_loaded < my_tiles) vp = st.pt[++page_v].v + v_off;
         }
     };
 

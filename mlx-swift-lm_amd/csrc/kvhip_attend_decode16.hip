@@ -136,16 +136,20 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 
     // ---- per-lane addresses inside a tile; tiles of one wavefront are a page apart -----------
     // K block tb, lane (n, jj): row of token tok(tb, n) = 16 (n / 4) + 4 tb + n % 4, segment jj
-    const size_t k_step = (size_t)st.BH * st.k_cell, v_step = (size_t)st.BH * st.v_cell;
-    const size_t ksb_step = (size_t)st.BH * st.ksb_cell, vsb_step = (size_t)st.BH * st.vsb_cell;
-    const int page0 = tile0 >> 2, tip = tile0 & 3;
-    const char *kp = st.k + ((size_t)page0 * st.BH + bh) * st.k_cell + (size_t)tip * TILE * st.k_row
-                     + (size_t)(16 * (n >> 2) + (n & 3)) * st.k_row + jj * (KWL * 4);
-    const char *vp = st.v + ((size_t)page0 * st.BH + bh) * st.v_cell + (size_t)tip * D * VROW
-                     + (size_t)n * VROW + jj * (VWL * 4);
+    // each page is found through the page table (a scalar load per plane pair); the offsets below are
+    // the same in every page
+    const int tip = tile0 & 3;
+    int page_k = my_tiles > 0 ? tile0 >> 2 : 0, page_v = page_k;
+    const size_t k_off = (size_t)bh * st.k_cell + (size_t)tip * TILE * st.k_row
+                         + (size_t)(16 * (n >> 2) + (n & 3)) * st.k_row + jj * (KWL * 4);
+    const size_t v_off = (size_t)bh * st.v_cell + (size_t)tip * D * VROW + (size_t)n * VROW + jj * (VWL * 4);
     // (scale, bias) pairs of this lane group's 16 tokens, 16 jj .. 16 jj + 15
-    const char *ksp = st.ksb + ((size_t)page0 * st.BH + bh) * st.ksb_cell + (size_t)(tip * TILE + 16 * jj) * st.ksb_row;
-    const char *vsp = st.vsb + ((size_t)page0 * st.BH + bh) * st.vsb_cell + (size_t)(tip * TILE + 16 * jj) * st.vsb_row;
+    const size_t ksb_off = (size_t)bh * st.ksb_cell + (size_t)(tip * TILE + 16 * jj) * st.ksb_row;
+    const size_t vsb_off = (size_t)bh * st.vsb_cell + (size_t)(tip * TILE + 16 * jj) * st.vsb_row;
+    const char *kp = st.pt[page_k].k + k_off;
+    const char *vp = st.pt[page_k].v + v_off;
+    const char *ksp = st.pt[page_k].ksb + ksb_off;
+    const char *vsp = st.pt[page_k].vsb + vsb_off;
     int base_next = tile0 * TILE;
 
     struct Tile {
@@ -186,8 +190,9 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         t.base = base_next;
         ++k_loaded;
         if (k_loaded < my_tiles) {  // wave-uniform: the same tile of the next page
-            kp += k_step;
-            ksp += ksb_step;
+            ++page_k;
+            kp = st.pt[page_k].k + k_off;
+            ksp = st.pt[page_k].ksb + ksb_off;
             base_next += PAGE;
         }
     };
@@ -211,8 +216,9 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         }
         ++v_loaded;
         if (v_loaded < my_tiles) {
-            vp += v_step;
-            vsp += vsb_step;
+            ++page_v;
+            vp = st.pt[page_v].v + v_off;
+            vsp = st.pt[page_v].vsb + vsb_off;
         }
     };
 

@@ -12,10 +12,12 @@ namespace kvhip {
 // ---------------------------------------------------------------------------
 // Page layout
 //
-// Cached rows live in fixed pages of PAGE tokens.  A plane (K data, V data and,
-// for quantized caches, K and V scale/bias pairs) is one allocation laid out
-// page-major: [page][b*Hkv + h][PAGE rows].  Growing a cache appends pages;
-// nothing already written moves relative to its page.
+// Cached rows live in fixed pages of PAGE tokens.  A page holds, for each plane (K data,
+// V data and, for quantized caches, K and V scale/bias pairs), one cell per (batch row,
+// kv head): [b*Hkv + h][PAGE rows].  Pages are found through a page table in device
+// memory (one PageEntry per page: the address of the page's cells in each plane), so
+// they need not be contiguous: growing a cache allocates further pages and appends
+// their entries; nothing already written moves or is copied.
 //
 //  K plane   one row per token in the reference's own order: Dk elements (full
 //            precision) or Dk*bits/32 packed uint32 words in MLX's bit order.  A
@@ -38,11 +40,17 @@ constexpr int PAGE_SHIFT = 8;
 constexpr int TILE = 64;       // tokens per V tile; 4 tiles per page
 constexpr int MAXRUNS = 8;
 
+// Where page p keeps its [BH] cells of each plane (ksb / vsb: quantized caches only).
+// (K and its pairs are adjacent, V and its pairs likewise: a kernel fetches each half with one load.)
+struct PageEntry {
+    char *k = nullptr;
+    char *ksb = nullptr;
+    char *v = nullptr;
+    char *vsb = nullptr;
+};
+
 struct Store {
-    char *k = nullptr;    // K plane
-    char *v = nullptr;    // V plane
-    char *ksb = nullptr;  // K (scale,bias) plane, quantized only
-    char *vsb = nullptr;  // V (scale,bias) plane, quantized only
+    const PageEntry *pt = nullptr;  // page table (device memory), indexed by slot >> PAGE_SHIFT
     int32_t BH = 0;       // B * Hkv
     int32_t Dk = 0, Dv = 0;
     int32_t dtype = 0;    // kvhip_dtype of cached values / of scales and biases
@@ -76,17 +84,18 @@ struct MaskDev {
 
 #if defined(__HIPCC__)
 // ---- device-side address helpers -------------------------------------------
+// A wave-uniform slot makes the table lookup a scalar load.
 __device__ __forceinline__ const char *k_row_ptr(const Store &st, int bh, int slot) {
-    return st.k + ((size_t)(slot >> PAGE_SHIFT) * st.BH + bh) * st.k_cell + (size_t)(slot & (PAGE - 1)) * st.k_row;
+    return st.pt[slot >> PAGE_SHIFT].k + (size_t)bh * st.k_cell + (size_t)(slot & (PAGE - 1)) * st.k_row;
 }
 __device__ __forceinline__ const char *ksb_row_ptr(const Store &st, int bh, int slot) {
-    return st.ksb + ((size_t)(slot >> PAGE_SHIFT) * st.BH + bh) * st.ksb_cell + (size_t)(slot & (PAGE - 1)) * st.ksb_row;
+    return st.pt[slot >> PAGE_SHIFT].ksb + (size_t)bh * st.ksb_cell + (size_t)(slot & (PAGE - 1)) * st.ksb_row;
 }
 __device__ __forceinline__ const char *vsb_row_ptr(const Store &st, int bh, int slot) {
-    return st.vsb + ((size_t)(slot >> PAGE_SHIFT) * st.BH + bh) * st.vsb_cell + (size_t)(slot & (PAGE - 1)) * st.vsb_row;
+    return st.pt[slot >> PAGE_SHIFT].vsb + (size_t)bh * st.vsb_cell + (size_t)(slot & (PAGE - 1)) * st.vsb_row;
 }
 __device__ __forceinline__ const char *v_cell_ptr(const Store &st, int bh, int slot) {
-    return st.v + ((size_t)(slot >> PAGE_SHIFT) * st.BH + bh) * st.v_cell;
+    return st.pt[slot >> PAGE_SHIFT].v + (size_t)bh * st.v_cell;
 }
 // Full-precision pages are interleaved in 16-byte chunks inside every 64-token tile, so that a
 // wavefront whose lanes are the 64 tokens (K) or 64 adjacent columns (V) reads 1 KB contiguous
@@ -103,7 +112,7 @@ __device__ __forceinline__ size_t vfp_off(const Store &st, int slot, int d) {
     return (size_t)(t >> 6) * ((size_t)TILE * st.Dv * st.es) + ((size_t)(tk / epc) * st.Dv + d) * 16 + (size_t)(tk % epc) * st.es;
 }
 __device__ __forceinline__ const char *k_cell_ptr(const Store &st, int bh, int slot) {
-    return st.k + ((size_t)(slot >> PAGE_SHIFT) * st.BH + bh) * st.k_cell;
+    return st.pt[slot >> PAGE_SHIFT].k + (size_t)bh * st.k_cell;
 }
 // bit position of token t (0..63 inside its tile) within the V tile row of a column
 template <int BITS> __device__ __forceinline__ int v_bitpos(int t) {
@@ -180,12 +189,25 @@ hipError_t launch_import_quant(const Store &st, const void *const srcs[6], int n
 // Device-to-device copy of slots between two stores of identical geometry, through a row map:
 // dst slot i <- src slot of presented row i.
 hipError_t launch_compact_fp(const Store &src, const Runs &runs, const Store &dst, int nrows, hipStream_t s);
+// Rows [0, rows) of the full-precision store `src` quantized into the same slots of `dst`
+// (`KVCacheSimple.toQuantized`), and the reverse (`QuantizedKVCache.toUnquantized`): one pass
+// from pages to pages, no dense copy in between.
+hipError_t launch_requant_pages(const Store &src, const Store &dst, int rows, hipStream_t s);
+hipError_t launch_dequant_pages(const Store &q, const Store &dst, int rows, hipStream_t s);
 hipError_t launch_affine_quantize(const void *src, int64_t rows, int D, int gs, int bits, int dtype,
                                   uint32_t *wq, void *scales, void *biases, hipStream_t s);
 hipError_t launch_affine_dequantize(const uint32_t *wq, const void *scales, const void *biases,
                                     int64_t rows, int D, int gs, int bits, int dtype, void *dst,
                                     hipStream_t s);
 hipError_t launch_mask_materialize(const kvhip_mask_plan_t &plan, uint8_t *dst, hipStream_t s);
+// Zero / copy `bytes` of device memory with a kernel (16-byte aligned pointers and sizes).
+hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s);
+hipError_t launch_copy_bytes(void *dst, const void *src, size_t bytes, hipStream_t s);
+// Page-table entries [first, first + count): page first + i keeps its cells at base.x + i * stride.x
+// for each plane x (pages backed by one allocation lie at a regular stride).
+hipError_t launch_set_pages(PageEntry *pt, int first, int count, PageEntry base, const size_t stride[4], hipStream_t s);
+// Every plane of pages [0, pages) of `src` into the same pages of `dst` (stores of one geometry).
+hipError_t launch_copy_pages(const Store &src, const Store &dst, int pages, hipStream_t s);
 
 struct AttendArgs {
     Store st;

@@ -61,11 +61,11 @@ __global__ void rope_apply_kernel(RopeDev r, const char *x, char *out, int L, in
 //   code_out  one byte per element (for the transposed V assembly)
 //   sb_row    (scale,bias) pairs of dtype DT per group
 //   scales/biases separate arrays of dtype DT per group
-template <int DT, int BITS>
-__device__ __forceinline__ void quantize_row_wave(const void *src, int D, int gs, int lane,
-                                                  uint32_t *k_words, uint8_t *code_out, void *sb_row,
-                                                  void *scales, void *biases, const RopeDev *rope = nullptr,
-                                                  int pos = 0) {
+// `load(d)` hands element d of the row as float.
+template <int DT, int BITS, class LOAD>
+__device__ __forceinline__ void quantize_row_wave_from(LOAD load, int D, int gs, int lane,
+                                                       uint32_t *k_words, uint8_t *code_out, void *sb_row,
+                                                       void *scales, void *biases) {
     const float nb = (float)((1 << BITS) - 1);
     const int K = gs > 64 ? gs / 64 : 1;
     const int width = gs < 64 ? gs : 64;
@@ -76,7 +76,7 @@ __device__ __forceinline__ void quantize_row_wave(const void *src, int D, int gs
         for (int k = 0; k < K; ++k) {
             const int d = base + k * 64 + lane;
             if (d < D) {
-                w[k] = rope ? rope_elem<DT>(*rope, src, d, pos) : Elem<DT>::load(src, d);
+                w[k] = load(d);
                 mn = fminf(mn, w[k]);
                 mx = fmaxf(mx, w[k]);
             }
@@ -107,6 +107,16 @@ __device__ __forceinline__ void quantize_row_wave(const void *src, int D, int gs
             }
         }
     }
+}
+
+template <int DT, int BITS>
+__device__ __forceinline__ void quantize_row_wave(const void *src, int D, int gs, int lane,
+                                                  uint32_t *k_words, uint8_t *code_out, void *sb_row,
+                                                  void *scales, void *biases, const RopeDev *rope = nullptr,
+                                                  int pos = 0) {
+    quantize_row_wave_from<DT, BITS>(
+        [&](int d) { return rope ? rope_elem<DT>(*rope, src, d, pos) : Elem<DT>::load(src, d); }, D, gs, lane, k_words,
+        code_out, sb_row, scales, biases);
 }
 
 // grid (rows, BH): one new row per workgroup, scattered into the chunk-interleaved tile.
@@ -140,10 +150,11 @@ __global__ void append_fp_kernel(Store st, const char *keys, const char *values,
 // the tile; V codes are staged as bytes in LDS and then merged into the transposed
 // tile rows, touching only the token positions this append writes.
 // (ROPE = false carries no rotation code: the single-token decode append stays as small as it was)
-template <int DT, int BITS, bool ROPE>
-__global__ void __launch_bounds__(256)
-append_quant_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, int n,
-                    RopeDev rope) {
+// PAGED: the new rows are rows [src0, src0 + n) of the full-precision page store `src` (a cache
+// being converted) instead of dense arrays.
+template <int DT, int BITS, bool ROPE, bool PAGED>
+__device__ __forceinline__ void append_quant_body(const Store &st, const Store &src, const char *keys, const char *values,
+                                                  int L, int src0, int slot0, int n, const RopeDev &rope) {
     extern __shared__ uint8_t vcodes[];  // [64][Dv]
     const int bh = blockIdx.y;
     const int tile = (slot0 >> 6) + blockIdx.x;
@@ -169,12 +180,22 @@ append_quant_kernel(Store st, const char *keys, const char *values, int L, int s
     for (int item = wave; item < 2 * (hi - lo); item += 4) {
         const int slot = lo + (item >> 1);
         const int l = src0 + (slot - slot0);
-        if ((item & 1) == 0) {
+        uint32_t *kw = reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot)));
+        if constexpr (PAGED) {
+            if ((item & 1) == 0) {
+                const char *kc = k_cell_ptr(src, bh, l);
+                quantize_row_wave_from<DT, BITS>([&](int d) { return Elem<DT>::load(kc + kfp_off(src, l, d), 0); }, st.Dk, st.gs,
+                                                 lane, kw, nullptr, const_cast<char *>(ksb_row_ptr(st, bh, slot)), nullptr, nullptr);
+            } else {
+                const char *vc = v_cell_ptr(src, bh, l);
+                quantize_row_wave_from<DT, BITS>([&](int d) { return Elem<DT>::load(vc + vfp_off(src, l, d), 0); }, st.Dv, st.gs,
+                                                 lane, nullptr, vcodes + (slot & (TILE - 1)) * st.Dv,
+                                                 const_cast<char *>(vsb_row_ptr(st, bh, slot)), nullptr, nullptr);
+            }
+        } else if ((item & 1) == 0) {
             const char *krow = keys + ((size_t)bh * L + l) * st.Dk * st.es;
-            quantize_row_wave<DT, BITS>(krow, st.Dk, st.gs, lane,
-                                        reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot))),
-                                        nullptr, const_cast<char *>(ksb_row_ptr(st, bh, slot)), nullptr, nullptr,
-                                        ROPE ? &rope : nullptr, ROPE ? rope_pos(rope, bh, l) : 0);
+            quantize_row_wave<DT, BITS>(krow, st.Dk, st.gs, lane, kw, nullptr, const_cast<char *>(ksb_row_ptr(st, bh, slot)),
+                                        nullptr, nullptr, ROPE ? &rope : nullptr, ROPE ? rope_pos(rope, bh, l) : 0);
         } else {
             const char *vrow = values + ((size_t)bh * L + l) * st.Dv * st.es;
             quantize_row_wave<DT, BITS>(vrow, st.Dv, st.gs, lane, nullptr, vcodes + (slot & (TILE - 1)) * st.Dv,
@@ -201,6 +222,23 @@ append_quant_kernel(Store st, const char *keys, const char *values, int L, int s
             *p = (old & ~mbits) | nbits;
         }
     }
+}
+
+// grid (64-token tiles touched, BH), 256 threads.  Each wavefront quantizes rows of
+// the tile; V codes are staged as bytes in LDS and then merged into the transposed
+// tile rows, touching only the token positions this append writes.
+// (ROPE = false carries no rotation code: the single-token decode append stays as small as it was)
+template <int DT, int BITS, bool ROPE>
+__global__ void __launch_bounds__(256)
+append_quant_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, int n,
+                    RopeDev rope) {
+    append_quant_body<DT, BITS, ROPE, false>(st, st, keys, values, L, src0, slot0, n, rope);
+}
+
+// The same for rows [row0, row0 + n) of a full-precision page store, written to the same slots of `st`.
+template <int DT, int BITS>
+__global__ void __launch_bounds__(256) requant_rows_kernel(Store st, Store src, int row0, int n) {
+    append_quant_body<DT, BITS, false, true>(st, src, nullptr, nullptr, 0, row0, row0, n, RopeDev());
 }
 
 // ---- whole 64-token tiles (prompt-sized appends) -----------------------------------------
@@ -312,9 +350,12 @@ template <int DT> __device__ __forceinline__ uint32_t pack_scale_bias(float scal
 // affine parameters -- four exact divisions, the costly part -- are worked out once per group
 // instead of once per lane: lane j of a group takes chunk-instance j (and j + GL, ...), writes
 // that group's (scale, bias) pair, and the other lanes fetch bias and reciprocal from it.
-template <int DT, int BITS, int NC, int GL, bool ROPE>
-__global__ void __launch_bounds__(256)
-append_quant_tile_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, RopeDev rope) {
+// PAGED: the 64 rows are tile `l_t / 64` of the full-precision page store `src` (a cache being
+// converted) instead of rows of dense arrays: K chunks are read from the interleaved tile where
+// they lie, the V tile (stored by column) is turned back into rows through LDS.
+template <int DT, int BITS, int NC, int GL, bool ROPE, bool PAGED>
+__device__ __forceinline__ void append_quant_tile_body(const Store &st, const Store &src, const char *keys, const char *values,
+                                                       int L, int src0, int slot0, const RopeDev &rope) {
     constexpr int D = 32 * NC;
     constexpr int GS = 8 * GL;
     constexpr int TPR = D / 8;   // threads per row
@@ -324,17 +365,41 @@ append_quant_tile_kernel(Store st, const char *keys, const char *values, int L, 
     constexpr int SH = GL < NI ? GL : NI;  // lanes of a group that work out parameters
     constexpr int PER = NI / SH;           // chunk-instances per such lane
     __shared__ __attribute__((aligned(8))) uint8_t vcodes[TILE * VP];
+    __shared__ __attribute__((aligned(16))) uint8_t vstage[PAGED ? TILE * D * 2 : 16];  // the source V tile as stored
     const int bh = blockIdx.y;
     const int slot_t = slot0 + blockIdx.x * TILE;
     const int l_t = src0 + blockIdx.x * TILE;
-    const char *kbase = keys + ((size_t)bh * L + l_t) * D * 2;
-    const char *vbase = values + ((size_t)bh * L + l_t) * D * 2;
+    const char *kbase = PAGED ? nullptr : keys + ((size_t)bh * L + l_t) * D * 2;
+    const char *vbase = PAGED ? nullptr : values + ((size_t)bh * L + l_t) * D * 2;
     u4v kraw[NC], vraw[NC];
+    if constexpr (PAGED) {
+        const char *kt = k_cell_ptr(src, bh, l_t) + kfp_off(src, l_t, 0);   // tile start: [chunk][token][16 B]
+        const char *vt = v_cell_ptr(src, bh, l_t) + vfp_off(src, l_t, 0);   // tile start: [8-token chunk][column][16 B]
 #pragma unroll
-    for (int e = 0; e < NC; ++e) {
-        const int c = e * 256 + threadIdx.x;
-        kraw[e] = *reinterpret_cast<const u4v *>(kbase + (size_t)c * 16);
-        vraw[e] = *reinterpret_cast<const u4v *>(vbase + (size_t)c * 16);
+        for (int e = 0; e < NC; ++e) {
+            const int c = e * 256 + threadIdx.x;
+            const int r = c / TPR, ch = c - r * TPR;
+            kraw[e] = *reinterpret_cast<const u4v *>(kt + ((size_t)ch * TILE + r) * 16);
+            *reinterpret_cast<u4v *>(vstage + (size_t)c * 16) = *reinterpret_cast<const u4v *>(vt + (size_t)c * 16);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < NC; ++e) {
+            const int c = e * 256 + threadIdx.x;
+            const int r = c / TPR, dd = (c - r * TPR) * 8;
+            const uint16_t *col = reinterpret_cast<const uint16_t *>(vstage) + ((size_t)(r >> 3) * D + dd) * 8 + (r & 7);
+            uint32_t u[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) u[j] = (uint32_t)col[(2 * j) * 8] | ((uint32_t)col[(2 * j + 1) * 8] << 16);
+            vraw[e] = u4v{u[0], u[1], u[2], u[3]};
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < NC; ++e) {
+            const int c = e * 256 + threadIdx.x;
+            kraw[e] = *reinterpret_cast<const u4v *>(kbase + (size_t)c * 16);
+            vraw[e] = *reinterpret_cast<const u4v *>(vbase + (size_t)c * 16);
+        }
     }
     const RopeDev no_rope;
     const float nb = (float)((1 << BITS) - 1);
@@ -345,7 +410,7 @@ append_quant_tile_kernel(Store st, const char *keys, const char *values, int L, 
     const int r_t = threadIdx.x / TPR;          // row of this thread's chunk 0; chunk e lies 256 / TPR rows further
     const int d0 = (threadIdx.x - r_t * TPR) * 8;
     const int page_off = (slot_t & (PAGE - 1));
-    const size_t cell_idx = (size_t)(slot_t >> PAGE_SHIFT) * st.BH + bh;
+    const PageEntry page = st.pt[slot_t >> PAGE_SHIFT];  // a tile lies inside one page
 #pragma unroll
     for (int e0 = 0; e0 < NC; e0 += EB) {
         float w[NI][8], mn[NI], mx[NI];
@@ -383,8 +448,8 @@ append_quant_tile_kernel(Store st, const char *keys, const char *values, int L, 
             if (pos < SH) {
                 const int i = psel + k * SH;  // this lane's chunk-instance
                 const int row = page_off + r_t + (e0 + i / 2) * (256 / TPR);
-                char *sb = (i & 1) ? const_cast<char *>(st.vsb) + cell_idx * st.vsb_cell + (size_t)row * st.vsb_row
-                                   : const_cast<char *>(st.ksb) + cell_idx * st.ksb_cell + (size_t)row * st.ksb_row;
+                char *sb = (i & 1) ? page.vsb + (size_t)bh * st.vsb_cell + (size_t)row * st.vsb_row
+                                   : page.ksb + (size_t)bh * st.ksb_cell + (size_t)row * st.ksb_row;
                 reinterpret_cast<uint32_t *>(sb)[d0 / GS] = pack_scale_bias<DT>(sc[k], bi[k]);
             }
         }
@@ -434,6 +499,42 @@ append_quant_tile_kernel(Store st, const char *keys, const char *values, int L, 
             out[wi] = word;
         }
         *reinterpret_cast<u4v *>(cell + (size_t)d * (TILE * BITS / 8) + 16 * q) = u4v{out[0], out[1], out[2], out[3]};
+    }
+}
+
+template <int DT, int BITS, int NC, int GL, bool ROPE>
+__global__ void __launch_bounds__(256)
+append_quant_tile_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, RopeDev rope) {
+    append_quant_tile_body<DT, BITS, NC, GL, ROPE, false>(st, st, keys, values, L, src0, slot0, rope);
+}
+
+// grid (tiles, BH): tiles [0, gridDim.x) of the full-precision store `src` into the same slots of `st`
+template <int DT, int BITS, int NC, int GL>
+__global__ void __launch_bounds__(256) requant_tile_kernel(Store st, Store src) {
+    append_quant_tile_body<DT, BITS, NC, GL, false, true>(st, src, nullptr, nullptr, 0, 0, 0, RopeDev());
+}
+
+// grid (64-token tiles, BH): rows [0, rows) of a quantized store as full-precision rows of `dst`
+// (`MLX.dequantized`: scale * code + bias in float32, rounded once to the dtype)
+template <int DT, int BITS>
+__global__ void __launch_bounds__(256) dequant_pages_kernel(Store q, Store dst, int rows) {
+    const int bh = blockIdx.y;
+    const int lo = blockIdx.x * TILE, hi = min(rows, lo + TILE);
+    constexpr int per = 32 / BITS;
+    for (int idx = threadIdx.x; idx < (hi - lo) * q.Dk; idx += 256) {
+        const int t = idx / q.Dk, d = idx - t * q.Dk, slot = lo + t;
+        const uint32_t c = (reinterpret_cast<const uint32_t *>(k_row_ptr(q, bh, slot))[d / per] >> ((d % per) * BITS)) & ((1u << BITS) - 1u);
+        const char *sb = ksb_row_ptr(q, bh, slot);
+        const float sc = Elem<DT>::load(sb, 2 * (d / q.gs)), bi = Elem<DT>::load(sb, 2 * (d / q.gs) + 1);
+        Elem<DT>::store(const_cast<char *>(k_cell_ptr(dst, bh, slot)) + kfp_off(dst, slot, d), 0, __fadd_rn(__fmul_rn(sc, (float)c), bi));
+    }
+    const char *vcell = v_cell_ptr(q, bh, lo);
+    for (int idx = threadIdx.x; idx < (hi - lo) * q.Dv; idx += 256) {
+        const int d = idx / (hi - lo), t = idx - d * (hi - lo), slot = lo + t;   // consecutive threads: consecutive tokens of a column
+        const uint32_t c = v_code_load<BITS>(vcell + v_row_off(q, lo, d), t);
+        const char *sb = vsb_row_ptr(q, bh, slot);
+        const float sc = Elem<DT>::load(sb, 2 * (d / q.gs)), bi = Elem<DT>::load(sb, 2 * (d / q.gs) + 1);
+        Elem<DT>::store(const_cast<char *>(v_cell_ptr(dst, bh, slot)) + vfp_off(dst, slot, d), 0, __fadd_rn(__fmul_rn(sc, (float)c), bi));
     }
 }
 
@@ -819,6 +920,54 @@ hipError_t launch_append_quant(const Store &st, const void *keys, const void *va
     return launch_append_quant_rows(st, keys, values, L, a0 + t.tiles * TILE, b0 + t.tiles * TILE, t.tail, s, r);
 }
 
+hipError_t launch_requant_pages(const Store &src, const Store &st, int rows, hipStream_t s) {
+    if (rows <= 0) return hipSuccess;
+    const int tiles = (rows + TILE - 1) / TILE;
+    const bool tiled = st.es == 2 && st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 128 || st.Dk == 256) &&
+                       (st.bits == 4 || st.bits == 8) && (st.gs == 32 || st.gs == 64 || st.gs == 128) && st.Dk % st.gs == 0;
+    dim3 grid(tiles, st.BH), block(256);
+    if (!tiled) {
+        const size_t lds = (size_t)TILE * st.Dv;
+#define CALL(DT, BITS) hipLaunchKernelGGL((requant_rows_kernel<DT, BITS>), grid, block, lds, s, st, src, 0, rows)
+        KV_DISPATCH_DT_BITS(st.dtype, st.bits, CALL);
+#undef CALL
+        return hipGetLastError();
+    }
+    // whole tiles, the last one included: its rows past `rows` hold zeros or rows trimmed earlier, and
+    // what they quantize to lies past the new cache's offset, where the next append overwrites it
+#define RQ(DT, BITS, NC, GL) hipLaunchKernelGGL((requant_tile_kernel<DT, BITS, NC, GL>), grid, block, 0, s, st, src)
+#define RQ_GL(DT, BITS, NC)                            \
+    do {                                               \
+        if (st.gs == 32) RQ(DT, BITS, NC, 4);          \
+        else if (st.gs == 64) RQ(DT, BITS, NC, 8);     \
+        else RQ(DT, BITS, NC, 16);                     \
+    } while (0)
+#define RQ_NC(DT, BITS)                              \
+    do {                                             \
+        if (st.Dk == 64) RQ_GL(DT, BITS, 2);         \
+        else if (st.Dk == 128) RQ_GL(DT, BITS, 4);   \
+        else RQ_GL(DT, BITS, 8);                     \
+    } while (0)
+    if (st.dtype == KVHIP_F16) {
+        if (st.bits == 4) RQ_NC(0, 4); else RQ_NC(0, 8);
+    } else {
+        if (st.bits == 4) RQ_NC(1, 4); else RQ_NC(1, 8);
+    }
+#undef RQ_NC
+#undef RQ_GL
+#undef RQ
+    return hipGetLastError();
+}
+
+hipError_t launch_dequant_pages(const Store &q, const Store &dst, int rows, hipStream_t s) {
+    if (rows <= 0) return hipSuccess;
+    dim3 grid((rows + TILE - 1) / TILE, q.BH), block(256);
+#define CALL(DT, BITS) hipLaunchKernelGGL((dequant_pages_kernel<DT, BITS>), grid, block, 0, s, q, dst, rows)
+    KV_DISPATCH_DT_BITS(q.dtype, q.bits, CALL);
+#undef CALL
+    return hipGetLastError();
+}
+
 hipError_t launch_export_fp(const Store &st, const Runs &runs, int row_begin, int count, int dst_row0,
                             int dst_rows, void *dst_k, void *dst_v, hipStream_t s) {
     if (count <= 0) return hipSuccess;
@@ -894,6 +1043,72 @@ hipError_t launch_affine_dequantize(const uint32_t *wq, const void *scales, cons
                        (const char *)biases, rows, D, gs, (char *)dst)
     KV_DISPATCH_DT_BITS(dtype, bits, CALL);
 #undef CALL
+    return hipGetLastError();
+}
+
+// Plain fills and copies of plane memory run as kernels: they see virtual addresses only, so a
+// range may span any number of separately mapped physical chunks, and no memset node ends up in
+// a stream capture.  16-byte aligned pointers and sizes.
+__global__ void __launch_bounds__(256) fill_zero_kernel(u4v *dst, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = u4v{0u, 0u, 0u, 0u};
+}
+__global__ void __launch_bounds__(256) copy_bytes_kernel(u4v *dst, const u4v *src, size_t n16) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
+// one thread per new page-table entry
+__global__ void set_pages_kernel(PageEntry *pt, int first, int count, PageEntry base, size_t sk, size_t sv, size_t sksb, size_t svsb) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    PageEntry e;
+    e.k = base.k + (size_t)i * sk;
+    e.v = base.v + (size_t)i * sv;
+    e.ksb = base.ksb ? base.ksb + (size_t)i * sksb : nullptr;
+    e.vsb = base.vsb ? base.vsb + (size_t)i * svsb : nullptr;
+    pt[first + i] = e;
+}
+
+// grid (pages, 4 planes): the [BH] cells of one plane of one page, 16 bytes per thread and step
+__global__ void __launch_bounds__(256) copy_pages_kernel(Store src, Store dst) {
+    const PageEntry a = src.pt[blockIdx.x], b = dst.pt[blockIdx.x];
+    const int plane = blockIdx.y;
+    const char *from = plane == 0 ? a.k : plane == 1 ? a.v : plane == 2 ? a.ksb : a.vsb;
+    char *to = plane == 0 ? b.k : plane == 1 ? b.v : plane == 2 ? b.ksb : b.vsb;
+    const size_t cell = plane == 0 ? src.k_cell : plane == 1 ? src.v_cell : plane == 2 ? src.ksb_cell : src.vsb_cell;
+    const size_t n16 = (size_t)src.BH * cell / 16;
+    for (size_t i = threadIdx.x; i < n16; i += 256) reinterpret_cast<u4v *>(to)[i] = reinterpret_cast<const u4v *>(from)[i];
+}
+
+hipError_t launch_set_pages(PageEntry *pt, int first, int count, PageEntry base, const size_t stride[4], hipStream_t s) {
+    if (count <= 0) return hipSuccess;
+    hipLaunchKernelGGL(set_pages_kernel, dim3((count + 63) / 64), dim3(64), 0, s, pt, first, count, base, stride[0], stride[1],
+                       stride[2], stride[3]);
+    return hipGetLastError();
+}
+
+hipError_t launch_copy_pages(const Store &src, const Store &dst, int pages, hipStream_t s) {
+    if (pages <= 0) return hipSuccess;
+    hipLaunchKernelGGL(copy_pages_kernel, dim3(pages, src.bits ? 4 : 2), dim3(256), 0, s, src, dst);
+    return hipGetLastError();
+}
+
+hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s) {
+    if (bytes == 0) return hipSuccess;
+    if (((uintptr_t)dst | bytes) & 15) return hipErrorInvalidValue;
+    const size_t n16 = bytes / 16;
+    const unsigned grid = (unsigned)std::min<size_t>((n16 + 255) / 256, 256 * 16);
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(grid), dim3(256), 0, s, static_cast<u4v *>(dst), n16);
+    return hipGetLastError();
+}
+
+hipError_t launch_copy_bytes(void *dst, const void *src, size_t bytes, hipStream_t s) {
+    if (bytes == 0) return hipSuccess;
+    if (((uintptr_t)dst | (uintptr_t)src | bytes) & 15) return hipErrorInvalidValue;
+    const size_t n16 = bytes / 16;
+    const unsigned grid = (unsigned)std::min<size_t>((n16 + 255) / 256, 256 * 16);
+    hipLaunchKernelGGL(copy_bytes_kernel, dim3(grid), dim3(256), 0, s, static_cast<u4v *>(dst), static_cast<const u4v *>(src), n16);
     return hipGetLastError();
 }
 

@@ -140,6 +140,11 @@ class _Cache:
         return self._lib.kvhip_cache_capacity(self._h)
 
     @property
+    def device_rows(self):
+        """Rows the device pages allocated so far can hold."""
+        return self._lib.kvhip_cache_device_rows(self._h)
+
+    @property
     def presented_length(self):
         return self._lib.kvhip_cache_presented_length(self._h)
 
