@@ -117,7 +117,8 @@ const char *kvhip_version(void);
 const char *kvhip_last_error_message(void);
 /* Binds the library to HIP device `device` (default 0) and checks it is gfx950. */
 kvhip_status kvhip_init(int32_t device);
-/* Blocks until all work enqueued on `stream` is done (tests; `eval(cache)` LLMModel.swift:56-58). */
+/* Blocks until all work enqueued on `stream` is done (tests; `eval(cache)` LLMModel.swift:56-58).
+ * Also releases device memory of freed caches and replaced buffers whose last readers are done. */
 kvhip_status kvhip_sync(void *stream);
 /* 0 = choose the fastest kernel for the shape (default); 1 = always the generic kernel. */
 void kvhip_set_kernel_policy(int32_t policy);
@@ -139,11 +140,17 @@ kvhip_status kvhip_profile_read(int32_t *out_launches, double *out_total_ms);
 /* ---- lifetime ---------------------------------------------------------- */
 /* KVCacheSimple() / RotatingKVCache(maxSize:keep:step:) / QuantizedKVCache(groupSize:bits:) */
 kvhip_status kvhip_cache_create(const kvhip_config *config, kvhip_cache **out_cache);
-/* Safe with NULL. */
+/* Safe with NULL.  Does not wait for the device: the cache's memory is released once the work
+ * enqueued on the stream it was last used with has run (by a later kvhip_sync / kvhip_cache_reserve,
+ * or at once if that stream is idle). */
 void kvhip_cache_free(kvhip_cache *cache);
 /* `copy()` (KVCache.swift:525-533, :877-885, :1177-1185): independent deep copy. */
 kvhip_status kvhip_cache_copy(const kvhip_cache *cache, void *stream, kvhip_cache **out_cache);
-/* Optional: pre-size device storage for `tokens` cached rows so later updates never reallocate. */
+/* Optional: allocate the device pages for `tokens` cached rows in one piece.  Updates grow a cache by
+ * themselves (further pages are allocated and entered into its page table; nothing is copied and the
+ * call does not wait for the device), so this only saves those allocations.  It has no stream
+ * argument: its zero-fill runs on the default stream and the call waits for it, so that a first
+ * update on any stream is ordered after it. */
 kvhip_status kvhip_cache_reserve(kvhip_cache *cache, int32_t B, int32_t Hkv, int32_t Dk, int32_t Dv,
                                  int32_t dtype, int64_t tokens);
 
@@ -325,7 +332,8 @@ kvhip_status kvhip_cache_stage_commit(kvhip_cache *cache, int64_t retaining, voi
  */
 kvhip_status kvhip_cache_logical_view(const kvhip_cache *cache, int64_t tail, int64_t *out_rows,
                                       void *dst_keys, void *dst_values, void *stream);
-/* `KVCacheSimple.toQuantized(groupSize:bits:)` (KVCache.swift:486-523): bulk quantize on the device. */
+/* `KVCacheSimple.toQuantized(groupSize:bits:)` (KVCache.swift:486-523): one kernel that quantizes
+ * from the full-precision pages into the new cache's pages (no dense copy, no wait for the device). */
 kvhip_status kvhip_cache_to_quantized(const kvhip_cache *cache, int32_t group_size, int32_t bits,
                                       void *stream, kvhip_cache **out_cache);
 /* `QuantizedKVCache.toUnquantized()` (KVCache.swift:1188-1209). */
