@@ -124,17 +124,18 @@ kvhip_status kvhip_sync(void *stream);
 void kvhip_set_kernel_policy(int32_t policy);
 /*
  * Measurement hooks (no counterpart in the reference, which times whole
- * generations with wall clocks, Evaluate.swift:2467).  While enabled, every
- * launch of the dominant attention kernel (split-sequence decode or prefill tile) is bracketed by HIP
- * events on the stream it is launched on.  kvhip_profile_read waits for those
- * events, returns the number of launches and their summed duration in
- * milliseconds, and clears the record.
+ * generations with wall clocks, Evaluate.swift:2467).  kvhip_profile_enable(n) with n > 0
+ * brackets every n-th launch of the dominant attention kernel (split-sequence decode or
+ * prefill tile) with HIP events on the stream it is launched on (n = 1: every launch; a
+ * larger n keeps the event packets, a few microseconds per bracket, out of most steps of a
+ * timed loop); 0 switches it off.  kvhip_profile_read waits for those events, returns the
+ * number of bracketed launches and their summed duration in milliseconds, and clears the record.
  */
 /* Which kernel family the last attention call on this thread's library state used:
  * 0 generic, 1 matrix-core decode (quantized), 2 matrix-core decode (full precision),
  * 3 matrix-core chunked-prefill tile; -1 before the first call.  For tests and reports. */
 int32_t kvhip_last_attend_kernel(void);
-void kvhip_profile_enable(int32_t on);
+void kvhip_profile_enable(int32_t every);
 kvhip_status kvhip_profile_read(int32_t *out_launches, double *out_total_ms);
 
 /* ---- lifetime ---------------------------------------------------------- */

@@ -468,7 +468,9 @@ kvhip_status ring_compact_if_needed(kvhip_cache *c, hipStream_t stream) {
 }
 
 // ---- the three update paths ----------------------------------------------------
-kvhip_status update_simple(kvhip_cache *c, const void *k, const void *v, int L, hipStream_t stream) {
+// `launch` false: everything but the append itself (pages, counters); the caller enqueues the
+// write of rows [offset - L, offset) some other way.
+kvhip_status update_simple(kvhip_cache *c, const void *k, const void *v, int L, hipStream_t stream, bool launch = true) {
     // KVCache.swift:404-447
     const int64_t prev = c->offset;
     int64_t ref_len = c->ref_len;
@@ -478,8 +480,10 @@ kvhip_status update_simple(kvhip_cache *c, const void *k, const void *v, int L, 
         ref_len = c->has_buffers ? ((prev % c->step) != 0 ? prev : c->ref_len) + grow : grow;
     }
     KV_TRY(ensure_slots(c, prev + L, stream));
-    if (c->kind == KVHIP_KIND_QUANTIZED) KV_HIP(launch_append_quant(c->st, k, v, L, 0, (int)prev, L, stream, c->rope));
-    else KV_HIP(launch_append_fp(c->st, k, v, L, 0, (int)prev, L, stream, c->rope));
+    if (launch) {
+        if (c->kind == KVHIP_KIND_QUANTIZED) KV_HIP(launch_append_quant(c->st, k, v, L, 0, (int)prev, L, stream, c->rope));
+        else KV_HIP(launch_append_fp(c->st, k, v, L, 0, (int)prev, L, stream, c->rope));
+    }
     // the host counters move only once the device work is enqueued
     c->ref_len = ref_len;
     c->has_buffers = true;
@@ -656,7 +660,7 @@ void kvhip_set_kernel_policy(int32_t policy) { g_policy = policy; }
 
 int32_t kvhip_last_attend_kernel(void) { return g_last_kernel; }
 
-void kvhip_profile_enable(int32_t on) { profile_enable(on != 0); }
+void kvhip_profile_enable(int32_t every) { profile_enable(every); }
 
 kvhip_status kvhip_profile_read(int32_t *out_launches, double *out_total_ms) {
     if (!out_launches || !out_total_ms) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
@@ -872,8 +876,12 @@ kvhip_status bind_workspace(kvhip_cache *c, AttendArgs &a, size_t need, float *f
     return KVHIP_OK;
 }
 
+// new_k / new_v: the rows of a single-token step whose bookkeeping is done but whose write is
+// still owed (quantized caches); the decode kernel takes them along when it can, else they are
+// appended by a launch of their own first.
 kvhip_status attend_impl(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, int32_t L, int32_t D, float scale,
-                         const kvhip_mask *mask, void *out, void *stream, float *fixed, size_t fixed_bytes) {
+                         const kvhip_mask *mask, void *out, void *stream, float *fixed, size_t fixed_bytes,
+                         const void *new_k = nullptr, const void *new_v = nullptr) {
     if (!c || !q || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
     const bool staged_view = c->staging && !c->stage_view.empty();
     if (!c->has_geom || (!c->has_buffers && !staged_view) || c->presented <= 0)
@@ -915,6 +923,14 @@ kvhip_status attend_impl(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, i
         }
     }
     hipStream_t s = S(c, stream);
+    if (new_k) {
+        if (g_policy == 0 && attend_decode_fuses_append(a)) {
+            a.new_k = new_k;
+            a.new_v = new_v;
+        } else {
+            KV_HIP(launch_append_quant(c->st, new_k, new_v, 1, 0, (int)c->offset - 1, 1, s, nullptr));
+        }
+    }
     if (g_policy == 0 && attend_decode_supported(a)) {
         KV_TRY(bind_workspace(c, a, attend_decode_workspace(a), fixed, fixed_bytes, s));
         KV_HIP(launch_attend_decode(a, s));
@@ -950,6 +966,19 @@ kvhip_status kvhip_cache_update_attend(kvhip_cache *c, const void *q, const void
                                        int32_t B, int32_t Hq, int32_t Hkv, int32_t L, int32_t Dk,
                                        int32_t Dv, int32_t dtype, float scale, const kvhip_mask *mask,
                                        void *out, void *stream) {
+    // One new token into a quantized cache: the decode kernel quantizes the row itself, so the
+    // step is a single launch.  The bookkeeping of `updateQuantized` runs here as usual.
+    if (c && k && v && q && out && L == 1 && c->kind == KVHIP_KIND_QUANTIZED && !c->staging && !c->rope &&
+        (dtype == KVHIP_F16 || dtype == KVHIP_BF16) && (!mask || mask->mode == KVHIP_MASK_NONE) && c->has_geom &&
+        c->has_buffers && c->B == B && c->Hkv == Hkv && c->st.Dk == Dk && c->st.Dv == Dv && c->st.dtype == dtype) {
+        KV_TRY(update_simple(c, k, v, 1, S(c, stream), false));
+        const kvhip_status st = attend_impl(c, q, B, Hq, L, Dk, scale, mask, out, stream, nullptr, 0, k, v);
+        if (st != KVHIP_OK) {  // nothing was written: take the row back
+            c->offset -= 1;
+            c->presented = c->offset;
+        }
+        return st;
+    }
     KV_TRY(kvhip_cache_update(c, k, v, B, Hkv, L, Dk, Dv, dtype, stream));
     return kvhip_cache_attend(c, q, B, Hq, L, Dk, scale, mask, out, stream);
 }

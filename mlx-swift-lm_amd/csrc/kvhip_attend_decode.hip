@@ -363,6 +363,35 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         full_hi = min(full_hi, a.T - 1);
     }
 
+    // ---- the step's new row, when it is still to be written (unmasked single-token decode) -----
+    // Slot T - 1 lies in the last tile, which exactly one wavefront of one workgroup reads (spans
+    // are equal and cover every tile): that wavefront quantizes the row into the cache before it
+    // requests any tile, with the arithmetic of the append kernel, so its own later loads of the
+    // tile see it.  The V code goes into its column's packed word read-modify-write.
+    if constexpr (MM == 0 && RG == 1) {
+        if (a.new_k != nullptr) {  // wave-uniform
+            const int slot = a.T - 1, tl = slot >> 6;
+            if (tl >= tile_begin && tl < tile_end && ((tl - tile_begin) % NW) == wave) {
+                const char *krow = static_cast<const char *>(a.new_k) + (size_t)bh * D * 2;
+                const char *vrow = static_cast<const char *>(a.new_v) + (size_t)bh * D * 2;
+                quantize_row_wave_from<DT, BITS>([&](int d) { return Elem<DT>::load(krow, d); }, D, GS, lane,
+                                                 reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot))),
+                                                 [](int, uint32_t) {}, const_cast<char *>(ksb_row_ptr(st, bh, slot)), nullptr, nullptr);
+                char *vcell = const_cast<char *>(v_cell_ptr(st, bh, slot));
+                const int bp = v_bitpos<BITS>(slot & (TILE - 1));
+                quantize_row_wave_from<DT, BITS>(
+                    [&](int d) { return Elem<DT>::load(vrow, d); }, D, GS, lane, nullptr,
+                    [&](int d, uint32_t code) {
+                        uint32_t *p = reinterpret_cast<uint32_t *>(vcell + v_row_off(st, slot, d)) + (bp >> 5);
+                        *p = (*p & ~(((1u << BITS) - 1u) << (bp & 31))) | (code << (bp & 31));
+                    },
+                    const_cast<char *>(vsb_row_ptr(st, bh, slot)), nullptr, nullptr);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            }
+        }
+    }
+
     // The K half (codes, scales, row bookkeeping) and the V half of tile number k_loaded /
     // v_loaded of this wavefront (clamped to its last tile, so loads past the end stay
     // unconditional and in bounds).
@@ -1083,15 +1112,27 @@ Plan plan_for(const AttendArgs &a) {
     return p;
 }
 
-bool g_profile = false;
+int g_profile = 0;        // 0 off, n: bracket every n-th launch of the dominant kernel
+int g_profile_count = 0;  // launches seen since it was enabled
+bool g_profile_open = false;
 std::vector<hipEvent_t> g_events;  // begin/end pairs
 
 }  // namespace
 
-void profile_enable(bool on) { g_profile = on; }
+void profile_enable(int every) {
+    g_profile = every > 0 ? every : 0;
+    g_profile_count = 0;
+    g_profile_open = false;
+}
 
-void profile_mark(hipStream_t s, bool) {
+void profile_mark(hipStream_t s, bool begin) {
     if (!g_profile) return;
+    if (begin) {
+        g_profile_open = (g_profile_count++ % g_profile) == 0;
+        if (!g_profile_open) return;
+    } else if (!g_profile_open) {
+        return;
+    }
     hipEvent_t e;
     if (hipEventCreate(&e) != hipSuccess) return;
     (void)hipEventRecord(e, s);
@@ -1149,6 +1190,14 @@ bool attend_decode_supported(const AttendArgs &a) {
     if (s.Dk == 128) return s.gs == 64 || s.gs == 128 || (s.gs == 32 && (R <= 4 || s.bits == 4));
     if (s.Dk == 256) return R <= 4 && (s.gs == 64 || s.gs == 128);  // more rows: the prefill tile
     return false;
+}
+
+// The 4-row quantized kernel without a mask writes the step's new row itself.
+bool attend_decode_fuses_append(const AttendArgs &a) {
+    if (!attend_decode_supported(a) || a.st.bits == 0 || a.L != 1) return false;
+    if ((a.Hq / a.Hkv) * a.L > 4 || a.mask.mode != KVHIP_MASK_NONE) return false;
+    static const bool off = getenv("KVHIP_NO_FUSED_APPEND") != nullptr;  // measurement aid
+    return !off;
 }
 
 // 5..16 rows per kv head of a quantized cache go to the 16x16x32 kernel

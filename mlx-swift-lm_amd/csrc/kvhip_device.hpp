@@ -93,4 +93,57 @@ __device__ __forceinline__ uint32_t group_or(uint32_t v, int width) {
     return v;
 }
 
+// One wavefront quantizes one row of D elements (groupwise affine, MLX's CPU algorithm).
+// `load(d)` hands element d of the row as float; `code_sink(d, code)` receives every code.
+// Optional outputs:
+//   k_words   packed codes in MLX order (D*BITS/32 words)
+//   sb_row    (scale, bias) pairs of dtype DT per group
+//   scales / biases   separate arrays of dtype DT per group
+template <int DT, int BITS, class LOAD, class SINK>
+__device__ __forceinline__ void quantize_row_wave_from(LOAD load, int D, int gs, int lane,
+                                                       uint32_t *k_words, SINK code_sink, void *sb_row,
+                                                       void *scales, void *biases) {
+    const float nb = (float)((1 << BITS) - 1);
+    const int K = gs > 64 ? gs / 64 : 1;
+    const int width = gs < 64 ? gs : 64;
+    constexpr int per = 32 / BITS;
+    for (int base = 0; base < D; base += 64 * K) {
+        float w[2] = {0.f, 0.f};
+        float mn = INFINITY, mx = -INFINITY;
+        for (int k = 0; k < K; ++k) {
+            const int d = base + k * 64 + lane;
+            if (d < D) {
+                w[k] = load(d);
+                mn = fminf(mn, w[k]);
+                mx = fmaxf(mx, w[k]);
+            }
+        }
+        group_minmax(mn, mx, width);
+        float scale, bias;
+        affine_params(mn, mx, nb, scale, bias);
+        for (int k = 0; k < K; ++k) {
+            const int d = base + k * 64 + lane;
+            const bool valid = d < D;
+            const uint32_t code = valid ? affine_code(w[k], scale, bias, nb) : 0u;
+            if (k_words) {
+                const uint32_t word = group_or(code << ((d % per) * BITS), per);
+                if (valid && (lane % per) == 0) k_words[d / per] = word;
+            }
+            if (valid) code_sink(d, code);
+        }
+        const int d0 = base + lane;
+        if (d0 < D && (d0 % gs) == 0) {
+            const int g = d0 / gs;
+            if (sb_row) {
+                Elem<DT>::store(sb_row, 2 * g, scale);
+                Elem<DT>::store(sb_row, 2 * g + 1, bias);
+            }
+            if (scales) {
+                Elem<DT>::store(scales, g, scale);
+                Elem<DT>::store(biases, g, bias);
+            }
+        }
+    }
+}
+
 }  // namespace kvhip

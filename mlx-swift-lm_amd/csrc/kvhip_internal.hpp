@@ -221,7 +221,15 @@ struct AttendArgs {
     MaskDev mask;
     float *workspace = nullptr;
     size_t workspace_bytes = 0;
+    // Single-token decode over a quantized cache (`attentionWithCacheUpdate` with L = 1): the new
+    // row [BH, 1, D] of keys and values, still to be quantized into slot T - 1.  The decode kernel
+    // does it itself -- the wavefront that reads the last tile writes the row first -- so a step is
+    // one launch.  NULL: the row is already in the cache.
+    const void *new_k = nullptr;
+    const void *new_v = nullptr;
 };
+// Whether launch_attend_decode quantizes a.new_k / a.new_v itself for these arguments.
+bool attend_decode_fuses_append(const AttendArgs &a);
 // Bytes of scratch each kernel family needs for these arguments.
 size_t attend_generic_workspace(const AttendArgs &a);
 hipError_t launch_attend_generic(const AttendArgs &a, hipStream_t s);
@@ -239,7 +247,7 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s);
 hipError_t launch_attend_decode16(const AttendArgs &a, int tiles_total, int tiles_per_wg, int nsplit, hipStream_t s);
 hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, hipStream_t s);
 // Event bracket around the dominant kernel while profiling is enabled.
-void profile_enable(bool on);
+void profile_enable(int every);
 void profile_mark(hipStream_t s, bool begin);
 hipError_t profile_read(int *launches, double *total_ms);
 

@@ -61,54 +61,6 @@ __global__ void rope_apply_kernel(RopeDev r, const char *x, char *out, int L, in
 //   code_out  one byte per element (for the transposed V assembly)
 //   sb_row    (scale,bias) pairs of dtype DT per group
 //   scales/biases separate arrays of dtype DT per group
-// `load(d)` hands element d of the row as float.
-template <int DT, int BITS, class LOAD>
-__device__ __forceinline__ void quantize_row_wave_from(LOAD load, int D, int gs, int lane,
-                                                       uint32_t *k_words, uint8_t *code_out, void *sb_row,
-                                                       void *scales, void *biases) {
-    const float nb = (float)((1 << BITS) - 1);
-    const int K = gs > 64 ? gs / 64 : 1;
-    const int width = gs < 64 ? gs : 64;
-    constexpr int per = 32 / BITS;
-    for (int base = 0; base < D; base += 64 * K) {
-        float w[2] = {0.f, 0.f};
-        float mn = INFINITY, mx = -INFINITY;
-        for (int k = 0; k < K; ++k) {
-            const int d = base + k * 64 + lane;
-            if (d < D) {
-                w[k] = load(d);
-                mn = fminf(mn, w[k]);
-                mx = fmaxf(mx, w[k]);
-            }
-        }
-        group_minmax(mn, mx, width);
-        float scale, bias;
-        affine_params(mn, mx, nb, scale, bias);
-        for (int k = 0; k < K; ++k) {
-            const int d = base + k * 64 + lane;
-            const bool valid = d < D;
-            const uint32_t code = valid ? affine_code(w[k], scale, bias, nb) : 0u;
-            if (k_words) {
-                const uint32_t word = group_or(code << ((d % per) * BITS), per);
-                if (valid && (lane % per) == 0) k_words[d / per] = word;
-            }
-            if (code_out && valid) code_out[d] = (uint8_t)code;
-        }
-        const int d0 = base + lane;
-        if (d0 < D && (d0 % gs) == 0) {
-            const int g = d0 / gs;
-            if (sb_row) {
-                Elem<DT>::store(sb_row, 2 * g, scale);
-                Elem<DT>::store(sb_row, 2 * g + 1, bias);
-            }
-            if (scales) {
-                Elem<DT>::store(scales, g, scale);
-                Elem<DT>::store(biases, g, bias);
-            }
-        }
-    }
-}
-
 template <int DT, int BITS>
 __device__ __forceinline__ void quantize_row_wave(const void *src, int D, int gs, int lane,
                                                   uint32_t *k_words, uint8_t *code_out, void *sb_row,
@@ -116,7 +68,7 @@ __device__ __forceinline__ void quantize_row_wave(const void *src, int D, int gs
                                                   int pos = 0) {
     quantize_row_wave_from<DT, BITS>(
         [&](int d) { return rope ? rope_elem<DT>(*rope, src, d, pos) : Elem<DT>::load(src, d); }, D, gs, lane, k_words,
-        code_out, sb_row, scales, biases);
+        [&](int d, uint32_t code) { if (code_out) code_out[d] = (uint8_t)code; }, sb_row, scales, biases);
 }
 
 // grid (rows, BH): one new row per workgroup, scattered into the chunk-interleaved tile.
@@ -185,11 +137,13 @@ __device__ __forceinline__ void append_quant_body(const Store &st, const Store &
             if ((item & 1) == 0) {
                 const char *kc = k_cell_ptr(src, bh, l);
                 quantize_row_wave_from<DT, BITS>([&](int d) { return Elem<DT>::load(kc + kfp_off(src, l, d), 0); }, st.Dk, st.gs,
-                                                 lane, kw, nullptr, const_cast<char *>(ksb_row_ptr(st, bh, slot)), nullptr, nullptr);
+                                                 lane, kw, [](int, uint32_t) {}, const_cast<char *>(ksb_row_ptr(st, bh, slot)),
+                                                 nullptr, nullptr);
             } else {
                 const char *vc = v_cell_ptr(src, bh, l);
+                uint8_t *vc_out = vcodes + (slot & (TILE - 1)) * st.Dv;
                 quantize_row_wave_from<DT, BITS>([&](int d) { return Elem<DT>::load(vc + vfp_off(src, l, d), 0); }, st.Dv, st.gs,
-                                                 lane, nullptr, vcodes + (slot & (TILE - 1)) * st.Dv,
+                                                 lane, nullptr, [&](int d, uint32_t code) { vc_out[d] = (uint8_t)code; },
                                                  const_cast<char *>(vsb_row_ptr(st, bh, slot)), nullptr, nullptr);
             }
         } else if ((item & 1) == 0) {

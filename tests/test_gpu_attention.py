@@ -13,7 +13,7 @@ import kvhip
 from kvhip import _lib as L
 from oracle import c_oracle as CO
 from oracle import kv_oracle as O
-from tests.util import NAME, dev, err_stats, np32, randn
+from tests.util import NAME, bits_equal, dev, err_stats, np32, randn
 
 pytestmark = pytest.mark.gpu
 
@@ -422,3 +422,40 @@ def test_ring_in_temporal_order_with_lengths(policy):
     out = c.attend(qd, 1.0 / np.sqrt(D), kvhip.MaskMode.window_mask(T - Lq, 0, lengths=torch.from_numpy(lengths)))
     ref = CO.sdpa(q, ok, ov, 1.0 / np.sqrt(D), m, name)
     check(out, ref, "ring, temporal order, lengths")
+
+
+@pytest.mark.parametrize("dtype,bits,gs,D,B,Hq,Hkv", [
+    (torch.float16, 4, 64, 128, 3, 8, 2), (torch.bfloat16, 4, 64, 128, 2, 4, 4), (torch.float16, 8, 64, 64, 1, 16, 4),
+    (torch.float16, 4, 32, 128, 2, 8, 2), (torch.float16, 8, 128, 256, 1, 4, 2), (torch.bfloat16, 8, 32, 64, 2, 6, 2),
+    (torch.float16, 4, 64, 256, 2, 8, 4),
+])
+def test_single_token_steps_write_their_row_inside_the_decode_kernel(dtype, bits, gs, D, B, Hq, Hkv):
+    """`attentionWithCacheUpdate` with one new token and no mask on a quantized cache is one launch: the decode
+    kernel quantizes the new row into the cache itself.  Codes, scale / bias pairs and offsets must be the
+    append kernel's (the oracle's) bit for bit after every step -- across octets, 64-token tiles, pages and
+    trims -- and the outputs the oracle's within the bound."""
+    rng = np.random.default_rng(bits * 7 + D + gs)
+    cache = kvhip.QuantizedKVCache(gs, bits)
+    ocache = O.QuantizedKVCache(gs, bits, NAME[dtype])
+    scale = D ** -0.5
+    tol = 1e-2 if dtype == torch.float16 else 1.6e-2
+    for start, steps, trim in [(1, 9, 0), (52, 14, 3), (250, 9, 0), (1500, 5, 2)]:
+        n = start - ocache.offset
+        if n > 0:
+            k, kd = randn(rng, (B, Hkv, n, D), dtype, 1.5)
+            v, vd = randn(rng, (B, Hkv, n, D), dtype, 0.7)
+            cache.update_quantized(kd, vd, fetch=False)
+            ocache.update_quantized(k, v)
+        for _ in range(steps):
+            q, qd = randn(rng, (B, Hq, 1, D), dtype)
+            k, kd = randn(rng, (B, Hkv, 1, D), dtype, 1.5)
+            v, vd = randn(rng, (B, Hkv, 1, D), dtype, 0.7)
+            got = np32(cache.update_attend(qd, kd, vd, scale))
+            assert kvhip.load().kvhip_last_attend_kernel() == 1
+            ref = O.attention_with_cache_update(q, k, v, ocache, scale, O.Mask.NONE, NAME[dtype])
+            mx, mean = err_stats(got, ref)
+            assert mx <= tol and mean <= 1e-3, (ocache.offset, mx, mean)
+            assert cache.offset == ocache.offset
+        for i, (a, b) in enumerate(zip(cache.state, ocache.get_state())):
+            assert np.array_equal(np32(a), b) if i % 3 == 0 else bits_equal(a, b, dtype), (start, i)
+        assert cache.trim(trim) == ocache.trim(trim)
