@@ -53,9 +53,11 @@ def main():
     ap.add_argument("--cpu-steps", type=int, default=5, help="decode steps timed on the CPU baseline after one warm-up (0 = skip)")
     ap.add_argument("--reserve", action="store_true",
                     help="pre-size the cache's pages (default: grow from empty, as the reference does)")
-    ap.add_argument("--workload", default="cfg3", choices=["cfg3", "cfg1", "cfg2", "cfg4", "cfg5"],
+    ap.add_argument("--workload", default="cfg3", choices=["cfg3", "cfg1", "cfg2", "cfg4", "cfg5", "prefill"],
                     help="cfg3 (default) is the configuration the metric is quoted on; the others are the "
                          "remaining BASELINE.json configs (reported as one JSON object each)")
+    ap.add_argument("--prefill-shape", default=None,
+                    help="with --workload prefill: one shape B,Hq,Hkv,D,L,T,dtype (dtype f16 or bf16) instead of the table")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy 4 times (reference point for rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -261,6 +263,40 @@ def other_workload(args, torch, kvhip, L, dev):
         n, ms = C.c_int32(), C.c_double()
         L.check(lib.kvhip_profile_read(C.byref(n), C.byref(ms)))
         return ms.value / max(n.value, 1), n.value
+
+    if args.workload == "prefill":
+        # the chunked-prefill tile on its own: L new rows attending causally over T cached keys (the new rows
+        # included), KVCacheSimple; flops = 4 * B * Hq * D * (keys each row sees)
+        shapes = [(1, 32, 8, 128, 2048, 8192, "f16"), (1, 32, 8, 128, 2048, 8192, "bf16"), (4, 32, 8, 128, 512, 4096, "f16"),
+                  (1, 32, 8, 128, 4096, 4096, "f16"), (2, 16, 4, 64, 2048, 4096, "f16"), (4, 8, 4, 256, 512, 4608, "f16"),
+                  (4, 8, 4, 256, 512, 4608, "bf16")]
+        if args.prefill_shape:
+            f = args.prefill_shape.split(",")
+            shapes = [tuple(int(x) for x in f[:6]) + (f[6],)]
+        rows = []
+        for Bn, Hq, Hkv, D, Lq, T, dn in shapes:
+            dtype = torch.float16 if dn == "f16" else torch.bfloat16
+            cache = kvhip.KVCacheSimple()
+            k = torch.randn(Bn, Hkv, T, D, generator=g, device=dev).to(dtype)
+            cache.update(k, k.flip(-1), fetch=False)
+            q = torch.randn(Bn, Hq, Lq, D, generator=g, device=dev).to(dtype)
+            mask = kvhip.MaskMode.causal()
+            for _ in range(2):
+                cache.attend(q, D ** -0.5, mask)
+            torch.cuda.synchronize()
+            lib.kvhip_profile_enable(1)
+            for _ in range(args.steps if args.steps != 256 else 10):
+                cache.attend(q, D ** -0.5, mask)
+            torch.cuda.synchronize()
+            lib.kvhip_profile_enable(0)
+            ms, n = kernel_ms()
+            keys = sum(T - Lq + i + 1 for i in range(Lq))
+            fl = 4.0 * Bn * Hq * keys * D
+            rows.append({"shape": f"B{Bn} {Hq}q/{Hkv}kv D{D} {dn}, {Lq} new rows over {T} keys, causal", "launches": n,
+                         "kernel_ms": round(ms, 4), "TFLOPs": round(fl / ms / 1e9, 1),
+                         "frac_of_2.5PF": round(fl / ms / 1e9 / 2500.0, 4)})
+            del cache, k, q
+        return {"workload": "chunked-prefill tile (prefill_fp_kernel) on its own", "results": rows}
 
     if args.workload == "cfg1":
         # the reference's own CPU-runnable case: B1, 16q/4kv, D64, fp16, 8-bit g64; prefill 512 under

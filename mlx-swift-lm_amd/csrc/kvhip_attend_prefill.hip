@@ -15,6 +15,8 @@
 // with the online softmax in fp32 between them.  Masks are evaluated from indices
 // (causal, window, lengths, left padding) or read from the caller's array; for the
 // symbolic ones whole key tiles outside the visible range are skipped.
+#include <cstdlib>
+
 #include "kvhip_mask.hpp"
 
 namespace kvhip {
@@ -200,6 +202,7 @@ prefill_kernel(AttendArgs a, int nsplit) {
     const int kt = tid / KT, kpart = tid % KT;
     const bool k_on = KT == 8 || tid < BN * KT;   // with 4 threads per row the upper half has no K work
 
+    PageCursor page_cur(st, min(tile_lo * BN, max(a.slots - 1, 0)));  // tiles of 32 slots: the entry is fetched once per eight tiles
     auto fetch = [&](int tile) {
         const int slot0 = tile * BN;
         if (tid < BN) {
@@ -209,19 +212,21 @@ prefill_kernel(AttendArgs a, int nsplit) {
             else row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
             row_reg = (row >= 0 && row < a.T) ? row : -1;
         }
-        const char *cell = v_cell_ptr(st, bh, slot0);
+        const PageEntry &pe = page_cur.at(st, slot0);
+        const int in_page = slot0 & (PAGE - 1);
+        const char *cell = pe.v + (size_t)bh * st.v_cell;
         if (k_on) {
-            const uint32_t *w = reinterpret_cast<const uint32_t *>(k_row_ptr(st, bh, slot0 + kt)) + kpart * KQW;
+            const uint32_t *w = reinterpret_cast<const uint32_t *>(pe.k + (size_t)bh * st.k_cell + (size_t)(in_page + kt) * st.k_row) + kpart * KQW;
 #pragma unroll
             for (int e = 0; e < KQW; ++e) kq[e] = w[e];
             // 8 threads per row: the D/8 codes of this thread lie in one group (group sizes are >= 32 >= D/8);
             // 4 threads per row: in at most two, the first code's and the last code's
-            const uint32_t *sbp = reinterpret_cast<const uint32_t *>(ksb_row_ptr(st, bh, slot0 + kt));
+            const uint32_t *sbp = reinterpret_cast<const uint32_t *>(pe.ksb + (size_t)bh * st.ksb_cell + (size_t)(in_page + kt) * st.ksb_row);
             ksb_raw = sbp[(kpart * CPT) / st.gs];
             if constexpr (KT != 8) ksb_raw_hi = sbp[(kpart * CPT + CPT - 1) / st.gs];
         }
         if (tid < BN) {
-            const uint32_t *sb = reinterpret_cast<const uint32_t *>(vsb_row_ptr(st, bh, slot0 + tid));
+            const uint32_t *sb = reinterpret_cast<const uint32_t *>(pe.vsb + (size_t)bh * st.vsb_cell + (size_t)(in_page + tid) * st.vsb_row);
 #pragma unroll
             for (int gg = 0; gg < D / 32; ++gg)
                 if (gg < D / st.gs) vsb_raw[gg] = sb[gg];
@@ -499,6 +504,8 @@ bool attend_prefill_supported(const AttendArgs &a) {
 // used when that would leave the grid too small to fill 256 CUs twice over.
 static bool prefill_wide(const AttendArgs &a) {
     const int R = (a.Hq / a.Hkv) * a.L;
+    static const int forced = getenv("KVHIP_PREFILL_WIDE") ? atoi(getenv("KVHIP_PREFILL_WIDE")) : -1;  // measurement aid
+    if (forced >= 0) return forced != 0 && a.st.Dk <= 128;
     return (size_t)((R + 127) / 128) * a.st.BH >= 512 && a.st.Dk <= 128;
 }
 

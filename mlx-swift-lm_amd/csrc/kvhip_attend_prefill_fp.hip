@@ -17,6 +17,13 @@
 // that every query row of the workgroup sees completely skip all mask tests.
 #include "kvhip_mask.hpp"
 
+#ifndef KVHIP_PREFILL_LM
+#define KVHIP_PREFILL_LM 1
+#endif
+#ifndef KVHIP_PREFILL_BF16_P
+#define KVHIP_PREFILL_BF16_P 1
+#endif
+
 namespace kvhip {
 
 namespace {
@@ -36,7 +43,8 @@ typedef __attribute__((address_space(3))) uint32_t LDS_U32;
 // vector-memory operations complete in order, so an operation it does not count only makes a wait
 // stricter.
 __device__ __forceinline__ void load_to_lds(const void *src, const void *lds_wave_base) {
-    const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(LDS_U32 *)lds_wave_base);
+    // (the low half of a flat address inside the LDS aperture is the LDS address itself)
+    const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds_wave_base);
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(base) : "memory", "m0");
 }
 union Op8 {
@@ -52,6 +60,16 @@ constexpr float RAISE = 8.f;  // log2 units
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ uint32_t rn_h2(float lo, float hi) {  // round to nearest even
     return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
+}
+// two non-negative finite floats -> two bf16 (round to nearest even) in one dword
+__device__ __forceinline__ uint32_t rn_bf2(float lo, float hi) {
+    const uint32_t a = __float_as_uint(lo), b = __float_as_uint(hi);
+    return ((a + 0x7fffu + ((a >> 16) & 1u)) >> 16) | ((b + 0x7fffu + ((b >> 16) & 1u)) & 0xffff0000u);
+}
+// the probabilities of one lane as the PV operand: fp16, or bf16 for bf16 caches on the direct path
+template <bool BF> __device__ __forceinline__ u4 pack_p(const float (&p)[2][4]) {
+    if constexpr (BF) return u4{rn_bf2(p[0][0], p[0][1]), rn_bf2(p[0][2], p[0][3]), rn_bf2(p[1][0], p[1][1]), rn_bf2(p[1][2], p[1][3])};
+    else return u4{rn_h2(p[0][0], p[0][1]), rn_h2(p[0][2], p[0][3]), rn_h2(p[1][0], p[1][1]), rn_h2(p[1][2], p[1][3])};
 }
 // two bf16 (one dword) -> two fp16, exact for every bf16 inside the fp16 range
 __device__ __forceinline__ uint32_t bf2_to_h2(uint32_t w) {
@@ -88,7 +106,11 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     // one filled while this one is contracted.  fp16 caches move V the same way, [8-token
     // chunk][column]; bf16 V is staged through registers (converted to fp16 on the way) into two
     // padded buffers of V^T.
-    constexpr bool VDMA = DT == 0;
+    // bf16 caches keep V as bf16 too: the probabilities are then rounded to bf16 for the PV matrix-core
+    // instruction (the reference's softmax output is an array of the cache's dtype as well), so that V
+    // needs no conversion and takes the direct path.  KVHIP_PREFILL_BF16_P = 0 brings back fp16
+    // probabilities with V converted to fp16 while it is staged through registers.
+    constexpr bool VDMA = DT == 0 || KVHIP_PREFILL_BF16_P;
     constexpr int NB = 2;
     // (one array per buffer, K then V, selected by constants after inlining: the compiler follows
     // loads into LDS per variable, and a read of one buffer then need not wait for the loads in
@@ -145,7 +167,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     // factor -- so that the maximum can be taken on the raw scores and the scale folded into one
     // multiply-add; the denominators ride on the matrix cores (lacc = ones . P^T sums the same
     // rounded probabilities the numerator uses; all 16 rows of the block hold the same sums).
-    constexpr bool LM = D <= 128 && DT == 0;
+    constexpr bool LM = D <= 128 && DT == 0 && KVHIP_PREFILL_LM;
     const bool flip = LM && a.scale < 0.f;
     const float sl2 = LM ? fmaxf(fabsf(a.scale) * LOG2E, 1e-30f) : a.scale * LOG2E;
 
@@ -232,9 +254,11 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         u4 v[NC];
     };
     Stg setA;
+    // tiles of 32 slots: the page-table entry is fetched once per eight tiles
+    PageCursor page_fetch(st, min(tile_lo * BN, max(a.slots - 1, 0))), page_dma = page_fetch;
     [[maybe_unused]] auto fetch = [&](int tile, Stg &g) __attribute__((always_inline)) {
         const int slot0 = tile * BN;
-        const char *vbase = v_cell_ptr(st, bh, slot0) + vfp_off(st, slot0, 0);
+        const char *vbase = page_fetch.at(st, slot0).v + (size_t)bh * st.v_cell + vfp_off(st, slot0, 0);
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
             const int c = min(e * 256 + tid, CH - 1);
@@ -273,8 +297,9 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             const bool full = __all(row >= keep_lo && row <= keep_hi);  // the first 32 lanes of wavefront 0
             if (tid == 0) full_s[buf] = full;
         }
-        const char *kbase = k_cell_ptr(st, bh, slot0) + kfp_off(st, slot0, 0);
-        const char *vbase = v_cell_ptr(st, bh, slot0) + vfp_off(st, slot0, 0);
+        const PageEntry &pe = page_dma.at(st, slot0);
+        const char *kbase = pe.k + (size_t)bh * st.k_cell + kfp_off(st, slot0, 0);
+        const char *vbase = pe.v + (size_t)bh * st.v_cell + vfp_off(st, slot0, 0);
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
             const int c = min(e * 256 + tid, CH - 1);
@@ -475,7 +500,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                     psum += p[mt][i];
                 }
             l_run[qt] += psum;
-            pb[qt].v = u4{rn_h2(p[0][0], p[0][1]), rn_h2(p[0][2], p[0][3]), rn_h2(p[1][0], p[1][1]), rn_h2(p[1][2], p[1][3])};
+            pb[qt].v = pack_p<DT == 1 && VDMA>(p);
         
         }
 
@@ -498,7 +523,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             for (int x = 0; x < 4; ++x)
 #pragma unroll
                 for (int qt = 0; qt < QT; ++qt)
-                    oacc[qt][d0 + x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va[x].h, pb[qt].h, oacc[qt][d0 + x], 0, 0, 0);
+                    oacc[qt][d0 + x] = mfma_qk<(DT == 1 && VDMA) ? 1 : 0>(va[x], pb[qt], oacc[qt][d0 + x]);
         }
         // What was requested at the top of this step has to land before the barrier: it has had the
         // whole step for it, so the wait is short, and an LDS read of the next step never meets a load

@@ -114,6 +114,33 @@ __device__ __forceinline__ size_t vfp_off(const Store &st, int slot, int d) {
 __device__ __forceinline__ const char *k_cell_ptr(const Store &st, int bh, int slot) {
     return st.pt[slot >> PAGE_SHIFT].k + (size_t)bh * st.k_cell;
 }
+// The page-table entry of the page that holds a wave-uniform `slot`, fetched again only when the
+// page changes: a kernel that walks the slots in tiles smaller than a page keeps the entry in
+// scalar registers across the tiles of one page.
+__device__ __forceinline__ char *wave_uniform(char *p) {  // tells the compiler: keep it in scalar registers
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<char *>(((uint64_t)hi << 32) | lo);
+}
+struct PageCursor {
+    int page;
+    PageEntry e;
+    __device__ __forceinline__ void fetch(const Store &st, int p) {
+        page = p;
+        const PageEntry &src = st.pt[p];
+        e.k = wave_uniform(src.k);
+        e.ksb = wave_uniform(src.ksb);
+        e.v = wave_uniform(src.v);
+        e.vsb = wave_uniform(src.vsb);
+    }
+    // starts on the page of `slot` (any slot the kernel may read: the entry is valid from the start)
+    __device__ __forceinline__ PageCursor(const Store &st, int slot) { fetch(st, __builtin_amdgcn_readfirstlane(slot >> PAGE_SHIFT)); }
+    __device__ __forceinline__ const PageEntry &at(const Store &st, int slot) {
+        const int p = __builtin_amdgcn_readfirstlane(slot >> PAGE_SHIFT);
+        if (p != page) fetch(st, p);
+        return e;
+    }
+};
 // bit position of token t (0..63 inside its tile) within the V tile row of a column
 template <int BITS> __device__ __forceinline__ int v_bitpos(int t) {
     if (BITS == 4) return 32 * (t >> 3) + 4 * (((t & 7) >> 1) + 4 * (t & 1));

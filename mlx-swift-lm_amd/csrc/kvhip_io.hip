@@ -419,7 +419,7 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
             codes8<BITS>(w[i], scale, bias, inv, q);
             if ((i & 1) == 0) {
                 // ---- K: packed words in natural order --------------------------------------------
-                uint32_t *kw = reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot_t + r)));
+                uint32_t *kw = reinterpret_cast<uint32_t *>(page.k + (size_t)bh * st.k_cell + (size_t)(page_off + r) * st.k_row);
                 if (BITS == 4) {
                     kw[d0 / 8] = pack_nibbles(q[0], q[1], q[2], q[3]) | (pack_nibbles(q[4], q[5], q[6], q[7]) << 16);
                 } else {
@@ -438,7 +438,7 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
     // continue the same row, so the tile rows are written contiguously
     constexpr int TPW = 32 / BITS;        // tokens per word
     constexpr int CPR = TILE / TPW / 4;   // 16-byte chunks per row
-    char *cell = const_cast<char *>(v_cell_ptr(st, bh, slot_t)) + v_row_off(st, slot_t, 0);
+    char *cell = page.v + (size_t)bh * st.v_cell + v_row_off(st, slot_t, 0);
     for (int c = threadIdx.x; c < D * CPR; c += 256) {
         const int d = c / CPR, q = c - d * CPR;
         uint32_t out[4];
@@ -505,6 +505,7 @@ append_fp_tile_kernel(Store st, const char *keys, const char *values, int L, int
     const int l_t = src0 + blockIdx.x * TILE;
     const char *kbase = keys + ((size_t)bh * L + l_t) * D * 2;
     const char *vbase = values + ((size_t)bh * L + l_t) * D * 2;
+    char *kcell = st.pt[slot_t >> PAGE_SHIFT].k + (size_t)bh * st.k_cell;  // a tile lies inside one page
     u4v kraw[NC], vraw[NC];
 #pragma unroll
     for (int e = 0; e < NC; ++e) {
@@ -535,7 +536,7 @@ append_fp_tile_kernel(Store st, const char *keys, const char *values, int L, int
             }
             k = u4v{u[0], u[1], u[2], u[3]};
         }
-        *reinterpret_cast<u4v *>(const_cast<char *>(k_cell_ptr(st, bh, slot_t)) + kfp_off(st, slot_t + r, d0)) = k;
+        *reinterpret_cast<u4v *>(kcell + kfp_off(st, slot_t + r, d0)) = k;
         uint32_t *vrow = &vt[r * VPW + d0 / 2];
         vrow[0] = vraw[e].x;
         vrow[1] = vraw[e].y;
