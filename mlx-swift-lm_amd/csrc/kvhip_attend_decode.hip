@@ -31,6 +31,11 @@
 
 #include "kvhip_mask.hpp"
 
+// piece buffers of the full-precision decode kernel (at most the D / 32 pieces of one tile)
+#ifndef KVHIP_DECODE_FP_NBUF
+#define KVHIP_DECODE_FP_NBUF(D, RG) 2
+#endif
+
 namespace kvhip {
 
 namespace {
@@ -815,18 +820,26 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         }
     };
 
-    uint32_t bufA[PW], bufB[PW];
-    // piece order per tile: K0 .. K(NP-1), V0 .. V(NP-1); piece n lives in buffer n & 1
-    // (NP = 1: K in A, V in B;  NP >= 2: even pieces in A, odd in B)
-    auto buf_of = [&](int n) -> uint32_t * { return (n & 1) ? bufB : bufA; };
+    // piece order per tile: K0 .. K(NP-1), V0 .. V(NP-1); piece n lives in buffer n % NBUF and piece
+    // n + NBUF is requested as soon as piece n has been consumed.  Two buffers: four (32 KB per
+    // wavefront in flight) measured slower on the short launches they were meant for (a 4096-row
+    // sliding window at D = 256, one tile per wavefront: 17.4 us against 15.7 us).
+    constexpr int NBUF = KVHIP_DECODE_FP_NBUF(D, RG);
+    uint32_t bufs[NBUF][PW];
+    auto buf_of = [&](int n) -> uint32_t * { return bufs[n % NBUF]; };
+    // request piece n (counted from the start of a tile; past its end: of the next tile) into `buf`
+    auto request = [&](uint32_t *buf, int n) __attribute__((always_inline)) {
+        n %= 2 * NP;
+        if (n < NP) load_k(buf, n);
+        else load_v(buf, n - NP);
+    };
 
     if (my_tiles > 0) {
         // (the queries first: loads complete in order, and a wait for queries requested after the
         // first pieces would be a wait for those pieces too -- in every iteration, the compiler
         // placing one wait for all ways into the loop)
         load_queries();
-        load_k(buf_of(0), 0);
-        if (NP > 1) load_k(buf_of(1), 1); else load_v(buf_of(1), 0);
+        static_for<NBUF>([&](auto N) { request(buf_of(decltype(N)::value), decltype(N)::value); });
         for (int done = 0; done < my_tiles; ++done) {
             int row;
             if (IDENT) row = slot_cur;
@@ -849,11 +862,8 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                     for (int rg = 0; rg < RG; ++rg)
                         sacc[rg] = BF ? mfma444_bf<s>(qa[rg][x], o, sacc[rg]) : mfma444<s>(qa[rg][x], o, sacc[rg]);
                 });
-                // the buffer is free: request the piece two ahead in the order K.., V..
-                constexpr int n2 = x + 2;
-                if constexpr (n2 < NP) load_k(buf, n2);
-                else if constexpr (n2 < 2 * NP) load_v(buf, n2 - NP);
-                else load_k(buf, n2 - 2 * NP);  // NP == 1: the next tile's K
+                // the buffer is free: request the piece NBUF ahead in the order K.., V.., next tile's K..
+                request(buf, x + NBUF);
             });
             // ---- online softmax ----------------------------------------------------------
             Op pa[RG], pl[RG];
@@ -932,11 +942,7 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                         }
                     }
                 });
-                // request the piece two ahead: the rest of V, then the next tile's K
-                constexpr int n2 = NP + x + 2;
-                if constexpr (n2 < 2 * NP) load_v(buf, n2 - NP);
-                else if constexpr (n2 < 3 * NP) load_k(buf, n2 - 2 * NP);
-                else load_v(buf, n2 - 3 * NP);  // NP == 1: the next tile's V
+                request(buf, NP + x + NBUF);
             });
             slot_cur += PAGE;
         }
@@ -1002,7 +1008,7 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 // row and write the output row
 template <int D, int DT>
 __global__ void __launch_bounds__((D + 63) / 64 * 64)
-combine_kernel(AttendArgs a, int nsplit, int rr) {
+combine_kernel(AttendArgs a, int nsplit, int rr, int ragged) {
     constexpr int NT = (D + 63) / 64 * 64;
     __shared__ float w_s[512];  // weight of each span for this row (nsplit <= 512)
     __shared__ float red_s[4];
@@ -1011,7 +1017,13 @@ combine_kernel(AttendArgs a, int nsplit, int rr) {
     const int r = a.Hq / a.Hkv;
     const int rep = i / a.L, l = i - rep * a.L;
     const size_t sstride = (size_t)rr * (D + 2);
-    const float *part = a.workspace + (size_t)bh * nsplit * sstride + (size_t)i * (D + 2);
+    size_t first_slot = (size_t)bh * nsplit;
+    if (ragged) {  // span slots shared over the batch in proportion to length: this row's are [first, first + count)
+        const RaggedSpan rs = ragged_span(a.mask, a.B, a.L, a.T, (a.slots + TILE - 1) / TILE, nsplit, -1, b, WAVES);
+        first_slot = (size_t)hk * nsplit + rs.first;
+        nsplit = rs.count;
+    }
+    const float *part = a.workspace + first_slot * sstride + (size_t)i * (D + 2);
     const int t = threadIdx.x;
     const int d = t < D ? t : 0;  // threads past the last column read column 0 and write nothing
     // every span's (max, sum) in one parallel round of loads, reduced through LDS
@@ -1095,6 +1107,14 @@ Plan plan_for(const AttendArgs &a) {
     const bool ident = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
     if (a.mask.mode == KVHIP_MASK_WINDOW && (a.mask.left_pad || a.mask.lengths) && forced_tiles <= 0 && ident) {
         p.tiles_per_wg = 0;
+        // the 16-row kernel goes further: a kv head's span slots are shared by its batch rows in
+        // proportion to their lengths (ragged_span), as many slots as workgroups are resident at once
+        static const bool prop_on = getenv("KVHIP_PROPORTIONAL_SPANS") != nullptr;
+        if (a.st.bits != 0 && p.rg >= 2 && a.B <= 64 && prop_on) {
+            p.tiles_per_wg = -1;
+            p.nsplit = std::max(512 / a.Hkv, 2 * a.B);
+            if (p.nsplit > 512) p.nsplit = 512;  // (more than 256 batch rows would be needed: not with B <= 64)
+        }
     } else if (a.st.bits != 0 && p.nsplit >= 2 && want <= 4 && p.rg == 1 && a.mask.mode != KVHIP_MASK_ARRAY &&
                forced_tiles <= 0) {
         // 128 pairs or more: workgroups of 8 wavefronts, one per CU -- the same wavefronts per CU
@@ -1156,13 +1176,13 @@ hipError_t profile_read(int *launches, double *total_ms) {
     return hipSuccess;
 }
 
-hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s) {
+hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s, int ragged) {
     const int R = (a.Hq / a.Hkv) * a.L;
     dim3 grid(R, a.st.BH);
 #define CMB(D)                                                                                       \
     do {                                                                                             \
-        if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL((combine_kernel<D, 0>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows); \
-        else hipLaunchKernelGGL((combine_kernel<D, 1>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows);       \
+        if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL((combine_kernel<D, 0>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows, ragged); \
+        else hipLaunchKernelGGL((combine_kernel<D, 1>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows, ragged);       \
     } while (0)
     if (a.st.Dk == 64) CMB(64);
     else if (a.st.Dk == 80) CMB(80);
@@ -1209,7 +1229,8 @@ static bool use_decode16(const AttendArgs &a, const Plan &p) { return a.st.bits 
 size_t attend_decode_workspace(const AttendArgs &a) {
     const Plan p = plan_for(a);
     const int rows = use_decode16(a, p) ? 16 : 4 * p.rg;
-    return (size_t)a.st.BH * p.nsplit * rows * (a.st.Dk + 2) * sizeof(float);
+    const size_t slots = p.tiles_per_wg < 0 ? (size_t)a.Hkv * p.nsplit : (size_t)a.st.BH * p.nsplit;
+    return slots * rows * (a.st.Dk + 2) * sizeof(float);
 }
 
 hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
@@ -1237,7 +1258,7 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
         }                                                                                                 \
         profile_mark(s, false);                                                                           \
         if (p.nsplit > 1)                                                                                 \
-            hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG); \
+            hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG, 0); \
     } while (0)
 #define DEC_RG(BITS, D, GS, DT) DEC(BITS, D, GS, DT, 1) /* more rows: the 16-row kernel above */
     if (use_decode16(a_in, p)) {
@@ -1245,7 +1266,7 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
         hipError_t e = launch_attend_decode16(a_in, p.tiles_total, p.tiles_per_wg, p.nsplit, s);
         profile_mark(s, false);
         if (e != hipSuccess) return e;
-        if (p.nsplit > 1) return launch_combine(a_in, p.nsplit, 16, s);
+        if (p.nsplit > 1) return launch_combine(a_in, p.nsplit, 16, s, p.tiles_per_wg < 0 ? 1 : 0);
         return hipSuccess;
     }
 #define DEC_DT(BITS, D, GS)                                \
@@ -1271,7 +1292,7 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
                            p.tiles_per_wg, p.nsplit);                                                     \
         profile_mark(s, false);                                                                           \
         if (p.nsplit > 1)                                                                                 \
-            hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG); \
+            hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG, 0); \
     } while (0)
 #define FP_MI(D, DT, RG)                                          \
     do {                                                          \

@@ -515,7 +515,11 @@ static int prefill_splits(const AttendArgs &a) {
     const int R = (a.Hq / a.Hkv) * a.L;
     const bool wide = prefill_wide(a);
     const size_t wgs = (size_t)((R + (wide ? 127 : 63)) / (wide ? 128 : 64)) * a.st.BH;
-    int n = (int)(768 / (wgs ? wgs : 1));
+    // as many workgroups as are resident at once: three per CU, two at D = 256 (LDS) -- a part more
+    // than that starts a second round that leaves half the CUs idle
+    static const int forced = getenv("KVHIP_PREFILL_TARGET") ? atoi(getenv("KVHIP_PREFILL_TARGET")) : 0;  // measurement aid
+    const int target = forced > 0 ? forced : (a.st.Dk >= 256 ? 512 : 768);
+    int n = (int)(target / (wgs ? wgs : 1));
     const int tiles = (a.slots + BN - 1) / BN;
     if (n > tiles / 8) n = tiles / 8;
     if (n > 8) n = 8;

@@ -269,7 +269,8 @@ bool attend_prefill_supported(const AttendArgs &a);
 size_t attend_prefill_workspace(const AttendArgs &a);
 // Merge `nsplit` partials per query row, laid out [bh][split][rows][D+2] in a.workspace
 // (out[D] unnormalised, running max, running sum), and write the normalised rows to a.out.
-hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s);
+// ragged: the partials lie in span slots shared over the batch (ragged_span, kvhip_mask.hpp)
+hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s, int ragged = 0);
 hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s);
 hipError_t launch_attend_decode16(const AttendArgs &a, int tiles_total, int tiles_per_wg, int nsplit, hipStream_t s);
 hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, hipStream_t s);
