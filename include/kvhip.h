@@ -120,7 +120,8 @@ kvhip_status kvhip_init(int32_t device);
 /* Blocks until all work enqueued on `stream` is done (tests; `eval(cache)` LLMModel.swift:56-58).
  * Also releases device memory of freed caches and replaced buffers whose last readers are done. */
 kvhip_status kvhip_sync(void *stream);
-/* 0 = choose the fastest kernel for the shape (default); 1 = always the generic kernel. */
+/* 0 = choose the fastest kernel for the shape (default); 1 = always the generic kernel.
+ * The setting, kvhip_last_attend_kernel and the profile record below belong to the calling thread. */
 void kvhip_set_kernel_policy(int32_t policy);
 /*
  * Measurement hooks (no counterpart in the reference, which times whole

@@ -19,8 +19,9 @@ namespace {
 
 thread_local std::string g_err;
 thread_local bool g_has_err = false;
-int g_policy = 0;
-int g_last_kernel = -1;
+// per calling thread, like the error state: caches driven from different threads do not share them
+thread_local int g_policy = 0;
+thread_local int g_last_kernel = -1;
 bool g_inited = false;
 
 kvhip_status fail(kvhip_status code, const std::string &msg) {

@@ -1132,10 +1132,11 @@ Plan plan_for(const AttendArgs &a) {
     return p;
 }
 
-int g_profile = 0;        // 0 off, n: bracket every n-th launch of the dominant kernel
-int g_profile_count = 0;  // launches seen since it was enabled
-bool g_profile_open = false;
-std::vector<hipEvent_t> g_events;  // begin/end pairs
+// (per calling thread: a thread brackets and reads its own launches)
+thread_local int g_profile = 0;        // 0 off, n: bracket every n-th launch of the dominant kernel
+thread_local int g_profile_count = 0;  // launches seen since it was enabled
+thread_local bool g_profile_open = false;
+thread_local std::vector<hipEvent_t> g_events;  // begin/end pairs
 
 }  // namespace
 

@@ -42,6 +42,13 @@ typedef __attribute__((address_space(3))) uint32_t LDS_U32;
 // cannot prove on every path which buffer the load fills.  Its waits for its own loads stay correct:
 // vector-memory operations complete in order, so an operation it does not count only makes a wait
 // stricter.
+// INVARIANT for anyone who edits this kernel: (1) every wavefront of the workgroup issues the same
+// number of these loads per step (the repeated tail chunks at D = 80 / 96 exist for that), because
+// the hand-placed `s_waitcnt vmcnt(N)` count them; (2) a step ends with vmcnt(0) and a barrier before
+// any wavefront reads the buffer the loads fill; (3) vector-memory operations of one wavefront
+// complete in order on this hardware -- the compiler's own waits for register loads rely on that
+// when an uncounted LDS load sits between them.  A new load inside the loop, or a different order of
+// `stage` / `fetch` / `dma`, has to keep all three.
 __device__ __forceinline__ void load_to_lds(const void *src, const void *lds_wave_base) {
     // (the low half of a flat address inside the LDS aperture is the LDS address itself)
     const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds_wave_base);

@@ -256,6 +256,12 @@ template <int GL> __device__ __forceinline__ void group_minmax_dpp(float &mn, fl
 // absolute (|quotient| <= 2^8), of the correctly rounded quotient, which can only change the
 // rounded integer when the quotient sits that close to a half-integer.  Those elements (about
 // one in 10^4) are redone with the exact division, so the codes are the reference's bit for bit.
+// INVARIANT for anyone who edits this: the guard band (0.5 - 0.4999 = 1e-4) must stay above the
+// largest error the fast quotient can have, which grows with the quotient: at |quotient| = 255 the
+// reciprocal's one ulp plus the product's rounding come to about 4.6e-5.  Widening the code range
+// (more than 8 bits) or replacing v_rcp_f32 by something less accurate needs a wider band; the
+// known answers at 254.5 (tests/quantizer_kats.py, scale 3/256) and the tie stress in
+// tests/test_gpu_cache.py fail if the band is too narrow.
 template <int BITS>
 __device__ __forceinline__ void codes8(const float (&w)[8], float scale, float bias, float inv, float (&q)[8]) {
     const float nb = (float)((1 << BITS) - 1);

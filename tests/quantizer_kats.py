@@ -109,6 +109,22 @@ CASES = [
         scale_bits=0xBF80, bias_bits=0x437F,
         wrong="codes 254, 253 for the last two under round-half-away",
     ),
+    dict(
+        # Exact ties at the top of the 8-bit code range with a scale that is not a power of two (the
+        # whole-tile device quantizer forms quotients with the hardware reciprocal and must redo these
+        # with the exact division: its guard band around half-integers has to hold up to 254.5).
+        #   s = 3/256: w_max = 255 s = 765/256, w_min = 0: scale = -(765/256)/255 = -3/256 exactly,
+        #   edge = w_max, q0 = -255, scale = edge / q0 = -3/256, bias = 765/256.  Codes (w_max - w) / s:
+        #   3/512 = 0.5 s -> 254.5 -> 254;  9/512 = 1.5 s -> 253.5 -> 254;  15/512 = 2.5 s -> 252.5 -> 252;
+        #   765/512 = 127.5 s -> 127.5 -> 128;  0 -> 255;  w_max -> 0.
+        #   float16(-3/256) = -1.5 * 2^-7 = 0xA200, float16(765/256) = 1.494140625 * 2 = 0x41FA.
+        name="8-bit ties at 254.5 with scale 3/256",
+        dtype="float16", bits=8,
+        head=[765 / 256, 0.0, 3 / 512, 9 / 512, 15 / 512], fill=765 / 512,
+        codes=[0, 255, 254, 254, 252], fill_code=128,
+        scale_bits=0xA200, bias_bits=0x41FA,
+        wrong="255 / 253 / 253 / 127 where a quotient a few 1e-5 off the tie is rounded as it stands",
+    ),
 ]
 
 
