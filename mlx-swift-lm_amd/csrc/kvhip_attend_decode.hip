@@ -105,9 +105,7 @@ __device__ __forceinline__ float uniform(float v) {  // v is the same in every l
     return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
 }
 __device__ __forceinline__ uint16_t f2h_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
-__device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
-    return (uint32_t)f2h_bits(lo) | ((uint32_t)f2h_bits(hi) << 16);
-}
+__device__ __forceinline__ uint32_t pack_h2(float lo, float hi) { return pk_h2(lo, hi); }
 
 // value held by lane (l ^ 1) / (l ^ 2) of the same quad
 __device__ __forceinline__ uint32_t quad_xor1(uint32_t v) {

@@ -44,9 +44,7 @@ constexpr float LOG2E = 1.4426950408889634f;
 constexpr float TWO24 = 16777216.0f;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ uint32_t pack_h2(float lo, float hi) {
-    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
-}
+__device__ __forceinline__ uint32_t pack_h2(float lo, float hi) { return pk_h2(lo, hi); }
 // scale / bias of a raw (scale, bias) pair; for fp16 the widening folds into the consuming fma
 template <int DT> __device__ __forceinline__ float sb_scale(uint32_t raw) {
     if (DT == 0) return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);

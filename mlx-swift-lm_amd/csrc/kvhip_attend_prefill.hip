@@ -41,7 +41,7 @@ constexpr float RAISE = 5.545177444479562f;  // 8 ln 2
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ uint16_t h_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
-__device__ __forceinline__ uint32_t h2_bits(float lo, float hi) { return (uint32_t)h_bits(lo) | ((uint32_t)h_bits(hi) << 16); }
+__device__ __forceinline__ uint32_t h2_bits(float lo, float hi) { return pk_h2(lo, hi); }
 
 // BITS 0: full precision (DT 0 fp16 / 1 bf16); 4 / 8: quantized (scales of dtype DT).
 // QT = 16-row query tiles per wavefront (2: 128 rows per workgroup, 1: 64 rows, chosen by

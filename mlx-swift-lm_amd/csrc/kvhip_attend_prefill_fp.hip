@@ -24,6 +24,9 @@
 #define KVHIP_PREFILL_BF16_P 1
 #endif
 
+#ifndef KV_SB
+#define KV_SB __builtin_amdgcn_sched_barrier(0)
+#endif
 namespace kvhip {
 
 namespace {
@@ -42,17 +45,21 @@ typedef __attribute__((address_space(3))) uint32_t LDS_U32;
 // cannot prove on every path which buffer the load fills.  Its waits for its own loads stay correct:
 // vector-memory operations complete in order, so an operation it does not count only makes a wait
 // stricter.
-// INVARIANT for anyone who edits this kernel: (1) every wavefront of the workgroup issues the same
-// number of these loads per step (the repeated tail chunks at D = 80 / 96 exist for that), because
-// the hand-placed `s_waitcnt vmcnt(N)` count them; (2) a step ends with vmcnt(0) and a barrier before
-// any wavefront reads the buffer the loads fill; (3) vector-memory operations of one wavefront
-// complete in order on this hardware -- the compiler's own waits for register loads rely on that
-// when an uncounted LDS load sits between them.  A new load inside the loop, or a different order of
-// `stage` / `fetch` / `dma`, has to keep all three.
-__device__ __forceinline__ void load_to_lds(const void *src, const void *lds_wave_base) {
+// INVARIANT for anyone who edits this kernel: (1) an iteration ends with vmcnt(0) and a barrier before
+// any wavefront reads the buffer the loads fill, and every wavefront of the workgroup runs the same
+// iterations with the same requests (which variant of an iteration it runs may differ); (2)
+// vector-memory operations of one wavefront complete in order on this hardware -- the compiler's own
+// waits for register loads rely on that when an uncounted LDS load sits between them.
+// (address = wave-uniform 64-bit `base` in scalar registers + the lane's unsigned 32-bit byte offset)
+__device__ __forceinline__ void load_to_lds(const char *base, uint32_t lane_off, const void *lds_wave_base) {
     // (the low half of a flat address inside the LDS aperture is the LDS address itself)
-    const uint32_t base = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds_wave_base);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(base) : "memory", "m0");
+    const uint32_t lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds_wave_base);
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    // (readfirstlane returns a signed int: without the casts the low half would be sign-extended over the high one)
+    const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
+    const uint64_t sb = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(sb), "s"(lds) : "memory", "m0");
 }
 union Op8 {
     h8 h;
@@ -65,14 +72,8 @@ constexpr float LOG2E = 1.4426950408889634f;
 constexpr float RAISE = 8.f;  // log2 units
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
-__device__ __forceinline__ uint32_t rn_h2(float lo, float hi) {  // round to nearest even
-    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
-}
-// two non-negative finite floats -> two bf16 (round to nearest even) in one dword
-__device__ __forceinline__ uint32_t rn_bf2(float lo, float hi) {
-    const uint32_t a = __float_as_uint(lo), b = __float_as_uint(hi);
-    return ((a + 0x7fffu + ((a >> 16) & 1u)) >> 16) | ((b + 0x7fffu + ((b >> 16) & 1u)) & 0xffff0000u);
-}
+__device__ __forceinline__ uint32_t rn_h2(float lo, float hi) { return pk_h2(lo, hi); }    // round to nearest even
+__device__ __forceinline__ uint32_t rn_bf2(float lo, float hi) { return pk_bf2(lo, hi); }
 // the probabilities of one lane as the PV operand: fp16, or bf16 for bf16 caches on the direct path
 template <bool BF> __device__ __forceinline__ u4 pack_p(const float (&p)[2][4]) {
     if constexpr (BF) return u4{rn_bf2(p[0][0], p[0][1]), rn_bf2(p[0][2], p[0][3]), rn_bf2(p[1][0], p[1][1]), rn_bf2(p[1][2], p[1][3])};
@@ -85,20 +86,45 @@ __device__ __forceinline__ uint32_t bf2_to_h2(uint32_t w) {
 
 __device__ __forceinline__ int st_BH(const AttendArgs &a) { return a.st.BH; }
 
-template <int DT> __device__ __forceinline__ f4 mfma_qk(const Op8 &a, const Op8 &b, f4 c) {
-    if constexpr (DT == 0) return __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, c, 0, 0, 0);
-    else return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, c, 0, 0, 0);
+// c += a . b and c = a . b on the matrix cores.  DT: 0 fp16 operands, 1 bf16 operands.
+template <int DT> __device__ __forceinline__ void mfma_acc(f4 &c, const Op8 &a, const Op8 &b) {
+    if constexpr (DT == 0) c = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, c, 0, 0, 0);
+    else c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, c, 0, 0, 0);
+}
+template <int DT> __device__ __forceinline__ void mfma_new(f4 &c, const Op8 &a, const Op8 &b) {
+    c = f4{0.f, 0.f, 0.f, 0.f};
+    mfma_acc<DT>(c, a, b);
+}
+// The same accumulation for the output accumulators, which live across the whole loop, written as
+// assembly with the accumulator as both input and output.  As a builtin the compiler gave most of
+// these instructions a new destination register, so that the accumulators wandered through the
+// register file and were copied back (36 64-bit moves per query block) at the loop's back edge.
+// What the compiler no longer does for these is insert the wait states between a matrix-core write
+// and a vector-ALU read of the same registers: the only such reads are the rescaling in `raise` and
+// the final normalisation, both of which sit behind a barrier (and cross-lane exchanges) that follow
+// the last of these instructions.  Waits for the LDS data that feed the operands are still inserted
+// by the compiler, which tracks registers, not opcodes.
+template <int DT> __device__ __forceinline__ void mfma_acc_inplace(f4 &c, const Op8 &a, const Op8 &b) {
+    if constexpr (DT == 0) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a.v), "v"(b.v));
+    else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a.v), "v"(b.v));
 }
 
 // D = 256 runs 64 query rows per workgroup only: 128 rows need the accumulator registers of
 // a whole SIMD lane (one wavefront per SIMD), which measured slower (0.34 ms against 0.29 ms
 // for a 512 x 4607 chunk at B4, 8 query heads).
+//
+// The loop is software-pipelined over the key tiles: iteration t issues S^T(t+1) = K(t+1) Q^T on
+// the matrix cores and, between those instructions, the vector-ALU half of the softmax of tile t
+// (scale, exp2, rounding to 16 bits), whose scores iteration t-1 left in registers; then
+// out^T += V(t)^T P(t)^T; then the mask, the tile maximum and the (rare) raise of the reference
+// maximum for tile t+1.  One wavefront so keeps the matrix cores and the vector ALU busy at the
+// same time, which the in-order issue of a tile-at-a-time loop (scores -> softmax -> PV, each
+// waiting for the one before) cannot.  K is requested two tiles ahead and V one tile ahead, each
+// into the buffer of its tile's parity; one barrier per iteration.
 template <int D, int DT, bool IDENT, int QT, int MM>
 __global__ void __launch_bounds__(256, 2)
 prefill_fp_kernel(AttendArgs a, int nsplit) {
     constexpr int BM = 64 * QT;
-    constexpr int VS = BN + 4;    // halves per V^T row in LDS: 18 dwords, so the 16 rows an operand
-                                  // read touches fall in distinct banks
     constexpr int S = (D + 31) / 32;  // contraction steps over the head dim (the last one partly zero at D = 80)
     constexpr int NDT = D / 16;   // 16-row tiles of out^T
     constexpr int NC = (D + 63) / 64;  // rounds of 256 16-byte chunks, for K and for V
@@ -108,38 +134,25 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     // row -- the unused tail that the repeated loads fill with finite values -- against query
     // operands that are zero there.
     static_assert(4 * S * BN <= ((D + 63) / 64) * 256, "the padded contraction stays inside the staged buffer");
-    // K tiles move from global memory straight into LDS (no registers, no LDS store instructions):
-    // two buffers, each the tile's 16-byte chunks in page order, [8-element chunk][token], the other
-    // one filled while this one is contracted.  fp16 caches move V the same way, [8-token
-    // chunk][column]; bf16 V is staged through registers (converted to fp16 on the way) into two
-    // padded buffers of V^T.
-    // bf16 caches keep V as bf16 too: the probabilities are then rounded to bf16 for the PV matrix-core
-    // instruction (the reference's softmax output is an array of the cache's dtype as well), so that V
-    // needs no conversion and takes the direct path.  KVHIP_PREFILL_BF16_P = 0 brings back fp16
-    // probabilities with V converted to fp16 while it is staged through registers.
-    constexpr bool VDMA = DT == 0 || KVHIP_PREFILL_BF16_P;
-    constexpr int NB = 2;
-    // (one array per buffer, K then V, selected by constants after inlining: the compiler follows
-    // loads into LDS per variable, and a read of one buffer then need not wait for the loads in
-    // flight into the other)
+    // K and V tiles move from global memory straight into LDS (no registers, no LDS store
+    // instructions): per parity of the tile one buffer for K, the tile's 16-byte chunks in page order
+    // [8-element chunk][token], and one for V, [8-token chunk][column].  bf16 caches keep K and V as
+    // bf16: the probabilities are rounded to bf16 for the PV matrix-core instruction (the reference's
+    // softmax output is an array of the cache's dtype as well).
     // 16-bit elements reserved for a tile's K (and for its V): whole rounds of 256 chunks.  With a head
     // size that is not a multiple of 64 (80, 96) the last round is partly empty: its wavefronts past the
     // tile's last chunk repeat that chunk into the unused tail, so that every wavefront issues the same
-    // number of loads and the hand-placed waits below count alike in all of them.
+    // number of loads.
     constexpr int KSZ = NC * 256 * 8;
-    __shared__ __attribute__((aligned(16))) uint16_t KV0[VDMA ? 2 * KSZ : KSZ], KV1[VDMA ? 2 * KSZ : KSZ];
-    __shared__ __attribute__((aligned(16))) _Float16 Vpad[2][VDMA ? 8 : D * VS];
-    auto Ks = [&](int buf) __attribute__((always_inline)) -> uint16_t * { return buf == 0 ? KV0 : KV1; };
-    auto Vs = [&](int buf) __attribute__((always_inline)) -> _Float16 * {
-        if constexpr (VDMA) return reinterpret_cast<_Float16 *>(buf == 0 ? KV0 : KV1) + KSZ;
-        else return Vpad[buf];
-    };
-    __shared__ int rows_s[NB][BN];
-    __shared__ int full_s[NB];
+    __shared__ __attribute__((aligned(16))) uint16_t KV0[2 * KSZ], KV1[2 * KSZ];
+    auto Ks = [&](int par) __attribute__((always_inline)) -> uint16_t * { return par == 0 ? KV0 : KV1; };
+    auto Vs = [&](int par) __attribute__((always_inline)) -> uint16_t * { return (par == 0 ? KV0 : KV1) + KSZ; };
+    __shared__ int rows_s[2][BN];
+    __shared__ int full_s[2];
 
     const Store &st = a.st;
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, jj = lane >> 4;
     // Workgroups go to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  All
     // query blocks of one (batch, kv-head) pair re-read that pair's K and V, so they are given
@@ -168,15 +181,18 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
     const int row0 = blk_x * BM + wave * 16 * QT;  // first query row of this wavefront
     const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
-    // Fast softmax (fp16 caches up to D = 128; D = 256 has no registers to spare, and bf16 keeps its
-    // float32 denominators): scores enter as exp2(s * sl2 - m) with sl2 >= 0 -- a negative scale
+    // Scores enter the softmax as exp2(s * ef - m) with ef = |scale| log2 e > 0 -- a negative scale
     // flips the sign of the query operands instead (exact), a zero one becomes a vanishing positive
-    // factor -- so that the maximum can be taken on the raw scores and the scale folded into one
-    // multiply-add; the denominators ride on the matrix cores (lacc = ones . P^T sums the same
-    // rounded probabilities the numerator uses; all 16 rows of the block hold the same sums).
+    // factor -- so that the maximum can be taken on the raw scores and the scale folds into one
+    // multiply-add.  Under an array mask the mask step leaves s * ef (+ the additive term) in the
+    // score registers and the factor is 1.
+    // fp16 caches up to D = 128: the denominators ride on the matrix cores (lacc = ones . P^T sums the
+    // same rounded probabilities the numerator uses; all 16 rows of the block hold the same sums).
+    // D = 256 has no registers to spare, and bf16 keeps float32 denominators.
     constexpr bool LM = D <= 128 && DT == 0 && KVHIP_PREFILL_LM;
-    const bool flip = LM && a.scale < 0.f;
-    const float sl2 = LM ? fmaxf(fabsf(a.scale) * LOG2E, 1e-30f) : a.scale * LOG2E;
+    const bool flip = a.scale < 0.f;
+    const float sl2 = fmaxf(fabsf(a.scale) * LOG2E, 1e-30f);
+    const float ef = MM == 2 ? 1.f : sl2;
 
     // ---- query operands: B of S^T = K . Q^T; lane (n, jj) holds q[row][32 s + 8 jj ..] raw ----
     Op8 qop[QT][S];
@@ -251,129 +267,78 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         tile_hi = min(tile_hi, tile_lo + span);
     }
 
-    // ---- staging ------------------------------------------------------------------------
-    // chunk c = e * 256 + tid.  K: slot c % 32 of the tile, 8-element chunk c / 32.  V: column
-    // c % D, 8-token chunk c / D of the 32 tokens of this tile.
-    // V through registers: a tile's V is requested one iteration before it is written to LDS and two
-    // before it is contracted.
-    constexpr int LEAD = 2;
-    struct Stg {
-        u4 v[NC];
-    };
-    Stg setA;
-    // tiles of 32 slots: the page-table entry is fetched once per eight tiles
-    PageCursor page_fetch(st, min(tile_lo * BN, max(a.slots - 1, 0))), page_dma = page_fetch;
-    [[maybe_unused]] auto fetch = [&](int tile, Stg &g) __attribute__((always_inline)) {
-        const int slot0 = tile * BN;
-        const char *vbase = page_fetch.at(st, slot0).v + (size_t)bh * st.v_cell + vfp_off(st, slot0, 0);
-#pragma unroll
-        for (int e = 0; e < NC; ++e) {
-            const int c = min(e * 256 + tid, CH - 1);
-            g.v[e] = *reinterpret_cast<const u4 *>(vbase + (size_t)(c / D) * (D * 16) + (c % D) * 16);
-        }
-    };
-    [[maybe_unused]] auto stage = [&](int buf, const Stg &g) __attribute__((always_inline)) {
-#pragma unroll
-        for (int e = 0; e < NC; ++e) {
-            const int c = e * 256 + tid;
-            if (c >= CH) continue;
-            u4 v = g.v[e];
-            if (DT == 1) v = u4{bf2_to_h2(v.x), bf2_to_h2(v.y), bf2_to_h2(v.z), bf2_to_h2(v.w)};
-            u2 *vd = reinterpret_cast<u2 *>(&Vs(buf)[(c % D) * VS + (c / D) * 8]);  // rows are 8-byte aligned
-            vd[0] = u2{v.x, v.y};
-            vd[1] = u2{v.z, v.w};
-        }
-    };
-
+    // ---- requests -------------------------------------------------------------------------
     // direct global -> LDS: lane i of a wavefront's load lands at the wavefront's LDS base + 16 i, so
-    // chunk c = e * 256 + tid goes to slot c of the buffer.  With V loaded the same way, K slot
-    // (chunk cc, position pos) takes token 8 ((pos & 15) / 4) + 4 (pos / 16) + pos % 4, the order in
-    // which the S^T accumulators of one lane cover the eight tokens of one V chunk (so K operand
-    // reads are contiguous across lanes and P never moves), and V slots are the page's own order;
-    // with V^T staged through registers K slots are the tokens in order.
-    auto dma = [&](int tile, int buf) __attribute__((always_inline)) {
+    // chunk c = e * 256 + tid goes to slot c of the buffer.  K slot (chunk cc, position pos) takes
+    // token 8 ((pos & 15) / 4) + 4 (pos / 16) + pos % 4, the order in which the S^T accumulators of one
+    // lane cover the eight tokens of one V chunk (so K operand reads are contiguous across lanes and P
+    // never moves), and V slots are the page's own order.
+    // A tile of 32 slots inside its page cell (16-bit elements): the 64-token tile t64 starts at
+    // t64 * 64 * D * 2 bytes in both planes; its K chunk (cc, token) lies at (cc * 64 + token) * 16, its
+    // V chunk (8-token chunk tc, column) at (tc * D + column) * 16.
+    const size_t cell_k = (size_t)bh * st.k_cell, cell_v = (size_t)bh * st.v_cell;
+    PageCursor page_k(st, min(tile_lo * BN, max(a.slots - 1, 0))), page_v = page_k;
+    // the lane's byte offsets inside a tile, one per round of 256 chunks
+    uint32_t koff[NC], voff[NC];
+#pragma unroll
+    for (int e = 0; e < NC; ++e) {
+        const int c = min(e * 256 + tid, CH - 1);
+        const int pos = c % BN;
+        const int tok = 8 * ((pos & 15) >> 2) + 4 * (pos >> 4) + (pos & 3);
+        koff[e] = (uint32_t)((c / BN) * (TILE * 16) + tok * 16);
+        voff[e] = (uint32_t)(c * 16);
+    }
+    auto dma_k = [&](int tile, int par) __attribute__((always_inline)) {
         const int slot0 = tile * BN;
         if (tid < BN) {
             const int pos = tid;
-            const int slot = slot0 + (VDMA ? 8 * ((pos & 15) >> 2) + 4 * (pos >> 4) + (pos & 3) : pos);
+            const int slot = slot0 + 8 * ((pos & 15) >> 2) + 4 * (pos >> 4) + (pos & 3);
             int row;
             if (IDENT) row = slot;
             else row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
             row = (row >= 0 && row < a.T) ? row : -1;
-            rows_s[buf][tid] = row;  // the row of the token in K slot `tid`
+            rows_s[par][tid] = row;  // the row of the token in K slot `tid`
             const bool full = __all(row >= keep_lo && row <= keep_hi);  // the first 32 lanes of wavefront 0
-            if (tid == 0) full_s[buf] = full;
+            if (tid == 0) full_s[par] = full;
         }
-        const PageEntry &pe = page_dma.at(st, slot0);
-        const char *kbase = pe.k + (size_t)bh * st.k_cell + kfp_off(st, slot0, 0);
-        const char *vbase = pe.v + (size_t)bh * st.v_cell + vfp_off(st, slot0, 0);
+        const int t = slot0 & (PAGE - 1);
+        const char *kbase = page_k.at(st, slot0).k + cell_k + (size_t)(t >> 6) * (TILE * D * 2) + (t & 63) * 16;
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
-            const int c = min(e * 256 + tid, CH - 1);
-            const int pos = c % BN;
-            const int tok = VDMA ? 8 * ((pos & 15) >> 2) + 4 * (pos >> 4) + (pos & 3) : pos;
-            const int cw = e * 256 + (tid & ~63);  // the wavefront's first slot
-            load_to_lds(kbase + (size_t)(c / BN) * (TILE * 16) + tok * 16, &Ks(buf)[cw * 8]);
-            if constexpr (VDMA) load_to_lds(vbase + (size_t)c * 16, &Vs(buf)[cw * 8]);
+            // whole rounds differ by a constant, which goes to the scalar base; a partly empty last
+            // round (its tail repeats the tile's last chunk) keeps its own lane offsets
+            if (D % 64 == 0) load_to_lds(kbase + e * 8 * (TILE * 16), koff[0], &Ks(par)[(e * 256 + 64 * wave) * 8]);
+            else load_to_lds(kbase, koff[e], &Ks(par)[(e * 256 + 64 * wave) * 8]);
         }
     };
-    // all but the `newer` most recent vector-memory operations of this wavefront have completed
-    auto wait_older = [&](auto N) __attribute__((always_inline)) {
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(decltype(N)::value) : "memory");
+    auto dma_v = [&](int tile, int par) __attribute__((always_inline)) {
+        const int slot0 = tile * BN;
+        const int t = slot0 & (PAGE - 1);
+        const char *vbase = page_v.at(st, slot0).v + cell_v + (size_t)(t >> 6) * (TILE * D * 2) + ((t & 63) >> 3) * (D * 16);
+#pragma unroll
+        for (int e = 0; e < NC; ++e) {
+            if (D % 64 == 0) load_to_lds(vbase + e * 256 * 16, voff[0], &Vs(par)[(e * 256 + 64 * wave) * 8]);
+            else load_to_lds(vbase, voff[e], &Vs(par)[(e * 256 + 64 * wave) * 8]);
+        }
+    };
+    auto wait_all_loads = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+
+    // ---- S^T = K . Q^T of one tile: acc[qt][mt] rows = tokens 16 mt + 4 jj + i, column = query n -----
+    // operand reads: K slot (chunk 4 s + jj, position 16 mt + n)
+    auto read_k = [&](int par, int s, Op8 (&ka)[2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+            ka[mt].v = *reinterpret_cast<const u4 *>(&Ks(par)[((4 * s + jj) * BN + 16 * mt + n) * 8]);
     };
 
-    // (fast softmax) raise query block qt's reference maximum to what the tile holds and rescale
-    auto raise = [&](int qt, float tmax) __attribute__((always_inline)) {
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-        const float mn = fmaxf(m_run[qt], tmax);
-        const float alpha = (mn == -INFINITY) ? 1.f : exp2_fast(m_run[qt] - mn);
-        m_run[qt] = mn;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) lacc[LM ? qt : 0][i] *= alpha;
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) oacc[qt][dt][i] *= alpha;
-    };
-    // one tile: `cur` is the LDS buffer that holds it, `g` the register set that holds the next one
-    auto step = [&](int tile, int cur, Stg &g) __attribute__((always_inline)) {
-        // The other buffers were last read in the previous step, which ended with a barrier.
-        // V^T first (the tile fetched in the previous step; its registers are then free for the tile
-        // after it), the K request last: the compiler's waits for those registers -- it does not
-        // count the K request -- must not meet it.
-        if constexpr (!VDMA) {
-            if (tile + 1 < tile_hi) stage(cur ^ 1, g);
-            if (tile + LEAD < tile_hi) fetch(tile + LEAD, g);
-        }
-        if (tile + 1 < tile_hi) dma(tile + 1, cur ^ 1);
-
-        // ---- S^T = K . Q^T: acc[qt][mt] rows = tokens 16 mt + 4 jj + i, column = query n -----
-        f4 sacc[QT][2];
-#pragma unroll
-        for (int qt = 0; qt < QT; ++qt)
-#pragma unroll
-            for (int mt = 0; mt < 2; ++mt) sacc[qt][mt] = f4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt) {
-            Op8 ka[S];
-#pragma unroll
-            for (int s = 0; s < S; ++s)
-                ka[s].v = *reinterpret_cast<const u4 *>(&Ks(cur)[((4 * s + jj) * BN + 16 * mt + n) * 8]);
-#pragma unroll
-            for (int s = 0; s < S; ++s)
-#pragma unroll
-                for (int qt = 0; qt < QT; ++qt) sacc[qt][mt] = mfma_qk<DT>(ka[s], qop[qt][s], sacc[qt][mt]);
-        }
-        const bool tile_full = full_s[cur] != 0;
+    // ---- mask of a tile whose scores are in `sc` (raw): excluded keys become -inf; under an array
+    // mask the scores are scaled here and additive terms added -----------------------------------
+    auto apply_mask = [&](int par, f4 (&sc)[QT][2]) __attribute__((always_inline)) {
         int trow[2][4];
-        if (MM == 2 || !tile_full) {
 #pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
+        for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) trow[mt][i] = rows_s[cur][16 * mt + 4 * jj + i];  // by K slot
-        }
-
+            for (int i = 0; i < 4; ++i) trow[mt][i] = rows_s[par][16 * mt + 4 * jj + i];  // by K slot
         // a boolean array mask is read four keys at a time where this lane's four rows are consecutive
         [[maybe_unused]] bool vec_ok[2] = {false, false};
         if constexpr (MM == 2) {
@@ -382,15 +347,6 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                 vec_ok[mt] = a.mask.dtype == KVHIP_BOOL && trow[mt][0] >= 0 && trow[mt][3] == trow[mt][0] + 3 &&
                              trow[mt][1] == trow[mt][0] + 1 && trow[mt][2] == trow[mt][0] + 2;
         }
-
-        // ---- online softmax per query column; P^T stays in place as the PV B operand ------
-        // Scores stay in the log2 domain: x = s * (scale * log2 e), p = exp2(x - m).  m is a reference
-        // value rather than the exact running maximum: it is the same in the four lanes that share a
-        // query and is raised (to the maximum seen) only when a score exceeds it by more than RAISE,
-        // so p stays below 2^RAISE (exact in fp16, whose relative precision does not depend on
-        // magnitude) and the accumulators are rescaled a handful of times per query, not on every
-        // tile that happens to hold a new maximum.
-        Op8 pb[QT];
 #pragma unroll
         for (int qt = 0; qt < QT; ++qt) {
             [[maybe_unused]] uint32_t mword[2] = {0u, 0u};
@@ -403,163 +359,250 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                         mword[mt] = w[0];
                     }
             }
-            if constexpr (LM) {
-                if (MM != 2 && tile_full) {
-                    // every key of the tile counts for every query
-                    float tmax = fmaxf(fmaxf(fmaxf(sacc[qt][0][0], sacc[qt][0][1]), fmaxf(sacc[qt][0][2], sacc[qt][0][3])),
-                                       fmaxf(fmaxf(sacc[qt][1][0], sacc[qt][1][1]), fmaxf(sacc[qt][1][2], sacc[qt][1][3])));
-                    tmax *= sl2;
-                    if (__any(tmax > m_run[qt] + RAISE)) raise(qt, tmax);
-                    const float mu = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt];
-                    float p[2][4];
-#pragma unroll
-                    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) p[mt][i] = exp2_fast(__builtin_fmaf(sacc[qt][mt][i], sl2, -mu));
-                    pb[qt].v = u4{rn_h2(p[0][0], p[0][1]), rn_h2(p[0][2], p[0][3]), rn_h2(p[1][0], p[1][1]), rn_h2(p[1][2], p[1][3])};
-                } else {
-                    float x[2][4];
-                    float tmax = -INFINITY;
-#pragma unroll
-                    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            float x_ = sacc[qt][mt][i] * sl2;
-                            const int row = trow[mt][i];
-                            if (row >= 0 && q_ok[qt]) {
-                                if constexpr (MM == 1) {
-                                    if (!sym_mask_keep(sym, q_l[qt], row)) x_ = -INFINITY;
-                                } else if constexpr (MM == 2) {
-                                    if (vec_ok[mt]) {
-                                        if (((mword[mt] >> (8 * i)) & 0xffu) == 0u) x_ = -INFINITY;
-                                    } else {
-                                        float add;
-                                        const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
-                                        x_ = keep ? x_ + add * LOG2E : -INFINITY;
-                                    }
-                                }
-                            } else {
-                                x_ = -INFINITY;
-                            }
-                            x[mt][i] = x_;
-                            tmax = fmaxf(tmax, x_);
-                        }
-                    if (__any(tmax > m_run[qt] + RAISE)) raise(qt, tmax);
-                    const float mu = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt];
-                    float p[2][4];
-#pragma unroll
-                    for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) p[mt][i] = exp2_fast(x[mt][i] - mu);  // exp2(-inf) = 0 for excluded keys
-                    pb[qt].v = u4{rn_h2(p[0][0], p[0][1]), rn_h2(p[0][2], p[0][3]), rn_h2(p[1][0], p[1][1]), rn_h2(p[1][2], p[1][3])};
-                }
-                lacc[LM ? qt : 0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones.h, pb[qt].h, lacc[LM ? qt : 0], 0, 0, 0);
-                continue;
-            }
-            float x[2][4];
-            float tmax = -INFINITY;
 #pragma unroll
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float x_ = sacc[qt][mt][i] * sl2;
-                    if (MM == 2 || !tile_full) {  // workgroup-uniform
-                        const int row = trow[mt][i];
-                        if (row >= 0 && q_ok[qt]) {
-                            if constexpr (MM == 1) {
-                                if (!sym_mask_keep(sym, q_l[qt], row)) x_ = -INFINITY;
-                            } else if constexpr (MM == 2) {
-                                if (vec_ok[mt]) {
-                                    if (((mword[mt] >> (8 * i)) & 0xffu) == 0u) x_ = -INFINITY;
-                                } else {
-                                    float add;
-                                    const bool keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
-                                    x_ = keep ? x_ + add * LOG2E : -INFINITY;
-                                }
+                    float x_ = sc[qt][mt][i];
+                    if constexpr (MM == 2) x_ *= sl2;
+                    const int row = trow[mt][i];
+                    bool keep = row >= 0 && q_ok[qt];
+                    if constexpr (MM == 1) {
+                        keep = keep && sym_mask_keep(sym, q_l[qt], row);
+                    } else if constexpr (MM == 2) {
+                        if (keep) {
+                            if (vec_ok[mt]) {
+                                keep = ((mword[mt] >> (8 * i)) & 0xffu) != 0u;
+                            } else {
+                                float add;
+                                keep = mask_keep(a.mask, b, q_h[qt], q_l[qt], row, a.L, a.T, add);
+                                x_ += add * LOG2E;
                             }
-                        } else {
-                            x_ = -INFINITY;
                         }
                     }
-                    x[mt][i] = x_;
-                    tmax = fmaxf(tmax, x_);
+                    sc[qt][mt][i] = keep ? x_ : -INFINITY;
                 }
-            if (__any(tmax > m_run[qt] + RAISE)) {  // a handful of times per query
-                tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
-                tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-                const float mn = fmaxf(m_run[qt], tmax);
-                const float alpha = (mn == -INFINITY) ? 1.f : exp2_fast(m_run[qt] - mn);
-                m_run[qt] = mn;
-                l_run[qt] *= alpha;
+        }
+    };
+
+    // ---- tile maximum and the reference maximum ---------------------------------------------
+    // Scores stay in the log2 domain: x = s * ef, p = exp2(x - m).  m is a reference value rather than
+    // the exact running maximum: it is the same in the four lanes that share a query and is raised (to
+    // the maximum seen) only when a score exceeds it by more than RAISE, so p stays below 2^RAISE
+    // (exact in fp16, whose relative precision does not depend on magnitude) and the accumulators are
+    // rescaled a handful of times per query, not on every tile that happens to hold a new maximum.
+    auto raise = [&](int qt, float tmax) __attribute__((always_inline)) {
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+        const float mn = fmaxf(m_run[qt], tmax);
+        const float alpha = (mn == -INFINITY) ? 1.f : exp2_fast(m_run[qt] - mn);
+        m_run[qt] = mn;
+        if constexpr (LM) {
 #pragma unroll
-                for (int dt = 0; dt < NDT; ++dt)
+            for (int i = 0; i < 4; ++i) lacc[LM ? qt : 0][i] *= alpha;
+        } else {
+            l_run[qt] *= alpha;
+        }
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) oacc[qt][dt][i] *= alpha;
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) oacc[qt][dt][i] *= alpha;
+    };
+    auto tile_max = [&](const f4 (&sc)[QT][2], int qt) __attribute__((always_inline)) -> float {
+        return ef * fmaxf(fmaxf(fmaxf(sc[qt][0][0], sc[qt][0][1]), fmaxf(sc[qt][0][2], sc[qt][0][3])),
+                          fmaxf(fmaxf(sc[qt][1][0], sc[qt][1][1]), fmaxf(sc[qt][1][2], sc[qt][1][3])));
+    };
+    // whether the tile whose scores are in `sc` exceeds some query's reference maximum by more than
+    // RAISE (wavefront-uniform; a handful of times per query)
+    auto needs_raise = [&](const f4 (&sc)[QT][2]) __attribute__((always_inline)) -> bool {
+        bool need = false;
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) need = need || tile_max(sc, qt) > m_run[qt] + RAISE;
+        return __any(need);
+    };
+    auto do_raise = [&](const f4 (&sc)[QT][2]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+            const float tmax = tile_max(sc, qt);
+            if (__any(tmax > m_run[qt] + RAISE)) raise(qt, tmax);
+        }
+    };
+
+    // ---- one iteration: tile `tile` (parity PAR) has its scores in `sc`; `sn` receives tile + 1's ---
+    // (MASKED: tile + 1 needs its mask evaluated -- a variant of the whole iteration rather than a
+    // branch inside it, so that the scores have one definition per variant and the paths join
+    // without register copies)
+    // The iteration itself never touches the reference maxima or rescales the accumulators: it only
+    // reports (`need`) that tile + 1 calls for it, and the loop below leaves its fast part to do so.
+    // With the rescaling inside the fast loop the compiler joined the rescaled and the untouched
+    // accumulators through register copies on the path that does not rescale: 36 moves per query block
+    // and tile, and spills.
+    auto body = [&](auto HAS_NEXT_, auto PAR_, auto MASKED_, int tile, f4 (&sc)[QT][2], f4 (&sn)[QT][2], bool &need) __attribute__((always_inline)) {
+        constexpr bool HAS_NEXT = decltype(HAS_NEXT_)::value;
+        constexpr int PAR = decltype(PAR_)::value;
+        constexpr bool MASKED = decltype(MASKED_)::value;
+        // the buffers requested into were last read in the previous iteration, which ended with a barrier
+        if (tile + 2 < tile_hi) dma_k(tile + 2, PAR);
+        if constexpr (HAS_NEXT) dma_v(tile + 1, PAR ^ 1);
+
+        float negmu[QT], pr[QT][2][4];
+        Op8 pb[QT];
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) negmu[qt] = (m_run[qt] == -INFINITY) ? 0.f : -m_run[qt];
+        // probability `idx` of this lane: query block idx / 8, accumulator idx % 8
+        auto softmax_slice = [&](int idx) __attribute__((always_inline)) {
+            const int qt = idx >> 3, mt = (idx >> 2) & 1, i = idx & 3;
+            const float p = exp2_fast(__builtin_fmaf(sc[qt][mt][i], ef, negmu[qt]));  // exp2(-inf) = 0 for excluded keys
+            pr[qt][mt][i] = p;
+            if constexpr (!LM) l_run[qt] += p;
+            if (i & 1) {
+                const uint32_t w = DT == 1 ? rn_bf2(pr[qt][mt][i - 1], p) : rn_h2(pr[qt][mt][i - 1], p);
+                pb[qt].v[2 * mt + (i >> 1)] = w;
             }
-            const float mu = (m_run[qt] == -INFINITY) ? 0.f : m_run[qt];
-            float psum = 0.f;
-            float p[2][4];
+        };
+        constexpr int NP = 8 * QT;      // probabilities per lane and tile
+        // the first V operands are asked for before the matrix cores start on the next tile's scores
+        constexpr int VG = 2;           // V operands (16 columns each) per group
+        constexpr int NG = (NDT + VG - 1) / VG;
+        Op8 va[2][VG];
+        auto read_v = [&](int g, Op8 (&dst)[VG]) __attribute__((always_inline)) {
 #pragma unroll
-            for (int mt = 0; mt < 2; ++mt)
+            for (int x = 0; x < VG; ++x)
+                if (VG * g + x < NDT)  // tokens 8 jj .. 8 jj + 7 of column 16 (VG g + x) + n: one chunk
+                    dst[x].v = *reinterpret_cast<const u4 *>(&Vs(PAR)[(jj * D + 16 * (VG * g + x) + n) * 8]);
+        };
+        if constexpr (HAS_NEXT) {
+            constexpr int NM = 2 * S * QT;  // matrix-core instructions of the next tile's scores
+            // K operands are asked for AHEAD contraction steps ahead, V's first group near the end
+            constexpr int AHEAD = QT == 1 ? 2 : 1;
+            constexpr int KA = S < AHEAD + 1 ? S : AHEAD + 1;
+            Op8 ka[KA][2];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    p[mt][i] = exp2_fast(x[mt][i] - mu);  // exp2(-inf) = 0 for excluded keys
-                    psum += p[mt][i];
-                }
-            l_run[qt] += psum;
-            pb[qt].v = pack_p<DT == 1 && VDMA>(p);
-        
+            for (int s = 0; s < (S < AHEAD ? S : AHEAD); ++s) read_k(PAR ^ 1, s, ka[s % KA]);
+            KV_SB;
+#pragma unroll
+            for (int k = 0; k < NM; ++k) {
+                // 2 QT independent accumulator chains, taken in turn
+                const int s = k / (2 * QT), mt = (k / QT) & 1, qt = k % QT;
+                if (k % (2 * QT) == 0 && s + AHEAD < S) read_k(PAR ^ 1, s + AHEAD, ka[(s + AHEAD) % KA]);
+                if (k == (NM > 2 * QT ? NM - 2 * QT : 0)) read_v(0, va[0]);
+                if (s == 0) mfma_new<DT>(sn[qt][mt], ka[s % KA][mt], qop[qt][s]);
+                else mfma_acc<DT>(sn[qt][mt], ka[s % KA][mt], qop[qt][s]);
+#pragma unroll
+                for (int idx = k * NP / NM; idx < (k + 1) * NP / NM; ++idx) softmax_slice(idx);
+                KV_SB;
+            }
+        } else {
+            read_v(0, va[0]);
+#pragma unroll
+            for (int idx = 0; idx < NP; ++idx) softmax_slice(idx);
         }
 
-        // ---- out^T += V^T . P^T: A = V^T rows (tokens 4jj..4jj+3 and 16+4jj..) from LDS -------
+        // ---- out^T += V^T . P^T: A = V^T chunks from LDS, B = the probabilities where they are ----
+        if constexpr (LM) {
 #pragma unroll
-        for (int d0 = 0; d0 < NDT; d0 += 4) {
-            Op8 va[4];
-#pragma unroll
-            for (int x = 0; x < 4; ++x) {
-                if constexpr (VDMA) {  // tokens 8 jj .. 8 jj + 7 of column 16 (d0 + x) + n: one chunk
-                    va[x].v = *reinterpret_cast<const u4 *>(&Vs(cur)[(jj * D + 16 * (d0 + x) + n) * 8]);
-                } else {
-                    const _Float16 *vrow = &Vs(cur)[(16 * (d0 + x) + n) * VS];
-                    const u2 lo = *reinterpret_cast<const u2 *>(vrow + 4 * jj);
-                    const u2 hi = *reinterpret_cast<const u2 *>(vrow + 16 + 4 * jj);
-                    va[x].v = u4{lo.x, lo.y, hi.x, hi.y};
-                }
-            }
-#pragma unroll
-            for (int x = 0; x < 4; ++x)
-#pragma unroll
-                for (int qt = 0; qt < QT; ++qt)
-                    oacc[qt][d0 + x] = mfma_qk<(DT == 1 && VDMA) ? 1 : 0>(va[x], pb[qt], oacc[qt][d0 + x]);
+            for (int qt = 0; qt < QT; ++qt)
+                mfma_acc<0>(lacc[LM ? qt : 0], ones, pb[qt]);
         }
-        // What was requested at the top of this step has to land before the barrier: it has had the
-        // whole step for it, so the wait is short, and an LDS read of the next step never meets a load
-        // in flight into its own buffer.  (Leaving the newest LDS request in flight across the
-        // barrier, with a third buffer, measured the same.)
-        // A plain barrier instead of __syncthreads(): nothing but LDS traffic (drained here) has to
-        // be ordered across it.
-        wait_older(std::integral_constant<int, 0>{});
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            if (g + 1 < NG) read_v(g + 1, va[(g + 1) & 1]);
+#pragma unroll
+            for (int x = 0; x < VG; ++x)
+                if (VG * g + x < NDT) {
+#pragma unroll
+                    for (int qt = 0; qt < QT; ++qt)
+                        mfma_acc<DT>(oacc[qt][VG * g + x], va[g & 1][x], pb[qt]);
+                }
+        }
+
+        need = false;
+        if constexpr (HAS_NEXT) {
+            if constexpr (MASKED) apply_mask(PAR ^ 1, sn);
+            need = needs_raise(sn);
+        }
+        // What was requested at the top has to land before the barrier: it has had the whole
+        // iteration for it, so the wait is short, and no LDS read of the next iteration meets a load
+        // in flight into its buffer.  A plain barrier instead of __syncthreads(): nothing but LDS
+        // traffic (drained here) has to be ordered across it.
+        wait_all_loads();
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     };
+
     if (tile_lo < tile_hi) {
-        dma(tile_lo, 0);
-        if constexpr (!VDMA) {
-            fetch(tile_lo, setA);
-            stage(0, setA);
-            if (tile_lo + 1 < tile_hi) fetch(tile_lo + 1, setA);
-        }
+        dma_k(tile_lo, 0);
+        dma_v(tile_lo, 0);
+        if (tile_lo + 1 < tile_hi) dma_k(tile_lo + 1, 1);
     }
-    wait_older(std::integral_constant<int, 0>{});
+    wait_all_loads();
     // (the same wait once more in a form the compiler's bookkeeping sees: it then knows that the
     // query operands have arrived, and does not wait for them -- and with them for every load just
     // issued -- inside the loop)
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), others untouched
     __syncthreads();
-    // (unrolled by the two buffers, so that every LDS address is a constant plus the lane's)
-    for (int tile = tile_lo; tile < tile_hi; tile += 2) {
-        step(tile, 0, setA);
-        if (tile + 1 >= tile_hi) break;
-        step(tile + 1, 1, setA);
+    if (tile_lo < tile_hi) {
+        f4 sa[QT][2], sb[QT][2];
+        {  // scores of the first tile
+#pragma unroll
+            for (int s = 0; s < S; ++s) {
+                Op8 ka[2];
+                read_k(0, s, ka);
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                    for (int qt = 0; qt < QT; ++qt) {
+                        if (s == 0) mfma_new<DT>(sa[qt][mt], ka[mt], qop[qt][s]);
+                        else mfma_acc<DT>(sa[qt][mt], ka[mt], qop[qt][s]);
+                    }
+            }
+            if (MM == 2 || full_s[0] == 0) apply_mask(0, sa);
+            do_raise(sa);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // K buffer 0 is free again
+        using T_ = std::true_type;
+        using F_ = std::false_type;
+        using P0 = std::integral_constant<int, 0>;
+        using P1 = std::integral_constant<int, 1>;
+        int tile = tile_lo;
+        // whether the tile after `tile` (parity par) needs its mask evaluated: workgroup-uniform
+        auto next_masked = [&](int par) __attribute__((always_inline)) -> bool {
+            return MM == 2 || __builtin_amdgcn_readfirstlane(full_s[par]) == 0;
+        };
+        // one iteration with the variant chosen at run time; false after the last tile
+        auto iterate = [&](auto PAR_, f4 (&sc)[QT][2], f4 (&sn)[QT][2], bool &need) __attribute__((always_inline)) -> bool {
+            constexpr int PAR = decltype(PAR_)::value;
+            if (tile + 1 < tile_hi) {
+                if (next_masked(PAR ^ 1)) body(T_{}, PAR_, T_{}, tile, sc, sn, need);
+                else if constexpr (MM != 2) body(T_{}, PAR_, F_{}, tile, sc, sn, need);
+                ++tile;
+                return true;
+            }
+            body(F_{}, PAR_, F_{}, tile, sc, sn, need);
+            return false;
+        };
+        for (;;) {
+            // the fast loop: two iterations (one per buffer parity) per round, left when a tile's scores
+            // call for a higher reference maximum -- after an even number of iterations (`odd` false:
+            // the next tile's scores are in sa) or an odd one (in sb)
+            bool more = true, need = false, odd = false;
+            for (;;) {
+                more = iterate(P0{}, sa, sb, need);
+                odd = true;
+                if (!more || need) break;
+                more = iterate(P1{}, sb, sa, need);
+                odd = false;
+                if (!more || need) break;
+            }
+            if (!more) break;
+            if (odd) {  // back to an even count through one iteration outside the fast loop
+                do_raise(sb);
+                more = iterate(P1{}, sb, sa, need);
+                if (!more) break;
+                if (need) do_raise(sa);
+            } else {
+                do_raise(sa);
+            }
+        }
     }
 
     // ---- normalise and store: lane (n, jj) holds out[q = n][d = 16 dt + 4 jj + i] ------------
@@ -595,8 +638,8 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                 w.x = rn_h2(o0, o1);
                 w.y = rn_h2(o2, o3);
             } else {
-                w.x = (uint32_t)Elem<1>::bits(o0) | ((uint32_t)Elem<1>::bits(o1) << 16);
-                w.y = (uint32_t)Elem<1>::bits(o2) | ((uint32_t)Elem<1>::bits(o3) << 16);
+                w.x = rn_bf2(o0, o1);
+                w.y = rn_bf2(o2, o3);
             }
             *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(a.out) + ooff + 16 * dt + 4 * jj) = w;
         }

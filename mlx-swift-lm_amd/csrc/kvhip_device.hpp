@@ -55,6 +55,18 @@ __device__ __forceinline__ float finfo_min_dt(int dt) {
     return dt == 0 ? -65504.0f : (dt == 1 ? -3.3895313892515355e38f : -3.4028234663852886e38f);
 }
 
+// Two floats -> two 16-bit floats in one dword (low half first), rounded to nearest even by the
+// packed converts of gfx950 (v_cvt_pk_f16_f32 / v_cvt_pk_bf16_f32): one instruction per pair.
+typedef float kv_f2 __attribute__((ext_vector_type(2)));
+typedef _Float16 kv_h2 __attribute__((ext_vector_type(2)));
+typedef __bf16 kv_b2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_h2(float lo, float hi) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((kv_f2{lo, hi}), kv_h2));
+}
+__device__ __forceinline__ uint32_t pk_bf2(float lo, float hi) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((kv_f2{lo, hi}), kv_b2));
+}
+
 // Affine parameters of one group from its extrema, in float32, step for step as
 // MLX's CPU quantizer computes them (call sites KVCache.swift:1069-1070).
 __device__ __forceinline__ void affine_params(float w_min, float w_max, float n_bins, float &scale,
