@@ -290,16 +290,16 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     }
     auto dma_k = [&](int tile, int par) __attribute__((always_inline)) {
         const int slot0 = tile * BN;
-        if (tid < BN) {
-            const int pos = tid;
+        if (wave == (tile & 3) && lane < BN) {  // the wavefronts take this in turn
+            const int pos = lane;
             const int slot = slot0 + 8 * ((pos & 15) >> 2) + 4 * (pos >> 4) + (pos & 3);
             int row;
             if (IDENT) row = slot;
             else row = slot < a.slots ? slot_to_row(a.runs, slot) : -1;
             row = (row >= 0 && row < a.T) ? row : -1;
-            rows_s[par][tid] = row;  // the row of the token in K slot `tid`
-            const bool full = __all(row >= keep_lo && row <= keep_hi);  // the first 32 lanes of wavefront 0
-            if (tid == 0) full_s[par] = full;
+            rows_s[par][pos] = row;  // the row of the token in K slot `pos`
+            const bool full = __all(row >= keep_lo && row <= keep_hi);  // (the 32 active lanes)
+            if (lane == 0) full_s[par] = full;
         }
         const int t = slot0 & (PAGE - 1);
         const char *kbase = page_k.at(st, slot0).k + cell_k + (size_t)(t >> 6) * (TILE * D * 2) + (t & 63) * 16;
@@ -333,12 +333,52 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
 
     // ---- mask of a tile whose scores are in `sc` (raw): excluded keys become -inf; under an array
     // mask the scores are scaled here and additive terms added -----------------------------------
+    // An index-only mask (causal, window, per-batch lengths and left padding) keeps, for one query, an
+    // interval of key rows: [q_lo, q_lo + q_span] per query block of this lane (empty for a query row
+    // past the end), tested with one unsigned comparison per key.
+    [[maybe_unused]] int q_lo[QT];
+    [[maybe_unused]] uint32_t q_span[QT];
+    if constexpr (MM == 1) {
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) {
+            int lo, hi;
+            if (sym.mode == KVHIP_MASK_CAUSAL) {
+                lo = 0;
+                hi = a.T - a.L + q_l[qt];
+            } else {
+                const int li = sym.offset + q_l[qt];
+                lo = sym.pad_b;
+                hi = min(li, sym.len_b - 1);
+                if (sym.window > 0) lo = max(lo, li - sym.window + 1);
+            }
+            lo = max(lo, 0);
+            hi = min(hi, a.T - 1);
+            const bool any = q_ok[qt] && hi >= lo;
+            q_lo[qt] = any ? lo : 0;
+            q_span[qt] = any ? (uint32_t)(hi - lo) : 0u;
+            if (!any) q_lo[qt] = 0x40000000;  // no row reaches it: row - q_lo wraps to a huge unsigned value
+        }
+    }
     auto apply_mask = [&](int par, f4 (&sc)[QT][2]) __attribute__((always_inline)) {
         int trow[2][4];
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) trow[mt][i] = rows_s[par][16 * mt + 4 * jj + i];  // by K slot
+            for (int i = 0; i < 4; ++i) trow[mt][i] = rows_s[par][16 * mt + 4 * jj + i];  // by K slot; -1: no row
+        if constexpr (MM != 2) {
+#pragma unroll
+            for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        bool keep;
+                        if constexpr (MM == 1) keep = (uint32_t)(trow[mt][i] - q_lo[qt]) <= q_span[qt];
+                        else keep = trow[mt][i] >= 0 && q_ok[qt];
+                        sc[qt][mt][i] = keep ? sc[qt][mt][i] : -INFINITY;
+                    }
+            return;
+        }
         // a boolean array mask is read four keys at a time where this lane's four rows are consecutive
         [[maybe_unused]] bool vec_ok[2] = {false, false};
         if constexpr (MM == 2) {
@@ -363,13 +403,10 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float x_ = sc[qt][mt][i];
-                    if constexpr (MM == 2) x_ *= sl2;
+                    float x_ = sc[qt][mt][i] * sl2;
                     const int row = trow[mt][i];
                     bool keep = row >= 0 && q_ok[qt];
-                    if constexpr (MM == 1) {
-                        keep = keep && sym_mask_keep(sym, q_l[qt], row);
-                    } else if constexpr (MM == 2) {
+                    if constexpr (MM == 2) {
                         if (keep) {
                             if (vec_ok[mt]) {
                                 keep = ((mword[mt] >> (8 * i)) & 0xffu) != 0u;
