@@ -23,6 +23,26 @@
 #ifndef KVHIP_PREFILL_BF16_P
 #define KVHIP_PREFILL_BF16_P 1
 #endif
+// how far ahead of their use the matrix-core operands are read from LDS (registers permitting):
+// per query-block count (1: 16 query rows per wavefront, 2: 32)
+#ifndef KVHIP_PF_VG1
+#define KVHIP_PF_VG1 2
+#endif
+#ifndef KVHIP_PF_VG2
+#define KVHIP_PF_VG2 2
+#endif
+#ifndef KVHIP_PF_NVB1
+#define KVHIP_PF_NVB1 2
+#endif
+#ifndef KVHIP_PF_NVB2
+#define KVHIP_PF_NVB2 2
+#endif
+#ifndef KVHIP_PF_AHEAD1
+#define KVHIP_PF_AHEAD1 2
+#endif
+#ifndef KVHIP_PF_AHEAD2
+#define KVHIP_PF_AHEAD2 1
+#endif
 
 #ifndef KV_SB
 #define KV_SB __builtin_amdgcn_sched_barrier(0)
@@ -487,21 +507,26 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
 #pragma unroll
         for (int qt = 0; qt < QT; ++qt) negmu[qt] = (m_run[qt] == -INFINITY) ? 0.f : -m_run[qt];
         // probability `idx` of this lane: query block idx / 8, accumulator idx % 8
-        auto softmax_slice = [&](int idx) __attribute__((always_inline)) {
+        // (the rounding of a pair of probabilities to 16 bits trails their exp2 by two probabilities, so
+        // that it does not wait for a result just asked for)
+        auto round_pair = [&](int idx) __attribute__((always_inline)) {  // idx: the odd member of the pair
             const int qt = idx >> 3, mt = (idx >> 2) & 1, i = idx & 3;
-            const float p = exp2_fast(__builtin_fmaf(sc[qt][mt][i], ef, negmu[qt]));  // exp2(-inf) = 0 for excluded keys
-            pr[qt][mt][i] = p;
-            if constexpr (!LM) l_run[qt] += p;
-            if (i & 1) {
-                const uint32_t w = DT == 1 ? rn_bf2(pr[qt][mt][i - 1], p) : rn_h2(pr[qt][mt][i - 1], p);
-                pb[qt].v[2 * mt + (i >> 1)] = w;
-            }
+            const float p0 = pr[qt][mt][i - 1], p1 = pr[qt][mt][i];
+            if constexpr (!LM) l_run[qt] += p0 + p1;
+            pb[qt].v[2 * mt + (i >> 1)] = DT == 1 ? rn_bf2(p0, p1) : rn_h2(p0, p1);
         };
         constexpr int NP = 8 * QT;      // probabilities per lane and tile
-        // the first V operands are asked for before the matrix cores start on the next tile's scores
-        constexpr int VG = 2;           // V operands (16 columns each) per group
+        auto softmax_slice = [&](int idx) __attribute__((always_inline)) {
+            const int qt = idx >> 3, mt = (idx >> 2) & 1, i = idx & 3;
+            pr[qt][mt][i] = exp2_fast(__builtin_fmaf(sc[qt][mt][i], ef, negmu[qt]));  // exp2(-inf) = 0 for excluded keys
+            if ((idx & 1) && idx >= 3) round_pair(idx - 2);
+            if (idx == NP - 1) round_pair(idx);
+        };
+        // V operands (16 columns each) are read in groups of VG, NVB - 1 groups ahead of their use
+        constexpr int VG = QT == 1 ? KVHIP_PF_VG1 : KVHIP_PF_VG2;
+        constexpr int NVB = QT == 1 ? KVHIP_PF_NVB1 : KVHIP_PF_NVB2;
         constexpr int NG = (NDT + VG - 1) / VG;
-        Op8 va[2][VG];
+        Op8 va[NVB][VG];
         auto read_v = [&](int g, Op8 (&dst)[VG]) __attribute__((always_inline)) {
 #pragma unroll
             for (int x = 0; x < VG; ++x)
@@ -511,7 +536,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         if constexpr (HAS_NEXT) {
             constexpr int NM = 2 * S * QT;  // matrix-core instructions of the next tile's scores
             // K operands are asked for AHEAD contraction steps ahead, V's first group near the end
-            constexpr int AHEAD = QT == 1 ? 2 : 1;
+            constexpr int AHEAD = QT == 1 ? KVHIP_PF_AHEAD1 : KVHIP_PF_AHEAD2;
             constexpr int KA = S < AHEAD + 1 ? S : AHEAD + 1;
             Op8 ka[KA][2];
 #pragma unroll
@@ -522,7 +547,10 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                 // 2 QT independent accumulator chains, taken in turn
                 const int s = k / (2 * QT), mt = (k / QT) & 1, qt = k % QT;
                 if (k % (2 * QT) == 0 && s + AHEAD < S) read_k(PAR ^ 1, s + AHEAD, ka[(s + AHEAD) % KA]);
-                if (k == (NM > 2 * QT ? NM - 2 * QT : 0)) read_v(0, va[0]);
+                if (k == (NM > 2 * QT ? NM - 2 * QT : 0)) {
+#pragma unroll
+                    for (int g = 0; g < NVB - 1 && g < NG; ++g) read_v(g, va[g]);
+                }
                 if (s == 0) mfma_new<DT>(sn[qt][mt], ka[s % KA][mt], qop[qt][s]);
                 else mfma_acc<DT>(sn[qt][mt], ka[s % KA][mt], qop[qt][s]);
 #pragma unroll
@@ -530,7 +558,8 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
                 KV_SB;
             }
         } else {
-            read_v(0, va[0]);
+#pragma unroll
+            for (int g = 0; g < NVB - 1 && g < NG; ++g) read_v(g, va[g]);
 #pragma unroll
             for (int idx = 0; idx < NP; ++idx) softmax_slice(idx);
         }
@@ -543,13 +572,13 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         }
 #pragma unroll
         for (int g = 0; g < NG; ++g) {
-            if (g + 1 < NG) read_v(g + 1, va[(g + 1) & 1]);
+            if (g + NVB - 1 < NG) read_v(g + NVB - 1, va[(g + NVB - 1) % NVB]);
 #pragma unroll
             for (int x = 0; x < VG; ++x)
                 if (VG * g + x < NDT) {
 #pragma unroll
                     for (int qt = 0; qt < QT; ++qt)
-                        mfma_acc<DT>(oacc[qt][VG * g + x], va[g & 1][x], pb[qt]);
+                        mfma_acc<DT>(oacc[qt][VG * g + x], va[g % NVB][x], pb[qt]);
                 }
         }
 
@@ -562,8 +591,12 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         // iteration for it, so the wait is short, and no LDS read of the next iteration meets a load
         // in flight into its buffer.  A plain barrier instead of __syncthreads(): nothing but LDS
         // traffic (drained here) has to be ordered across it.
+#ifndef KVHIP_PROBE_NOWAIT  // (timing probe: results are wrong without the wait)
         wait_all_loads();
+#endif
+#ifndef KVHIP_PROBE_NOBARRIER
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#endif
     };
 
     if (tile_lo < tile_hi) {
@@ -601,15 +634,20 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         using P0 = std::integral_constant<int, 0>;
         using P1 = std::integral_constant<int, 1>;
         int tile = tile_lo;
-        // whether the tile after `tile` (parity par) needs its mask evaluated: workgroup-uniform
-        auto next_masked = [&](int par) __attribute__((always_inline)) -> bool {
-            return MM == 2 || __builtin_amdgcn_readfirstlane(full_s[par]) == 0;
-        };
         // one iteration with the variant chosen at run time; false after the last tile
         auto iterate = [&](auto PAR_, f4 (&sc)[QT][2], f4 (&sn)[QT][2], bool &need) __attribute__((always_inline)) -> bool {
             constexpr int PAR = decltype(PAR_)::value;
-            if (tile + 1 < tile_hi) {
-                if (next_masked(PAR ^ 1)) body(T_{}, PAR_, T_{}, tile, sc, sn, need);
+            const bool has_next = tile + 1 < tile_hi;
+            // whether tile + 1 needs its mask evaluated (workgroup-uniform): with slots in presented
+            // order a comparison of its ends with the rows every query keeps, else the flag its
+            // request left in LDS -- asked for before the requests below are formed, which hide its latency
+            bool masked = true;
+            if constexpr (MM != 2) {
+                if constexpr (IDENT) masked = !((tile + 1) * BN >= keep_lo && (tile + 1) * BN + (BN - 1) <= keep_hi);
+                else masked = full_s[PAR ^ 1] == 0;
+            }
+            if (has_next) {
+                if (__builtin_amdgcn_readfirstlane(masked)) body(T_{}, PAR_, T_{}, tile, sc, sn, need);
                 else if constexpr (MM != 2) body(T_{}, PAR_, F_{}, tile, sc, sn, need);
                 ++tile;
                 return true;
@@ -642,6 +680,9 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         }
     }
 
+#if defined(KVHIP_PROBE_NOWAIT)
+    wait_all_loads();
+#endif
     // ---- normalise and store: lane (n, jj) holds out[q = n][d = 16 dt + 4 jj + i] ------------
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
