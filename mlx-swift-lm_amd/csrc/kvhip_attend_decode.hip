@@ -137,22 +137,23 @@ __device__ __forceinline__ void quad_transpose(uint32_t x[4], int lane) {
 }
 
 // load N consecutive dwords with the widest vector accesses
-template <int N> __device__ __forceinline__ void load_words(uint32_t *dst, const char *p) {
+// (from device memory: a `gptr`, so that the loads are GLOBAL rather than FLAT ones)
+template <int N> __device__ __forceinline__ void load_words(uint32_t *dst, gptr p) {
     if constexpr (N % 4 == 0) {
 #pragma unroll
         for (int i = 0; i < N / 4; ++i) {
-            const uint4 v = reinterpret_cast<const uint4 *>(p)[i];
+            const kv_u4 v = ld_global<kv_u4>(p, i);
             dst[4 * i] = v.x; dst[4 * i + 1] = v.y; dst[4 * i + 2] = v.z; dst[4 * i + 3] = v.w;
         }
     } else if constexpr (N % 2 == 0) {
 #pragma unroll
         for (int i = 0; i < N / 2; ++i) {
-            const uint2 v = reinterpret_cast<const uint2 *>(p)[i];
+            const kv_u2 v = ld_global<kv_u2>(p, i);
             dst[2 * i] = v.x; dst[2 * i + 1] = v.y;
         }
     } else {
 #pragma unroll
-        for (int i = 0; i < N; ++i) dst[i] = reinterpret_cast<const uint32_t *>(p)[i];
+        for (int i = 0; i < N; ++i) dst[i] = ld_global<uint32_t>(p, i);
     }
 }
 
@@ -351,10 +352,10 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     const size_t v_off = (size_t)bh * st.v_cell + (size_t)tip * D * VROW;
     const size_t ksb_off = (size_t)bh * st.ksb_cell + (size_t)tip * TILE * st.ksb_row;
     const size_t vsb_off = (size_t)bh * st.vsb_cell + (size_t)tip * TILE * st.vsb_row;
-    const char *kp = st.pt[page_k].k + k_off;
-    const char *vp = st.pt[page_k].v + v_off;
-    const char *ksp = st.pt[page_k].ksb + ksb_off;
-    const char *vsp = st.pt[page_k].vsb + vsb_off;
+    gptr kp = as_global(st.pt[page_k].k) + k_off;
+    gptr vp = as_global(st.pt[page_k].v) + v_off;
+    gptr ksp = as_global(st.pt[page_k].ksb) + ksb_off;
+    gptr vsp = as_global(st.pt[page_k].vsb) + vsb_off;
     const uint32_t k_lane = lane * st.k_row, v_lane = lane * VROW;
     const uint32_t ksb_lane = lane * st.ksb_row, vsb_lane = lane * st.vsb_row;
     int slot_next = tile0 * TILE + lane;  // slot of this lane's token in the tile loaded next
@@ -418,8 +419,8 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         ++k_loaded;
         if (k_loaded < my_tiles) {  // wave-uniform: step to the same tile of the next page
             page_k += PSTEP;
-            kp = st.pt[page_k].k + k_off;
-            ksp = st.pt[page_k].ksb + ksb_off;
+            kp = as_global(st.pt[page_k].k) + k_off;
+            ksp = as_global(st.pt[page_k].ksb) + ksb_off;
             slot_next += PAGE * PSTEP;
             base_next += PAGE * PSTEP;
         }
@@ -442,8 +443,8 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         ++v_loaded;
         if (v_loaded < my_tiles) {
             page_v += PSTEP;
-            vp = st.pt[page_v].v + v_off;
-            vsp = st.pt[page_v].vsb + vsb_off;
+            vp = as_global(st.pt[page_v].v) + v_off;
+            vsp = as_global(st.pt[page_v].vsb) + vsb_off;
         }
     };
     auto load_tile = [&](T &t) {
@@ -785,6 +786,9 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     constexpr int VROW = TILE * 2;  // bytes of one V tile row
     const size_t k_off = (size_t)bh * st.k_cell + (size_t)tip * TILE * st.k_row;
     const size_t v_off = (size_t)bh * st.v_cell + (size_t)tip * D * VROW;
+    // (plain pointers, hence FLAT loads, on purpose: as GLOBAL loads with a scalar base the short launches
+    // of this kernel measured 0.4-1 us slower -- 19.1 against 18.7 us on a 4096-row ring at D = 256,
+    // 10.4-11.2 against 9.1-10.1 us at 1024 rows of D = 128 -- and the long ones the same)
     const char *kp = st.pt[page_k].k + k_off;
     const char *vp = st.pt[page_k].v + v_off;
     // chunk-interleaved tiles: chunk j of the lane's token (K) or column (V) sits 16 * lane bytes into
@@ -1105,6 +1109,9 @@ Plan plan_for(const AttendArgs &a) {
     const bool ident = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
     if (a.mask.mode == KVHIP_MASK_WINDOW && (a.mask.left_pad || a.mask.lengths) && forced_tiles <= 0 && ident) {
         p.tiles_per_wg = 0;
+        // KVHIP_RAGGED_SPANS (read once) forces the number of spans per batch row: a measurement aid
+        static const int forced_spans = getenv("KVHIP_RAGGED_SPANS") ? atoi(getenv("KVHIP_RAGGED_SPANS")) : 0;
+        if (forced_spans > 0) p.nsplit = std::min(forced_spans, 512);
         // the 16-row kernel goes further: a kv head's span slots are shared by its batch rows in
         // proportion to their lengths (ragged_span), as many slots as workgroups are resident at once
         static const bool prop_on = getenv("KVHIP_PROPORTIONAL_SPANS") != nullptr;

@@ -141,8 +141,9 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         tile_begin = t_lo + split * per;
         tile_end = min(t_hi, tile_begin + per);
     }
-    const int tile0 = tile_begin + wave;
-    const int my_tiles = tile0 < tile_end ? (tile_end - tile0 + WAVES - 1) / WAVES : 0;
+    // (wave-uniform by construction; saying so keeps the page walk in scalar registers and scalar loads)
+    const int tile0 = __builtin_amdgcn_readfirstlane(tile_begin + wave);
+    const int my_tiles = __builtin_amdgcn_readfirstlane(tile0 < tile_end ? (tile_end - tile0 + WAVES - 1) / WAVES : 0);
     int full_lo = 0, full_hi = a.T - 1;  // rows every query row keeps
     if constexpr (MM == 1) {
         sym_mask_full_range(sym, full_lo, full_hi);
@@ -163,10 +164,12 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     // (scale, bias) pairs of this lane group's 16 tokens, 16 jj .. 16 jj + 15
     const size_t ksb_off = (size_t)bh * st.ksb_cell + (size_t)(tip * TILE + 16 * jj) * st.ksb_row;
     const size_t vsb_off = (size_t)bh * st.vsb_cell + (size_t)(tip * TILE + 16 * jj) * st.vsb_row;
-    const char *kp = st.pt[page_k].k + k_off;
-    const char *vp = st.pt[page_k].v + v_off;
-    const char *ksp = st.pt[page_k].ksb + ksb_off;
-    const char *vsp = st.pt[page_k].vsb + vsb_off;
+    // The plane bases of the wavefront's next tile stay wave-uniform (scalar registers) until the loads
+    // that use them are formed: the entry of the following page is asked for right after a tile's loads
+    // are issued and its latency passes behind the tile's arithmetic.  (Adding the lane's offset as soon
+    // as the entry arrived put a wait for the scalar load into every tile: 44 -> 50 us on a ragged
+    // batch of 16 rows.)
+    gptr kb = as_global(st.pt[page_k].k), vb = as_global(st.pt[page_k].v), ksb_b = as_global(st.pt[page_k].ksb), vsb_b = as_global(st.pt[page_k].vsb);
     int base_next = tile0 * TILE;
 
     struct Tile {
@@ -178,20 +181,21 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 
     int k_loaded = 0, v_loaded = 0;
     auto load_k = [&](Tile &t) __attribute__((always_inline)) {
+        const gptr kp = kb + k_off, ksp = ksb_b + ksb_off;
 #pragma unroll
         for (int tb = 0; tb < 4; ++tb)
 #pragma unroll
             for (int g = 0; g < G; ++g) {
-                const char *p = kp + (size_t)(4 * tb) * st.k_row + g * (GS * BITS / 8);
+                const gptr p = kp + (size_t)(4 * tb) * st.k_row + g * (GS * BITS / 8);
                 if constexpr (KWL == 1) {
-                    t.k[tb][g][0] = *reinterpret_cast<const uint32_t *>(p);
+                    t.k[tb][g][0] = ld_global<uint32_t>(p);
                 } else if constexpr (KWL == 2) {
-                    const u2 w = *reinterpret_cast<const u2 *>(p);
+                    const u2 w = ld_global<u2>(p);
                     t.k[tb][g][0] = w.x; t.k[tb][g][1] = w.y;
                 } else {
 #pragma unroll
                     for (int e = 0; e < KWL / 4; ++e) {
-                        const u4 w = reinterpret_cast<const u4 *>(p)[e];
+                        const u4 w = ld_global<u4>(p, e);
                         t.k[tb][g][4 * e] = w.x; t.k[tb][g][4 * e + 1] = w.y;
                         t.k[tb][g][4 * e + 2] = w.z; t.k[tb][g][4 * e + 3] = w.w;
                     }
@@ -200,7 +204,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         // 16 tokens x G pairs of 4 bytes: contiguous rows of G * 4 bytes
 #pragma unroll
         for (int e = 0; e < 16 * G / 4; ++e) {
-            const u4 w = reinterpret_cast<const u4 *>(ksp)[e];
+            const u4 w = ld_global<u4>(ksp, e);
             (&t.ksb[0][0])[4 * e] = w.x; (&t.ksb[0][0])[4 * e + 1] = w.y;
             (&t.ksb[0][0])[4 * e + 2] = w.z; (&t.ksb[0][0])[4 * e + 3] = w.w;
         }
@@ -208,34 +212,35 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         ++k_loaded;
         if (k_loaded < my_tiles) {  // wave-uniform: the same tile of the next page
             ++page_k;
-            kp = st.pt[page_k].k + k_off;
-            ksp = st.pt[page_k].ksb + ksb_off;
+            kb = as_global(st.pt[page_k].k);
+            ksb_b = as_global(st.pt[page_k].ksb);
             base_next += PAGE;
         }
     };
     auto load_v = [&](Tile &t) __attribute__((always_inline)) {
+        const gptr vp = vb + v_off, vsp = vsb_b + vsb_off;
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
-            const char *p = vp + (size_t)(16 * db) * VROW;
+            const gptr p = vp + (size_t)(16 * db) * VROW;
             if constexpr (VWL == 2) {
-                const u2 w = *reinterpret_cast<const u2 *>(p);
+                const u2 w = ld_global<u2>(p);
                 t.v[db][0] = w.x; t.v[db][1] = w.y;
             } else {
-                const u4 w = *reinterpret_cast<const u4 *>(p);
+                const u4 w = ld_global<u4>(p);
                 t.v[db][0] = w.x; t.v[db][1] = w.y; t.v[db][2] = w.z; t.v[db][3] = w.w;
             }
         }
 #pragma unroll
         for (int e = 0; e < 16 * G / 4; ++e) {
-            const u4 w = reinterpret_cast<const u4 *>(vsp)[e];
+            const u4 w = ld_global<u4>(vsp, e);
             (&t.vsb[0][0])[4 * e] = w.x; (&t.vsb[0][0])[4 * e + 1] = w.y;
             (&t.vsb[0][0])[4 * e + 2] = w.z; (&t.vsb[0][0])[4 * e + 3] = w.w;
         }
         ++v_loaded;
         if (v_loaded < my_tiles) {
             ++page_v;
-            vp = st.pt[page_v].v + v_off;
-            vsp = st.pt[page_v].vsb + vsb_off;
+            vb = as_global(st.pt[page_v].v);
+            vsb_b = as_global(st.pt[page_v].vsb);
         }
     };
 

@@ -114,6 +114,18 @@ __device__ __forceinline__ size_t vfp_off(const Store &st, int slot, int d) {
 __device__ __forceinline__ const char *k_cell_ptr(const Store &st, int bh, int slot) {
     return st.pt[slot >> PAGE_SHIFT].k + (size_t)bh * st.k_cell;
 }
+// A pointer taken from the page table is a plain `char *` to the compiler, which then emits FLAT loads
+// for it: those count on both the vector-memory and the LDS/scalar counter, and since they may
+// complete through either path a wait for one of them has to be a wait for all -- a tile's loads can
+// no longer stay in flight behind the previous tile's.  `gptr` states that the memory is device
+// memory (address space 1): the loads become GLOBAL loads with counted, in-order waits.
+typedef uint32_t kv_u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t kv_u2 __attribute__((ext_vector_type(2)));
+#define KV_GLOBAL __attribute__((address_space(1)))
+typedef const KV_GLOBAL char *gptr;
+__device__ __forceinline__ gptr as_global(const void *p) { return (gptr) reinterpret_cast<const char *>(p); }
+template <class T> __device__ __forceinline__ T ld_global(gptr p) { return *reinterpret_cast<const KV_GLOBAL T *>(p); }
+template <class T> __device__ __forceinline__ T ld_global(gptr p, int i) { return reinterpret_cast<const KV_GLOBAL T *>(p)[i]; }
 // The page-table entry of the page that holds a wave-uniform `slot`, fetched again only when the
 // page changes: a kernel that walks the slots in tiles smaller than a page keeps the entry in
 // scalar registers across the tiles of one page.
