@@ -314,14 +314,15 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int tl = 4 * tb + i;
-                float s_ = 0.f;
+                // q . (s c + b) per group = s (q . c) + b sum(q); the 2^24 of the masked-code operands is
+                // taken out of the sum over the groups (one multiply-add instead of one multiply per group)
+                float sc_ = 0.f, sb_ = 0.f;
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
-                    const float s24 = sacc[tb][g][i] * TWO24;
-                    s_ = __builtin_fmaf(sb_bias<DT>(t.ksb[tl][g]), qsum[g], s_);
-                    s_ = __builtin_fmaf(sb_scale<DT>(t.ksb[tl][g]), s24, s_);
+                    sc_ = __builtin_fmaf(sb_scale<DT>(t.ksb[tl][g]), sacc[tb][g][i], sc_);
+                    sb_ = __builtin_fmaf(sb_bias<DT>(t.ksb[tl][g]), qsum[g], sb_);
                 }
-                x[tl] = round_dt<DT>(s_);
+                x[tl] = round_dt<DT>(__builtin_fmaf(sc_, TWO24, sb_));
             }
         if (MM == 2 && a.mask.dtype == KVHIP_BOOL && t.base + (TILE - 1) < a.T) {
             // a boolean array over a whole tile: this lane's 16 tokens are 16 consecutive bytes of its
@@ -376,6 +377,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         float pv[G][16];
 #pragma unroll
         for (int tl = 0; tl < 16; ++tl) {
+            // (the difference first: a masked score is finfo(T).min, whose product with log2 e overflows for bfloat16)
             const float p = fast_exp2((x[tl] - mu) * LOG2E);  // exp2(-inf) = 0 for dead slots
             l_part += p;
             // positions 2, 3, 6, 7 of a 4-bit operand meet high nibbles (x16)
