@@ -169,6 +169,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     auto Vs = [&](int par) __attribute__((always_inline)) -> uint16_t * { return (par == 0 ? KV0 : KV1) + KSZ; };
     __shared__ int rows_s[2][BN];
     __shared__ int full_s[2];
+    __shared__ int seg_lo_s[MAXRUNS], seg_hi_s[MAXRUNS], nseg_s;  // tile segments to visit (ring presentations)
 
     const Store &st = a.st;
     const int tid = threadIdx.x;
@@ -279,12 +280,96 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             tile_hi = min(tile_hi, (a.T + BN - 1) / BN);
         }
     }
-    // optional split of the key range (small grids): each part leaves an
+    // The tiles to visit, in slot order, as up to NSEG segments; position v of the visiting order is tile
+    // vt_of(v).  With slots in presented order that is the one range found above.  A ring presented
+    // through a run table keeps its rows in rotated order, so the rows no query of this block can see
+    // (older than the window, newer than the block) lie somewhere inside the slot range: thread 0 maps
+    // the visible row range through every run to slot tiles, sorts and merges them (a few dozen scalar
+    // steps, once per workgroup), and whole tiles of invisible rows are never requested -- 14 of 144
+    // tiles for a 512-row chunk over a 4096-row window.
+    constexpr int NSEG = 4;
+    int seg_start[NSEG], seg_cnt[NSEG];
+#pragma unroll
+    for (int k = 0; k < NSEG; ++k) seg_start[k] = seg_cnt[k] = 0;
+    seg_start[0] = tile_lo;
+    seg_cnt[0] = max(tile_hi - tile_lo, 0);
+    if constexpr (!IDENT && MM == 1) {
+        if (tid == 0) {
+            const int i_first = blk_x * BM, i_last = min(R, i_first + BM) - 1;
+            const bool spans = (i_first / a.L) != (i_last / a.L);
+            const int l_min = spans ? 0 : i_first % a.L, l_max = spans ? a.L - 1 : i_last % a.L;
+            int vis_lo = 0, vis_hi = a.T - a.L + l_max;  // rows some query of the block may see
+            if (sym.mode != KVHIP_MASK_CAUSAL) {
+                vis_lo = sym.pad_b;
+                vis_hi = min(sym.offset + l_max, sym.len_b - 1);
+                if (sym.window > 0) vis_lo = max(vis_lo, sym.offset + l_min - sym.window + 1);
+            }
+            vis_lo = max(vis_lo, 0);
+            vis_hi = min(vis_hi, a.T - 1);
+            int ns = 0;
+#pragma unroll
+            for (int i = 0; i < MAXRUNS; ++i) {
+                if (i < a.runs.n) {
+                    const int r_lo = max(vis_lo, a.runs.row0[i]), r_hi = min(vis_hi, a.runs.row0[i] + a.runs.len[i] - 1);
+                    if (r_lo <= r_hi) {
+                        const int t_lo = (a.runs.phys0[i] + r_lo - a.runs.row0[i]) / BN;
+                        const int t_hi = (a.runs.phys0[i] + r_hi - a.runs.row0[i]) / BN;
+                        int pos = ns;  // insertion by first tile
+                        while (pos > 0 && seg_lo_s[pos - 1] > t_lo) {
+                            seg_lo_s[pos] = seg_lo_s[pos - 1];
+                            seg_hi_s[pos] = seg_hi_s[pos - 1];
+                            --pos;
+                        }
+                        seg_lo_s[pos] = t_lo;
+                        seg_hi_s[pos] = t_hi;
+                        ++ns;
+                    }
+                }
+            }
+            int m = 0;  // merge what overlaps or touches
+            for (int i = 0; i < ns; ++i) {
+                if (m > 0 && seg_lo_s[i] <= seg_hi_s[m - 1] + 1) {
+                    seg_hi_s[m - 1] = max(seg_hi_s[m - 1], seg_hi_s[i]);
+                } else {
+                    seg_lo_s[m] = seg_lo_s[i];
+                    seg_hi_s[m] = seg_hi_s[i];
+                    ++m;
+                }
+            }
+            if (m > NSEG) {  // more pieces than are kept: one range over all of them (nothing wrong, nothing skipped)
+                seg_hi_s[0] = seg_hi_s[m - 1];
+                m = 1;
+            }
+            nseg_s = m;
+        }
+        __syncthreads();
+        const int m = __builtin_amdgcn_readfirstlane(nseg_s);
+#pragma unroll
+        for (int k = 0; k < NSEG; ++k) {
+            const int lo = k < m ? __builtin_amdgcn_readfirstlane(seg_lo_s[k]) : 0;
+            const int hi = k < m ? __builtin_amdgcn_readfirstlane(seg_hi_s[k]) : -1;
+            seg_start[k] = lo;
+            seg_cnt[k] = hi - lo + 1;
+        }
+    }
+    auto vt_of = [&](int v) __attribute__((always_inline)) -> int {
+        int t = seg_start[0] + v, rem = v - seg_cnt[0];
+#pragma unroll
+        for (int k = 1; k < NSEG; ++k) {
+            if (rem >= 0) t = seg_start[k] + rem;
+            rem -= seg_cnt[k];
+        }
+        return t;
+    };
+    int v_lo = 0, v_hi = 0;
+#pragma unroll
+    for (int k = 0; k < NSEG; ++k) v_hi += seg_cnt[k];
+    // optional split of the visiting order (small grids): each part leaves an
     // unnormalised partial per query row, merged by the decode path's combine kernel
     if (nsplit > 1) {
-        const int span = (tile_hi - tile_lo + nsplit - 1) / nsplit;
-        tile_lo = tile_lo + split * span;
-        tile_hi = min(tile_hi, tile_lo + span);
+        const int span = (v_hi + nsplit - 1) / nsplit;
+        v_lo = split * span;
+        v_hi = min(v_hi, v_lo + span);
     }
 
     // ---- requests -------------------------------------------------------------------------
@@ -297,7 +382,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     // t64 * 64 * D * 2 bytes in both planes; its K chunk (cc, token) lies at (cc * 64 + token) * 16, its
     // V chunk (8-token chunk tc, column) at (tc * D + column) * 16.
     const size_t cell_k = (size_t)bh * st.k_cell, cell_v = (size_t)bh * st.v_cell;
-    PageCursor page_k(st, min(tile_lo * BN, max(a.slots - 1, 0))), page_v = page_k;
+    PageCursor page_k(st, min(vt_of(v_lo) * BN, max(a.slots - 1, 0))), page_v = page_k;
     // the lane's byte offsets inside a tile, one per round of 256 chunks
     uint32_t koff[NC], voff[NC];
 #pragma unroll
@@ -499,8 +584,8 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         constexpr int PAR = decltype(PAR_)::value;
         constexpr bool MASKED = decltype(MASKED_)::value;
         // the buffers requested into were last read in the previous iteration, which ended with a barrier
-        if (tile + 2 < tile_hi) dma_k(tile + 2, PAR);
-        if constexpr (HAS_NEXT) dma_v(tile + 1, PAR ^ 1);
+        if (tile + 2 < v_hi) dma_k(vt_of(tile + 2), PAR);  // (`tile`: the position in the visiting order)
+        if constexpr (HAS_NEXT) dma_v(vt_of(tile + 1), PAR ^ 1);
 
         float negmu[QT], pr[QT][2][4];
         Op8 pb[QT];
@@ -599,10 +684,10 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
 #endif
     };
 
-    if (tile_lo < tile_hi) {
-        dma_k(tile_lo, 0);
-        dma_v(tile_lo, 0);
-        if (tile_lo + 1 < tile_hi) dma_k(tile_lo + 1, 1);
+    if (v_lo < v_hi) {
+        dma_k(vt_of(v_lo), 0);
+        dma_v(vt_of(v_lo), 0);
+        if (v_lo + 1 < v_hi) dma_k(vt_of(v_lo + 1), 1);
     }
     wait_all_loads();
     // (the same wait once more in a form the compiler's bookkeeping sees: it then knows that the
@@ -610,7 +695,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     // issued -- inside the loop)
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), others untouched
     __syncthreads();
-    if (tile_lo < tile_hi) {
+    if (v_lo < v_hi) {
         f4 sa[QT][2], sb[QT][2];
         {  // scores of the first tile
 #pragma unroll
@@ -633,17 +718,17 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         using F_ = std::false_type;
         using P0 = std::integral_constant<int, 0>;
         using P1 = std::integral_constant<int, 1>;
-        int tile = tile_lo;
+        int tile = v_lo;  // position in the visiting order
         // one iteration with the variant chosen at run time; false after the last tile
         auto iterate = [&](auto PAR_, f4 (&sc)[QT][2], f4 (&sn)[QT][2], bool &need) __attribute__((always_inline)) -> bool {
             constexpr int PAR = decltype(PAR_)::value;
-            const bool has_next = tile + 1 < tile_hi;
+            const bool has_next = tile + 1 < v_hi;
             // whether tile + 1 needs its mask evaluated (workgroup-uniform): with slots in presented
             // order a comparison of its ends with the rows every query keeps, else the flag its
             // request left in LDS -- asked for before the requests below are formed, which hide its latency
             bool masked = true;
             if constexpr (MM != 2) {
-                if constexpr (IDENT) masked = !((tile + 1) * BN >= keep_lo && (tile + 1) * BN + (BN - 1) <= keep_hi);
+                if constexpr (IDENT) masked = !(vt_of(tile + 1) * BN >= keep_lo && vt_of(tile + 1) * BN + (BN - 1) <= keep_hi);
                 else masked = full_s[PAR ^ 1] == 0;
             }
             if (has_next) {
