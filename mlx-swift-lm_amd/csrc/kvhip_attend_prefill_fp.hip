@@ -199,6 +199,9 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             split = t / BH;
         }
     }
+    // Under a causal or window mask the later query blocks see more keys: they are given the lower
+    // workgroup ids, which the hardware starts first, so that the launch does not end on its longest blocks.
+    if (MM == 1) blk_x = nblk - 1 - blk_x;
     const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
     const int row0 = blk_x * BM + wave * 16 * QT;  // first query row of this wavefront
     const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
