@@ -122,6 +122,15 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             part_slot = (size_t)hk * nsplit + blockIdx.x;
         }
     }
+    if constexpr (MM == 1) {
+        // a ragged batch whose rows divide their own ranges over the same number of spans: long and short
+        // rows are paired on the CUs (balanced_row)
+        if (tiles_per_wg == 0 && a.B <= 64 && a.B > 2) {
+            b = __builtin_amdgcn_readfirstlane(balanced_row(a.mask, a.B, a.L, a.T, tiles_total, b));
+            bh = b * a.Hkv + hk;
+            part_slot = (size_t)bh * nsplit + split;
+        }
+    }
     const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
     int tile_begin = split * tiles_per_wg;
     int tile_end = min(tiles_total, tile_begin + tiles_per_wg);

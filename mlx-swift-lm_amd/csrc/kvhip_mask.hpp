@@ -179,4 +179,37 @@ __device__ __forceinline__ RaggedSpan ragged_span(const MaskDev &m, int B, int L
     return r;
 }
 
+// ---- which batch row a workgroup row takes, for ragged batches ------------------------------------
+// Workgroups are started in id order, one per CU and then a second one per CU, so rows v and v + B/2 of a
+// launch of 512 workgroups share CUs.  Taking the batch rows in order of their visible length -- the first
+// half of the workgroup rows in descending order, the second half in ascending order -- pairs the longest
+// row with the shortest on the same CUs, the second longest with the second shortest, and so on, instead of
+// whatever the batch order happens to pair.  Every workgroup computes the same permutation (one lane
+// per batch row, B <= 64); partial results are still indexed by the batch row itself, so nothing
+// downstream changes.
+__device__ __forceinline__ int balanced_row(const MaskDev &m, int B, int L, int T, int tiles_total, int v) {
+    const int lane = threadIdx.x & 63;
+    int tiles = -1;
+    if (lane < B) {
+        const SymMask s = sym_mask_init(m, lane, L, T);
+        int vis_lo, vis_hi;
+        sym_mask_row_range(s, vis_lo, vis_hi);
+        int t_lo = max(0, vis_lo) >> 6, t_hi = min(tiles_total, (min(vis_hi, T - 1) >> 6) + 1);
+        if (sym_mask_some_row_empty(s)) {
+            t_lo = 0;
+            t_hi = tiles_total;
+        }
+        tiles = max(t_hi - t_lo, 0);
+    }
+    int rank = 0;  // rows that come before this lane's: more tiles, or as many and a lower index
+    for (int j = 0; j < B; ++j) {
+        const int tj = __shfl(tiles, j);
+        rank += (tj > tiles || (tj == tiles && j < lane)) ? 1 : 0;
+    }
+    const int h = (B + 1) / 2;
+    const int want = v < h ? v : B - 1 - (v - h);
+    const unsigned long long hit = __ballot(lane < B && rank == want);
+    return hit ? __ffsll(hit) - 1 : v;
+}
+
 }  // namespace kvhip
