@@ -224,8 +224,18 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform
     const int blk = lane >> 2, qi = lane & 3;  // lane group (MFMA block) and position in it
-    const int bh = blockIdx.y, split = blockIdx.x;
-    const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
+    int bh = blockIdx.y;
+    const int split = blockIdx.x;
+    int b = bh / a.Hkv;
+    const int hk = bh - b * a.Hkv;
+    if constexpr (MM == 1) {
+        // a ragged batch whose rows divide their own ranges over the same number of spans: long and short
+        // rows are paired on the CUs (balanced_row); partials stay indexed by the batch row itself
+        if (tiles_per_wg == 0 && a.B <= 64 && a.B > 2) {
+            b = __builtin_amdgcn_readfirstlane(balanced_row(a.mask, a.B, a.L, a.T, tiles_total, b));
+            bh = b * a.Hkv + hk;
+        }
+    }
     const int r = a.Hq / a.Hkv;
     const int R = r * a.L;
 
