@@ -67,7 +67,7 @@ typedef struct {
     int32_t max_size;   /* RotatingKVCache(maxSize:) */
     int32_t keep;       /* RotatingKVCache(keep:) */
     int32_t group_size; /* QuantizedKVCache(groupSize:) :931 */
-    int32_t bits;       /* QuantizedKVCache(bits:), affine mode; 2, 4 or 8 */
+    int32_t bits;       /* QuantizedKVCache(bits:), affine mode; 2, 3, 4, 5, 6 or 8 */
 } kvhip_config;
 
 /* MLXFast.ScaledDotProductAttentionMaskMode as the attention entry points take it. */
@@ -230,7 +230,7 @@ kvhip_status kvhip_cache_fetch(const kvhip_cache *cache, void *dst_keys, void *d
  * queries [B,Hq,L,Dk] and out [B,Hq,L,Dv] in the cache's dtype.
  * Every dtype, bit width, head size, group size and mask is accepted.  The tuned kernels take
  * float16 / bfloat16 caches with Dk == Dv in {64, 96, 128, 256} (also 80 when not quantized;
- * quantized: 4 or 8 bits, group size 32, 64 or 128); anything else (float32, 2-bit codes, other head sizes) runs on a plain kernel
+ * quantized: 4 or 8 bits, group size 32, 64 or 128); anything else (float32, 2-, 3-, 5- and 6-bit codes, other head sizes) runs on a plain kernel
  * that is 50-75 times slower at 8k keys.  kvhip_last_attend_kernel() tells which one ran.
  */
 kvhip_status kvhip_cache_attend(kvhip_cache *cache, const void *queries, int32_t B, int32_t Hq,

@@ -24,6 +24,9 @@ thread_local int g_policy = 0;
 thread_local int g_last_kernel = -1;
 bool g_inited = false;
 
+// code widths of MLX's affine quantization
+bool affine_bits_ok(int bits) { return bits == 2 || bits == 3 || bits == 4 || bits == 5 || bits == 6 || bits == 8; }
+
 kvhip_status fail(kvhip_status code, const std::string &msg) {
     g_err = msg;
     g_has_err = true;
@@ -209,8 +212,8 @@ kvhip_status set_geometry(kvhip_cache *c, int B, int Hkv, int Dk, int Dv, int dt
     s.dtype = dtype;
     s.es = elem_size(dtype);
     if (c->kind == KVHIP_KIND_QUANTIZED) {
-        if (c->bits != 2 && c->bits != 4 && c->bits != 8)
-            return fail(KVHIP_ERR_UNSUPPORTED, "affine KV quantization is implemented for 2, 4 and 8 bits");
+        if (!affine_bits_ok(c->bits))
+            return fail(KVHIP_ERR_UNSUPPORTED, "affine KV quantization is implemented for 2, 3, 4, 5, 6 and 8 bits");
         if (Dk % c->gs || Dv % c->gs) return fail(KVHIP_ERR_INVALID_ARG, "head dim not divisible by the group size");
         s.bits = c->bits;
         s.gs = c->gs;
@@ -1419,7 +1422,7 @@ kvhip_status kvhip_cache_to_unquantized(const kvhip_cache *c, void *stream, kvhi
 kvhip_status kvhip_affine_quantize(const void *src, int64_t rows, int32_t D, int32_t gs, int32_t bits,
                                    int32_t dtype, uint32_t *wq, void *scales, void *biases, void *stream) {
     if (!src || !wq || !scales || !biases) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
-    if (bits != 2 && bits != 4 && bits != 8) return fail(KVHIP_ERR_UNSUPPORTED, "bits must be 2, 4 or 8");
+    if (!affine_bits_ok(bits)) return fail(KVHIP_ERR_UNSUPPORTED, "bits must be 2, 3, 4, 5, 6 or 8");
     if ((gs != 32 && gs != 64 && gs != 128) || D % gs) return fail(KVHIP_ERR_INVALID_ARG, "group size must be 32, 64 or 128 and divide D");
     if (dtype < 0 || dtype > 2) return fail(KVHIP_ERR_INVALID_ARG, "bad dtype");
     KV_HIP(launch_affine_quantize(src, rows, D, gs, bits, dtype, wq, scales, biases, S(stream)));
@@ -1430,7 +1433,7 @@ kvhip_status kvhip_affine_dequantize(const uint32_t *wq, const void *scales, con
                                      int64_t rows, int32_t D, int32_t gs, int32_t bits, int32_t dtype,
                                      void *dst, void *stream) {
     if (!wq || !scales || !biases || !dst) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
-    if (bits != 2 && bits != 4 && bits != 8) return fail(KVHIP_ERR_UNSUPPORTED, "bits must be 2, 4 or 8");
+    if (!affine_bits_ok(bits)) return fail(KVHIP_ERR_UNSUPPORTED, "bits must be 2, 3, 4, 5, 6 or 8");
     if (D % gs) return fail(KVHIP_ERR_INVALID_ARG, "group size must divide D");
     if (dtype < 0 || dtype > 2) return fail(KVHIP_ERR_INVALID_ARG, "bad dtype");
     KV_HIP(launch_affine_dequantize(wq, scales, biases, rows, D, gs, bits, dtype, dst, S(stream)));

@@ -64,12 +64,17 @@ attend_generic_kernel(AttendArgs a, int slots_pad) {
                 const char *sb = ksb_row_ptr(st, bh, slot);
                 for (int g = 0; g < st.Dk / st.gs; ++g) {
                     const float sc = Elem<DT>::load(sb, 2 * g), bi = Elem<DT>::load(sb, 2 * g + 1);
-                    for (int w0 = g * st.gs / per; w0 < (g + 1) * st.gs / per; ++w0) {
-                        const uint32_t word = krow[w0];
-                        for (int i = 0; i < per; ++i) {
-                            const uint32_t c = (word >> (i * BB)) & ((1u << BB) - 1u);
-                            sum += qs[w0 * per + i] * (sc * (float)c + bi);
+                    if constexpr ((32 % BB) == 0) {
+                        for (int w0 = g * st.gs / per; w0 < (g + 1) * st.gs / per; ++w0) {
+                            const uint32_t word = krow[w0];
+                            for (int i = 0; i < per; ++i) {
+                                const uint32_t c = (word >> (i * BB)) & ((1u << BB) - 1u);
+                                sum += qs[w0 * per + i] * (sc * (float)c + bi);
+                            }
                         }
+                    } else {  // 3, 5, 6 bits: codes straddle words of the row's bit stream
+                        for (int d = g * st.gs; d < (g + 1) * st.gs; ++d)
+                            sum += qs[d] * (sc * (float)stream_code<BB>(krow, d) + bi);
                     }
                 }
                 s = round_dt<DT>(sum);
@@ -156,6 +161,9 @@ hipError_t launch_attend_generic(const AttendArgs &a, hipStream_t s) {
         case 0: GEN_DT(0); break;
         case 2: GEN_DT(2); break;
         case 4: GEN_DT(4); break;
+        case 3: GEN_DT(3); break;
+        case 5: GEN_DT(5); break;
+        case 6: GEN_DT(6); break;
         default: GEN_DT(8); break;
     }
 #undef GEN_DT

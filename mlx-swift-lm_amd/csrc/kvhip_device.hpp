@@ -138,8 +138,23 @@ __device__ __forceinline__ void quantize_row_wave_from(LOAD load, int D, int gs,
             const bool valid = d < D;
             const uint32_t code = valid ? affine_code(w[k], scale, bias, nb) : 0u;
             if (k_words) {
-                const uint32_t word = group_or(code << ((d % per) * BITS), per);
-                if (valid && (lane % per) == 0) k_words[d / per] = word;
+                if constexpr ((32 % BITS) == 0) {
+                    const uint32_t word = group_or(code << ((d % per) * BITS), per);
+                    if (valid && (lane % per) == 0) k_words[d / per] = word;
+                } else {
+                    // 3, 5 and 6 bits: the 64 codes of this pass are 2 BITS whole words of the row's bit stream;
+                    // lane w < 2 BITS collects the codes that touch word w (at most 32 / BITS + 2 of them)
+                    const int j0 = (32 * lane) / BITS;
+                    uint32_t word = 0u;
+#pragma unroll
+                    for (int i = 0; i < 32 / BITS + 2; ++i) {
+                        const int j = j0 + i;
+                        const uint32_t c = __shfl(code, j & 63);
+                        if (j < 64 && j * BITS < 32 * lane + 32) word |= stream_bits(c, j * BITS, lane);
+                    }
+                    const int wi = (base + k * 64) * BITS / 32 + lane;
+                    if (lane < 2 * BITS && wi < D * BITS / 32) k_words[wi] = word;
+                }
             }
             if (valid) code_sink(d, code);
         }

@@ -157,7 +157,21 @@ struct PageCursor {
 template <int BITS> __device__ __forceinline__ int v_bitpos(int t) {
     if (BITS == 4) return 32 * (t >> 3) + 4 * (((t & 7) >> 1) + 4 * (t & 1));
     if (BITS == 8) return 32 * (t >> 2) + 8 * (((t & 3) >> 1) + 2 * (t & 1));
-    return 2 * t;  // BITS == 2
+    return BITS * t;  // 2 bits, and the widths that do not divide 32 (3, 5, 6): a plain bit stream over the tile
+}
+// Packed codes are a little-endian bit stream: code j of a row occupies bits [j BITS, (j + 1) BITS) of the row's
+// words.  For 2, 4 and 8 bits that is "element k of a 32-bit word at bits [k BITS, (k + 1) BITS)"; for 3, 5 and 6
+// bits it is MLX's 8 / 8 / 4 codes in 3 / 5 / 3 bytes, low code first, where a code may straddle two words.
+template <int BITS> __device__ __forceinline__ uint32_t stream_code(const uint32_t *w, int j) {
+    const int bit = j * BITS, sh = bit & 31;
+    uint32_t v = w[bit >> 5] >> sh;
+    if ((32 % BITS) != 0 && sh + BITS > 32) v |= w[(bit >> 5) + 1] << (32 - sh);
+    return v & ((1u << BITS) - 1u);
+}
+// the bits that a value `c` placed at bit `pos` of a stream contributes to word `w` of it
+__device__ __forceinline__ uint32_t stream_bits(uint32_t c, int pos, int w) {
+    const int rel = pos - 32 * w;
+    return rel >= 0 ? (rel < 32 ? (c << rel) : 0u) : (c >> -rel);
 }
 // (quantized pages) byte offset, inside the page cell, of the V tile row (tile of `slot`, column d)
 __device__ __forceinline__ size_t v_row_off(const Store &st, int slot, int d) {
@@ -165,6 +179,7 @@ __device__ __forceinline__ size_t v_row_off(const Store &st, int slot, int d) {
     return ((size_t)((slot & (PAGE - 1)) >> 6) * st.Dv + d) * row_bytes;
 }
 template <int BITS> __device__ __forceinline__ uint32_t v_code_load(const char *vrow, int t) {
+    if ((32 % BITS) != 0) return stream_code<BITS>(reinterpret_cast<const uint32_t *>(vrow), t);
     const int bp = v_bitpos<BITS>(t);
     return (reinterpret_cast<const uint32_t *>(vrow)[bp >> 5] >> (bp & 31)) & ((1u << BITS) - 1u);
 }

@@ -118,14 +118,15 @@ __device__ __forceinline__ void append_quant_body(const Store &st, const Store &
     const int t_lo = lo & (TILE - 1), t_hi = t_lo + (hi - lo);
     // the words of a V tile row this append touches, and this thread's first merge item:
     // its old word is requested now, so a single-token append does not wait for it later
-    const int w_lo = t_lo / TPW, nw = (t_hi - 1) / TPW - w_lo + 1;
+    // (for 3, 5 and 6 bits a token's code may straddle two words of the row's bit stream)
+    const int w_lo = (t_lo * BITS) >> 5, nw = ((t_hi * BITS - 1) >> 5) - w_lo + 1;
     const int items = st.Dv * nw;
     char *cell = const_cast<char *>(v_cell_ptr(st, bh, lo));
     auto word_ptr = [&](int u) -> uint32_t * {
         const int d = u / nw, w = w_lo + (u - d * nw);
         return reinterpret_cast<uint32_t *>(cell + v_row_off(st, lo, d)) + w;
     };
-    const bool partial = (t_lo % TPW) != 0 || (t_hi % TPW) != 0;  // some word keeps old tokens
+    const bool partial = ((t_lo * BITS) & 31) != 0 || ((t_hi * BITS) & 31) != 0;  // some word keeps old tokens
     uint32_t old0 = 0;
     if (partial && (int)threadIdx.x < items) old0 = *word_ptr(threadIdx.x);
     // (row, K or V) pairs go round the four wavefronts, so one new token uses two of them
@@ -160,12 +161,23 @@ __device__ __forceinline__ void append_quant_body(const Store &st, const Store &
     for (int u = threadIdx.x; u < items; u += blockDim.x) {
         const int d = u / nw, w = w_lo + (u - d * nw);
         uint32_t nbits = 0, mbits = 0;
-        for (int tt = 0; tt < TPW; ++tt) {
-            const int t = w * TPW + tt;
-            if (t >= t_lo && t < t_hi) {
-                const int bp = v_bitpos<BITS>(t) & 31;
-                nbits |= (uint32_t)vcodes[t * st.Dv + d] << bp;
-                mbits |= ((1u << BITS) - 1u) << bp;
+        if constexpr ((32 % BITS) == 0) {
+            for (int tt = 0; tt < TPW; ++tt) {
+                const int t = w * TPW + tt;
+                if (t >= t_lo && t < t_hi) {
+                    const int bp = v_bitpos<BITS>(t) & 31;
+                    nbits |= (uint32_t)vcodes[t * st.Dv + d] << bp;
+                    mbits |= ((1u << BITS) - 1u) << bp;
+                }
+            }
+        } else {
+            const int t0 = (32 * w) / BITS;  // the first token with bits in word w
+            for (int tt = 0; tt < TPW + 2; ++tt) {
+                const int t = t0 + tt;
+                if (t >= t_lo && t < t_hi && t * BITS < 32 * w + 32) {
+                    nbits |= stream_bits(vcodes[t * st.Dv + d], t * BITS, w);
+                    mbits |= stream_bits((1u << BITS) - 1u, t * BITS, w);
+                }
             }
         }
         uint32_t *p = word_ptr(u);
@@ -480,10 +492,9 @@ template <int DT, int BITS>
 __global__ void __launch_bounds__(256) dequant_pages_kernel(Store q, Store dst, int rows) {
     const int bh = blockIdx.y;
     const int lo = blockIdx.x * TILE, hi = min(rows, lo + TILE);
-    constexpr int per = 32 / BITS;
     for (int idx = threadIdx.x; idx < (hi - lo) * q.Dk; idx += 256) {
         const int t = idx / q.Dk, d = idx - t * q.Dk, slot = lo + t;
-        const uint32_t c = (reinterpret_cast<const uint32_t *>(k_row_ptr(q, bh, slot))[d / per] >> ((d % per) * BITS)) & ((1u << BITS) - 1u);
+        const uint32_t c = stream_code<BITS>(reinterpret_cast<const uint32_t *>(k_row_ptr(q, bh, slot)), d);
         const char *sb = ksb_row_ptr(q, bh, slot);
         const float sc = Elem<DT>::load(sb, 2 * (d / q.gs)), bi = Elem<DT>::load(sb, 2 * (d / q.gs) + 1);
         Elem<DT>::store(const_cast<char *>(k_cell_ptr(dst, bh, slot)) + kfp_off(dst, slot, d), 0, __fadd_rn(__fmul_rn(sc, (float)c), bi));
@@ -630,14 +641,23 @@ __global__ void export_quant_kernel(Store st, int which, int nrows, char *dst) {
         for (int w = threadIdx.x; w < W; w += blockDim.x) d[w] = s[w];
     } else if (which == 3) {
         constexpr int per = 32 / BITS;
-        const int W = st.Dv / per;
+        const int W = st.Dv * BITS / 32;
         const char *cell = v_cell_ptr(st, bh, slot);
         const int t = slot & (TILE - 1);
         uint32_t *d = reinterpret_cast<uint32_t *>(dst) + ((size_t)bh * nrows + slot) * W;
         for (int w = threadIdx.x; w < W; w += blockDim.x) {
             uint32_t word = 0;
-            for (int i = 0; i < per; ++i)
-                word |= v_code_load<BITS>(cell + v_row_off(st, slot, w * per + i), t) << (i * BITS);
+            if constexpr ((32 % BITS) == 0) {
+                for (int i = 0; i < per; ++i)
+                    word |= v_code_load<BITS>(cell + v_row_off(st, slot, w * per + i), t) << (i * BITS);
+            } else {
+                const int j0 = (32 * w) / BITS;  // the first column with bits in word w of the row's bit stream
+                for (int i = 0; i < per + 2; ++i) {
+                    const int j = j0 + i;
+                    if (j < st.Dv && j * BITS < 32 * w + 32)
+                        word |= stream_bits(v_code_load<BITS>(cell + v_row_off(st, slot, j), t), j * BITS, w);
+                }
+            }
             d[w] = word;
         }
     } else {
@@ -662,8 +682,7 @@ __global__ void import_quant_kernel(Store st, const uint32_t *kw, const char *ks
     const int bh = blockIdx.y;
     const int lo = blockIdx.x * TILE, hi = min(nrows, lo + TILE);
     const int es = st.es;
-    constexpr int per = 32 / BITS;
-    const int Wk = st.Dk / per, Wv = st.Dv / per, Gk = st.Dk / st.gs, Gv = st.Dv / st.gs;
+    const int Wk = st.Dk * BITS / 32, Wv = st.Dv * BITS / 32, Gk = st.Dk / st.gs, Gv = st.Dv / st.gs;
     for (int slot = lo; slot < hi; ++slot) {
         const size_t r = (size_t)bh * nrows + slot;
         uint32_t *kd = reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot)));
@@ -691,15 +710,22 @@ __global__ void import_quant_kernel(Store st, const uint32_t *kw, const char *ks
     }
     char *cell = const_cast<char *>(v_cell_ptr(st, bh, lo));
     constexpr int TPW = 32 / BITS;
-    constexpr int WPR = TILE / TPW;
+    constexpr int WPR = TILE * BITS / 32;
     for (int u = threadIdx.x; u < st.Dv * WPR; u += blockDim.x) {
         const int d = u / WPR, w = u - d * WPR;
         uint32_t nbits = 0;
-        for (int tt = 0; tt < TPW; ++tt) {
-            const int t = w * TPW + tt;
-            if (lo + t < hi) {
-                const uint32_t word = vw[((size_t)bh * nrows + lo + t) * Wv + d / per];
-                nbits |= ((word >> ((d % per) * BITS)) & ((1u << BITS) - 1u)) << (v_bitpos<BITS>(t) & 31);
+        if constexpr ((32 % BITS) == 0) {
+            for (int tt = 0; tt < TPW; ++tt) {
+                const int t = w * TPW + tt;
+                if (lo + t < hi)
+                    nbits |= stream_code<BITS>(vw + ((size_t)bh * nrows + lo + t) * Wv, d) << (v_bitpos<BITS>(t) & 31);
+            }
+        } else {
+            const int t0 = (32 * w) / BITS;  // the first token with bits in word w of the tile row
+            for (int tt = 0; tt < TPW + 2; ++tt) {
+                const int t = t0 + tt;
+                if (t < TILE && lo + t < hi && t * BITS < 32 * w + 32)
+                    nbits |= stream_bits(stream_code<BITS>(vw + ((size_t)bh * nrows + lo + t) * Wv, d), t * BITS, w);
             }
         }
         reinterpret_cast<uint32_t *>(cell + v_row_off(st, lo, d))[w] = nbits;
@@ -722,10 +748,9 @@ template <int DT, int BITS>
 __global__ void affine_dequantize_kernel(const uint32_t *wq, const char *scales, const char *biases,
                                          int64_t rows, int D, int gs, char *dst) {
     const int64_t row = blockIdx.x;
-    constexpr int per = 32 / BITS;
-    const int W = D / per, G = D / gs;
+    const int W = D * BITS / 32, G = D / gs;
     for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        const uint32_t c = (wq[row * W + d / per] >> ((d % per) * BITS)) & ((1u << BITS) - 1u);
+        const uint32_t c = stream_code<BITS>(wq + row * W, d);
         const float s = Elem<DT>::load(scales, row * G + d / gs);
         const float b = Elem<DT>::load(biases, row * G + d / gs);
         Elem<DT>::store(dst, row * D + d, __fadd_rn(__fmul_rn(s, (float)c), b));
@@ -755,6 +780,9 @@ __global__ void mask_materialize_kernel(kvhip_mask_plan_t p, uint8_t *dst) {
     do {                                                                                       \
         if ((BITSV) == 4) { if ((DTV) == 0) { CALL(0, 4); } else if ((DTV) == 1) { CALL(1, 4); } else { CALL(2, 4); } } \
         else if ((BITSV) == 8) { if ((DTV) == 0) { CALL(0, 8); } else if ((DTV) == 1) { CALL(1, 8); } else { CALL(2, 8); } } \
+        else if ((BITSV) == 3) { if ((DTV) == 0) { CALL(0, 3); } else if ((DTV) == 1) { CALL(1, 3); } else { CALL(2, 3); } } \
+        else if ((BITSV) == 5) { if ((DTV) == 0) { CALL(0, 5); } else if ((DTV) == 1) { CALL(1, 5); } else { CALL(2, 5); } } \
+        else if ((BITSV) == 6) { if ((DTV) == 0) { CALL(0, 6); } else if ((DTV) == 1) { CALL(1, 6); } else { CALL(2, 6); } } \
         else { if ((DTV) == 0) { CALL(0, 2); } else if ((DTV) == 1) { CALL(1, 2); } else { CALL(2, 2); } } \
     } while (0)
 
@@ -963,9 +991,16 @@ hipError_t launch_compact_fp(const Store &src, const Runs &runs, const Store &ds
 hipError_t launch_export_quant(const Store &st, int which, int nrows, void *dst, hipStream_t s) {
     if (nrows <= 0) return hipSuccess;
     dim3 grid(nrows, st.BH), block(64);
-    if (st.bits == 4) hipLaunchKernelGGL(export_quant_kernel<4>, grid, block, 0, s, st, which, nrows, (char *)dst);
-    else if (st.bits == 8) hipLaunchKernelGGL(export_quant_kernel<8>, grid, block, 0, s, st, which, nrows, (char *)dst);
-    else hipLaunchKernelGGL(export_quant_kernel<2>, grid, block, 0, s, st, which, nrows, (char *)dst);
+#define EXP(BITS) hipLaunchKernelGGL(export_quant_kernel<BITS>, grid, block, 0, s, st, which, nrows, (char *)dst)
+    switch (st.bits) {
+        case 4: EXP(4); break;
+        case 8: EXP(8); break;
+        case 3: EXP(3); break;
+        case 5: EXP(5); break;
+        case 6: EXP(6); break;
+        default: EXP(2); break;
+    }
+#undef EXP
     return hipGetLastError();
 }
 
@@ -976,7 +1011,14 @@ hipError_t launch_import_quant(const Store &st, const void *const srcs[6], int n
     hipLaunchKernelGGL(import_quant_kernel<BITS>, grid, block, 0, s, st, (const uint32_t *)srcs[0],   \
                        (const char *)srcs[1], (const char *)srcs[2], (const uint32_t *)srcs[3],       \
                        (const char *)srcs[4], (const char *)srcs[5], nrows)
-    if (st.bits == 4) IMP(4); else if (st.bits == 8) IMP(8); else IMP(2);
+    switch (st.bits) {
+        case 4: IMP(4); break;
+        case 8: IMP(8); break;
+        case 3: IMP(3); break;
+        case 5: IMP(5); break;
+        case 6: IMP(6); break;
+        default: IMP(2); break;
+    }
 #undef IMP
     return hipGetLastError();
 }

@@ -286,9 +286,9 @@ class _Cache:
         L.check(self._lib.kvhip_cache_state_import(self._h, n, ptrs, shapes, dts, _stream()))
         torch.cuda.current_stream().synchronize()
         if self.kind == L.KIND_QUANTIZED:
-            per = 32 // self.bits
-            self._shape = (arrays[0].shape[0], arrays[0].shape[1], arrays[0].shape[3] * per,
-                           arrays[3].shape[3] * per, arrays[1].dtype)
+            bits = self.bits
+            self._shape = (arrays[0].shape[0], arrays[0].shape[1], arrays[0].shape[3] * 32 // bits,
+                           arrays[3].shape[3] * 32 // bits, arrays[1].dtype)
         else:
             self._shape = (arrays[0].shape[0], arrays[0].shape[1], arrays[0].shape[3], arrays[1].shape[3],
                            arrays[0].dtype)

@@ -34,6 +34,10 @@ Parity status of each function
   (oracle/kv_oracle.c).  No output of MLX itself is held by the reference for
   packed codes or scale / bias bits, so against the MLX binary this stays
   **parity unpinned**; against the published algorithm it is pinned.
+  The packing of 3-, 5- and 6-bit codes (8 / 8 / 4 codes in 3 / 5 / 3 bytes, low
+  code first) is likewise restated from that file and pinned only by byte patterns
+  worked out by hand (tests/test_oracle_kat.py) and by the pack / unpack round trip:
+  **parity unpinned** against the MLX binary.
 * `quantized_matmul` / `softmax_last` rounding points and accumulation order:
   **parity unpinned** (tolerance-level only).  `softmax(precise: false)`, which
   KVCache.swift:2416 calls, accumulates in the input dtype on MLX's CPU backend
@@ -124,11 +128,16 @@ def affine_quantize(w: np.ndarray, group_size: int, bits: int, dtype: str):
         code  = clamp(rint((w - bias) / scale), 0, 2^bits - 1)   with the float32 scale/bias
         scales = T(scale), biases = T(bias)
 
-    Element k of each run of 32/bits codes occupies bits [k*bits, (k+1)*bits)
-    of one uint32 word. Returns (wq uint32 [..., D*bits/32], scales f32-as-T
-    [..., D/group_size], biases likewise).
+    Packing: for 2, 4 and 8 bits element k of each run of 32/bits codes occupies
+    bits [k*bits, (k+1)*bits) of one uint32 word.  For 3, 5 and 6 bits MLX packs
+    8 / 8 / 4 codes, low code first, into a 24 / 40 / 24-bit integer stored as
+    3 / 5 / 3 little-endian bytes; the row's bytes are then read as uint32 words.
+    Both are the same thing: the row is a little-endian bit stream in which code j
+    occupies bits [j*bits, (j+1)*bits), and `pack_codes` builds exactly that.
+    Returns (wq uint32 [..., D*bits/32], scales f32-as-T [..., D/group_size],
+    biases likewise).
     """
-    assert bits in (2, 4, 8), "power-of-two bit widths only"
+    assert bits in (2, 3, 4, 5, 6, 8), "MLX's affine code widths"
     w = np.asarray(w, dtype=np.float32)
     D = w.shape[-1]
     assert D % group_size == 0
@@ -151,18 +160,37 @@ def affine_quantize(w: np.ndarray, group_size: int, bits: int, dtype: str):
         q = np.rint((g - bias[..., None]) / scale[..., None]).astype(np.float32)
     q = np.minimum(np.maximum(q, np.float32(0)), n_bins)
     codes = q.astype(np.uint32).reshape(w.shape[:-1] + (D,))
-    per = 32 // bits
-    c = codes.reshape(w.shape[:-1] + (D // per, per))
-    shifts = (np.arange(per, dtype=np.uint32) * np.uint32(bits))
-    wq = np.bitwise_or.reduce(c << shifts, axis=-1).astype(np.uint32)
-    return wq, round_to(scale, dtype), round_to(bias, dtype)
+    return pack_codes(codes, bits), round_to(scale, dtype), round_to(bias, dtype)
+
+
+def pack_codes(codes: np.ndarray, bits: int) -> np.ndarray:
+    """codes [..., D] (each < 2^bits) -> uint32 [..., D*bits/32]: code j at bits [j*bits, (j+1)*bits)
+    of the row read as a little-endian bit stream (see `affine_quantize`)."""
+    codes = np.asarray(codes, dtype=np.uint32)
+    D = codes.shape[-1]
+    assert (D * bits) % 32 == 0
+    if 32 % bits == 0:
+        per = 32 // bits
+        c = codes.reshape(codes.shape[:-1] + (D // per, per))
+        shifts = (np.arange(per, dtype=np.uint32) * np.uint32(bits))
+        return np.bitwise_or.reduce(c << shifts, axis=-1).astype(np.uint32)
+    one = ((codes[..., None] >> np.arange(bits, dtype=np.uint32)) & np.uint32(1)).astype(np.uint8)
+    stream = np.packbits(one.reshape(codes.shape[:-1] + (D * bits,)), axis=-1, bitorder="little")
+    return np.ascontiguousarray(stream).view("<u4").astype(np.uint32)
 
 
 def unpack_codes(wq: np.ndarray, bits: int) -> np.ndarray:
-    per = 32 // bits
-    shifts = (np.arange(per, dtype=np.uint32) * np.uint32(bits))
-    c = (wq[..., None] >> shifts) & np.uint32((1 << bits) - 1)
-    return c.reshape(wq.shape[:-1] + (wq.shape[-1] * per,))
+    wq = np.asarray(wq, dtype=np.uint32)
+    if 32 % bits == 0:
+        per = 32 // bits
+        shifts = (np.arange(per, dtype=np.uint32) * np.uint32(bits))
+        c = (wq[..., None] >> shifts) & np.uint32((1 << bits) - 1)
+        return c.reshape(wq.shape[:-1] + (wq.shape[-1] * per,))
+    stream = np.ascontiguousarray(wq.astype("<u4")).view(np.uint8)
+    one = np.unpackbits(stream, axis=-1, bitorder="little")
+    D = wq.shape[-1] * 32 // bits
+    one = one.reshape(wq.shape[:-1] + (D, bits)).astype(np.uint32)
+    return (one << np.arange(bits, dtype=np.uint32)).sum(axis=-1).astype(np.uint32)
 
 
 def _dequant_f32(wq, scales, biases, group_size, bits):

@@ -55,7 +55,7 @@ def omask(mask, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("bits,gs,D", [(8, 64, 64), (4, 64, 128), (4, 32, 64), (2, 64, 128), (4, 64, 256), (8, 128, 256),
-                                        (8, 32, 128), (4, 32, 96), (8, 32, 96)])
+                                        (8, 32, 128), (4, 32, 96), (8, 32, 96), (3, 64, 128), (5, 32, 96), (6, 64, 64)])
 @pytest.mark.parametrize("r", [1, 4])
 def test_quantized_attention_modes(policy, dtype, bits, gs, D, r):
     rng = np.random.default_rng(bits + D + r)

@@ -24,7 +24,7 @@ def positioned(lo, hi, D=2, dtype=torch.float16):
 
 # ------------------------------------------------------------------ quantizer
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
 @pytest.mark.parametrize("gs", [32, 64, 128])
 def test_affine_quantize_bit_exact(dtype, bits, gs):
     rng = np.random.default_rng(bits * 100 + gs)
@@ -93,6 +93,9 @@ def check_quantized_state(cache, ocache, dtype):
 @pytest.mark.parametrize("dtype,bits,gs,D", [
     (torch.float16, 4, 64, 128), (torch.float16, 8, 64, 64), (torch.bfloat16, 4, 32, 64),
     (torch.float32, 8, 64, 128), (torch.float16, 2, 64, 128), (torch.float16, 4, 128, 256),
+    # code widths that do not divide 32: a code may straddle two words of a K row / of a V tile row
+    (torch.float16, 3, 64, 128), (torch.bfloat16, 5, 32, 96), (torch.float16, 6, 64, 64), (torch.float32, 3, 32, 96),
+    (torch.bfloat16, 6, 128, 256), (torch.float16, 5, 64, 128),
 ])
 def test_quantized_cache_append_trim_state(dtype, bits, gs, D):
     rng = np.random.default_rng(11)
@@ -293,6 +296,11 @@ def test_simple_to_quantized_and_back(dtype):
     q = c.to_quantized(64, 4)
     oq = o.to_quantized(64, 4)
     check_quantized_state(q, oq, dtype)
+    for bits in (3, 5, 6):
+        qb, ob = c.to_quantized(32, bits), o.to_quantized(32, bits)
+        check_quantized_state(qb, ob, dtype)
+        for a, b in zip(qb.to_unquantized().state, ob.to_unquantized().get_state()):
+            assert bits_equal(a, b, dtype)
     # empty Simple, offset 7, toQuantized(128, 4) -> ["256","7","128","4"] (KVCacheTests.swift:526-536)
     e = kvhip.KVCacheSimple()
     e.offset = 7

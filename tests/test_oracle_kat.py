@@ -288,7 +288,7 @@ def test_quantize_numpy_vs_scalar_c(bits, gs, dtype):
     assert np.array_equal(da, db)
 
 
-@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("bits", [3, 4, 5, 6, 8])
 def test_quantize_closed_forms(bits):
     gs, D = 64, 128
     nb = (1 << bits) - 1
@@ -350,7 +350,7 @@ def test_compression_matches_reference_documentation(bits, bytes_per_group):
     assert wq.size * 4 + s.size * 2 + b.size * 2 == bytes_per_group
 
 
-@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
 def test_quantize_invariants(bits):
     rng = np.random.default_rng(7)
     w = O.round_to(rng.standard_normal((64, 128)).astype(np.float32) * 3, "float16")
@@ -366,11 +366,41 @@ def test_quantize_invariants(bits):
     uncovered = np.maximum(0, (g.max(-1) - g.min(-1)) - nb * np.abs(s))
     assert np.all(err <= (np.abs(s) * 0.5 + uncovered) * (1 + 1e-5) + 1e-6)
     # little-endian nibble order: element k of a word sits at bits [k*bits, (k+1)*bits)
-    per = 32 // bits
-    assert codes[3, per + 1] == (wq[3, 1] >> bits) & ((1 << bits) - 1)
+    if 32 % bits == 0:
+        per = 32 // bits
+        assert codes[3, per + 1] == (wq[3, 1] >> bits) & ((1 << bits) - 1)
     # the extreme element |edge| reproduces exactly (bias == edge, code 0)
     edge = np.where(np.abs(g.min(-1)) > np.abs(g.max(-1)), g.min(-1), g.max(-1))
     assert np.array_equal(b, edge)
+
+
+@pytest.mark.parametrize("bits,codes,packed", [
+    # 3 bits, 8 codes in 3 bytes: 1 + 2*8 + 3*64 + 4*512 + 5*4096 + 6*32768 + 7*262144 + 0 = 0x1F58D1
+    (3, [1, 2, 3, 4, 5, 6, 7, 0], [0xD1, 0x58, 0x1F]),
+    # 6 bits, 4 codes in 3 bytes: 1 + 2*64 + 3*4096 + 63*262144 = 0xFC3081
+    (6, [1, 2, 3, 63], [0x81, 0x30, 0xFC]),
+    # 5 bits, 8 codes in 5 bytes: 1 + 2*2^5 + 3*2^10 + 4*2^15 + 5*2^20 + 6*2^25 + 7*2^30 + 31*2^35 = 0xF9CC520C41
+    (5, [1, 2, 3, 4, 5, 6, 7, 31], [0x41, 0x0C, 0x52, 0xCC, 0xF9]),
+])
+def test_odd_width_packing_known_bytes(bits, codes, packed):
+    """MLX packs 3-, 5- and 6-bit codes 8 / 8 / 4 at a time, low code first, into 3 / 5 / 3 bytes
+    (`quantize<T, U>`, mlx/backend/cpu/quantized.cpp, reached from KVCache.swift:1069-1070); the
+    expected bytes are worked out by hand above, not taken from a restatement."""
+    n = 32 * len(codes)  # whole uint32 words
+    row = np.asarray(codes * 32, np.uint32)
+    wq = O.pack_codes(row[None], bits)
+    assert wq.dtype == np.uint32 and wq.shape == (1, n * bits // 32)
+    stream = wq.astype("<u4").view(np.uint8)[0]
+    assert [int(x) for x in stream[:len(packed)]] == packed
+    assert [int(x) for x in stream] == packed * 32
+    assert np.array_equal(O.unpack_codes(wq, bits)[0], row)
+    # through the quantizer: integers 0 .. nb with both ends present -> code(x) = nb - x exactly
+    nb = (1 << bits) - 1
+    group = [nb - c for c in codes] * (32 // len(codes))
+    group[0], group[1] = nb, 0  # both extremes in every group whatever the codes above are
+    w = np.asarray(group * len(codes), np.float32)[None]
+    q, s, b = O.affine_quantize(w, 32, bits, "float32")
+    assert np.array_equal(O.unpack_codes(q, bits)[0], (nb - w[0]).astype(np.uint32))
 
 
 # ---------------------------------------------------------------- attention
