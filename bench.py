@@ -47,7 +47,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--context", type=int, default=32768)
     ap.add_argument("--batch", type=int, default=32)
-    ap.add_argument("--head-dim", type=int, default=128, help="head size of the cfg3-shaped run (64, 128, 256)")
+    ap.add_argument("--head-dim", type=int, default=128, help="head size of the cfg3-shaped run (64, 96, 128, 256)")
+    ap.add_argument("--tokens", type=int, default=1,
+                    help="new tokens per step of the cfg3-shaped run (more than 1: a causal multi-token step, "
+                         "as a speculative verify makes; needs --cpu-steps 0)")
     ap.add_argument("--group-size", type=int, default=64, help="quantization group size (32, 64, 128)")
     ap.add_argument("--bits", type=int, default=4, help="code width (4, 8)")
     ap.add_argument("--cpu-steps", type=int, default=5, help="decode steps timed on the CPU baseline after one warm-up (0 = skip)")
@@ -84,10 +87,12 @@ def main():
         print(json.dumps(other_workload(args, torch, kvhip, L, dev)))
         return
     nb, ctx = args.batch, args.context
-    D, GS, BITS = args.head_dim, args.group_size, args.bits
+    D, GS, BITS, NT = args.head_dim, args.group_size, args.bits, args.tokens
+    if NT > 1 and args.cpu_steps > 0:
+        sys.exit("bench.py: --tokens above 1 is timed on the GPU only; pass --cpu-steps 0")
     # per cached token and kv head: K and V codes + (scale, bias) pairs of 2 x 2 bytes per group
     ROW_BYTES = 2 * (D * BITS // 8 + (D // GS) * 4)
-    headline = (nb, ctx, D, GS, BITS) == (32, 32768, 128, 64, 4)
+    headline = (nb, ctx, D, GS, BITS, NT) == (32, 32768, 128, 64, 4, 1)
     g = torch.Generator(device=dev)
     g.manual_seed(0)
     ch = (10.0 ** (torch.rand(D, generator=g, device=dev) * 2 - 1)).to(torch.float32)
@@ -114,9 +119,15 @@ def main():
     pf_rows = sorted(n for _, _, n in pf_events)[len(pf_events) // 2]
     pf_bytes = nb * HKV * pf_rows * (2 * D * 2 + ROW_BYTES)
     nsteps = args.warmup + args.steps
-    qs = torch.randn(nsteps, nb, HQ, 1, D, generator=g, device=dev).to(torch.float16)
-    ks = (torch.randn(nsteps, nb, HKV, 1, D, generator=g, device=dev) * ch).to(torch.float16)
-    vs = (torch.randn(nsteps, nb, HKV, 1, D, generator=g, device=dev) * ch).to(torch.float16)
+    qs = torch.randn(nsteps, nb, HQ, NT, D, generator=g, device=dev).to(torch.float16)
+    ks = (torch.randn(nsteps, nb, HKV, NT, D, generator=g, device=dev) * ch).to(torch.float16)
+    vs = (torch.randn(nsteps, nb, HKV, NT, D, generator=g, device=dev) * ch).to(torch.float16)
+    causal = kvhip.MaskMode.causal()
+
+    def step(i):
+        if NT == 1:
+            return cache.update_attend(qs[i], ks[i], vs[i], scale)
+        return kvhip.attention_with_cache_update(qs[i], ks[i], vs[i], cache, scale, causal)
     scale = 1.0 / D ** 0.5
     torch.cuda.synchronize()
 
@@ -129,7 +140,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     for i in range(args.warmup):
-        out = cache.update_attend(qs[i], ks[i], vs[i], scale)
+        out = step(i)
     torch.cuda.synchronize()
     # every 8th launch of the timed region is bracketed by HIP events (each bracket costs a few
     # microseconds of stream time, which would otherwise sit in every step)
@@ -137,7 +148,7 @@ def main():
     t_first = cache.offset + 1
     t0 = time.perf_counter()
     for i in range(args.warmup, nsteps):
-        out = cache.update_attend(qs[i], ks[i], vs[i], scale)
+        out = step(i)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     lib.kvhip_profile_enable(0)
@@ -146,7 +157,7 @@ def main():
     t_last = cache.offset
     elapsed = t1 - t0
     ms_per_step = 1e3 * elapsed / args.steps
-    tok_s = nb * args.steps / elapsed
+    tok_s = nb * NT * args.steps / elapsed
 
     mean_t = 0.5 * (t_first + t_last)
     alg_bytes = nb * HKV * mean_t * ROW_BYTES
@@ -154,7 +165,9 @@ def main():
     if launches.value > 0:
         kernel_ms = kms.value / launches.value
         achieved = alg_bytes / (kernel_ms * 1e-3) / 1e9
-        roofline = {"bound": "hbm", "kernel": f"decode_kernel<{BITS},{D},{GS},f16>", "achieved": round(achieved, 1),
+        rows = (HQ // HKV) * NT
+        kname = "decode16_kernel" if (rows > 4 or D == 96) else "decode_kernel"
+        roofline = {"bound": "hbm", "kernel": f"{kname}<{BITS},{D},{GS},f16>", "achieved": round(achieved, 1),
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                     "kernel_ms": round(kernel_ms, 5), "algorithmic_bytes": int(alg_bytes),
                     "launches_timed": int(launches.value),
@@ -233,7 +246,7 @@ def main():
         "dtype": f"f16 ({BITS}-bit affine codes, fp32 accumulate)", "data": "synthetic",
         "config": {"workload": ("configs[2]: " if headline else "configs[2]'s shape varied: ") +
                                f"QuantizedKVCache {BITS}-bit g{GS}, 32q/8kv heads, head_dim {D}, "
-                               f"batch {nb}, context {ctx}+, quantize-on-append + fused dequant-SDPA, one layer",
+                               f"batch {nb}, context {ctx}+, {NT} token(s) per step, quantize-on-append + fused dequant-SDPA, one layer",
                    "batch": nb, "context_first": int(t_first), "context_last": int(t_last)},
         "roofline": roofline, "cpu_baseline": cpu, "parity": parity,
         "prefill_append": {"rows": pf_rows, "ms": round(pf_ms, 3), "GB/s": round(pf_bytes / (pf_ms * 1e-3) / 1e9, 1),

@@ -1130,7 +1130,7 @@ Plan plan_for(const AttendArgs &a) {
             p.nsplit = std::max(512 / a.Hkv, 2 * a.B);
             if (p.nsplit > 512) p.nsplit = 512;  // (more than 256 batch rows would be needed: not with B <= 64)
         }
-    } else if (a.st.bits != 0 && p.nsplit >= 2 && want <= 4 && p.rg == 1 && a.mask.mode != KVHIP_MASK_ARRAY &&
+    } else if (a.st.bits != 0 && p.nsplit >= 2 && want <= 4 && p.rg == 1 && a.st.Dk != 96 && a.mask.mode != KVHIP_MASK_ARRAY &&
                forced_tiles <= 0) {
         // 128 pairs or more: workgroups of 8 wavefronts, one per CU -- the same wavefronts per CU
         // with half the spans.  With 256 pairs a workgroup takes its pair's whole sequence: the
@@ -1222,8 +1222,8 @@ bool attend_decode_supported(const AttendArgs &a) {
     if (a.runs.n != 1 || a.runs.row0[0] != 0 || a.runs.phys0[0] != 0) return false;
     if (s.bits != 4 && s.bits != 8) return false;
     if (s.Dk == 64) return s.gs == 32 || s.gs == 64;
-    // 5..16 rows of group size 32 at D = 128: the 16-row kernel is built for 4-bit codes only
-    if (s.Dk == 128) return s.gs == 64 || s.gs == 128 || (s.gs == 32 && (R <= 4 || s.bits == 4));
+    if (s.Dk == 96) return s.gs == 32;  // every row count on the 16-row kernel
+    if (s.Dk == 128) return s.gs == 32 || s.gs == 64 || s.gs == 128;
     if (s.Dk == 256) return R <= 4 && (s.gs == 64 || s.gs == 128);  // more rows: the prefill tile
     return false;
 }
@@ -1231,7 +1231,7 @@ bool attend_decode_supported(const AttendArgs &a) {
 // The 4-row quantized kernel without a mask writes the step's new row itself.
 bool attend_decode_fuses_append(const AttendArgs &a) {
     if (!attend_decode_supported(a) || a.st.bits == 0 || a.L != 1) return false;
-    if ((a.Hq / a.Hkv) * a.L > 4 || a.mask.mode != KVHIP_MASK_NONE) return false;
+    if ((a.Hq / a.Hkv) * a.L > 4 || a.mask.mode != KVHIP_MASK_NONE || a.st.Dk == 96) return false;
     static const bool off = getenv("KVHIP_NO_FUSED_APPEND") != nullptr;  // measurement aid
     return !off;
 }
@@ -1240,7 +1240,8 @@ bool attend_decode_fuses_append(const AttendArgs &a) {
 // (kvhip_attend_decode16.hip), which always carries 16 rows: measured faster than the 4-row
 // broadcast contraction from 8 rows up (B16, 8 kv heads, 8192 tokens: 37 us against 43 us at
 // 8 rows, 36 us against 87 us at 16).
-static bool use_decode16(const AttendArgs &a, const Plan &p) { return a.st.bits != 0 && p.rg >= 2; }
+// Head size 96 (a row and a half of the 4-row kernel's 64-column halves) takes it for every row count.
+static bool use_decode16(const AttendArgs &a, const Plan &p) { return a.st.bits != 0 && (p.rg >= 2 || a.st.Dk == 96); }
 
 size_t attend_decode_workspace(const AttendArgs &a) {
     const Plan p = plan_for(a);

@@ -55,6 +55,22 @@ template <int DT> __device__ __forceinline__ float sb_bias(uint32_t raw) {
     return __uint_as_float(raw & 0xffff0000u);
 }
 
+// 4 bytes per lane from global memory straight into LDS: lane i's land at `lds_wave_base` + 4 i (the base is
+// the same for the whole wavefront; address = wave-uniform `base` in scalar registers + the lane's unsigned
+// 32-bit byte offset).  Written as assembly: the compiler does not count it among the vector-memory
+// operations in flight, which only makes its own waits stricter (such operations complete in order); the
+// kernel waits for it by hand (s_waitcnt vmcnt(0)) before it reads what the load fills.
+__device__ __forceinline__ void load_dword_to_lds(gptr base, uint32_t lane_off, const void *lds_wave_base) {
+    // (the low half of a flat address inside the LDS aperture is the LDS address itself)
+    const uint32_t lds = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds_wave_base);
+    const uint64_t b = (uint64_t)base;
+    // (readfirstlane returns a signed int: without the casts the low half would be sign-extended over the high one)
+    const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));
+    const uint64_t sb = ((uint64_t)b_hi << 32) | (uint64_t)b_lo;
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(lane_off), "s"(sb), "s"(lds) : "memory", "m0");
+}
+
 // 8 codes -> one 8-element operand.  4 bit: one word, element order (c0,c4,c1,c5,c2,c6,c3,c7),
 // registers 1 and 3 hold high nibbles (x16).  8 bit: two words, order (c0,c2,c1,c3,c4,c6,c5,c7).
 template <int BITS> struct Codes;
@@ -94,6 +110,13 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     constexpr int VWL = 16 * BITS / 32;          // words per lane and V row: its 16 tokens
     constexpr int VROW = 64 * BITS / 8;          // bytes of one V tile row
     constexpr int RR = 16;
+    // Three or four groups per row (group size 32 at D = 96 / 128): the (scale, bias) pairs of a tile -- 64 tokens
+    // x G pairs per side, 2 G registers per token of the lane group if held in registers -- go from global memory
+    // straight into LDS one tile ahead and are read from there four tokens at a time when they are used.
+    constexpr bool SB_LDS = G >= 3;
+    constexpr int SB_PAD = G == 4 ? 4 : 0;       // words between the 64-word pieces (G = 4: a piece per lane group; keeps the groups' reads on different banks)
+    constexpr int SB_JJ = 16 * G + SB_PAD;       // words from one lane group's pairs to the next
+    constexpr int SB_WORDS = SB_LDS ? G * (64 + SB_PAD) : 4;
     const Store &st = a.st;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -105,6 +128,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     size_t part_slot = (size_t)bh * nsplit + split;  // where this workgroup's partial goes
 
     __shared__ float cbuf[WAVES][RR][D + 2];
+    __shared__ __attribute__((aligned(16))) uint32_t sbuf[WAVES][2][2][SB_WORDS];  // [wavefront][tile parity][K, V][pairs]
 
     // ---- span of this workgroup (as in the 4-row kernel) -----------------------------------
     // tiles_per_wg < 0: a ragged batch, grid (nsplit span slots, kv heads): the slots of a kv head are
@@ -184,8 +208,38 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     struct Tile {
         uint32_t k[4][G][KWL];
         uint32_t v[NDB][VWL];
-        uint32_t ksb[16][G], vsb[16][G];  // raw (scale, bias) pairs per token of the lane group
+        uint32_t ksb[SB_LDS ? 1 : 16][G], vsb[SB_LDS ? 1 : 16][G];  // raw (scale, bias) pairs per token of the lane group
         int base;                          // first slot of the tile
+    };
+    // (SB_LDS) the pairs of the wavefront's tile number `i`, both sides, into the buffer of that parity; the plane
+    // bases walk the page table on their own, one page ahead, like the code planes'
+    int page_sb = page_k, sb_issued = 0;
+    gptr ksb_n = ksb_b, vsb_n = vsb_b;
+    auto dma_sb = [&]() __attribute__((always_inline)) {
+        const size_t tile_off = (size_t)tip * TILE;
+        const gptr ks = ksb_n + (size_t)bh * st.ksb_cell + tile_off * st.ksb_row;
+        const gptr vs = vsb_n + (size_t)bh * st.vsb_cell + tile_off * st.vsb_row;
+        const int par = sb_issued & 1;
+#pragma unroll
+        for (int c = 0; c < G; ++c) {
+            load_dword_to_lds(ks, (uint32_t)(c * 256 + lane * 4), &sbuf[wave][par][0][c * (64 + SB_PAD)]);
+            load_dword_to_lds(vs, (uint32_t)(c * 256 + lane * 4), &sbuf[wave][par][1][c * (64 + SB_PAD)]);
+        }
+        ++sb_issued;
+        if (sb_issued < my_tiles) {
+            ++page_sb;
+            ksb_n = as_global(st.pt[page_sb].ksb);
+            vsb_n = as_global(st.pt[page_sb].vsb);
+        }
+    };
+    // (SB_LDS) the pairs of tokens 4 tb .. 4 tb + 3 of the lane group, `side` 0 K / 1 V: out[i * G + g]
+    auto sb_quad = [&](int par, int side, int tb, uint32_t (&out)[4 * G]) __attribute__((always_inline)) {
+        const u4 *p = reinterpret_cast<const u4 *>(&sbuf[wave][par][side][SB_JJ * jj + 4 * G * tb]);
+#pragma unroll
+        for (int e = 0; e < G; ++e) {
+            const u4 w = p[e];
+            out[4 * e] = w.x; out[4 * e + 1] = w.y; out[4 * e + 2] = w.z; out[4 * e + 3] = w.w;
+        }
     };
 
     int k_loaded = 0, v_loaded = 0;
@@ -211,18 +265,20 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 }
             }
         // 16 tokens x G pairs of 4 bytes: contiguous rows of G * 4 bytes
+        if constexpr (!SB_LDS) {
 #pragma unroll
-        for (int e = 0; e < 16 * G / 4; ++e) {
-            const u4 w = ld_global<u4>(ksp, e);
-            (&t.ksb[0][0])[4 * e] = w.x; (&t.ksb[0][0])[4 * e + 1] = w.y;
-            (&t.ksb[0][0])[4 * e + 2] = w.z; (&t.ksb[0][0])[4 * e + 3] = w.w;
+            for (int e = 0; e < 16 * G / 4; ++e) {
+                const u4 w = ld_global<u4>(ksp, e);
+                (&t.ksb[0][0])[4 * e] = w.x; (&t.ksb[0][0])[4 * e + 1] = w.y;
+                (&t.ksb[0][0])[4 * e + 2] = w.z; (&t.ksb[0][0])[4 * e + 3] = w.w;
+            }
         }
         t.base = base_next;
         ++k_loaded;
         if (k_loaded < my_tiles) {  // wave-uniform: the same tile of the next page
             ++page_k;
             kb = as_global(st.pt[page_k].k);
-            ksb_b = as_global(st.pt[page_k].ksb);
+            if constexpr (!SB_LDS) ksb_b = as_global(st.pt[page_k].ksb);
             base_next += PAGE;
         }
     };
@@ -239,17 +295,19 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 t.v[db][0] = w.x; t.v[db][1] = w.y; t.v[db][2] = w.z; t.v[db][3] = w.w;
             }
         }
+        if constexpr (!SB_LDS) {
 #pragma unroll
-        for (int e = 0; e < 16 * G / 4; ++e) {
-            const u4 w = ld_global<u4>(vsp, e);
-            (&t.vsb[0][0])[4 * e] = w.x; (&t.vsb[0][0])[4 * e + 1] = w.y;
-            (&t.vsb[0][0])[4 * e + 2] = w.z; (&t.vsb[0][0])[4 * e + 3] = w.w;
+            for (int e = 0; e < 16 * G / 4; ++e) {
+                const u4 w = ld_global<u4>(vsp, e);
+                (&t.vsb[0][0])[4 * e] = w.x; (&t.vsb[0][0])[4 * e + 1] = w.y;
+                (&t.vsb[0][0])[4 * e + 2] = w.z; (&t.vsb[0][0])[4 * e + 3] = w.w;
+            }
         }
         ++v_loaded;
         if (v_loaded < my_tiles) {
             ++page_v;
             vb = as_global(st.pt[page_v].v);
-            vsb_b = as_global(st.pt[page_v].vsb);
+            if constexpr (!SB_LDS) vsb_b = as_global(st.pt[page_v].vsb);
         }
     };
 
@@ -302,7 +360,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 
     Op8 pb[G][2];  // probabilities of the tile in flight: per group (pre-scaled by V's scale), step u
 
-    auto compute_qk_softmax = [&](const Tile &t) __attribute__((always_inline)) {
+    auto compute_qk_softmax = [&](const Tile &t, int par) __attribute__((always_inline)) {
         // ---- S^T blocks --------------------------------------------------------------------
         f4 sacc[4][G];
 #pragma unroll
@@ -319,7 +377,9 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         // ---- scores of row n for this lane group's 16 tokens: local token 4 tb + i ---------------
         float x[16];
 #pragma unroll
-        for (int tb = 0; tb < 4; ++tb)
+        for (int tb = 0; tb < 4; ++tb) {
+            uint32_t kq[4 * G];
+            if constexpr (SB_LDS) sb_quad(par, 0, tb, kq);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int tl = 4 * tb + i;
@@ -328,11 +388,13 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 float sc_ = 0.f, sb_ = 0.f;
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
-                    sc_ = __builtin_fmaf(sb_scale<DT>(t.ksb[tl][g]), sacc[tb][g][i], sc_);
-                    sb_ = __builtin_fmaf(sb_bias<DT>(t.ksb[tl][g]), qsum[g], sb_);
+                    const uint32_t raw = SB_LDS ? kq[i * G + g] : t.ksb[SB_LDS ? 0 : tl][g];
+                    sc_ = __builtin_fmaf(sb_scale<DT>(raw), sacc[tb][g][i], sc_);
+                    sb_ = __builtin_fmaf(sb_bias<DT>(raw), qsum[g], sb_);
                 }
                 x[tl] = round_dt<DT>(__builtin_fmaf(sc_, TWO24, sb_));
             }
+        }
         if (MM == 2 && a.mask.dtype == KVHIP_BOOL && t.base + (TILE - 1) < a.T) {
             // a boolean array over a whole tile: this lane's 16 tokens are 16 consecutive bytes of its
             // query row
@@ -385,16 +447,23 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         const float mu = (m_run == -INFINITY) ? 0.f : m_run;
         float pv[G][16];
 #pragma unroll
-        for (int tl = 0; tl < 16; ++tl) {
-            // (the difference first: a masked score is finfo(T).min, whose product with log2 e overflows for bfloat16)
-            const float p = fast_exp2((x[tl] - mu) * LOG2E);  // exp2(-inf) = 0 for dead slots
-            l_part += p;
-            // positions 2, 3, 6, 7 of a 4-bit operand meet high nibbles (x16)
-            const float ps = hi_of<BITS>(tl & 7) ? p * 0.0625f : p;
+        for (int tb = 0; tb < 4; ++tb) {
+            uint32_t vq[4 * G];
+            if constexpr (SB_LDS) sb_quad(par, 1, tb, vq);
 #pragma unroll
-            for (int g = 0; g < G; ++g) {
-                bacc[g] = __builtin_fmaf(p, sb_bias<DT>(t.vsb[tl][g]), bacc[g]);
-                pv[g][tl] = ps * sb_scale<DT>(t.vsb[tl][g]);
+            for (int i = 0; i < 4; ++i) {
+                const int tl = 4 * tb + i;
+                // (the difference first: a masked score is finfo(T).min, whose product with log2 e overflows for bfloat16)
+                const float p = fast_exp2((x[tl] - mu) * LOG2E);  // exp2(-inf) = 0 for dead slots
+                l_part += p;
+                // positions 2, 3, 6, 7 of a 4-bit operand meet high nibbles (x16)
+                const float ps = hi_of<BITS>(tl & 7) ? p * 0.0625f : p;
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    const uint32_t raw = SB_LDS ? vq[i * G + g] : t.vsb[SB_LDS ? 0 : tl][g];
+                    bacc[g] = __builtin_fmaf(p, sb_bias<DT>(raw), bacc[g]);
+                    pv[g][tl] = ps * sb_scale<DT>(raw);
+                }
             }
         }
 #pragma unroll
@@ -421,11 +490,20 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     // next tile before its PV
     if (my_tiles > 0) {
         Tile buf;
+        if constexpr (SB_LDS) dma_sb();
         load_k(buf);
         load_queries();
         for (int done = 0; done < my_tiles; ++done) {
-            load_v(buf);
-            compute_qk_softmax(buf);
+            if constexpr (SB_LDS) {
+                // K codes and pairs of this tile have arrived (everything requested so far); the pairs of the next
+                // tile go to the other buffer, whose last readers (the tile before this one) are long done
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                load_v(buf);
+                if (sb_issued < my_tiles) dma_sb();
+            } else {
+                load_v(buf);
+            }
+            compute_qk_softmax(buf, done & 1);
             load_k(buf);
             compute_pv(buf);
         }
@@ -519,14 +597,14 @@ hipError_t launch_attend_decode16(const AttendArgs &a, int tiles_total, int tile
     do {                                                \
         if (st.Dk == 64 && st.gs == 32) D16_DT(BITS, 64, 32);        \
         else if (st.Dk == 64) D16_DT(BITS, 64, 64);                  \
+        else if (st.Dk == 96) D16_DT(BITS, 96, 32);                  \
+        else if (st.gs == 32) D16_DT(BITS, 128, 32);                 \
         else if (st.gs == 64) D16_DT(BITS, 128, 64);                 \
         else D16_DT(BITS, 128, 128);                                 \
     } while (0)
-    // (group size 32 at D = 128 is built for 4-bit codes only: the 8-bit tile plus four groups of
-    // scale / bias registers no longer fits the register file; the caller sends that shape, and
-    // D = 256, whose partials exceed a workgroup's LDS, to the prefill tile)
-    if (st.bits == 4 && st.Dk == 128 && st.gs == 32) D16_DT(4, 128, 32);
-    else if (st.bits == 4) D16_Q(4);
+    // (head size 96 only divides by group size 32; D = 256, whose partials exceed a workgroup's LDS, is
+    // sent to the prefill tile by the caller)
+    if (st.bits == 4) D16_Q(4);
     else D16_Q(8);
 #undef D16_Q
 #undef D16_DT

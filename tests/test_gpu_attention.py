@@ -103,13 +103,14 @@ def test_quantized_attention_modes(policy, dtype, bits, gs, D, r):
     check(out, ref, "decode")
 
 
-@pytest.mark.parametrize("bits,D,gs", [(4, 128, 64), (8, 64, 64), (4, 128, 32), (8, 128, 32), (4, 64, 32)])
+@pytest.mark.parametrize("bits,D,gs", [(4, 128, 64), (8, 64, 64), (4, 128, 32), (8, 128, 32), (4, 64, 32), (4, 96, 32), (8, 96, 32)])
 @pytest.mark.parametrize("B,Hkv,T0", [(32, 8, 777), (64, 8, 300), (32, 8, 70)])
 def test_quantized_decode_many_pairs(bits, D, gs, B, Hkv, T0):
     """Many (batch, kv-head) pairs, the shape of the headline workload scaled down in length:
     with 256 pairs two spans per pair fold into one workgroup of 8 wavefronts that writes the
     output itself, with 512 pairs a single span of 4 does; both skip the partial-merge
-    kernel.  One token (no mask) and two tokens (causal) per step, against the oracle."""
+    kernel.  One token (no mask), two and four tokens (causal: 8 and 16 query rows per kv head, the 16-row
+    kernel, which also takes every row count of head size 96) per step, against the oracle."""
     rng = np.random.default_rng(B + T0 + bits)
     dtype, name = torch.float16, "float16"
     r = 4
@@ -120,14 +121,12 @@ def test_quantized_decode_many_pairs(bits, D, gs, B, Hkv, T0):
     c.update_quantized(kd, vd, fetch=False)
     o.update_quantized(k, v)
     scale = 1.0 / np.sqrt(D)
-    for Lq, mask, om in ((1, None, O.Mask.NONE), (2, kvhip.MaskMode.causal(), O.Mask.CAUSAL)):
+    for Lq, mask, om in ((1, None, O.Mask.NONE), (2, kvhip.MaskMode.causal(), O.Mask.CAUSAL), (4, kvhip.MaskMode.causal(), O.Mask.CAUSAL)):
         k, kd = randn(rng, (B, Hkv, Lq, D), dtype)
         v, vd = randn(rng, (B, Hkv, Lq, D), dtype)
         q, qd = randn(rng, (B, Hkv * r, Lq, D), dtype)
         out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
-        # group size 32 with 8-bit codes at D = 128 is built into the 4-row decode kernel only; more
-        # rows of it take the prefill tile
-        assert kvhip.load().kvhip_last_attend_kernel() == (3 if (gs, bits, D) == (32, 8, 128) and r * Lq > 4 else 1)
+        assert kvhip.load().kvhip_last_attend_kernel() == 1
         ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
         check(out, ref, f"L={Lq}")
 

@@ -103,7 +103,7 @@ def test_quantized_shapes_against_generic(seed):
     if gs > D:
         gs = 64
     if seed % 7 == 6:
-        D, gs = 96, 32  # the only group size that divides 96; every row count runs on the prefill tile
+        D, gs = 96, 32  # the only group size that divides 96 (16 rows or fewer: the 16-row kernel)
     bits = [4, 8][(seed // 9) % 2]
     dtype = [torch.float16, torch.bfloat16][(seed // 18) % 2]
     B, Hkv, r = int(rng.integers(1, 4)), int(rng.choice([1, 2])), int(rng.choice([1, 4, 8]))
