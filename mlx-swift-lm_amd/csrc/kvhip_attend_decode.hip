@@ -1200,10 +1200,11 @@ hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t
         if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL((combine_kernel<D, 0>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows, ragged); \
         else hipLaunchKernelGGL((combine_kernel<D, 1>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows, ragged);       \
     } while (0)
-    if (a.st.Dk == 64) CMB(64);
-    else if (a.st.Dk == 80) CMB(80);
-    else if (a.st.Dk == 96) CMB(96);
-    else if (a.st.Dk == 128) CMB(128);
+    // (the partials hold output columns: the head size of the values)
+    if (a.st.Dv == 64) CMB(64);
+    else if (a.st.Dv == 80) CMB(80);
+    else if (a.st.Dv == 96) CMB(96);
+    else if (a.st.Dv == 128) CMB(128);
     else CMB(256);
 #undef CMB
     return hipGetLastError();

@@ -492,6 +492,8 @@ prefill_kernel(AttendArgs a, int nsplit) {
 bool attend_prefill_supported(const AttendArgs &a) {
     const Store &s = a.st;
     if (s.dtype != KVHIP_F16 && s.dtype != KVHIP_BF16) return false;
+    // keys of 192 with values of 128 (the multi-head latent attention models), full precision only
+    if (s.Dk == 192 && s.Dv == 128 && s.bits == 0) return true;
     if (s.Dk != s.Dv) return false;
     // head sizes 80 (full precision only) and 96: every row count (no decode kernel is built for them)
     if (s.Dk != 64 && s.Dk != 128 && s.Dk != 256 && s.Dk != 96 && !(s.Dk == 80 && s.bits == 0)) return false;
@@ -524,14 +526,14 @@ static int prefill_splits(const AttendArgs &a) {
     if (n > tiles / 8) n = tiles / 8;
     if (n > 8) n = 8;
     if (n < 2) return 1;
-    if ((size_t)a.st.BH * n * R * (a.st.Dk + 2) * sizeof(float) > ((size_t)256 << 20)) return 1;
+    if ((size_t)a.st.BH * n * R * (a.st.Dv + 2) * sizeof(float) > ((size_t)256 << 20)) return 1;
     return n;
 }
 
 size_t attend_prefill_workspace(const AttendArgs &a) {
     const int n = prefill_splits(a);
     if (n <= 1) return 0;
-    return (size_t)a.st.BH * n * (a.Hq / a.Hkv) * a.L * (a.st.Dk + 2) * sizeof(float);
+    return (size_t)a.st.BH * n * (a.Hq / a.Hkv) * a.L * (a.st.Dv + 2) * sizeof(float);
 }
 
 hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {

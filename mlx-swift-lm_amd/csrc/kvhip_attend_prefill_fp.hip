@@ -141,19 +141,21 @@ template <int DT> __device__ __forceinline__ void mfma_acc_inplace(f4 &c, const 
 // same time, which the in-order issue of a tile-at-a-time loop (scores -> softmax -> PV, each
 // waiting for the one before) cannot.  K is requested two tiles ahead and V one tile ahead, each
 // into the buffer of its tile's parity; one barrier per iteration.
-template <int D, int DT, bool IDENT, int QT, int MM>
+// DK and DV are the head sizes of keys / queries and of values / outputs (192 and 128 for the multi-head
+// latent attention models, equal otherwise).
+template <int DK, int DV, int DT, bool IDENT, int QT, int MM>
 __global__ void __launch_bounds__(256, 2)
 prefill_fp_kernel(AttendArgs a, int nsplit) {
     constexpr int BM = 64 * QT;
-    constexpr int S = (D + 31) / 32;  // contraction steps over the head dim (the last one partly zero at D = 80)
-    constexpr int NDT = D / 16;   // 16-row tiles of out^T
-    constexpr int NC = (D + 63) / 64;  // rounds of 256 16-byte chunks, for K and for V
-    constexpr int CH = 4 * D;          // 16-byte chunks of a tile's K (and of its V); a multiple of 64
-    static_assert(D % 16 == 0, "out^T is built from 16-row tiles");
+    constexpr int S = (DK + 31) / 32;  // contraction steps over the head dim (the last one partly zero at D = 80)
+    constexpr int NDT = DV / 16;   // 16-row tiles of out^T
+    constexpr int NCK = (DK + 63) / 64, NCV = (DV + 63) / 64;  // rounds of 256 16-byte chunks, for K and for V
+    constexpr int CHK = 4 * DK, CHV = 4 * DV;  // 16-byte chunks of a tile's K and of its V; multiples of 64
+    static_assert(DK % 16 == 0 && DV % 16 == 0, "out^T is built from 16-row tiles");
     // A head size that is not a multiple of 32 (80): the last contraction step reads K chunks past the
     // row -- the unused tail that the repeated loads fill with finite values -- against query
     // operands that are zero there.
-    static_assert(4 * S * BN <= ((D + 63) / 64) * 256, "the padded contraction stays inside the staged buffer");
+    static_assert(4 * S * BN <= NCK * 256, "the padded contraction stays inside the staged buffer");
     // K and V tiles move from global memory straight into LDS (no registers, no LDS store
     // instructions): per parity of the tile one buffer for K, the tile's 16-byte chunks in page order
     // [8-element chunk][token], and one for V, [8-token chunk][column].  bf16 caches keep K and V as
@@ -163,8 +165,8 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     // size that is not a multiple of 64 (80, 96) the last round is partly empty: its wavefronts past the
     // tile's last chunk repeat that chunk into the unused tail, so that every wavefront issues the same
     // number of loads.
-    constexpr int KSZ = NC * 256 * 8;
-    __shared__ __attribute__((aligned(16))) uint16_t KV0[2 * KSZ], KV1[2 * KSZ];
+    constexpr int KSZ = NCK * 256 * 8, VSZ = NCV * 256 * 8;
+    __shared__ __attribute__((aligned(16))) uint16_t KV0[KSZ + VSZ], KV1[KSZ + VSZ];
     auto Ks = [&](int par) __attribute__((always_inline)) -> uint16_t * { return par == 0 ? KV0 : KV1; };
     auto Vs = [&](int par) __attribute__((always_inline)) -> uint16_t * { return (par == 0 ? KV0 : KV1) + KSZ; };
     __shared__ int rows_s[2][BN];
@@ -213,7 +215,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     // fp16 caches up to D = 128: the denominators ride on the matrix cores (lacc = ones . P^T sums the
     // same rounded probabilities the numerator uses; all 16 rows of the block hold the same sums).
     // D = 256 has no registers to spare, and bf16 keeps float32 denominators.
-    constexpr bool LM = D <= 128 && DT == 0 && KVHIP_PREFILL_LM;
+    constexpr bool LM = DK <= 128 && DV <= 128 && DT == 0 && KVHIP_PREFILL_LM;
     const bool flip = a.scale < 0.f;
     const float sl2 = fmaxf(fabsf(a.scale) * LOG2E, 1e-30f);
     const float ef = MM == 2 ? 1.f : sl2;
@@ -230,10 +232,10 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         q_l[qt] = q_ok[qt] ? i - rep * a.L : 0;
         q_h[qt] = hk * r + rep;
         const u4 *qp = reinterpret_cast<const u4 *>(
-            reinterpret_cast<const uint16_t *>(a.q) + ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D + 8 * jj);
+            reinterpret_cast<const uint16_t *>(a.q) + ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * DK + 8 * jj);
 #pragma unroll
         for (int s = 0; s < S; ++s) {
-            u4 w = (q_ok[qt] && (D % 32 == 0 || 32 * s + 8 * jj < D)) ? qp[4 * s] : u4{0, 0, 0, 0};
+            u4 w = (q_ok[qt] && (DK % 32 == 0 || 32 * s + 8 * jj < DK)) ? qp[4 * s] : u4{0, 0, 0, 0};
             if (flip) w ^= u4{0x80008000u, 0x80008000u, 0x80008000u, 0x80008000u};
             qop[qt][s].v = w;
         }
@@ -382,20 +384,21 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
     // lane cover the eight tokens of one V chunk (so K operand reads are contiguous across lanes and P
     // never moves), and V slots are the page's own order.
     // A tile of 32 slots inside its page cell (16-bit elements): the 64-token tile t64 starts at
-    // t64 * 64 * D * 2 bytes in both planes; its K chunk (cc, token) lies at (cc * 64 + token) * 16, its
-    // V chunk (8-token chunk tc, column) at (tc * D + column) * 16.
+    // t64 * 64 * DK * 2 bytes in the K plane and t64 * 64 * DV * 2 in the V plane; its K chunk (cc, token) lies at
+    // (cc * 64 + token) * 16, its V chunk (8-token chunk tc, column) at (tc * DV + column) * 16.
     const size_t cell_k = (size_t)bh * st.k_cell, cell_v = (size_t)bh * st.v_cell;
     PageCursor page_k(st, min(vt_of(v_lo) * BN, max(a.slots - 1, 0))), page_v = page_k;
     // the lane's byte offsets inside a tile, one per round of 256 chunks
-    uint32_t koff[NC], voff[NC];
+    uint32_t koff[NCK], voff[NCV];
 #pragma unroll
-    for (int e = 0; e < NC; ++e) {
-        const int c = min(e * 256 + tid, CH - 1);
+    for (int e = 0; e < NCK; ++e) {
+        const int c = min(e * 256 + tid, CHK - 1);
         const int pos = c % BN;
         const int tok = 8 * ((pos & 15) >> 2) + 4 * (pos >> 4) + (pos & 3);
         koff[e] = (uint32_t)((c / BN) * (TILE * 16) + tok * 16);
-        voff[e] = (uint32_t)(c * 16);
     }
+#pragma unroll
+    for (int e = 0; e < NCV; ++e) voff[e] = (uint32_t)(min(e * 256 + tid, CHV - 1) * 16);
     auto dma_k = [&](int tile, int par) __attribute__((always_inline)) {
         const int slot0 = tile * BN;
         if (wave == (tile & 3) && lane < BN) {  // the wavefronts take this in turn
@@ -410,22 +413,22 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
             if (lane == 0) full_s[par] = full;
         }
         const int t = slot0 & (PAGE - 1);
-        const char *kbase = page_k.at(st, slot0).k + cell_k + (size_t)(t >> 6) * (TILE * D * 2) + (t & 63) * 16;
+        const char *kbase = page_k.at(st, slot0).k + cell_k + (size_t)(t >> 6) * (TILE * DK * 2) + (t & 63) * 16;
 #pragma unroll
-        for (int e = 0; e < NC; ++e) {
+        for (int e = 0; e < NCK; ++e) {
             // whole rounds differ by a constant, which goes to the scalar base; a partly empty last
             // round (its tail repeats the tile's last chunk) keeps its own lane offsets
-            if (D % 64 == 0) load_to_lds(kbase + e * 8 * (TILE * 16), koff[0], &Ks(par)[(e * 256 + 64 * wave) * 8]);
+            if (DK % 64 == 0) load_to_lds(kbase + e * 8 * (TILE * 16), koff[0], &Ks(par)[(e * 256 + 64 * wave) * 8]);
             else load_to_lds(kbase, koff[e], &Ks(par)[(e * 256 + 64 * wave) * 8]);
         }
     };
     auto dma_v = [&](int tile, int par) __attribute__((always_inline)) {
         const int slot0 = tile * BN;
         const int t = slot0 & (PAGE - 1);
-        const char *vbase = page_v.at(st, slot0).v + cell_v + (size_t)(t >> 6) * (TILE * D * 2) + ((t & 63) >> 3) * (D * 16);
+        const char *vbase = page_v.at(st, slot0).v + cell_v + (size_t)(t >> 6) * (TILE * DV * 2) + ((t & 63) >> 3) * (DV * 16);
 #pragma unroll
-        for (int e = 0; e < NC; ++e) {
-            if (D % 64 == 0) load_to_lds(vbase + e * 256 * 16, voff[0], &Vs(par)[(e * 256 + 64 * wave) * 8]);
+        for (int e = 0; e < NCV; ++e) {
+            if (DV % 64 == 0) load_to_lds(vbase + e * 256 * 16, voff[0], &Vs(par)[(e * 256 + 64 * wave) * 8]);
             else load_to_lds(vbase, voff[e], &Vs(par)[(e * 256 + 64 * wave) * 8]);
         }
     };
@@ -619,7 +622,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
 #pragma unroll
             for (int x = 0; x < VG; ++x)
                 if (VG * g + x < NDT)  // tokens 8 jj .. 8 jj + 7 of column 16 (VG g + x) + n: one chunk
-                    dst[x].v = *reinterpret_cast<const u4 *>(&Vs(PAR)[(jj * D + 16 * (VG * g + x) + n) * 8]);
+                    dst[x].v = *reinterpret_cast<const u4 *>(&Vs(PAR)[(jj * DV + 16 * (VG * g + x) + n) * 8]);
         };
         if constexpr (HAS_NEXT) {
             constexpr int NM = 2 * S * QT;  // matrix-core instructions of the next tile's scores
@@ -784,17 +787,17 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         if (!q_ok[qt]) continue;
         if (nsplit > 1) {
             const int i = row0 + 16 * qt + n;
-            float *part = a.workspace + (((size_t)bh * nsplit + split) * R + i) * (D + 2);
+            float *part = a.workspace + (((size_t)bh * nsplit + split) * R + i) * (DV + 2);
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<f4 *>(part + 16 * dt + 4 * jj) = oacc[qt][dt];
             if (jj == 0) {
-                part[D] = m_run[qt] * 0.6931471805599453f;  // back from the log2 domain
-                part[D + 1] = l;
+                part[DV] = m_run[qt] * 0.6931471805599453f;  // back from the log2 domain
+                part[DV + 1] = l;
             }
             continue;
         }
         const float inv = l > 0.f ? 1.0f / l : 0.f;
-        const size_t ooff = ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D;
+        const size_t ooff = ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * DV;
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) {
             const float o0 = oacc[qt][dt][0] * inv, o1 = oacc[qt][dt][1] * inv;
@@ -821,17 +824,18 @@ hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, 
     dim3 grid((unsigned)((R + bm - 1) / bm) * st.BH * nsplit), block(256);  // linear: the kernel maps ids to tiles
     const bool ident = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
     const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
-#define PF_M(D, DT, QT, MM)                                                                                   \
+#define PF_M(DK, DV, DT, QT, MM)                                                                                   \
     do {                                                                                                      \
-        if (ident) hipLaunchKernelGGL((prefill_fp_kernel<D, DT, true, QT, MM>), grid, block, 0, s, a, nsplit);  \
-        else hipLaunchKernelGGL((prefill_fp_kernel<D, DT, false, QT, MM>), grid, block, 0, s, a, nsplit);       \
+        if (ident) hipLaunchKernelGGL((prefill_fp_kernel<DK, DV, DT, true, QT, MM>), grid, block, 0, s, a, nsplit);  \
+        else hipLaunchKernelGGL((prefill_fp_kernel<DK, DV, DT, false, QT, MM>), grid, block, 0, s, a, nsplit);       \
     } while (0)
-#define PF(D, DT, QT)                        \
+#define PF2(DK, DV, DT, QT)                        \
     do {                                     \
-        if (mm == 0) PF_M(D, DT, QT, 0);     \
-        else if (mm == 1) PF_M(D, DT, QT, 1); \
-        else PF_M(D, DT, QT, 2);             \
+        if (mm == 0) PF_M(DK, DV, DT, QT, 0);     \
+        else if (mm == 1) PF_M(DK, DV, DT, QT, 1); \
+        else PF_M(DK, DV, DT, QT, 2);             \
     } while (0)
+#define PF(D, DT, QT) PF2(D, D, DT, QT)
 #define PF_QT(D, DT)                 \
     do {                             \
         if (wide) PF(D, DT, 2);      \
@@ -842,7 +846,11 @@ hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, 
         if (st.dtype == KVHIP_F16) PF_QT(D, 0);   \
         else PF_QT(D, 1);                         \
     } while (0)
-    if (st.Dk == 64) PF_DT(64);
+    // keys of 192 with values of 128 (multi-head latent attention): 64 query rows per workgroup
+    if (st.Dk == 192 && st.Dv == 128) {
+        if (st.dtype == KVHIP_F16) PF2(192, 128, 0, 1);
+        else PF2(192, 128, 1, 1);
+    } else if (st.Dk == 64) PF_DT(64);
     else if (st.Dk == 80) PF_DT(80);
     else if (st.Dk == 96) PF_DT(96);
     else if (st.Dk == 128) PF_DT(128);
@@ -851,6 +859,7 @@ hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, 
 #undef PF_DT
 #undef PF_QT
 #undef PF
+#undef PF2
 #undef PF_M
     return hipGetLastError();
 }

@@ -175,7 +175,7 @@ def test_quantized_causal_close_to_full_precision(policy, r):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("Dk,Dv,r", [(128, 128, 4), (64, 32, 1), (256, 256, 2), (80, 80, 2), (96, 96, 4), (96, 96, 1)])
+@pytest.mark.parametrize("Dk,Dv,r", [(128, 128, 4), (64, 32, 1), (256, 256, 2), (80, 80, 2), (96, 96, 4), (96, 96, 1), (192, 128, 1), (192, 128, 4)])
 def test_simple_cache_attention(policy, dtype, Dk, Dv, r):
     rng = np.random.default_rng(Dk + r)
     B, Hkv = 2, 2
@@ -204,6 +204,36 @@ def test_simple_cache_attention(policy, dtype, Dk, Dv, r):
             addm = torch.where(mask.array, 0.0, -30000.0).to(dtype if dtype != torch.float32 else torch.float32)
             out = c.attend(qd, scale, kvhip.MaskMode.from_array(addm))
             check(out, ref, f"L={Lq} additive array")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_keys_of_192_values_of_128_on_the_prefill_tile(dtype):
+    """The multi-head latent attention models cache keys of 192 (qk_nope 128 + qk_rope 64) and values of
+    128 per head (DeepseekV3.swift:128-156, also DeepseekV2 / GLM4MOELite / MiMoV2Flash): prompt chunks,
+    single-token steps over a key range long enough to be split into parts and merged, and a ring."""
+    rng = np.random.default_rng(192)
+    name, Dk, Dv = NAME[dtype], 192, 128
+    scale = Dk ** -0.5
+    lib = kvhip.load()
+    B, H = 1, 2
+    c, o = kvhip.KVCacheSimple(), O.KVCacheSimple(name)
+    for Lq, mode in [(1100, "causal"), (1, "none"), (400, "causal"), (1, "none"), (5, "causal")]:
+        k, kd = randn(rng, (B, H, Lq, Dk), dtype)
+        v, vd = randn(rng, (B, H, Lq, Dv), dtype)
+        q, qd = randn(rng, (B, H, Lq, Dk), dtype)
+        mask, om = (kvhip.MaskMode.causal(), O.Mask.CAUSAL) if mode == "causal" else (kvhip.MaskMode.none(), O.Mask.NONE)
+        out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
+        assert lib.kvhip_last_attend_kernel() == 3 and tuple(out.shape) == (B, H, Lq, Dv)
+        check(out, O.attention_with_cache_update(q, k, v, o, scale, om, name), f"simple L={Lq}")
+    M = 256
+    c, o = kvhip.RotatingKVCache(M, keep=4), O.RotatingKVCache(M, keep=4, dtype=name)
+    for i, Lq in enumerate([64] * 7 + [1] * 6):
+        k, kd = randn(rng, (2, H, Lq, Dk), dtype)
+        v, vd = randn(rng, (2, H, Lq, Dv), dtype)
+        q, qd = randn(rng, (2, 2 * H, Lq, Dk), dtype)
+        out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, c.make_mask(Lq, M, False))
+        assert lib.kvhip_last_attend_kernel() == 3
+        check(out, O.attention_with_cache_update(q, k, v, o, scale, o.make_mask(Lq, M, False), name), f"ring step {i}")
 
 
 def test_rotating_attention_past_wrap_matches_never_rotated_reference(policy):
