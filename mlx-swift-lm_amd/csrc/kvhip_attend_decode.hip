@@ -1225,7 +1225,7 @@ bool attend_decode_supported(const AttendArgs &a) {
     if (s.Dk == 64) return s.gs == 32 || s.gs == 64;
     if (s.Dk == 96) return s.gs == 32;  // every row count on the 16-row kernel
     if (s.Dk == 128) return s.gs == 32 || s.gs == 64 || s.gs == 128;
-    if (s.Dk == 256) return R <= 4 && (s.gs == 64 || s.gs == 128);  // more rows: the prefill tile
+    if (s.Dk == 256) return s.gs == 64 || s.gs == 128;
     return false;
 }
 

@@ -99,8 +99,9 @@ template <int BITS> __device__ __forceinline__ constexpr int code_of(int p) {
 template <int BITS> __device__ __forceinline__ constexpr bool hi_of(int p) { return BITS == 4 && ((p >> 1) & 1); }
 
 // MM: 0 no mask, 1 index-only mask (causal / window with per-batch bounds), 2 array mask.
+// (8-bit codes at D = 256 take more than 256 registers: one workgroup per CU)
 template <int BITS, int D, int GS, int DT, int MM>
-__global__ void __launch_bounds__(WAVES * 64, 2)
+__global__ void __launch_bounds__(WAVES * 64, (D >= 256 && BITS == 8) ? 1 : 2)
 decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     using CD = Codes<BITS>;
     constexpr int G = D / GS;                    // quantization groups per row
@@ -110,10 +111,10 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     constexpr int VWL = 16 * BITS / 32;          // words per lane and V row: its 16 tokens
     constexpr int VROW = 64 * BITS / 8;          // bytes of one V tile row
     constexpr int RR = 16;
-    // Three or four groups per row (group size 32 at D = 96 / 128): the (scale, bias) pairs of a tile -- 64 tokens
+    // Three or four groups per row (group size 32 at D = 96 / 128, 64 at D = 256), and D = 256 with two: the (scale, bias) pairs of a tile -- 64 tokens
     // x G pairs per side, 2 G registers per token of the lane group if held in registers -- go from global memory
     // straight into LDS one tile ahead and are read from there four tokens at a time when they are used.
-    constexpr bool SB_LDS = G >= 3;
+    constexpr bool SB_LDS = G >= 3 || D >= 256;  // (D = 256: the accumulators alone take 64 registers)
     constexpr int SB_PAD = G == 4 ? 4 : 0;       // words between the 64-word pieces (G = 4: a piece per lane group; keeps the groups' reads on different banks)
     constexpr int SB_JJ = 16 * G + SB_PAD;       // words from one lane group's pairs to the next
     constexpr int SB_WORDS = SB_LDS ? G * (64 + SB_PAD) : 4;
@@ -598,12 +599,14 @@ hipError_t launch_attend_decode16(const AttendArgs &a, int tiles_total, int tile
         if (st.Dk == 64 && st.gs == 32) D16_DT(BITS, 64, 32);        \
         else if (st.Dk == 64) D16_DT(BITS, 64, 64);                  \
         else if (st.Dk == 96) D16_DT(BITS, 96, 32);                  \
+        else if (st.Dk == 256 && st.gs == 64) D16_DT(BITS, 256, 64); \
+        else if (st.Dk == 256) D16_DT(BITS, 256, 128);               \
         else if (st.gs == 32) D16_DT(BITS, 128, 32);                 \
         else if (st.gs == 64) D16_DT(BITS, 128, 64);                 \
         else D16_DT(BITS, 128, 128);                                 \
     } while (0)
-    // (head size 96 only divides by group size 32; D = 256, whose partials exceed a workgroup's LDS, is
-    // sent to the prefill tile by the caller)
+    // (head size 96 only divides by group size 32; D = 256 keeps 66 KB of partials in LDS -- one workgroup per
+    // CU at group size 64, whose instances also need more than 256 registers)
     if (st.bits == 4) D16_Q(4);
     else D16_Q(8);
 #undef D16_Q

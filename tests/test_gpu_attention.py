@@ -135,8 +135,9 @@ def test_quantized_decode_many_pairs(bits, D, gs, B, Hkv, T0):
 @pytest.mark.parametrize("bits,gs", [(4, 64), (8, 64), (4, 128), (8, 128)])
 @pytest.mark.parametrize("B,Hkv,r,T0", [(16, 8, 2, 777), (32, 8, 4, 300), (3, 2, 1, 2100)])
 def test_quantized_decode_head_size_256(dtype, bits, gs, B, Hkv, r, T0):
-    """Head size 256 (four or two groups per row) on the matrix-core decode kernel: one token
-    without a mask, then as many tokens as still make four query rows per kv head under .causal."""
+    """Head size 256 (four or two groups per row) on the matrix-core decode kernels: one token
+    without a mask, as many tokens as still make four query rows per kv head under .causal (the 4-row
+    kernel), then four tokens (up to 16 rows: the 16-row kernel)."""
     rng = np.random.default_rng(B + T0 + bits + gs)
     name, D = NAME[dtype], 256
     c = kvhip.QuantizedKVCache(gs, bits)
@@ -146,7 +147,8 @@ def test_quantized_decode_head_size_256(dtype, bits, gs, B, Hkv, r, T0):
     c.update_quantized(kd, vd, fetch=False)
     o.update_quantized(k, v)
     scale = 1.0 / np.sqrt(D)
-    for Lq, mask, om in ((1, None, O.Mask.NONE), (4 // r, kvhip.MaskMode.causal(), O.Mask.CAUSAL)):
+    for Lq, mask, om in ((1, None, O.Mask.NONE), (4 // r, kvhip.MaskMode.causal(), O.Mask.CAUSAL),
+                         (4, kvhip.MaskMode.causal(), O.Mask.CAUSAL), (3, kvhip.MaskMode.causal(), O.Mask.CAUSAL)):
         k, kd = randn(rng, (B, Hkv, Lq, D), dtype)
         v, vd = randn(rng, (B, Hkv, Lq, D), dtype)
         q, qd = randn(rng, (B, Hkv * r, Lq, D), dtype)
