@@ -188,7 +188,12 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         const int id = blockIdx.x;
         const int BH = st_BH(a);
         if ((BH & 7) == 0) {
-            const int xcd = id & 7, j = id >> 3;
+            const int xcd = id & 7;
+            int j = id >> 3;
+            // A grid of exactly two workgroups per CU is resident all at once and gets no balancing from the
+            // order of the ids.  Under a causal or window mask the two workgroups of a CU -- 32 apart among the
+            // 64 of their XCD -- then take a long and a short query block: the second 32 count backwards.
+            if (MM == 1 && gridDim.x == 512 && (j & 32)) j = 95 - j;
             const int per_pair = nblk * nsplit;
             const int h_local = j / per_pair, rem = j - h_local * per_pair;
             bh = h_local * 8 + xcd;
