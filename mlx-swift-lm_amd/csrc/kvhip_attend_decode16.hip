@@ -115,8 +115,9 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     // x G pairs per side, 2 G registers per token of the lane group if held in registers -- go from global memory
     // straight into LDS one tile ahead and are read from there four tokens at a time when they are used.
     constexpr bool SB_LDS = G >= 3 || D >= 256;  // (D = 256: the accumulators alone take 64 registers)
-    constexpr int SB_PAD = G == 4 ? 4 : 0;       // words between the 64-word pieces (G = 4: a piece per lane group; keeps the groups' reads on different banks)
-    constexpr int SB_JJ = 16 * G + SB_PAD;       // words from one lane group's pairs to the next
+    // words between the 64-word pieces the pairs arrive in (G = 2, 4: no lane group's pairs straddle two pieces;
+    // the gap keeps the four lane groups' reads on different banks)
+    constexpr int SB_PAD = (G == 4 || G == 2) ? 4 : 0;
     constexpr int SB_WORDS = SB_LDS ? G * (64 + SB_PAD) : 4;
     const Store &st = a.st;
     const int lane = threadIdx.x & 63;
@@ -235,7 +236,8 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     };
     // (SB_LDS) the pairs of tokens 4 tb .. 4 tb + 3 of the lane group, `side` 0 K / 1 V: out[i * G + g]
     auto sb_quad = [&](int par, int side, int tb, uint32_t (&out)[4 * G]) __attribute__((always_inline)) {
-        const u4 *p = reinterpret_cast<const u4 *>(&sbuf[wave][par][side][SB_JJ * jj + 4 * G * tb]);
+        const int first = 16 * G * jj;  // the lane group's first word among the tile's 64 G
+        const u4 *p = reinterpret_cast<const u4 *>(&sbuf[wave][par][side][first + SB_PAD * (first >> 6) + 4 * G * tb]);
 #pragma unroll
         for (int e = 0; e < G; ++e) {
             const u4 w = p[e];
@@ -351,10 +353,13 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     };
 
     // ---- running state: lane (n, jj) carries row n; m is equal in the four lanes of a row -------
-    float m_run = -INFINITY, l_part = 0.f, bacc[G];
+    // (float16 caches, 4-bit codes: the probabilities that meet high nibbles are formed already divided by 16
+    // and summed apart -- `l_hi`, `bacc_hi` -- so that no multiply brings them down; they rejoin at the end)
+    constexpr bool SPLIT_HI = DT == 0 && BITS == 4;
+    float m_run = -INFINITY, l_part = 0.f, bacc[G], l_hi = 0.f, bacc_hi[G];
     f4 oacc[NDB];
 #pragma unroll
-    for (int g = 0; g < G; ++g) bacc[g] = 0.f;
+    for (int g = 0; g < G; ++g) bacc[g] = bacc_hi[g] = 0.f;
 #pragma unroll
     for (int db = 0; db < NDB; ++db) oacc[db] = f4{0.f, 0.f, 0.f, 0.f};
     const float fill = finfo_min_dt(DT);
@@ -376,7 +381,10 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 }
             }
         // ---- scores of row n for this lane group's 16 tokens: local token 4 tb + i ---------------
-        float x[16];
+        // (float16 caches keep the rounded scores as float16: the maximum is taken on them and the exponent's
+        // multiply-add reads them directly, so they are never widened one by one)
+        using XT = typename std::conditional<DT == 0, _Float16, float>::type;
+        XT x[16];
 #pragma unroll
         for (int tb = 0; tb < 4; ++tb) {
             uint32_t kq[4 * G];
@@ -393,7 +401,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                     sc_ = __builtin_fmaf(sb_scale<DT>(raw), sacc[tb][g][i], sc_);
                     sb_ = __builtin_fmaf(sb_bias<DT>(raw), qsum[g], sb_);
                 }
-                x[tl] = round_dt<DT>(__builtin_fmaf(sc_, TWO24, sb_));
+                x[tl] = (XT)round_dt<DT>(__builtin_fmaf(sc_, TWO24, sb_));
             }
         }
         if (MM == 2 && a.mask.dtype == KVHIP_BOOL && t.base + (TILE - 1) < a.T) {
@@ -403,12 +411,12 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             if (row_ok) mask_bool_words<4>(a.mask, b, hk * r + row_rep, row_l, t.base + 16 * jj, mw);
 #pragma unroll
             for (int tl = 0; tl < 16; ++tl)
-                if (((mw[tl >> 2] >> (8 * (tl & 3))) & 0xffu) == 0u) x[tl] = fill;
+                if (((mw[tl >> 2] >> (8 * (tl & 3))) & 0xffu) == 0u) x[tl] = (XT)fill;
         } else if (MM == 2 || t.base < full_lo || t.base + (TILE - 1) > full_hi) {  // wave-uniform: edge tile
 #pragma unroll
             for (int tl = 0; tl < 16; ++tl) {
                 const int row = t.base + 16 * jj + tl;  // slots are presented rows
-                float s_ = x[tl];
+                float s_ = (float)x[tl];
                 if (row < a.T) {
                     if constexpr (MM == 1) {
                         if (!sym_mask_keep(sym, row_l, row)) s_ = fill;
@@ -423,12 +431,13 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 } else {
                     s_ = -INFINITY;
                 }
-                x[tl] = s_;
+                x[tl] = (XT)s_;
             }
         }
-        float tmax = x[0];
+        XT xmax = x[0];
 #pragma unroll
-        for (int tl = 1; tl < 16; ++tl) tmax = fmaxf(tmax, x[tl]);
+        for (int tl = 1; tl < 16; ++tl) xmax = x[tl] > xmax ? x[tl] : xmax;
+        float tmax = (float)xmax;
         // raise the row maximum only when some lane's own maximum exceeds it (rare after the
         // first tiles); it stays equal in the four lanes of a row
         if (__any(tmax > m_run)) {
@@ -438,14 +447,19 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             const float alpha = (mn == -INFINITY) ? 1.f : fast_exp2((m_run - mn) * LOG2E);
             m_run = mn;
             l_part *= alpha;
+            l_hi *= alpha;
 #pragma unroll
-            for (int g = 0; g < G; ++g) bacc[g] *= alpha;
+            for (int g = 0; g < G; ++g) {
+                bacc[g] *= alpha;
+                bacc_hi[g] *= alpha;
+            }
 #pragma unroll
             for (int db = 0; db < NDB; ++db)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) oacc[db][i] *= alpha;
         }
         const float mu = (m_run == -INFINITY) ? 0.f : m_run;
+        const float nmu = -mu * LOG2E;  // (float16: |mu| <= 65504, the product is finite)
         float pv[G][16];
 #pragma unroll
         for (int tb = 0; tb < 4; ++tb) {
@@ -454,16 +468,28 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int tl = 4 * tb + i;
-                // (the difference first: a masked score is finfo(T).min, whose product with log2 e overflows for bfloat16)
-                const float p = fast_exp2((x[tl] - mu) * LOG2E);  // exp2(-inf) = 0 for dead slots
-                l_part += p;
                 // positions 2, 3, 6, 7 of a 4-bit operand meet high nibbles (x16)
-                const float ps = hi_of<BITS>(tl & 7) ? p * 0.0625f : p;
+                const bool hi = hi_of<BITS>(tl & 7);
+                float p, ps;
+                if constexpr (DT == 0) {
+                    // one multiply-add on the float16 score; exp2(-inf) = 0 for dead slots
+                    ps = fast_exp2(__builtin_fmaf((float)x[tl], LOG2E, (SPLIT_HI && hi) ? nmu - 4.f : nmu));
+                    p = ps;
+                } else {
+                    // (the difference first: a masked score is finfo(T).min, whose product with log2 e overflows for bfloat16)
+                    p = fast_exp2((x[tl] - mu) * LOG2E);
+                    ps = hi ? p * 0.0625f : p;
+                }
+                if (SPLIT_HI && hi) l_hi += p;
+                else l_part += p;
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
                     const uint32_t raw = SB_LDS ? vq[i * G + g] : t.vsb[SB_LDS ? 0 : tl][g];
-                    bacc[g] = __builtin_fmaf(p, sb_bias<DT>(raw), bacc[g]);
-                    pv[g][tl] = ps * sb_scale<DT>(raw);
+                    if (SPLIT_HI && hi) bacc_hi[g] = __builtin_fmaf(p, sb_bias<DT>(raw), bacc_hi[g]);
+                    else bacc[g] = __builtin_fmaf(p, sb_bias<DT>(raw), bacc[g]);
+                    // (float16: written as a multiply-add so that the widening of the scale folds into it)
+                    if constexpr (DT == 0) pv[g][tl] = __builtin_fmaf(sb_scale<DT>(raw), ps, 0.f);
+                    else pv[g][tl] = ps * sb_scale<DT>(raw);
                 }
             }
         }
@@ -514,6 +540,11 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     }
 
     // ---- wavefront partial -> LDS: lane (n, jj) holds out^T[d = 16 db + 4 jj + i][row n] ---------
+    if constexpr (SPLIT_HI) {
+        l_part = __builtin_fmaf(l_hi, 16.f, l_part);
+#pragma unroll
+        for (int g = 0; g < G; ++g) bacc[g] = __builtin_fmaf(bacc_hi[g], 16.f, bacc[g]);
+    }
     l_part += __shfl_xor(l_part, 16);
     l_part += __shfl_xor(l_part, 32);
 #pragma unroll
