@@ -77,6 +77,25 @@ def test_quantized_group_size_fallback_survives_the_file(tmp_path):
     assert r.group_size == 32 and r.offset == 5
 
 
+@pytest.mark.parametrize("bits", [3, 5, 6])
+def test_code_widths_that_do_not_divide_32_survive_the_file(tmp_path, bits):
+    # the packed arrays are [.., D * bits / 32] uint32 words of a bit stream; restore order: state, then metaState
+    g = torch.Generator(device="cuda")
+    g.manual_seed(bits)
+    c = kvhip.QuantizedKVCache(32, bits)
+    k = torch.randn(2, 2, 70, 96, generator=g, device="cuda").half()
+    c.update_quantized(k, k.flip(-1), fetch=False)
+    assert tuple(c.state[0].shape) == (2, 2, 70, 96 * bits // 32)
+    url = tmp_path / "q.safetensors"
+    kvhip.save_prompt_cache(url, [c])
+    (r,), _ = kvhip.load_prompt_cache(url)
+    assert r.bits == bits and r.group_size == 32 and r.offset == 70 and r.meta_state == c.meta_state
+    for a, b in zip(r.state, c.state):
+        assert torch.equal(a, b)
+    q = torch.randn(2, 4, 1, 96, generator=g, device="cuda").half()
+    assert torch.equal(r.attend(q, 96 ** -0.5), c.attend(q, 96 ** -0.5))
+
+
 def write_fixture(path, class_name, array_count, metadata, shape=(1, 1, 1, 1)):
     # the fixture writer of KVCacheTests.swift:31-46
     arrays = {f"0.{i}": torch.zeros(shape, dtype=torch.float32) for i in range(array_count)}
