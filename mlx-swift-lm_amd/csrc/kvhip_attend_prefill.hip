@@ -43,6 +43,22 @@ __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ uint16_t h_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
 __device__ __forceinline__ uint32_t h2_bits(float lo, float hi) { return pk_h2(lo, hi); }
 
+// Codes become float16 values without an integer-to-float conversion: a code OR-ed into the mantissa of a
+// float16 constant (1024 for bits 0..9 of the mantissa, 64 for a nibble at bits 4..7) is that constant plus the
+// code, exactly; subtracting the constant leaves the code, and one packed multiply-add applies scale and bias
+// to two codes at a time (a single rounding to float16, which is what the tile holds in LDS anyway).
+__device__ __forceinline__ uint32_t deq_pair(uint32_t masked_or_magic, kv_h2 magic, kv_h2 sc, kv_h2 bi) {
+    kv_h2 x = __builtin_bit_cast(kv_h2, masked_or_magic);
+    x = x - magic;
+    x = __builtin_elementwise_fma(x, sc, bi);
+    return __builtin_bit_cast(uint32_t, x);
+}
+// position p of an aligned run of 8 codes of a K row in LDS holds code K_PERM<BITS>(p) of the run: the order in
+// which the masked words above yield their pairs; the query operands are permuted the same way
+template <int BITS> __device__ __forceinline__ constexpr int k_perm(int p) {
+    return BITS == 4 ? ((p >> 1) + 4 * (p & 1)) : ((p & 4) | ((p & 2) >> 1) | ((p & 1) << 1));
+}
+
 // BITS 0: full precision (DT 0 fp16 / 1 bf16); 4 / 8: quantized (scales of dtype DT).
 // QT = 16-row query tiles per wavefront (2: 128 rows per workgroup, 1: 64 rows, chosen by
 // the launcher so that the grid fills the chip).  MM: 0 no mask, 1 index-only mask
@@ -60,7 +76,7 @@ prefill_kernel(AttendArgs a, int nsplit) {
     __shared__ __attribute__((aligned(16))) _Float16 Vs[D * VS];
     __shared__ int rows_s[BN];
     __shared__ int tile_full_s;
-    __shared__ float sb_s[BN * 2 * (D / 32)];  // V (scale, bias) per token and group
+    __shared__ __attribute__((aligned(16))) _Float16 sb_s[(D / 32) * 2 * BN];  // V scales and biases: [group][scale, bias][token]
 
     const Store &st = a.st;
     const int tid = threadIdx.x;
@@ -115,15 +131,18 @@ prefill_kernel(AttendArgs a, int nsplit) {
         for (int s = 0; s < S; ++s) raw[s] = qp[4 * s];
 #pragma unroll
         for (int s = 0; s < S; ++s) {
+            float qv[8];
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
                 const uint32_t pair = raw[s][w];
                 float v0 = DT == 0 ? (float)__builtin_bit_cast(_Float16, (uint16_t)pair) : __uint_as_float(pair << 16);
                 float v1 = DT == 0 ? (float)__builtin_bit_cast(_Float16, (uint16_t)(pair >> 16)) : __uint_as_float(pair & 0xffff0000u);
-                v0 = q_ok[qt] ? round_dt<DT>(v0 * a.scale) : 0.f;  // the reference rounds q * scale to T
-                v1 = q_ok[qt] ? round_dt<DT>(v1 * a.scale) : 0.f;
-                qop[qt][s].u[w] = h2_bits(v0, v1);
+                qv[2 * w] = q_ok[qt] ? round_dt<DT>(v0 * a.scale) : 0.f;  // the reference rounds q * scale to T
+                qv[2 * w + 1] = q_ok[qt] ? round_dt<DT>(v1 * a.scale) : 0.f;
             }
+            // (the contraction order inside a run of 8 follows the staged K rows)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) qop[qt][s].u[w] = h2_bits(qv[k_perm<BITS>(2 * w)], qv[k_perm<BITS>(2 * w + 1)]);
         }
     }
 
@@ -260,6 +279,7 @@ prefill_kernel(AttendArgs a, int nsplit) {
             if (lane == 0) tile_full_s = full;
         }
         constexpr int per = 32 / BB;
+        const kv_h2 m1024 = kv_h2{(_Float16)1024.f, (_Float16)1024.f}, m64 = kv_h2{(_Float16)64.f, (_Float16)64.f};
         if (k_on) {
             float sc, bi, sc_hi = 0.f, bi_hi = 0.f;
             sb_pair(ksb_raw, sc, bi);
@@ -268,21 +288,31 @@ prefill_kernel(AttendArgs a, int nsplit) {
                 sb_pair(ksb_raw_hi, sc_hi, bi_hi);
                 g_lo = (kpart * CPT) / st.gs;
             }
+            const kv_h2 s_lo = kv_h2{(_Float16)sc, (_Float16)sc}, b_lo = kv_h2{(_Float16)bi, (_Float16)bi};
+            [[maybe_unused]] const kv_h2 s_hi = kv_h2{(_Float16)sc_hi, (_Float16)sc_hi}, b_hi = kv_h2{(_Float16)bi_hi, (_Float16)bi_hi};
             _Float16 *dst = Ks + kt * KS + kpart * CPT;
 #pragma unroll
             for (int e = 0; e < KQW; ++e) {
-                float s_ = sc, b_ = bi;
+                kv_h2 s_ = s_lo, b_ = b_lo;
                 if constexpr (KT != 8) {  // a packed word lies in one group (32 is a multiple of the codes per word)
                     if ((kpart * CPT + e * per) / st.gs != g_lo) {
-                        s_ = sc_hi;
-                        b_ = bi_hi;
+                        s_ = s_hi;
+                        b_ = b_hi;
                     }
                 }
-#pragma unroll
-                for (int x = 0; x < per; x += 2) {
-                    const float c0 = (float)((kq[e] >> (x * BB)) & ((1u << BB) - 1u));
-                    const float c1 = (float)((kq[e] >> ((x + 1) * BB)) & ((1u << BB) - 1u));
-                    *reinterpret_cast<uint32_t *>(dst + e * per + x) = h2_bits(s_ * c0 + b_, s_ * c1 + b_);
+                const uint32_t w = kq[e];
+                if constexpr (BB == 4) {  // codes (0,4) (1,5) (2,6) (3,7) of the word's 8
+                    u4 o;
+                    o.x = deq_pair((w & 0x000f000fu) | 0x64006400u, m1024, s_, b_);
+                    o.y = deq_pair((w & 0x00f000f0u) | 0x54005400u, m64, s_, b_);
+                    o.z = deq_pair(((w >> 8) & 0x000f000fu) | 0x64006400u, m1024, s_, b_);
+                    o.w = deq_pair(((w >> 8) & 0x00f000f0u) | 0x54005400u, m64, s_, b_);
+                    *reinterpret_cast<u4 *>(dst + e * 8) = o;
+                } else {  // codes (0,2) (1,3) of the word's 4
+                    uint2 o;
+                    o.x = deq_pair((w & 0x00ff00ffu) | 0x64006400u, m1024, s_, b_);
+                    o.y = deq_pair(((w >> 8) & 0x00ff00ffu) | 0x64006400u, m1024, s_, b_);
+                    *reinterpret_cast<uint2 *>(dst + e * 4) = o;
                 }
             }
         }
@@ -292,32 +322,47 @@ prefill_kernel(AttendArgs a, int nsplit) {
                 if (gg < D / st.gs) {
                     float s2, b2;
                     sb_pair(vsb_raw[gg], s2, b2);
-                    sb_s[(tid * 2) * (D / 32) + gg] = s2;
-                    sb_s[(tid * 2 + 1) * (D / 32) + gg] = b2;
+                    sb_s[(gg * 2) * BN + tid] = (_Float16)s2;
+                    sb_s[(gg * 2 + 1) * BN + tid] = (_Float16)b2;
                 }
         }
     
     };
     auto stage_v = [&]() {
+        const kv_h2 m1024 = kv_h2{(_Float16)1024.f, (_Float16)1024.f}, m64 = kv_h2{(_Float16)64.f, (_Float16)64.f};
 #pragma unroll
         for (int ci = 0; ci < VCOLS; ++ci) {
             const int c = tid + 256 * ci;
             if (c < 2 * D) {
                 const int d = c >> 1, part = c & 1;
-                _Float16 *dst = Vs + d * VS + part * 16;
+                uint32_t *dst = reinterpret_cast<uint32_t *>(Vs + d * VS + part * 16);
                 const int g = d / st.gs;
-                // token tt of the 16 sits at code position p(tt) of its word (V tile order)
+                // the 16 tokens' scales and biases, two tokens per word
+                const u4 *sp = reinterpret_cast<const u4 *>(sb_s + (g * 2) * BN + part * 16);
+                const u4 *bp = reinterpret_cast<const u4 *>(sb_s + (g * 2 + 1) * BN + part * 16);
+                const u4 sA = sp[0], sB = sp[1], bA = bp[0], bB = bp[1];
+                const uint32_t sw[8] = {sA.x, sA.y, sA.z, sA.w, sB.x, sB.y, sB.z, sB.w};
+                const uint32_t bw[8] = {bA.x, bA.y, bA.z, bA.w, bB.x, bB.y, bB.z, bB.w};
+                auto S2 = [&](int tp) { return __builtin_bit_cast(kv_h2, sw[tp]); };
+                auto B2 = [&](int tp) { return __builtin_bit_cast(kv_h2, bw[tp]); };
+                // a word of a V tile row yields its tokens two at a time in token order (V tile order)
+                if constexpr (BB == 4) {
 #pragma unroll
-                for (int tt = 0; tt < 16; tt += 2) {
-                    const int bp0 = v_bitpos<BB>(tt), bp1 = v_bitpos<BB>(tt + 1);
-                    const float c0 = (float)((vq[ci * VQW + (bp0 >> 5)] >> (bp0 & 31)) & ((1u << BB) - 1u));
-                    const float c1 = (float)((vq[ci * VQW + (bp1 >> 5)] >> (bp1 & 31)) & ((1u << BB) - 1u));
-                    const int t0 = part * 16 + tt;
-                    const float v0 = sb_s[(t0 * 2) * (D / 32) + g] * c0 + sb_s[(t0 * 2 + 1) * (D / 32) + g];
-                    const float v1 = sb_s[((t0 + 1) * 2) * (D / 32) + g] * c1 + sb_s[((t0 + 1) * 2 + 1) * (D / 32) + g];
-                    *reinterpret_cast<uint32_t *>(dst + tt) = h2_bits(v0, v1);
+                    for (int e = 0; e < 2; ++e) {  // 8 tokens per word
+                        const uint32_t w = vq[ci * VQW + e];
+                        dst[4 * e] = deq_pair((w & 0x000f000fu) | 0x64006400u, m1024, S2(4 * e), B2(4 * e));
+                        dst[4 * e + 1] = deq_pair((w & 0x00f000f0u) | 0x54005400u, m64, S2(4 * e + 1), B2(4 * e + 1));
+                        dst[4 * e + 2] = deq_pair(((w >> 8) & 0x000f000fu) | 0x64006400u, m1024, S2(4 * e + 2), B2(4 * e + 2));
+                        dst[4 * e + 3] = deq_pair(((w >> 8) & 0x00f000f0u) | 0x54005400u, m64, S2(4 * e + 3), B2(4 * e + 3));
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {  // 4 tokens per word
+                        const uint32_t w = vq[ci * VQW + e];
+                        dst[2 * e] = deq_pair((w & 0x00ff00ffu) | 0x64006400u, m1024, S2(2 * e), B2(2 * e));
+                        dst[2 * e + 1] = deq_pair(((w >> 8) & 0x00ff00ffu) | 0x64006400u, m1024, S2(2 * e + 1), B2(2 * e + 1));
+                    }
                 }
-            
             }
         }
     };
