@@ -60,7 +60,7 @@ def main():
                     help="cfg3 (default) is the configuration the metric is quoted on; the others are the "
                          "remaining BASELINE.json configs (reported as one JSON object each)")
     ap.add_argument("--prefill-shape", default=None,
-                    help="with --workload prefill: one shape B,Hq,Hkv,D,L,T,dtype (dtype f16 or bf16) instead of the table")
+                    help="with --workload prefill: one shape B,Hq,Hkv,D,L,T,dtype (dtype f16, bf16, q4 or q8; D may be 192/128) instead of the table")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy 4 times (reference point for rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -279,37 +279,47 @@ def other_workload(args, torch, kvhip, L, dev):
 
     if args.workload == "prefill":
         # the chunked-prefill tile on its own: L new rows attending causally over T cached keys (the new rows
-        # included), KVCacheSimple; flops = 4 * B * Hq * D * (keys each row sees)
+        # included); flops = 2 * B * Hq * (Dk + Dv) * (keys each row sees)
+        # dtype field: f16 / bf16 full precision; q4 / q8 a float16 QuantizedKVCache (group 64; 32 at D 96);
+        # a head size "192/128" is keys of 192 with values of 128
         shapes = [(1, 32, 8, 128, 2048, 8192, "f16"), (1, 32, 8, 128, 2048, 8192, "bf16"), (4, 32, 8, 128, 512, 4096, "f16"),
                   (1, 32, 8, 128, 4096, 4096, "f16"), (2, 16, 4, 64, 2048, 4096, "f16"), (4, 8, 4, 256, 512, 4608, "f16"),
-                  (4, 8, 4, 256, 512, 4608, "bf16")]
+                  (4, 8, 4, 256, 512, 4608, "bf16"), (1, 16, 16, "192/128", 2048, 8192, "f16"),
+                  (1, 16, 16, "192/128", 2048, 8192, "bf16"), (1, 32, 8, 128, 2048, 8192, "q4"), (1, 32, 8, 128, 2048, 8192, "q8"),
+                  (4, 16, 4, 64, 2048, 4096, "q8"), (4, 8, 4, 256, 512, 4608, "q4"), (1, 32, 8, 96, 2048, 8192, "q4")]
         if args.prefill_shape:
             f = args.prefill_shape.split(",")
-            shapes = [tuple(int(x) for x in f[:6]) + (f[6],)]
+            shapes = [tuple(x if "/" in x else int(x) for x in f[:6]) + (f[6],)]
         rows = []
         for Bn, Hq, Hkv, D, Lq, T, dn in shapes:
-            dtype = torch.float16 if dn == "f16" else torch.bfloat16
-            cache = kvhip.KVCacheSimple()
-            k = torch.randn(Bn, Hkv, T, D, generator=g, device=dev).to(dtype)
-            cache.update(k, k.flip(-1), fetch=False)
-            q = torch.randn(Bn, Hq, Lq, D, generator=g, device=dev).to(dtype)
+            Dk, Dv = (int(x) for x in D.split("/")) if isinstance(D, str) else (D, D)
+            dtype = torch.bfloat16 if dn == "bf16" else torch.float16
+            k = torch.randn(Bn, Hkv, T, Dk, generator=g, device=dev).to(dtype)
+            v = k.flip(-1)[..., :Dv].contiguous()
+            if dn in ("q4", "q8"):
+                cache = kvhip.QuantizedKVCache(64, int(dn[1]))
+                cache.update_quantized(k, v, fetch=False)
+            else:
+                cache = kvhip.KVCacheSimple()
+                cache.update(k, v, fetch=False)
+            q = torch.randn(Bn, Hq, Lq, Dk, generator=g, device=dev).to(dtype)
             mask = kvhip.MaskMode.causal()
             for _ in range(2):
-                cache.attend(q, D ** -0.5, mask)
+                cache.attend(q, Dk ** -0.5, mask)
             torch.cuda.synchronize()
             lib.kvhip_profile_enable(1)
             for _ in range(args.steps if args.steps != 256 else 10):
-                cache.attend(q, D ** -0.5, mask)
+                cache.attend(q, Dk ** -0.5, mask)
             torch.cuda.synchronize()
             lib.kvhip_profile_enable(0)
             ms, n = kernel_ms()
             keys = sum(T - Lq + i + 1 for i in range(Lq))
-            fl = 4.0 * Bn * Hq * keys * D
+            fl = 2.0 * Bn * Hq * keys * (Dk + Dv)
             rows.append({"shape": f"B{Bn} {Hq}q/{Hkv}kv D{D} {dn}, {Lq} new rows over {T} keys, causal", "launches": n,
                          "kernel_ms": round(ms, 4), "TFLOPs": round(fl / ms / 1e9, 1),
                          "frac_of_2.5PF": round(fl / ms / 1e9 / 2500.0, 4)})
-            del cache, k, q
-        return {"workload": "chunked-prefill tile (prefill_fp_kernel) on its own", "results": rows}
+            del cache, k, v, q
+        return {"workload": "chunked-prefill tiles (prefill_fp_kernel, prefill_kernel for quantized caches) on their own", "results": rows}
 
     if args.workload == "cfg1":
         # the reference's own CPU-runnable case: B1, 16q/4kv, D64, fp16, 8-bit g64; prefill 512 under
