@@ -1078,6 +1078,50 @@ combine_kernel(AttendArgs a, int nsplit, int rr, int ragged) {
     if (t < D) Elem<DT>::store(a.out, ((size_t)(b * a.Hq + hk * r + rep) * a.L + l) * D + d, o);
 }
 
+// The same merge for the prefill tiles' key-range parts: many query rows, at most 8 parts.  One wavefront per
+// query row, four rows per workgroup; a lane takes four adjacent columns; no LDS and no barrier (the
+// per-row workgroups above spend their time being launched: 22 us for 16 384 rows of 256 columns).
+template <int D, int DT>
+__global__ void __launch_bounds__(256) combine_rows_kernel(AttendArgs a, int nsplit, int rr) {
+    const int lane = threadIdx.x & 63;
+    const int i = blockIdx.x * 4 + (threadIdx.x >> 6), bh = blockIdx.y;
+    if (i >= rr) return;
+    const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
+    const int r = a.Hq / a.Hkv;
+    const int rep = i / a.L, l = i - rep * a.L;
+    const size_t sstride = (size_t)rr * (D + 2);
+    const float *part = a.workspace + (size_t)bh * nsplit * sstride + (size_t)i * (D + 2);
+    float m[8], w[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        m[s] = s < nsplit ? part[s * sstride + D] : -INFINITY;
+        mx = fmaxf(mx, m[s]);
+    }
+    float den = 0.f;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        w[s] = (m[s] == -INFINITY) ? 0.f : fast_exp2((m[s] - mx) * LOG2E);
+        if (s < nsplit) den += w[s] * part[s * sstride + D + 1];
+    }
+    if (lane >= D / 4) return;
+    float num[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+        if (s < nsplit) {
+            // (a row of partials is 8-byte aligned: D + 2 floats)
+            const float2 p0 = *reinterpret_cast<const float2 *>(part + s * sstride + 4 * lane);
+            const float2 p1 = *reinterpret_cast<const float2 *>(part + s * sstride + 4 * lane + 2);
+            num[0] += w[s] * p0.x;
+            num[1] += w[s] * p0.y;
+            num[2] += w[s] * p1.x;
+            num[3] += w[s] * p1.y;
+        }
+    const size_t ooff = ((size_t)(b * a.Hq + hk * r + rep) * a.L + l) * D + 4 * lane;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) Elem<DT>::store(a.out, ooff + c, den > 0.f ? num[c] / den : 0.f);
+}
+
 struct Plan {
     int tiles_total, tiles_per_wg, nsplit, rg, nw;
 };
@@ -1195,6 +1239,21 @@ hipError_t profile_read(int *launches, double *total_ms) {
 hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s, int ragged) {
     const int R = (a.Hq / a.Hkv) * a.L;
     dim3 grid(R, a.st.BH);
+    if (rows > 16 && !ragged && nsplit <= 8 && rows == R) {  // the prefill tiles' parts
+        dim3 grid4((R + 3) / 4, a.st.BH);
+#define CMBR(D)                                                                                      \
+    do {                                                                                             \
+        if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL((combine_rows_kernel<D, 0>), grid4, dim3(256), 0, s, a, nsplit, rows); \
+        else hipLaunchKernelGGL((combine_rows_kernel<D, 1>), grid4, dim3(256), 0, s, a, nsplit, rows); \
+    } while (0)
+        if (a.st.Dv == 64) CMBR(64);
+        else if (a.st.Dv == 80) CMBR(80);
+        else if (a.st.Dv == 96) CMBR(96);
+        else if (a.st.Dv == 128) CMBR(128);
+        else CMBR(256);
+#undef CMBR
+        return hipGetLastError();
+    }
 #define CMB(D)                                                                                       \
     do {                                                                                             \
         if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL((combine_kernel<D, 0>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows, ragged); \
