@@ -1080,34 +1080,37 @@ combine_kernel(AttendArgs a, int nsplit, int rr, int ragged) {
 
 // The same merge for the prefill tiles' key-range parts: many query rows, at most 8 parts.  One wavefront per
 // query row, four rows per workgroup; a lane takes four adjacent columns; no LDS and no barrier (the
-// per-row workgroups above spend their time being launched: 22 us for 16 384 rows of 256 columns).
+// per-row workgroups above spend their time being launched: 22 us for 16 384 rows of 256 columns).  Decode
+// launches keep the kernel above: with few rows and many parts it has the loads of a column in flight together
+// (configs[3]'s ring decode, 2 rows of 16 parts: 29.1 us per step against 31.7 us with this one).
 template <int D, int DT>
 __global__ void __launch_bounds__(256) combine_rows_kernel(AttendArgs a, int nsplit, int rr) {
     const int lane = threadIdx.x & 63;
     const int i = blockIdx.x * 4 + (threadIdx.x >> 6), bh = blockIdx.y;
-    if (i >= rr) return;
-    const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
     const int r = a.Hq / a.Hkv;
+    if (i >= r * a.L) return;  // (rr, the rows a part holds, may exceed the query rows there are)
+    const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
     const int rep = i / a.L, l = i - rep * a.L;
     const size_t sstride = (size_t)rr * (D + 2);
     const float *part = a.workspace + (size_t)bh * nsplit * sstride + (size_t)i * (D + 2);
-    float m[8], w[8];
+    constexpr int MAXP = 8;
+    float m[MAXP], w[MAXP];
     float mx = -INFINITY;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
+    for (int s = 0; s < MAXP; ++s) {
         m[s] = s < nsplit ? part[s * sstride + D] : -INFINITY;
         mx = fmaxf(mx, m[s]);
     }
     float den = 0.f;
 #pragma unroll
-    for (int s = 0; s < 8; ++s) {
+    for (int s = 0; s < MAXP; ++s) {
         w[s] = (m[s] == -INFINITY) ? 0.f : fast_exp2((m[s] - mx) * LOG2E);
         if (s < nsplit) den += w[s] * part[s * sstride + D + 1];
     }
     if (lane >= D / 4) return;
     float num[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int s = 0; s < 8; ++s)
+    for (int s = 0; s < MAXP; ++s)
         if (s < nsplit) {
             // (a row of partials is 8-byte aligned: D + 2 floats)
             const float2 p0 = *reinterpret_cast<const float2 *>(part + s * sstride + 4 * lane);
@@ -1335,7 +1338,7 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
         }                                                                                                 \
         profile_mark(s, false);                                                                           \
         if (p.nsplit > 1)                                                                                 \
-            hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG, 0); \
+            (void)launch_combine(a, p.nsplit, 4 * RG, s, 0);                                             \
     } while (0)
 #define DEC_RG(BITS, D, GS, DT) DEC(BITS, D, GS, DT, 1) /* more rows: the 16-row kernel above */
     if (use_decode16(a_in, p)) {
@@ -1369,7 +1372,7 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
                            p.tiles_per_wg, p.nsplit);                                                     \
         profile_mark(s, false);                                                                           \
         if (p.nsplit > 1)                                                                                 \
-            hipLaunchKernelGGL((combine_kernel<D, DT>), dim3(R, st.BH), dim3(D), 0, s, a, p.nsplit, 4 * RG, 0); \
+            (void)launch_combine(a, p.nsplit, 4 * RG, s, 0);                                             \
     } while (0)
 #define FP_MI(D, DT, RG)                                          \
     do {                                                          \
