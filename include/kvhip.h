@@ -257,7 +257,9 @@ kvhip_status kvhip_cache_attend_static(kvhip_cache *cache, const void *queries, 
                                        int32_t L, int32_t D, float scale, const kvhip_mask *mask,
                                        void *out, void *stream);
 
-/* `attentionWithCacheUpdate` (AttentionUtils.swift:37-95): update, then attend. */
+/* `attentionWithCacheUpdate` (AttentionUtils.swift:37-95): update, then attend.  A single new token without a
+ * mask is written by the decode kernel itself where one of them serves the call (quantized caches up to four
+ * query rows per kv head, 16-bit full-precision caches): the step then has no launch for the append. */
 kvhip_status kvhip_cache_update_attend(kvhip_cache *cache, const void *queries, const void *keys,
                                        const void *values, int32_t B, int32_t Hq, int32_t Hkv,
                                        int32_t L, int32_t Dk, int32_t Dv, int32_t dtype, float scale,

@@ -496,7 +496,10 @@ kvhip_status update_simple(kvhip_cache *c, const void *k, const void *v, int L, 
     return KVHIP_OK;
 }
 
-kvhip_status update_rotating(kvhip_cache *c, const void *k, const void *v, int L, hipStream_t stream) {
+// deferred_slot (single-token steps only): the row is not written here; its physical slot is handed back and
+// the caller sees to the write (the decode kernel takes it along).
+kvhip_status update_rotating(kvhip_cache *c, const void *k, const void *v, int L, hipStream_t stream,
+                             int32_t *deferred_slot = nullptr) {
     const int64_t M = c->max_size;
     if (L == 1) {
         // updateInPlace, KVCache.swift:684-740
@@ -518,7 +521,8 @@ kvhip_status update_rotating(kvhip_cache *c, const void *k, const void *v, int L
             return fail(KVHIP_ERR_STATE, "RotatingKVCache write cursor lies outside its buffer");
         KV_TRY(ring_compact_if_needed(c, stream));
         const int32_t slot = c->rows[(size_t)c->idx];
-        KV_HIP(launch_append_fp(c->st, k, v, 1, 0, slot, 1, stream, c->rope));
+        if (deferred_slot) *deferred_slot = slot;
+        else KV_HIP(launch_append_fp(c->st, k, v, 1, 0, slot, 1, stream, c->rope));
         c->offset += 1;
         c->idx += 1;
         c->presented = c->offset < M ? c->offset : c->ref_len;
@@ -880,12 +884,12 @@ kvhip_status bind_workspace(kvhip_cache *c, AttendArgs &a, size_t need, float *f
     return KVHIP_OK;
 }
 
-// new_k / new_v: the rows of a single-token step whose bookkeeping is done but whose write is
-// still owed (quantized caches); the decode kernel takes them along when it can, else they are
+// new_k / new_v: the rows of a single-token step whose bookkeeping is done but whose write into physical
+// slot `new_slot` is still owed; the decode kernel takes them along when it can, else they are
 // appended by a launch of their own first.
 kvhip_status attend_impl(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, int32_t L, int32_t D, float scale,
                          const kvhip_mask *mask, void *out, void *stream, float *fixed, size_t fixed_bytes,
-                         const void *new_k = nullptr, const void *new_v = nullptr) {
+                         const void *new_k = nullptr, const void *new_v = nullptr, int32_t new_slot = -1) {
     if (!c || !q || !out) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
     const bool staged_view = c->staging && !c->stage_view.empty();
     if (!c->has_geom || (!c->has_buffers && !staged_view) || c->presented <= 0)
@@ -931,8 +935,11 @@ kvhip_status attend_impl(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, i
         if (g_policy == 0 && attend_decode_fuses_append(a)) {
             a.new_k = new_k;
             a.new_v = new_v;
+            a.new_slot = new_slot;
+        } else if (c->st.bits != 0) {
+            KV_HIP(launch_append_quant(c->st, new_k, new_v, 1, 0, new_slot, 1, s, nullptr));
         } else {
-            KV_HIP(launch_append_quant(c->st, new_k, new_v, 1, 0, (int)c->offset - 1, 1, s, nullptr));
+            KV_HIP(launch_append_fp(c->st, new_k, new_v, 1, 0, new_slot, 1, s, nullptr));
         }
     }
     if (g_policy == 0 && attend_decode_supported(a)) {
@@ -976,11 +983,29 @@ kvhip_status kvhip_cache_update_attend(kvhip_cache *c, const void *q, const void
         (dtype == KVHIP_F16 || dtype == KVHIP_BF16) && (!mask || mask->mode == KVHIP_MASK_NONE) && c->has_geom &&
         c->has_buffers && c->B == B && c->Hkv == Hkv && c->st.Dk == Dk && c->st.Dv == Dv && c->st.dtype == dtype) {
         KV_TRY(update_simple(c, k, v, 1, S(c, stream), false));
-        const kvhip_status st = attend_impl(c, q, B, Hq, L, Dk, scale, mask, out, stream, nullptr, 0, k, v);
+        const kvhip_status st = attend_impl(c, q, B, Hq, L, Dk, scale, mask, out, stream, nullptr, 0, k, v, (int32_t)c->offset - 1);
         if (st != KVHIP_OK) {  // nothing was written: take the row back
             c->offset -= 1;
             c->presented = c->offset;
         }
+        return st;
+    }
+    // One new token into a full-precision cache of a 16-bit dtype (KVCacheSimple, or the in-place step of a
+    // RotatingKVCache): the decode kernel copies the row into its slot itself.  The bookkeeping of `update`
+    // runs here as usual; if the attention cannot be enqueued the row is written by the append kernel, so
+    // the cache holds what its counters say.
+    if (c && k && v && q && out && L == 1 && (c->kind == KVHIP_KIND_SIMPLE || c->kind == KVHIP_KIND_ROTATING) &&
+        !c->staging && !c->rope && (dtype == KVHIP_F16 || dtype == KVHIP_BF16) && (!mask || mask->mode == KVHIP_MASK_NONE) &&
+        c->has_geom && c->has_buffers && c->B == B && c->Hkv == Hkv && c->st.Dk == Dk && c->st.Dv == Dv && c->st.dtype == dtype) {
+        int32_t slot = -1;
+        if (c->kind == KVHIP_KIND_SIMPLE) {
+            KV_TRY(update_simple(c, k, v, 1, S(c, stream), false));
+            slot = (int32_t)c->offset - 1;
+        } else {
+            KV_TRY(update_rotating(c, k, v, 1, S(c, stream), &slot));
+        }
+        const kvhip_status st = attend_impl(c, q, B, Hq, L, Dk, scale, mask, out, stream, nullptr, 0, k, v, slot);
+        if (st != KVHIP_OK) (void)launch_append_fp(c->st, k, v, 1, 0, slot, 1, S(c, stream), nullptr);
         return st;
     }
     KV_TRY(kvhip_cache_update(c, k, v, B, Hkv, L, Dk, Dv, dtype, stream));

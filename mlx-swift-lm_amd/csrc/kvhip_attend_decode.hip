@@ -384,7 +384,7 @@ decode_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     // tile see it.  The V code goes into its column's packed word read-modify-write.
     if constexpr (MM == 0 && RG == 1) {
         if (a.new_k != nullptr) {  // wave-uniform
-            const int slot = a.T - 1, tl = slot >> 6;
+            const int slot = a.new_slot, tl = slot >> 6;
             if (tl >= tile_begin && tl < tile_end && ((tl - tile_begin) % NW) == wave) {
                 const char *krow = static_cast<const char *>(a.new_k) + (size_t)bh * D * 2;
                 const char *vrow = static_cast<const char *>(a.new_v) + (size_t)bh * D * 2;
@@ -790,6 +790,27 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     }
     const int tile0 = tile_begin + wave;
     const int my_tiles = tile0 < tile_end ? (tile_end - tile0 + WAVES - 1) / WAVES : 0;
+    // ---- the step's new row, when it is still to be written (unmasked single-token decode) -----
+    // Exactly one wavefront of one workgroup reads the tile of physical slot `new_slot` (spans are equal and
+    // cover every tile): it copies the row into the page before it requests any tile, so its own later
+    // loads of the tile see it.
+    if constexpr (MM == 0) {
+        if (a.new_k != nullptr) {  // wave-uniform
+            const int slot = a.new_slot, tl = slot >> 6;
+            if (tl >= tile_begin && tl < tile_end && ((tl - tile_begin) % WAVES) == wave) {
+                const uint16_t *krow = static_cast<const uint16_t *>(a.new_k) + (size_t)bh * D;
+                const uint16_t *vrow = static_cast<const uint16_t *>(a.new_v) + (size_t)bh * D;
+                char *kc = const_cast<char *>(k_cell_ptr(st, bh, slot));
+                char *vc = const_cast<char *>(v_cell_ptr(st, bh, slot));
+                if (lane < D / 8)  // one 16-byte chunk of the K row per lane
+                    *reinterpret_cast<uint4 *>(kc + kfp_off(st, slot, 8 * lane)) = *reinterpret_cast<const uint4 *>(krow + 8 * lane);
+                for (int d = lane; d < D; d += 64)
+                    *reinterpret_cast<uint16_t *>(vc + vfp_off(st, slot, d)) = vrow[d];
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            }
+        }
+    }
     // a wavefront's tiles are a page apart: each is found through the page table (a scalar load)
     const int tip = tile0 & 3;
     int page_k = my_tiles > 0 ? tile0 >> 2 : 0, page_v = page_k;
@@ -1291,12 +1312,13 @@ bool attend_decode_supported(const AttendArgs &a) {
     return false;
 }
 
-// The 4-row quantized kernel without a mask writes the step's new row itself.
+// The 4-row quantized kernel and the full-precision decode kernel, without a mask, write the step's new row themselves.
 bool attend_decode_fuses_append(const AttendArgs &a) {
-    if (!attend_decode_supported(a) || a.st.bits == 0 || a.L != 1) return false;
-    if ((a.Hq / a.Hkv) * a.L > 4 || a.mask.mode != KVHIP_MASK_NONE || a.st.Dk == 96) return false;
+    if (!attend_decode_supported(a) || a.L != 1 || a.mask.mode != KVHIP_MASK_NONE) return false;
     static const bool off = getenv("KVHIP_NO_FUSED_APPEND") != nullptr;  // measurement aid
-    return !off;
+    if (off) return false;
+    if (a.st.bits == 0) return true;  // the full-precision decode kernel, any of its row counts
+    return (a.Hq / a.Hkv) * a.L <= 4 && a.st.Dk != 96;
 }
 
 // 5..16 rows per kv head of a quantized cache go to the 16x16x32 kernel

@@ -275,14 +275,15 @@ struct AttendArgs {
     MaskDev mask;
     float *workspace = nullptr;
     size_t workspace_bytes = 0;
-    // Single-token decode over a quantized cache (`attentionWithCacheUpdate` with L = 1): the new
-    // row [BH, 1, D] of keys and values, still to be quantized into slot T - 1.  The decode kernel
-    // does it itself -- the wavefront that reads the last tile writes the row first -- so a step is
-    // one launch.  NULL: the row is already in the cache.
+    // Single-token decode (`attentionWithCacheUpdate` with L = 1): the new row [BH, 1, D] of keys and
+    // values, still to be written (quantized caches: quantized) into physical slot `new_slot`.  The decode
+    // kernel does it itself -- the wavefront that reads the slot's tile writes the row first -- so a
+    // step needs no launch for the append.  NULL: the row is already in the cache.
     const void *new_k = nullptr;
     const void *new_v = nullptr;
+    int new_slot = -1;
 };
-// Whether launch_attend_decode quantizes a.new_k / a.new_v itself for these arguments.
+// Whether launch_attend_decode writes a.new_k / a.new_v itself for these arguments.
 bool attend_decode_fuses_append(const AttendArgs &a);
 // Bytes of scratch each kernel family needs for these arguments.
 size_t attend_generic_workspace(const AttendArgs &a);
