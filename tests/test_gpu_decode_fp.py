@@ -7,7 +7,7 @@ import torch
 import kvhip
 from oracle import c_oracle as CO
 from oracle import kv_oracle as O
-from tests.util import NAME, dev, err_stats, np32, randn
+from tests.util import NAME, bits_equal, dev, err_stats, np32, randn
 
 pytestmark = pytest.mark.gpu
 
@@ -102,3 +102,41 @@ def test_rotating_decode_after_wrap(dtype):
         mx, mean = err_stats(np32(out), ref)
         assert mx <= 1e-2 and mean <= 1e-3, (i, mx, mean)
         assert c.meta_state == o.get_meta_state()
+
+
+@pytest.mark.parametrize("dtype,D,B,Hq,Hkv", [(torch.float16, 128, 2, 8, 2), (torch.bfloat16, 64, 1, 4, 4), (torch.bfloat16, 256, 2, 4, 2),
+                                              (torch.float16, 256, 1, 8, 2), (torch.float16, 96, 1, 4, 2)])
+@pytest.mark.parametrize("kind", ["simple", "ring"])
+def test_single_token_steps_write_their_row_inside_the_decode_kernel(kind, dtype, D, B, Hq, Hkv):
+    """`attentionWithCacheUpdate` with one new token and no mask on a 16-bit full-precision cache has no append
+    launch: the decode kernel copies the new row into its slot (KVCacheSimple: the next row; RotatingKVCache: the
+    slot of the in-place step, past the wrap as well).  After every run of steps the cache's state must equal
+    the oracle's bit for bit -- across 64-token tiles, pages, trims and ring wraps -- and every output the
+    oracle's within the bound.  Head size 96 has no decode kernel: there the row goes through the append kernel."""
+    rng = np.random.default_rng(D + B)
+    name = NAME[dtype]
+    if kind == "simple":
+        cache, ocache = kvhip.KVCacheSimple(), O.KVCacheSimple(name)
+    else:
+        cache, ocache = kvhip.RotatingKVCache(300, keep=4), O.RotatingKVCache(300, keep=4, dtype=name)
+    scale = D ** -0.5
+    for start, steps, trim in [(1, 9, 0), (60, 10, 3), (250, 12, 0), (290, 25, 2), (700, 6, 0)]:
+        n = start - ocache.offset
+        if n > 0:
+            k, kd = randn(rng, (B, Hkv, n, D), dtype)
+            v, vd = randn(rng, (B, Hkv, n, D), dtype)
+            cache.update(kd, vd, fetch=False)
+            ocache.update(k, v)
+        for _ in range(steps):
+            q, qd = randn(rng, (B, Hq, 1, D), dtype)
+            k, kd = randn(rng, (B, Hkv, 1, D), dtype)
+            v, vd = randn(rng, (B, Hkv, 1, D), dtype)
+            got = kvhip.attention_with_cache_update(qd, kd, vd, cache, scale)
+            assert kvhip.load().kvhip_last_attend_kernel() == (3 if D == 96 else 2)
+            ref = O.attention_with_cache_update(q, k, v, ocache, scale, O.Mask.NONE, name)
+            mx, mean = err_stats(np32(got), ref)
+            assert mx <= (1e-2 if dtype == torch.float16 else 1.6e-2) and mean <= 1e-3, (ocache.offset, mx, mean)
+            assert cache.offset == ocache.offset and cache.meta_state == ocache.get_meta_state()
+        for a, b in zip(cache.state, ocache.get_state()):
+            assert bits_equal(a, b, dtype), (kind, start)
+        assert cache.trim(trim) == ocache.trim(trim)
