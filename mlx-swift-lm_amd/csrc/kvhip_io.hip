@@ -129,8 +129,10 @@ __device__ __forceinline__ void append_quant_body(const Store &st, const Store &
     const bool partial = ((t_lo * BITS) & 31) != 0 || ((t_hi * BITS) & 31) != 0;  // some word keeps old tokens
     uint32_t old0 = 0;
     if (partial && (int)threadIdx.x < items) old0 = *word_ptr(threadIdx.x);
-    // (row, K or V) pairs go round the four wavefronts, so one new token uses two of them
-    for (int item = wave; item < 2 * (hi - lo); item += 4) {
+    // (row, K or V) pairs go round the wavefronts (four, or eight for appends of three rows and more), so one
+    // new token uses two of them
+    const int nwaves = blockDim.x >> 6;
+    for (int item = wave; item < 2 * (hi - lo); item += nwaves) {
         const int slot = lo + (item >> 1);
         const int l = src0 + (slot - slot0);
         uint32_t *kw = reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot)));
@@ -195,7 +197,7 @@ __device__ __forceinline__ void append_quant_body(const Store &st, const Store &
 // tile rows, touching only the token positions this append writes.
 // (ROPE = false carries no rotation code: the single-token decode append stays as small as it was)
 template <int DT, int BITS, bool ROPE>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(512)
 append_quant_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, int n,
                     RopeDev rope) {
     append_quant_body<DT, BITS, ROPE, false>(st, st, keys, values, L, src0, slot0, n, rope);
@@ -845,7 +847,8 @@ hipError_t launch_append_quant_rows(const Store &st, const void *keys, const voi
                                     int slot0, int n, hipStream_t s, const RopeDev &r) {
     if (n <= 0) return hipSuccess;
     const int ntile = ((slot0 + n - 1) >> 6) - (slot0 >> 6) + 1;
-    dim3 grid(ntile, st.BH), block(256);
+    // (a speculative-verify step appends 4 rows: 8 (row, K or V) items, one per wavefront)
+    dim3 grid(ntile, st.BH), block(n >= 3 ? 512 : 256);
     const size_t lds = (size_t)TILE * st.Dv;
 #define CALL(DT, BITS)                                                                                      \
     do {                                                                                                    \
