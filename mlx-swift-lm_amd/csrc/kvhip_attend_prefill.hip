@@ -93,7 +93,11 @@ prefill_kernel(AttendArgs a, int nsplit) {
         const int id = blockIdx.x;
         const int BH = a.st.BH;
         if ((BH & 7) == 0) {
-            const int xcd = id & 7, j = id >> 3;
+            const int xcd = id & 7;
+            int j = id >> 3;
+            // (a grid of exactly two workgroups per CU under a causal or window mask: the two workgroups of a CU,
+            // 32 apart among the 64 of their XCD, take a long and a short query block)
+            if (MM == 1 && gridDim.x == 512 && (j & 32)) j = 95 - j;
             const int per_pair = nblk * nsplit;
             const int h_local = j / per_pair, rem = j - h_local * per_pair;
             bh = h_local * 8 + xcd;
@@ -106,6 +110,9 @@ prefill_kernel(AttendArgs a, int nsplit) {
             split = t / BH;
         }
     }
+    // Under a causal or window mask the later query blocks see more keys: they get the lower workgroup ids,
+    // which the hardware starts first, so that the launch does not end on its longest blocks.
+    if (MM == 1) blk_x = nblk - 1 - blk_x;
     const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
     const int row0 = blk_x * BM + wave * 16 * QT;  // first query row of this wavefront
     const float fill = finfo_min_dt(DT);
