@@ -115,20 +115,6 @@ template <int DT> __device__ __forceinline__ void mfma_new(f4 &c, const Op8 &a, 
     c = f4{0.f, 0.f, 0.f, 0.f};
     mfma_acc<DT>(c, a, b);
 }
-// The same accumulation for the output accumulators, which live across the whole loop, written as
-// assembly with the accumulator as both input and output.  As a builtin the compiler gave most of
-// these instructions a new destination register, so that the accumulators wandered through the
-// register file and were copied back (36 64-bit moves per query block) at the loop's back edge.
-// What the compiler no longer does for these is insert the wait states between a matrix-core write
-// and a vector-ALU read of the same registers: the only such reads are the rescaling in `raise` and
-// the final normalisation, both of which sit behind a barrier (and cross-lane exchanges) that follow
-// the last of these instructions.  Waits for the LDS data that feed the operands are still inserted
-// by the compiler, which tracks registers, not opcodes.
-template <int DT> __device__ __forceinline__ void mfma_acc_inplace(f4 &c, const Op8 &a, const Op8 &b) {
-    if constexpr (DT == 0) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a.v), "v"(b.v));
-    else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a.v), "v"(b.v));
-}
-
 // D = 256 runs 64 query rows per workgroup only: 128 rows need the accumulator registers of
 // a whole SIMD lane (one wavefront per SIMD), which measured slower (0.34 ms against 0.29 ms
 // for a 512 x 4607 chunk at B4, 8 query heads).
