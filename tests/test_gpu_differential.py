@@ -152,3 +152,42 @@ def test_quantized_shapes_against_generic(seed):
     ulp = float(np.abs(ref).max()) * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10)
     assert d.max() <= max(MAX_ABS, 2 * ulp) and d.mean() <= max(MEAN_ABS, ulp / 4), \
         f"kernel {chosen}: max-abs {d.max():.3e} mean-abs {d.mean():.3e}"
+
+
+@pytest.mark.parametrize("kind,dtype,B,Hkv,L,extra", [
+    ("simple", torch.float16, 1, 8, 2048, 0), ("simple", torch.bfloat16, 2, 8, 1024, 512),
+    ("quantized", torch.float16, 1, 8, 2048, 0), ("quantized", torch.float16, 2, 8, 1024, 300),
+])
+def test_causal_grids_of_two_workgroups_per_cu(kind, dtype, B, Hkv, L, extra):
+    """A causal prompt chunk whose prefill grid is exactly 512 workgroups (4 query heads per kv head, 128 query
+    rows per workgroup): the kernels then pair a long and a short query block on every CU by renumbering the
+    workgroups, which must still hand every query block to exactly one of them -- checked against the generic
+    kernel over the same device cache."""
+    D, r = 128, 4
+    g = torch.Generator(device="cuda")
+    g.manual_seed(B * 1000 + L)
+
+    def rand(*shape):
+        return torch.randn(*shape, generator=g, device="cuda").to(dtype)
+
+    T = L + extra
+    if kind == "simple":
+        c = kvhip.KVCacheSimple()
+        c.update(rand(B, Hkv, T, D), rand(B, Hkv, T, D), fetch=False)
+    else:
+        c = kvhip.QuantizedKVCache(64, 4)
+        c.update_quantized(rand(B, Hkv, T, D), rand(B, Hkv, T, D), fetch=False)
+    assert (r * L // 128) * B * Hkv == 512
+    q = rand(B, Hkv * r, L, D)
+    lib = kvhip.load()
+    try:
+        lib.kvhip_set_kernel_policy(1)
+        ref = np32(c.attend(q, D ** -0.5, kvhip.MaskMode.causal()))
+        lib.kvhip_set_kernel_policy(0)
+        out = np32(c.attend(q, D ** -0.5, kvhip.MaskMode.causal()))
+        assert lib.kvhip_last_attend_kernel() == 3
+    finally:
+        lib.kvhip_set_kernel_policy(0)
+    d = np.abs(out.astype(np.float64) - ref.astype(np.float64))
+    ulp = float(np.abs(ref).max()) * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10)
+    assert np.isfinite(out).all() and d.max() <= max(MAX_ABS, ulp) and d.mean() <= max(MEAN_ABS, ulp / 4), (d.max(), d.mean())
