@@ -229,8 +229,8 @@ kvhip_status kvhip_cache_fetch(const kvhip_cache *cache, void *dst_keys, void *d
  * (KVCache.swift:2351-2447) for quantized ones.
  * queries [B,Hq,L,Dk] and out [B,Hq,L,Dv] in the cache's dtype.
  * Every dtype, bit width, head size, group size and mask is accepted.  The tuned kernels take
- * float16 / bfloat16 caches with Dk == Dv in {64, 96, 128, 256} (also 80, and keys of 192 with values
- * of 128, when not quantized; quantized: 4 or 8 bits, group size 32, 64 or 128); anything else
+ * float16 / bfloat16 caches with Dk == Dv in {64, 96, 128, 256}, keys of 192 with values of 128 (also
+ * 80 when not quantized; quantized: 4 or 8 bits, group size 32, 64 or 128); anything else
  * (float32, 2-, 3-, 5- and 6-bit codes, other head sizes) runs on a plain kernel
  * that is 50-75 times slower at 8k keys.  kvhip_last_attend_kernel() tells which one ran.
  */

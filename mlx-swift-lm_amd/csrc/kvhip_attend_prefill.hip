@@ -63,20 +63,22 @@ template <int BITS> __device__ __forceinline__ constexpr int k_perm(int p) {
 // QT = 16-row query tiles per wavefront (2: 128 rows per workgroup, 1: 64 rows, chosen by
 // the launcher so that the grid fills the chip).  MM: 0 no mask, 1 index-only mask
 // (causal / window, no memory access in the loop), 2 array mask.
-template <int BITS, int D, int DT, bool IDENT, int QT, int MM>
+// DK and DV are the head sizes of keys / queries and of values / outputs (192 and 128 for the multi-head latent
+// attention models, equal otherwise).
+template <int BITS, int DK, int DV, int DT, bool IDENT, int QT, int MM>
 __global__ void __launch_bounds__(256, 2)
 prefill_kernel(AttendArgs a, int nsplit) {
     static_assert(BITS == 4 || BITS == 8, "quantized caches only");
     constexpr int BM = 64 * QT;
-    constexpr int KS = D + 8;    // halves per K row in LDS (padded against bank conflicts)
+    constexpr int KS = DK + 8;   // halves per K row in LDS (padded against bank conflicts)
     constexpr int VS = BN + 4;   // halves per V^T row in LDS
-    constexpr int S = D / 32;    // contraction steps over the head dim
-    constexpr int NDT = D / 16;  // 16-row tiles of out^T
+    constexpr int S = DK / 32;   // contraction steps over the head dim
+    constexpr int NDT = DV / 16; // 16-row tiles of out^T
     __shared__ __attribute__((aligned(16))) _Float16 Ks[BN * KS];
-    __shared__ __attribute__((aligned(16))) _Float16 Vs[D * VS];
+    __shared__ __attribute__((aligned(16))) _Float16 Vs[DV * VS];
     __shared__ int rows_s[BN];
     __shared__ int tile_full_s;
-    __shared__ __attribute__((aligned(16))) _Float16 sb_s[(D / 32) * 2 * BN];  // V scales and biases: [group][scale, bias][token]
+    __shared__ __attribute__((aligned(16))) _Float16 sb_s[(DV / 32) * 2 * BN];  // V scales and biases: [group][scale, bias][token]
 
     const Store &st = a.st;
     const int tid = threadIdx.x;
@@ -132,7 +134,7 @@ prefill_kernel(AttendArgs a, int nsplit) {
         // rows past R read row (rep 0, l 0), which is in bounds, and are zeroed: no branch around the
         // loads, which are one 16-byte piece per contraction step, all in flight together
         const u4 *qp = reinterpret_cast<const u4 *>(
-            reinterpret_cast<const uint16_t *>(a.q) + ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D + 8 * jj);
+            reinterpret_cast<const uint16_t *>(a.q) + ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * DK + 8 * jj);
         u4 raw[S];
 #pragma unroll
         for (int s = 0; s < S; ++s) raw[s] = qp[4 * s];
@@ -214,16 +216,16 @@ prefill_kernel(AttendArgs a, int nsplit) {
     // (in flight while the current tile is contracted), then converted and written to LDS.
     constexpr int BB = BITS;
     // K: KT threads per token row, CPT codes each: 8 threads where that gives whole packed words
-    // (head sizes that are multiples of 64), 4 otherwise (96: 24 codes = 3 or 6 words, which may
+    // (head sizes 64, 128 and 256), 4 otherwise (96 / 192: 24 / 48 codes = whole words, which may
     // straddle two groups of 32)
-    constexpr int KT = (D % 64 == 0) ? 8 : 4;
-    constexpr int CPT = D / KT;
+    constexpr int KT = (DK == 64 || DK == 128 || DK == 256) ? 8 : 4;
+    constexpr int CPT = DK / KT;
     constexpr int KQW = CPT * BB / 32;            // packed words per thread for K
     static_assert((CPT * BB) % 32 == 0, "a thread's K codes are whole packed words");
     constexpr int VQW = 16 * BB / 32;             // packed words per thread and column for V
-    constexpr int VCOLS = (2 * D + 255) / 256;    // (column, half) items per thread for V
+    constexpr int VCOLS = (2 * DV + 255) / 256;    // (column, half) items per thread for V
     uint32_t kq[KQW], vq[VCOLS * VQW], ksb_raw = 0, ksb_raw_hi = 0;
-    uint32_t vsb_raw[D / 32];
+    uint32_t vsb_raw[DV / 32];
     int row_reg = -1;
     const int kt = tid / KT, kpart = tid % KT;
     const bool k_on = KT == 8 || tid < BN * KT;   // with 4 threads per row the upper half has no K work
@@ -254,14 +256,14 @@ prefill_kernel(AttendArgs a, int nsplit) {
         if (tid < BN) {
             const uint32_t *sb = reinterpret_cast<const uint32_t *>(pe.vsb + (size_t)bh * st.vsb_cell + (size_t)(in_page + tid) * st.vsb_row);
 #pragma unroll
-            for (int gg = 0; gg < D / 32; ++gg)
-                if (gg < D / st.gs) vsb_raw[gg] = sb[gg];
+            for (int gg = 0; gg < DV / 32; ++gg)
+                if (gg < DV / st.gs) vsb_raw[gg] = sb[gg];
         }
         const int tbase = slot0 & 32;
 #pragma unroll
         for (int ci = 0; ci < VCOLS; ++ci) {
             const int c = tid + 256 * ci;
-            if (c < 2 * D) {
+            if (c < 2 * DV) {
                 const int d = c >> 1, part = c & 1;
                 const uint32_t *vw = reinterpret_cast<const uint32_t *>(cell + v_row_off(st, slot0, d)) + (tbase + part * 16) * BB / 32;
 #pragma unroll
@@ -325,8 +327,8 @@ prefill_kernel(AttendArgs a, int nsplit) {
         }
         if (tid < BN) {
 #pragma unroll
-            for (int gg = 0; gg < D / 32; ++gg)
-                if (gg < D / st.gs) {
+            for (int gg = 0; gg < DV / 32; ++gg)
+                if (gg < DV / st.gs) {
                     float s2, b2;
                     sb_pair(vsb_raw[gg], s2, b2);
                     sb_s[(gg * 2) * BN + tid] = (_Float16)s2;
@@ -340,7 +342,7 @@ prefill_kernel(AttendArgs a, int nsplit) {
 #pragma unroll
         for (int ci = 0; ci < VCOLS; ++ci) {
             const int c = tid + 256 * ci;
-            if (c < 2 * D) {
+            if (c < 2 * DV) {
                 const int d = c >> 1, part = c & 1;
                 uint32_t *dst = reinterpret_cast<uint32_t *>(Vs + d * VS + part * 16);
                 const int g = d / st.gs;
@@ -520,18 +522,18 @@ prefill_kernel(AttendArgs a, int nsplit) {
         if (!q_ok[qt]) continue;
         if (nsplit > 1) {
             const int i = row0 + 16 * qt + n;
-            float *part = a.workspace + (((size_t)bh * nsplit + split) * R + i) * (D + 2);
+            float *part = a.workspace + (((size_t)bh * nsplit + split) * R + i) * (DV + 2);
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt)
                 *reinterpret_cast<f4 *>(part + 16 * dt + 4 * jj) = oacc[qt][dt];
             if (jj == 0) {
-                part[D] = m_run[qt];
-                part[D + 1] = l;
+                part[DV] = m_run[qt];
+                part[DV + 1] = l;
             }
             continue;
         }
         const float inv = l > 0.f ? 1.0f / l : 0.f;
-        const size_t ooff = ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D;
+        const size_t ooff = ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * DV;
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt)
 #pragma unroll
@@ -544,8 +546,9 @@ prefill_kernel(AttendArgs a, int nsplit) {
 bool attend_prefill_supported(const AttendArgs &a) {
     const Store &s = a.st;
     if (s.dtype != KVHIP_F16 && s.dtype != KVHIP_BF16) return false;
-    // keys of 192 with values of 128 (the multi-head latent attention models), full precision only
-    if (s.Dk == 192 && s.Dv == 128 && s.bits == 0) return true;
+    // keys of 192 with values of 128 (the multi-head latent attention models): full precision, or 4- / 8-bit codes
+    // in groups of 32 or 64 (the sizes that divide both)
+    if (s.Dk == 192 && s.Dv == 128 && (s.bits == 0 || ((s.bits == 4 || s.bits == 8) && (s.gs == 32 || s.gs == 64)))) return true;
     if (s.Dk != s.Dv) return false;
     // head sizes 80 (full precision only) and 96: every row count (no decode kernel is built for them)
     if (s.Dk != 64 && s.Dk != 128 && s.Dk != 256 && s.Dk != 96 && !(s.Dk == 80 && s.bits == 0)) return false;
@@ -602,8 +605,8 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
 #define PF_M(BITS, D, DT, QT, MM)                                                                         \
     do {                                                                                                  \
         profile_mark(s, true);                                                                            \
-        if (ident) hipLaunchKernelGGL((prefill_kernel<BITS, D, DT, true, QT, MM>), grid, block, 0, s, a, nsplit); \
-        else hipLaunchKernelGGL((prefill_kernel<BITS, D, DT, false, QT, MM>), grid, block, 0, s, a, nsplit);      \
+        if (ident) hipLaunchKernelGGL((prefill_kernel<BITS, D, D, DT, true, QT, MM>), grid, block, 0, s, a, nsplit); \
+        else hipLaunchKernelGGL((prefill_kernel<BITS, D, D, DT, false, QT, MM>), grid, block, 0, s, a, nsplit);      \
         profile_mark(s, false);                                                                           \
     } while (0)
 #define PF(BITS, D, DT, QT)                      \
@@ -622,9 +625,26 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
         if (st.dtype == KVHIP_F16) PF_QT(BITS, D, 0); \
         else PF_QT(BITS, D, 1);                  \
     } while (0)
+#define PF_MLA(BITS, DT)                                                                                   \
+    do {                                                                                                  \
+        profile_mark(s, true);                                                                            \
+        if (mm == 0) {                                                                                    \
+            if (ident) hipLaunchKernelGGL((prefill_kernel<BITS, 192, 128, DT, true, 1, 0>), grid, block, 0, s, a, nsplit);  \
+            else hipLaunchKernelGGL((prefill_kernel<BITS, 192, 128, DT, false, 1, 0>), grid, block, 0, s, a, nsplit);       \
+        } else if (mm == 1) {                                                                             \
+            if (ident) hipLaunchKernelGGL((prefill_kernel<BITS, 192, 128, DT, true, 1, 1>), grid, block, 0, s, a, nsplit);  \
+            else hipLaunchKernelGGL((prefill_kernel<BITS, 192, 128, DT, false, 1, 1>), grid, block, 0, s, a, nsplit);       \
+        } else {                                                                                          \
+            if (ident) hipLaunchKernelGGL((prefill_kernel<BITS, 192, 128, DT, true, 1, 2>), grid, block, 0, s, a, nsplit);  \
+            else hipLaunchKernelGGL((prefill_kernel<BITS, 192, 128, DT, false, 1, 2>), grid, block, 0, s, a, nsplit);       \
+        }                                                                                                 \
+        profile_mark(s, false);                                                                           \
+    } while (0)
 #define PF_D(BITS)                                    \
     do {                                              \
-        if (st.Dk == 64) PF_DT(BITS, 64);             \
+        if (st.Dk == 192) { /* keys 192 / values 128: 64 query rows per workgroup */ \
+            if (st.dtype == KVHIP_F16) PF_MLA(BITS, 0); else PF_MLA(BITS, 1);        \
+        } else if (st.Dk == 64) PF_DT(BITS, 64);             \
         else if (st.Dk == 96) PF_DT(BITS, 96);        \
         else if (st.Dk == 128) PF_DT(BITS, 128);      \
         else if (st.dtype == KVHIP_F16) PF(BITS, 256, 0, 1); /* 64 query rows per workgroup only */ \
@@ -640,6 +660,7 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
         if (e != hipSuccess) return e;
     }
 #undef PF_D
+#undef PF_MLA
 #undef PF_DT
 #undef PF_QT
 #undef PF

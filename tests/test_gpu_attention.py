@@ -238,6 +238,29 @@ def test_keys_of_192_values_of_128_on_the_prefill_tile(dtype):
         check(out, O.attention_with_cache_update(q, k, v, o, scale, o.make_mask(Lq, M, False), name), f"ring step {i}")
 
 
+@pytest.mark.parametrize("dtype,bits,gs", [(torch.float16, 4, 64), (torch.bfloat16, 8, 64), (torch.float16, 8, 32)])
+def test_quantized_keys_of_192_values_of_128_on_the_prefill_tile(dtype, bits, gs):
+    """The same head sizes in a QuantizedKVCache (group sizes 32 and 64 divide both): every row count runs on
+    the quantized prefill tile; codes and pairs equal the oracle's, outputs are the oracle's within the bound."""
+    rng = np.random.default_rng(bits + gs)
+    name, Dk, Dv = NAME[dtype], 192, 128
+    scale = Dk ** -0.5
+    lib = kvhip.load()
+    B, H, r = 2, 2, 2
+    c, o = kvhip.QuantizedKVCache(gs, bits), O.QuantizedKVCache(gs, bits, name)
+    for Lq, mode in [(330, "causal"), (1, "none"), (70, "causal"), (1, "none"), (4, "causal")]:
+        k, kd = randn(rng, (B, H, Lq, Dk), dtype)
+        v, vd = randn(rng, (B, H, Lq, Dv), dtype)
+        q, qd = randn(rng, (B, H * r, Lq, Dk), dtype)
+        mask, om = (kvhip.MaskMode.causal(), O.Mask.CAUSAL) if mode == "causal" else (kvhip.MaskMode.none(), O.Mask.NONE)
+        out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
+        assert lib.kvhip_last_attend_kernel() == 3 and tuple(out.shape) == (B, H * r, Lq, Dv)
+        check(out, O.attention_with_cache_update(q, k, v, o, scale, om, name), f"L={Lq}")
+    assert c.group_size == gs and c.offset == o.offset
+    for i, (a, b) in enumerate(zip(c.state, o.get_state())):
+        assert np.array_equal(np32(a), b) if i % 3 == 0 else bits_equal(a, b, dtype), i
+
+
 def test_rotating_attention_past_wrap_matches_never_rotated_reference(policy):
     # KVCacheTests.swift:1451-1491 (rtol = atol = 1e-5, float32)
     rng = np.random.default_rng(0)
