@@ -337,7 +337,10 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
     constexpr int EB = NC < 4 ? NC : 4;    // chunks of K and of V per batch
     constexpr int NI = 2 * EB;             // chunk-instances per batch: (chunk e0 + i / 2, K or V by i & 1)
     constexpr int SH = GL < NI ? GL : NI;  // lanes of a group that work out parameters
-    constexpr int PER = NI / SH;           // chunk-instances per such lane
+    constexpr int PER = (NI + SH - 1) / SH;  // chunk-instances per such lane (D = 96: six over four lanes, two of them take two)
+    // a row's TPR threads: where 256 is a multiple of TPR the rows of a thread's chunks are 256 / TPR apart and
+    // its columns the same; at D = 96 (12 threads per row) row and column are worked out per chunk
+    constexpr bool EVEN = 256 % TPR == 0;
     __shared__ __attribute__((aligned(8))) uint8_t vcodes[TILE * VP];
     __shared__ __attribute__((aligned(16))) uint8_t vstage[PAGED ? TILE * D * 2 : 16];  // the source V tile as stored
     const int bh = blockIdx.y;
@@ -382,7 +385,9 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
     const int psel = pos & (SH - 1);
     const int gbase4 = (lane & ~(GL - 1)) * 4;  // byte address (lane number x 4) of the group's first lane
     const int r_t = threadIdx.x / TPR;          // row of this thread's chunk 0; chunk e lies 256 / TPR rows further
-    const int d0 = (threadIdx.x - r_t * TPR) * 8;
+    const int d0_t = (threadIdx.x - r_t * TPR) * 8;
+    auto row_of = [&](int e) { return EVEN ? r_t + e * (256 / TPR) : (e * 256 + (int)threadIdx.x) / TPR; };
+    auto col_of = [&](int e) { return EVEN ? d0_t : ((e * 256 + (int)threadIdx.x) % TPR) * 8; };
     const int page_off = (slot_t & (PAGE - 1));
     const PageEntry page = st.pt[slot_t >> PAGE_SHIFT];  // a tile lies inside one page
 #pragma unroll
@@ -391,8 +396,9 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             const int e = e0 + i / 2;
+            const int d0 = col_of(e);
             if ((i & 1) == 0) {
-                const int r = r_t + e * (256 / TPR);
+                const int r = row_of(e);
                 if constexpr (ROPE) unpack8<DT>(kraw[e], kbase + (size_t)r * D * 2, d0, rope, rope_pos(rope, bh, l_t + r), w[i]);
                 else unpack8<DT>(kraw[e], nullptr, d0, no_rope, 0, w[i]);
             } else {
@@ -413,15 +419,17 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
         for (int k = 0; k < PER; ++k) {
             float a = mn[k * SH], b = mx[k * SH];
 #pragma unroll
-            for (int j = 1; j < SH; ++j) {
-                a = psel == j ? mn[k * SH + j] : a;
-                b = psel == j ? mx[k * SH + j] : b;
-            }
+            for (int j = 1; j < SH; ++j)
+                if (k * SH + j < NI) {
+                    a = psel == j ? mn[k * SH + j] : a;
+                    b = psel == j ? mx[k * SH + j] : b;
+                }
             affine_params(a, b, nb, sc[k], bi[k]);
             iv[k] = __builtin_amdgcn_rcpf(sc[k]);
-            if (pos < SH) {
+            if (pos < SH && psel + k * SH < NI) {
                 const int i = psel + k * SH;  // this lane's chunk-instance
-                const int row = page_off + r_t + (e0 + i / 2) * (256 / TPR);
+                const int row = page_off + row_of(e0 + i / 2);
+                const int d0 = col_of(e0 + i / 2);
                 char *sb = (i & 1) ? page.vsb + (size_t)bh * st.vsb_cell + (size_t)row * st.vsb_row
                                    : page.ksb + (size_t)bh * st.ksb_cell + (size_t)row * st.ksb_row;
                 reinterpret_cast<uint32_t *>(sb)[d0 / GS] = pack_scale_bias<DT>(sc[k], bi[k]);
@@ -430,7 +438,7 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             const int e = e0 + i / 2;
-            const int r = r_t + e * (256 / TPR);
+            const int r = row_of(e), d0 = col_of(e);
             const int src = gbase4 + (i % SH) * 4;
             const float scale = lane_value(src, sc[i / SH]);
             const float bias = lane_value(src, bi[i / SH]);
@@ -869,7 +877,7 @@ hipError_t launch_append_quant(const Store &st, const void *keys, const void *va
                                int slot0, int n, hipStream_t s, const RopeDev *rope) {
     if (n <= 0) return hipSuccess;
     const RopeDev r = rope ? *rope : RopeDev();
-    const bool tiled = st.es == 2 && st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 128 || st.Dk == 256) &&
+    const bool tiled = st.es == 2 && st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 96 || st.Dk == 128 || st.Dk == 256) &&
                        (st.bits == 4 || st.bits == 8) && (st.gs == 32 || st.gs == 64 || st.gs == 128) &&
                        st.Dk % st.gs == 0;
     const TileSplit t = tile_split(slot0, n);
@@ -895,6 +903,7 @@ hipError_t launch_append_quant(const Store &st, const void *keys, const void *va
 #define TILE_NC(DT, BITS)                              \
     do {                                               \
         if (st.Dk == 64) TILE_GL(DT, BITS, 2);         \
+        else if (st.Dk == 96) TILE_RP(DT, BITS, 3, 4); \
         else if (st.Dk == 128) TILE_GL(DT, BITS, 4);   \
         else TILE_GL(DT, BITS, 8);                     \
     } while (0)
@@ -915,7 +924,7 @@ hipError_t launch_append_quant(const Store &st, const void *keys, const void *va
 hipError_t launch_requant_pages(const Store &src, const Store &st, int rows, hipStream_t s) {
     if (rows <= 0) return hipSuccess;
     const int tiles = (rows + TILE - 1) / TILE;
-    const bool tiled = st.es == 2 && st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 128 || st.Dk == 256) &&
+    const bool tiled = st.es == 2 && st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 96 || st.Dk == 128 || st.Dk == 256) &&
                        (st.bits == 4 || st.bits == 8) && (st.gs == 32 || st.gs == 64 || st.gs == 128) && st.Dk % st.gs == 0;
     dim3 grid(tiles, st.BH), block(256);
     if (!tiled) {
@@ -937,6 +946,7 @@ hipError_t launch_requant_pages(const Store &src, const Store &st, int rows, hip
 #define RQ_NC(DT, BITS)                              \
     do {                                             \
         if (st.Dk == 64) RQ_GL(DT, BITS, 2);         \
+        else if (st.Dk == 96) RQ(DT, BITS, 3, 4);    \
         else if (st.Dk == 128) RQ_GL(DT, BITS, 4);   \
         else RQ_GL(DT, BITS, 8);                     \
     } while (0)

@@ -170,7 +170,7 @@ def test_quantized_prompt_append_on_rounding_ties(bits):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("bits", [4, 8])
-@pytest.mark.parametrize("D,gs", [(64, 32), (64, 64), (128, 32), (128, 64), (128, 128), (256, 32), (256, 64), (256, 128)])
+@pytest.mark.parametrize("D,gs", [(64, 32), (64, 64), (96, 32), (128, 32), (128, 64), (128, 128), (256, 32), (256, 64), (256, 128)])
 def test_quantized_prompt_append_every_tile_shape(dtype, bits, D, gs):
     """Whole 64-token tiles for every head size and group size the tile quantizer is built for (how
     many lanes share a group, and how many groups a lane works parameters out for, differ between
@@ -185,6 +185,21 @@ def test_quantized_prompt_append_every_tile_shape(dtype, bits, D, gs):
         cache.update_quantized(kd, vd, fetch=False)
         ocache.update_quantized(k, v)
         check_quantized_state(cache, ocache, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bits", [4, 8])
+def test_head_size_96_converts_by_whole_tiles(dtype, bits):
+    """`toQuantized` of a full-precision cache of head size 96 (twelve 16-byte chunks per row: a row's
+    threads do not divide the workgroup) gives the oracle's codes and pairs."""
+    rng = np.random.default_rng(96 + bits)
+    c, o = kvhip.KVCacheSimple(), O.KVCacheSimple(NAME[dtype])
+    for L in (200, 1, 70):
+        k, kd = randn(rng, (2, 3, L, 96), dtype, 2.0)
+        v, vd = randn(rng, (2, 3, L, 96), dtype, 0.5)
+        c.update(kd, vd, fetch=False)
+        o.update(k, v)
+    check_quantized_state(c.to_quantized(32, bits), o.to_quantized(32, bits), dtype)
 
 
 def test_quantized_group_size_fallback_and_errors():
