@@ -519,35 +519,33 @@ __global__ void __launch_bounds__(256) dequant_pages_kernel(Store q, Store dst, 
     }
 }
 
-// grid (whole tiles, BH), 256 threads; 16-bit dtypes, Dk == Dv == 32 NC
-template <int NC>
+// grid (whole tiles, BH), 256 threads; 16-bit dtypes, Dk == 32 NCK, Dv == 32 NCV
+template <int NCK, int NCV>
 __global__ void __launch_bounds__(256)
 append_fp_tile_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, RopeDev rope) {
-    constexpr int D = 32 * NC;
-    constexpr int TPR = D / 8;
+    constexpr int DK = 32 * NCK, D = 32 * NCV;
+    constexpr int TPRK = DK / 8, TPR = D / 8;
     constexpr int VPW = D / 2 + 1;  // dword pitch of a token's V row in LDS (odd: column reads spread over banks)
     __shared__ uint32_t vt[TILE * VPW];
     const int bh = blockIdx.y;
     const int slot_t = slot0 + blockIdx.x * TILE;
     const int l_t = src0 + blockIdx.x * TILE;
-    const char *kbase = keys + ((size_t)bh * L + l_t) * D * 2;
+    const char *kbase = keys + ((size_t)bh * L + l_t) * DK * 2;
     const char *vbase = values + ((size_t)bh * L + l_t) * D * 2;
     char *kcell = st.pt[slot_t >> PAGE_SHIFT].k + (size_t)bh * st.k_cell;  // a tile lies inside one page
-    u4v kraw[NC], vraw[NC];
+    u4v kraw[NCK], vraw[NCV];
 #pragma unroll
-    for (int e = 0; e < NC; ++e) {
-        const int c = e * 256 + threadIdx.x;
-        kraw[e] = *reinterpret_cast<const u4v *>(kbase + (size_t)c * 16);
-        vraw[e] = *reinterpret_cast<const u4v *>(vbase + (size_t)c * 16);
-    }
+    for (int e = 0; e < NCK; ++e) kraw[e] = *reinterpret_cast<const u4v *>(kbase + (size_t)(e * 256 + threadIdx.x) * 16);
 #pragma unroll
-    for (int e = 0; e < NC; ++e) {
+    for (int e = 0; e < NCV; ++e) vraw[e] = *reinterpret_cast<const u4v *>(vbase + (size_t)(e * 256 + threadIdx.x) * 16);
+#pragma unroll
+    for (int e = 0; e < NCK; ++e) {
         const int c = e * 256 + threadIdx.x;
-        const int r = c / TPR, d0 = (c - r * TPR) * 8;
+        const int r = c / TPRK, d0 = (c - r * TPRK) * 8;
         u4v k = kraw[e];
         if (rope.dims > 0 && d0 < rope.dims) {
             const int pos = rope_pos(rope, bh, l_t + r);
-            const char *row = kbase + (size_t)r * D * 2;
+            const char *row = kbase + (size_t)r * DK * 2;
             uint32_t u[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -564,6 +562,11 @@ append_fp_tile_kernel(Store st, const char *keys, const char *values, int L, int
             k = u4v{u[0], u[1], u[2], u[3]};
         }
         *reinterpret_cast<u4v *>(kcell + kfp_off(st, slot_t + r, d0)) = k;
+    }
+#pragma unroll
+    for (int e = 0; e < NCV; ++e) {
+        const int c = e * 256 + threadIdx.x;
+        const int r = c / TPR, d0 = (c - r * TPR) * 8;
         uint32_t *vrow = &vt[r * VPW + d0 / 2];
         vrow[0] = vraw[e].x;
         vrow[1] = vraw[e].y;
@@ -824,17 +827,21 @@ hipError_t launch_append_fp(const Store &st, const void *keys, const void *value
                             int slot0, int n, hipStream_t s, const RopeDev *rope) {
     if (n <= 0) return hipSuccess;
     const RopeDev r = rope ? *rope : RopeDev();
-    const bool tiled = st.es == 2 && st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 96 || st.Dk == 128 || st.Dk == 256);
+    const bool mla = st.Dk == 192 && st.Dv == 128;  // keys of 192 with values of 128
+    const bool tiled = st.es == 2 && ((st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 96 || st.Dk == 128 || st.Dk == 256)) || mla);
     const TileSplit t = tile_split(slot0, n);
     if (!tiled || t.tiles == 0) return launch_append_fp_rows(st, keys, values, L, src0, slot0, n, s, r);
     hipError_t e = launch_append_fp_rows(st, keys, values, L, src0, slot0, t.head, s, r);
     if (e != hipSuccess) return e;
     dim3 grid(t.tiles, st.BH), block(256);
     const int a0 = src0 + t.head, b0 = slot0 + t.head;
-    if (st.Dk == 64) hipLaunchKernelGGL(append_fp_tile_kernel<2>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, a0, b0, r);
-    else if (st.Dk == 96) hipLaunchKernelGGL(append_fp_tile_kernel<3>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, a0, b0, r);
-    else if (st.Dk == 128) hipLaunchKernelGGL(append_fp_tile_kernel<4>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, a0, b0, r);
-    else hipLaunchKernelGGL(append_fp_tile_kernel<8>, grid, block, 0, s, st, (const char *)keys, (const char *)values, L, a0, b0, r);
+#define FP_TILE(NCK, NCV) hipLaunchKernelGGL((append_fp_tile_kernel<NCK, NCV>), grid, block, 0, s, st, (const char *)keys, (const char *)values, L, a0, b0, r)
+    if (mla) FP_TILE(6, 4);
+    else if (st.Dk == 64) FP_TILE(2, 2);
+    else if (st.Dk == 96) FP_TILE(3, 3);
+    else if (st.Dk == 128) FP_TILE(4, 4);
+    else FP_TILE(8, 8);
+#undef FP_TILE
     e = hipGetLastError();
     if (e != hipSuccess) return e;
     return launch_append_fp_rows(st, keys, values, L, a0 + t.tiles * TILE, b0 + t.tiles * TILE, t.tail, s, r);

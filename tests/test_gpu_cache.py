@@ -251,16 +251,17 @@ def test_simple_cache_update_fetch_state(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("D", [64, 96, 128, 256])
+@pytest.mark.parametrize("D", [64, 96, 128, 256, (192, 128)])
 def test_simple_cache_prompt_sized_appends(dtype, D):
     """Appends that cover whole 64-token tiles take the tile kernel (head rows, tiles, tail rows)."""
     rng = np.random.default_rng(21)
     B, H = 2, 3
+    Dk, Dv = D if isinstance(D, tuple) else (D, D)
     c = kvhip.KVCacheSimple()
     o = O.KVCacheSimple(NAME[dtype])
     for L, trim in [(37, 0), (200, 5), (64, 0), (1, 0), (459, 3), (128, 0)]:
-        k, kd = randn(rng, (B, H, L, D), dtype)
-        v, vd = randn(rng, (B, H, L, D), dtype)
+        k, kd = randn(rng, (B, H, L, Dk), dtype)
+        v, vd = randn(rng, (B, H, L, Dv), dtype)
         gk, gv = c.update(kd, vd)
         ok, ov = o.update(k, v)
         assert np.array_equal(np32(gk), ok) and np.array_equal(np32(gv), ov)

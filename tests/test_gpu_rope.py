@@ -101,14 +101,15 @@ def test_fused_append_equals_rotate_then_append_simple_and_ring(dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("traditional", [False, True])
-def test_fused_prompt_sized_append_equals_rotate_then_append(dtype, traditional):
+@pytest.mark.parametrize("Dk,Dv,dims", [(128, 128, 128), (192, 128, 64)])
+def test_fused_prompt_sized_append_equals_rotate_then_append(dtype, traditional, Dk, Dv, dims):
     """Whole-tile appends rotate inside the tile kernel."""
     rng = np.random.default_rng(7)
-    rope = kvhip.RoPE(128, traditional=traditional, base=500000.0)
+    rope = kvhip.RoPE(dims, traditional=traditional, base=500000.0)
     fused, plain = kvhip.KVCacheSimple(), kvhip.KVCacheSimple()
     for Lq in (5, 200, 130):
-        _, k = randn(rng, (2, 2, Lq, 128), dtype)
-        _, v = randn(rng, (2, 2, Lq, 128), dtype)
+        _, k = randn(rng, (2, 2, Lq, Dk), dtype)
+        _, v = randn(rng, (2, 2, Lq, Dv), dtype)
         off = plain.offset
         fused.update_rope(rope, k, v)
         plain.update(kvhip.apply_rotary_position(rope, k, off), v, fetch=False)
