@@ -154,6 +154,75 @@ def test_quantized_shapes_against_generic(seed):
         f"kernel {chosen}: max-abs {d.max():.3e} mean-abs {d.mean():.3e}"
 
 
+@pytest.mark.parametrize("seed", range(48))
+def test_keys_of_192_values_of_128_against_generic(seed):
+    """Keys of 192 with values of 128 (multi-head latent attention) in all three cache kinds, every row
+    count on the prefill tiles: the tuned result against the generic kernel's."""
+    rng = np.random.default_rng(5000 + seed)
+    kind = ["simple", "rotating", "quantized"][seed % 3]
+    dtype = [torch.float16, torch.bfloat16][(seed // 3) % 2]
+    Dk, Dv = 192, 128
+    B, Hkv, r = int(rng.integers(1, 4)), int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 8]))
+    Lq = int(rng.choice([1, 1, 3, 16, 40, 70, 130]))
+    T0 = int(rng.choice([1, 31, 64, 200, 257, 700, 1300]))
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+
+    def rand(*shape):
+        return torch.randn(*shape, generator=g, device="cuda").to(dtype)
+
+    if kind == "simple":
+        c = kvhip.KVCacheSimple()
+    elif kind == "rotating":
+        c = kvhip.RotatingKVCache(int(rng.choice([96, 300, 1024])), keep=int(rng.choice([0, 4])))
+    else:
+        c = kvhip.QuantizedKVCache(int(rng.choice([32, 64])), int(rng.choice([4, 8])))
+    upd = c.update_quantized if kind == "quantized" else c.update
+    upd(rand(B, Hkv, T0, Dk), rand(B, Hkv, T0, Dv), fetch=False)
+    for _ in range(int(rng.integers(0, 40)) if kind == "rotating" else 0):
+        upd(rand(B, Hkv, 1, Dk), rand(B, Hkv, 1, Dv), fetch=False)
+    upd(rand(B, Hkv, Lq, Dk), rand(B, Hkv, Lq, Dv), fetch=False)
+    T = c.presented_length
+    Lq = min(Lq, T)
+    q = rand(B, Hkv * r, Lq, Dk)
+    which = rng.choice(["none", "causal", "window", "left_pad", "bool", "additive"])
+    if which == "none":
+        mask = kvhip.MaskMode.none()
+    elif which == "causal":
+        mask = kvhip.MaskMode.causal()
+    elif which == "window":
+        mask = kvhip.MaskMode.window_mask(T - Lq, int(rng.integers(1, T + 2)))
+    elif which == "left_pad":
+        pad = torch.from_numpy(rng.integers(0, max(T - Lq, 1), size=B).astype(np.int32))
+        mask = kvhip.MaskMode.window_mask(T - Lq, 0, left_pad=pad)
+    else:
+        shape = [(B, 1, Lq, T), (1, 1, Lq, T)][rng.integers(2)]
+        keep = rng.random(shape) < 0.7
+        keep[..., int(rng.integers(T))] = True
+        if which == "bool":
+            mask = kvhip.MaskMode.from_array(torch.from_numpy(keep).cuda())
+        else:
+            add = np.where(keep, rng.standard_normal(shape).astype(np.float32), -np.inf)
+            mask = kvhip.MaskMode.from_array(torch.from_numpy(add).to(dtype).cuda())
+    scale = Dk ** -0.5
+    print(f"seed {seed}: {kind} {dtype} B{B} Hkv{Hkv} r{r} L{Lq} T{T} mask {which}", flush=True)
+    lib = kvhip.load()
+    try:
+        lib.kvhip_set_kernel_policy(1)
+        ref = np32(c.attend(q, scale, mask))
+        lib.kvhip_set_kernel_policy(0)
+        out = np32(c.attend(q, scale, mask))
+        chosen = lib.kvhip_last_attend_kernel()
+    finally:
+        lib.kvhip_set_kernel_policy(0)
+    assert chosen == 3 and out.shape == (B, Hkv * r, Lq, Dv)
+    assert np.isfinite(ref).all() and np.isfinite(out).all()
+    d = np.abs(out.astype(np.float64) - ref.astype(np.float64))
+    ulp = float(np.abs(ref).max()) * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10)
+    assert d.max() <= max(MAX_ABS, 2 * ulp) and d.mean() <= max(MEAN_ABS, ulp / 4), \
+        f"max-abs {d.max():.3e} mean-abs {d.mean():.3e}"
+
+
 @pytest.mark.parametrize("kind,dtype,B,Hkv,L,extra", [
     ("simple", torch.float16, 1, 8, 2048, 0), ("simple", torch.bfloat16, 2, 8, 1024, 512),
     ("quantized", torch.float16, 1, 8, 2048, 0), ("quantized", torch.float16, 2, 8, 1024, 300),
