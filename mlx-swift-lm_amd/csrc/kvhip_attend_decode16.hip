@@ -434,10 +434,25 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 x[tl] = (XT)s_;
             }
         }
-        XT xmax = x[0];
+        // this lane's largest score: a tree of packed maxima (float16 scores sit two to a register) or of
+        // three-operand maxima -- a chain of compares and selects is sixteen dependent steps
+        float tmax;
+        if constexpr (DT == 0) {
+            typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+            h2v m2[8];
 #pragma unroll
-        for (int tl = 1; tl < 16; ++tl) xmax = x[tl] > xmax ? x[tl] : xmax;
-        float tmax = (float)xmax;
+            for (int u = 0; u < 8; ++u) m2[u] = h2v{x[2 * u], x[2 * u + 1]};
+#pragma unroll
+            for (int w = 4; w >= 1; w >>= 1)
+#pragma unroll
+                for (int u = 0; u < w; ++u) m2[u] = __builtin_elementwise_max(m2[u], m2[u + w]);
+            tmax = fmaxf((float)m2[0].x, (float)m2[0].y);
+        } else {
+            float m4[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) m4[u] = fmaxf(fmaxf((float)x[4 * u], (float)x[4 * u + 1]), fmaxf((float)x[4 * u + 2], (float)x[4 * u + 3]));
+            tmax = fmaxf(fmaxf(m4[0], m4[1]), fmaxf(m4[2], m4[3]));
+        }
         // raise the row maximum only when some lane's own maximum exceeds it (rare after the
         // first tiles); it stays equal in the four lanes of a row
         if (__any(tmax > m_run)) {
