@@ -327,22 +327,30 @@ template <int DT> __device__ __forceinline__ uint32_t pack_scale_bias(float scal
 // PAGED: the 64 rows are tile `l_t / 64` of the full-precision page store `src` (a cache being
 // converted) instead of rows of dense arrays: K chunks are read from the interleaved tile where
 // they lie, the V tile (stored by column) is turned back into rows through LDS.
-template <int DT, int BITS, int NC, int GL, bool ROPE, bool PAGED>
+// SIDE: 0 keys and values of one head size 32 NC; 1 the keys alone, 2 the values alone (caches whose keys and
+// values differ in head size take one launch for each, NC being that side's).
+template <int DT, int BITS, int NC, int GL, bool ROPE, bool PAGED, int SIDE = 0>
 __device__ __forceinline__ void append_quant_tile_body(const Store &st, const Store &src, const char *keys, const char *values,
                                                        int L, int src0, int slot0, const RopeDev &rope) {
     constexpr int D = 32 * NC;
     constexpr int GS = 8 * GL;
     constexpr int TPR = D / 8;   // threads per row
     constexpr int VP = D + 8;    // byte pitch of a token's V codes in LDS
-    constexpr int EB = NC < 4 ? NC : 4;    // chunks of K and of V per batch
-    constexpr int NI = 2 * EB;             // chunk-instances per batch: (chunk e0 + i / 2, K or V by i & 1)
+    constexpr bool DO_K = SIDE != 2, DO_V = SIDE != 1;
+    // chunks per batch (a divisor of NC; one side alone: a count whose instances share out evenly over a group's lanes)
+    constexpr int EB = SIDE == 0 ? (NC < 4 ? NC : 4) : (NC % 4 == 0 ? 4 : 2);
+    static_assert(NC % EB == 0, "a batch holds a whole number of chunks");
+    // chunk-instances per batch: both sides (chunk e0 + i / 2, K or V by i & 1), or one side's chunks e0 + i
+    constexpr int NI = SIDE == 0 ? 2 * EB : EB;
+    auto chunk_of = [](int i) { return SIDE == 0 ? i / 2 : i; };
+    auto is_v = [](int i) { return SIDE == 0 ? (i & 1) != 0 : SIDE == 2; };
     constexpr int SH = GL < NI ? GL : NI;  // lanes of a group that work out parameters
     constexpr int PER = (NI + SH - 1) / SH;  // chunk-instances per such lane (D = 96: six over four lanes, two of them take two)
     // a row's TPR threads: where 256 is a multiple of TPR the rows of a thread's chunks are 256 / TPR apart and
     // its columns the same; at D = 96 (12 threads per row) row and column are worked out per chunk
     constexpr bool EVEN = 256 % TPR == 0;
-    __shared__ __attribute__((aligned(8))) uint8_t vcodes[TILE * VP];
-    __shared__ __attribute__((aligned(16))) uint8_t vstage[PAGED ? TILE * D * 2 : 16];  // the source V tile as stored
+    __shared__ __attribute__((aligned(8))) uint8_t vcodes[DO_V ? TILE * VP : 8];
+    __shared__ __attribute__((aligned(16))) uint8_t vstage[PAGED && DO_V ? TILE * D * 2 : 16];  // the source V tile as stored
     const int bh = blockIdx.y;
     const int slot_t = slot0 + blockIdx.x * TILE;
     const int l_t = src0 + blockIdx.x * TILE;
@@ -356,12 +364,12 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
         for (int e = 0; e < NC; ++e) {
             const int c = e * 256 + threadIdx.x;
             const int r = c / TPR, ch = c - r * TPR;
-            kraw[e] = *reinterpret_cast<const u4v *>(kt + ((size_t)ch * TILE + r) * 16);
-            *reinterpret_cast<u4v *>(vstage + (size_t)c * 16) = *reinterpret_cast<const u4v *>(vt + (size_t)c * 16);
+            if constexpr (DO_K) kraw[e] = *reinterpret_cast<const u4v *>(kt + ((size_t)ch * TILE + r) * 16);
+            if constexpr (DO_V) *reinterpret_cast<u4v *>(vstage + (size_t)c * 16) = *reinterpret_cast<const u4v *>(vt + (size_t)c * 16);
         }
-        __syncthreads();
+        if constexpr (DO_V) __syncthreads();
 #pragma unroll
-        for (int e = 0; e < NC; ++e) {
+        for (int e = 0; e < (DO_V ? NC : 0); ++e) {
             const int c = e * 256 + threadIdx.x;
             const int r = c / TPR, dd = (c - r * TPR) * 8;
             const uint16_t *col = reinterpret_cast<const uint16_t *>(vstage) + ((size_t)(r >> 3) * D + dd) * 8 + (r & 7);
@@ -374,8 +382,8 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
 #pragma unroll
         for (int e = 0; e < NC; ++e) {
             const int c = e * 256 + threadIdx.x;
-            kraw[e] = *reinterpret_cast<const u4v *>(kbase + (size_t)c * 16);
-            vraw[e] = *reinterpret_cast<const u4v *>(vbase + (size_t)c * 16);
+            if constexpr (DO_K) kraw[e] = *reinterpret_cast<const u4v *>(kbase + (size_t)c * 16);
+            if constexpr (DO_V) vraw[e] = *reinterpret_cast<const u4v *>(vbase + (size_t)c * 16);
         }
     }
     const RopeDev no_rope;
@@ -395,9 +403,9 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
         float w[NI][8], mn[NI], mx[NI];
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int e = e0 + i / 2;
+            const int e = e0 + chunk_of(i);
             const int d0 = col_of(e);
-            if ((i & 1) == 0) {
+            if (!is_v(i)) {
                 const int r = row_of(e);
                 if constexpr (ROPE) unpack8<DT>(kraw[e], kbase + (size_t)r * D * 2, d0, rope, rope_pos(rope, bh, l_t + r), w[i]);
                 else unpack8<DT>(kraw[e], nullptr, d0, no_rope, 0, w[i]);
@@ -428,16 +436,16 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
             iv[k] = __builtin_amdgcn_rcpf(sc[k]);
             if (pos < SH && psel + k * SH < NI) {
                 const int i = psel + k * SH;  // this lane's chunk-instance
-                const int row = page_off + row_of(e0 + i / 2);
-                const int d0 = col_of(e0 + i / 2);
-                char *sb = (i & 1) ? page.vsb + (size_t)bh * st.vsb_cell + (size_t)row * st.vsb_row
+                const int row = page_off + row_of(e0 + chunk_of(i));
+                const int d0 = col_of(e0 + chunk_of(i));
+                char *sb = is_v(i) ? page.vsb + (size_t)bh * st.vsb_cell + (size_t)row * st.vsb_row
                                    : page.ksb + (size_t)bh * st.ksb_cell + (size_t)row * st.ksb_row;
                 reinterpret_cast<uint32_t *>(sb)[d0 / GS] = pack_scale_bias<DT>(sc[k], bi[k]);
             }
         }
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int e = e0 + i / 2;
+            const int e = e0 + chunk_of(i);
             const int r = row_of(e), d0 = col_of(e);
             const int src = gbase4 + (i % SH) * 4;
             const float scale = lane_value(src, sc[i / SH]);
@@ -445,7 +453,7 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
             const float inv = lane_value(src, iv[i / SH]);
             float q[8];
             codes8<BITS>(w[i], scale, bias, inv, q);
-            if ((i & 1) == 0) {
+            if (!is_v(i)) {
                 // ---- K: packed words in natural order --------------------------------------------
                 uint32_t *kw = reinterpret_cast<uint32_t *>(page.k + (size_t)bh * st.k_cell + (size_t)(page_off + r) * st.k_row);
                 if (BITS == 4) {
@@ -461,6 +469,7 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
             }
         }
     }
+    if constexpr (!DO_V) return;
     __syncthreads();
     // each thread assembles 16 bytes (4 words) of one transposed row; consecutive threads
     // continue the same row, so the tile rows are written contiguously
@@ -484,16 +493,16 @@ __device__ __forceinline__ void append_quant_tile_body(const Store &st, const St
     }
 }
 
-template <int DT, int BITS, int NC, int GL, bool ROPE>
+template <int DT, int BITS, int NC, int GL, bool ROPE, int SIDE = 0>
 __global__ void __launch_bounds__(256)
 append_quant_tile_kernel(Store st, const char *keys, const char *values, int L, int src0, int slot0, RopeDev rope) {
-    append_quant_tile_body<DT, BITS, NC, GL, ROPE, false>(st, st, keys, values, L, src0, slot0, rope);
+    append_quant_tile_body<DT, BITS, NC, GL, ROPE, false, SIDE>(st, st, keys, values, L, src0, slot0, rope);
 }
 
 // grid (tiles, BH): tiles [0, gridDim.x) of the full-precision store `src` into the same slots of `st`
-template <int DT, int BITS, int NC, int GL>
+template <int DT, int BITS, int NC, int GL, int SIDE = 0>
 __global__ void __launch_bounds__(256) requant_tile_kernel(Store st, Store src) {
-    append_quant_tile_body<DT, BITS, NC, GL, false, true>(st, src, nullptr, nullptr, 0, 0, 0, RopeDev());
+    append_quant_tile_body<DT, BITS, NC, GL, false, true, SIDE>(st, src, nullptr, nullptr, 0, 0, 0, RopeDev());
 }
 
 // grid (64-token tiles, BH): rows [0, rows) of a quantized store as full-precision rows of `dst`
@@ -887,12 +896,41 @@ hipError_t launch_append_quant(const Store &st, const void *keys, const void *va
     const bool tiled = st.es == 2 && st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 96 || st.Dk == 128 || st.Dk == 256) &&
                        (st.bits == 4 || st.bits == 8) && (st.gs == 32 || st.gs == 64 || st.gs == 128) &&
                        st.Dk % st.gs == 0;
+    // keys of 192 with values of 128: a launch for the keys and one for the values
+    const bool two_sided = st.es == 2 && st.Dk == 192 && st.Dv == 128 && (st.bits == 4 || st.bits == 8) && (st.gs == 32 || st.gs == 64);
     const TileSplit t = tile_split(slot0, n);
-    if (!tiled || t.tiles == 0) return launch_append_quant_rows(st, keys, values, L, src0, slot0, n, s, r);
+    if ((!tiled && !two_sided) || t.tiles == 0) return launch_append_quant_rows(st, keys, values, L, src0, slot0, n, s, r);
     hipError_t e = launch_append_quant_rows(st, keys, values, L, src0, slot0, t.head, s, r);
     if (e != hipSuccess) return e;
     dim3 grid(t.tiles, st.BH), block(256);
     const int a0 = src0 + t.head, b0 = slot0 + t.head;
+    if (two_sided) {
+#define SIDE_CALL(DT, BITS, NC, GL, RP, SIDE)                                                                          \
+    hipLaunchKernelGGL((append_quant_tile_kernel<DT, BITS, NC, GL, RP, SIDE>), grid, block, 0, s, st, (const char *)keys, \
+                       (const char *)values, L, a0, b0, r)
+#define SIDES(DT, BITS, GL)                                    \
+    do {                                                       \
+        if (r.dims > 0) SIDE_CALL(DT, BITS, 6, GL, true, 1);   \
+        else SIDE_CALL(DT, BITS, 6, GL, false, 1);             \
+        SIDE_CALL(DT, BITS, 4, GL, false, 2);                  \
+    } while (0)
+#define SIDES_GL(DT, BITS)                     \
+    do {                                       \
+        if (st.gs == 32) SIDES(DT, BITS, 4);   \
+        else SIDES(DT, BITS, 8);               \
+    } while (0)
+        if (st.dtype == KVHIP_F16) {
+            if (st.bits == 4) SIDES_GL(0, 4); else SIDES_GL(0, 8);
+        } else {
+            if (st.bits == 4) SIDES_GL(1, 4); else SIDES_GL(1, 8);
+        }
+#undef SIDES_GL
+#undef SIDES
+#undef SIDE_CALL
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        return launch_append_quant_rows(st, keys, values, L, a0 + t.tiles * TILE, b0 + t.tiles * TILE, t.tail, s, r);
+    }
 #define TILE_CALL(DT, BITS, NC, GL, RP)                                                                  \
     hipLaunchKernelGGL((append_quant_tile_kernel<DT, BITS, NC, GL, RP>), grid, block, 0, s, st, (const char *)keys, \
                        (const char *)values, L, a0, b0, r)
@@ -934,6 +972,27 @@ hipError_t launch_requant_pages(const Store &src, const Store &st, int rows, hip
     const bool tiled = st.es == 2 && st.Dk == st.Dv && (st.Dk == 64 || st.Dk == 96 || st.Dk == 128 || st.Dk == 256) &&
                        (st.bits == 4 || st.bits == 8) && (st.gs == 32 || st.gs == 64 || st.gs == 128) && st.Dk % st.gs == 0;
     dim3 grid(tiles, st.BH), block(256);
+    if (st.es == 2 && st.Dk == 192 && st.Dv == 128 && (st.bits == 4 || st.bits == 8) && (st.gs == 32 || st.gs == 64)) {
+        // keys of 192 with values of 128: a launch for the keys and one for the values
+#define RQS(DT, BITS, GL)                                                                                      \
+    do {                                                                                                       \
+        hipLaunchKernelGGL((requant_tile_kernel<DT, BITS, 6, GL, 1>), grid, block, 0, s, st, src);             \
+        hipLaunchKernelGGL((requant_tile_kernel<DT, BITS, 4, GL, 2>), grid, block, 0, s, st, src);             \
+    } while (0)
+#define RQS_GL(DT, BITS)                     \
+    do {                                     \
+        if (st.gs == 32) RQS(DT, BITS, 4);   \
+        else RQS(DT, BITS, 8);               \
+    } while (0)
+        if (st.dtype == KVHIP_F16) {
+            if (st.bits == 4) RQS_GL(0, 4); else RQS_GL(0, 8);
+        } else {
+            if (st.bits == 4) RQS_GL(1, 4); else RQS_GL(1, 8);
+        }
+#undef RQS_GL
+#undef RQS
+        return hipGetLastError();
+    }
     if (!tiled) {
         const size_t lds = (size_t)TILE * st.Dv;
 #define CALL(DT, BITS) hipLaunchKernelGGL((requant_rows_kernel<DT, BITS>), grid, block, lds, s, st, src, 0, rows)

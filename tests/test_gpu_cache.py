@@ -188,6 +188,27 @@ def test_quantized_prompt_append_every_tile_shape(dtype, bits, D, gs):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bits,gs", [(4, 64), (8, 64), (4, 32), (8, 32)])
+def test_keys_of_192_values_of_128_fill_and_convert_by_whole_tiles(dtype, bits, gs):
+    """Keys and values of different head sizes: whole tiles are quantized by a launch for the keys and one for
+    the values, on append and in `toQuantized`; codes and pairs are the oracle's."""
+    rng = np.random.default_rng(192 + bits + gs)
+    B, H = 2, 3
+    cache, ocache = kvhip.QuantizedKVCache(gs, bits), O.QuantizedKVCache(gs, bits, NAME[dtype])
+    c, o = kvhip.KVCacheSimple(), O.KVCacheSimple(NAME[dtype])
+    for L in (7, 210, 64, 1, 300):
+        k, kd = randn(rng, (B, H, L, 192), dtype, 3.0)
+        v, vd = randn(rng, (B, H, L, 128), dtype, 0.25)
+        cache.update_quantized(kd, vd, fetch=False)
+        ocache.update_quantized(k, v)
+        check_quantized_state(cache, ocache, dtype)
+        c.update(kd, vd, fetch=False)
+        o.update(k, v)
+    assert cache.group_size == gs
+    check_quantized_state(c.to_quantized(gs, bits), o.to_quantized(gs, bits), dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("bits", [4, 8])
 def test_head_size_96_converts_by_whole_tiles(dtype, bits):
     """`toQuantized` of a full-precision cache of head size 96 (twelve 16-byte chunks per row: a row's

@@ -118,15 +118,17 @@ def test_fused_prompt_sized_append_equals_rotate_then_append(dtype, traditional,
     assert torch.equal(fk, pk) and torch.equal(fv, pv)
 
 
-@pytest.mark.parametrize("bits,gs,D,dims", [(4, 64, 128, 96), (8, 32, 128, 96), (4, 32, 96, 96), (8, 32, 96, 48)])
+@pytest.mark.parametrize("bits,gs,D,dims", [(4, 64, 128, 96), (8, 32, 128, 96), (4, 32, 96, 96), (8, 32, 96, 48),
+                                            (4, 64, (192, 128), 64), (8, 32, (192, 128), 192)])
 def test_fused_quantize_on_append_equals_rotate_then_append(bits, gs, D, dims):
     rng = np.random.default_rng(3)
     dtype = torch.float16
+    Dk, Dv = D if isinstance(D, tuple) else (D, D)
     rope = kvhip.RoPE(dims, traditional=True, base=1e6)          # (partial rotation of a 128-wide head)
     fused, plain = kvhip.QuantizedKVCache(gs, bits), kvhip.QuantizedKVCache(gs, bits)
     for Lq in (70, 1, 1, 3, 190):
-        _, k = randn(rng, (2, 2, Lq, D), dtype)
-        _, v = randn(rng, (2, 2, Lq, D), dtype)
+        _, k = randn(rng, (2, 2, Lq, Dk), dtype)
+        _, v = randn(rng, (2, 2, Lq, Dv), dtype)
         off = plain.offset
         fused.update_rope(rope, k, v)
         plain.update_quantized(kvhip.apply_rotary_position(rope, k, off), v, fetch=False)
