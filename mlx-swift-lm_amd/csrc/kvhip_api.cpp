@@ -1111,10 +1111,11 @@ kvhip_status kvhip_cache_state_desc(const kvhip_cache *c, int32_t i, int64_t sha
 }
 
 kvhip_status kvhip_cache_state_export(const kvhip_cache *c, int32_t i, void *dst, void *stream) {
-    if (!c || !dst) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
+    if (!c) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
     if (i < 0 || i >= kvhip_cache_state_count(c)) return fail(KVHIP_ERR_INVALID_ARG, "state index out of range");
     const int64_t n = state_rows(c);
-    if (n == 0) return KVHIP_OK;
+    if (n == 0) return KVHIP_OK;  // (an array of no rows -- a cache trimmed back to empty -- has no address)
+    if (!dst) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
     if (c->kind == KVHIP_KIND_QUANTIZED) {
         KV_HIP(launch_export_quant(c->st, i, (int)n, dst, S(c, stream)));
         return KVHIP_OK;

@@ -223,6 +223,31 @@ def test_head_size_96_converts_by_whole_tiles(dtype, bits):
     check_quantized_state(c.to_quantized(32, bits), o.to_quantized(32, bits), dtype)
 
 
+@pytest.mark.parametrize("kind", ["simple", "quantized"])
+def test_state_of_a_cache_trimmed_back_to_empty(kind):
+    """Trimming every row leaves buffers with offset 0: `state` is then arrays of no rows (a slice `[..<0]`,
+    KVCache.swift:449-460, 1113-1130), which round-trip into a fresh cache."""
+    rng = np.random.default_rng(2)
+    k, kd = randn(rng, (2, 2, 5, 64), torch.float16)
+    if kind == "simple":
+        c, o = kvhip.KVCacheSimple(), O.KVCacheSimple("float16")
+        c.update(kd, kd, fetch=False)
+        o.update(k, k)
+    else:
+        c, o = kvhip.QuantizedKVCache(64, 4), O.QuantizedKVCache(64, 4, "float16")
+        c.update_quantized(kd, kd, fetch=False)
+        o.update_quantized(k, k)
+    assert c.trim(9) == o.trim(9) == 5 and c.offset == 0
+    st, ost = c.state, o.get_state()
+    assert [tuple(a.shape) for a in st] == [tuple(b.shape) for b in ost] and all(a.shape[2] == 0 for a in st)
+    fresh = kvhip.KVCacheSimple() if kind == "simple" else kvhip.QuantizedKVCache(64, 4)
+    fresh.state = st
+    fresh.meta_state = c.meta_state
+    assert fresh.offset == 0
+    (fresh.update_quantized if kind == "quantized" else fresh.update)(kd, kd, fetch=False)
+    assert fresh.offset == 5
+
+
 def test_quantized_group_size_fallback_and_errors():
     # KVCacheTests.swift:477-501: QuantizedKVCache(64, 4) fed D=32 -> groupSize 32
     rng = np.random.default_rng(0)
