@@ -1,0 +1,116 @@
+"""Drawn schedules against the oracle: appends of drawn widths, trims, copies, state round trips, conversions and
+decode sequences, each case a seed.  The fixed schedules of the other files pin the cases the reference's own tests
+name; these walk combinations nobody wrote down (one of them found that a cache trimmed back to empty could not
+export its state)."""
+import numpy as np
+import pytest
+import torch
+
+import kvhip
+from oracle import kv_oracle as O
+from tests.test_gpu_cache import check_quantized_state, drive_pair, positioned
+from tests.util import NAME, err_stats, np32, randn
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_quantized_append_trim_convert(seed):
+    """Codes and (scale, bias) pairs bit for bit after a drawn schedule, and after `toQuantized` of the same rows."""
+    rng = np.random.default_rng(9000 + seed)
+    dtype = [torch.float16, torch.bfloat16][seed % 2]
+    Dk, Dv, gss = [(64, 64, [32, 64]), (96, 96, [32]), (128, 128, [32, 64, 128]), (256, 256, [64, 128]),
+                   (192, 128, [32, 64])][seed % 5]
+    gs, bits = int(rng.choice(gss)), int(rng.choice([4, 8, 4, 8, 3, 6]))
+    B, H = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+    cache, oc = kvhip.QuantizedKVCache(gs, bits), O.QuantizedKVCache(gs, bits, NAME[dtype])
+    c, o = kvhip.KVCacheSimple(), O.KVCacheSimple(NAME[dtype])
+    for _ in range(int(rng.integers(3, 8))):
+        L = int(rng.choice([1, 2, 5, 63, 64, 65, 128, 130, 257, 400]))
+        k, kd = randn(rng, (B, H, L, Dk), dtype, float(rng.choice([0.1, 1.0, 30.0])))
+        v, vd = randn(rng, (B, H, L, Dv), dtype, float(rng.choice([0.1, 1.0, 30.0])))
+        cache.update_quantized(kd, vd, fetch=False)
+        oc.update_quantized(k, v)
+        c.update(kd, vd, fetch=False)
+        o.update(k, v)
+        t = int(rng.choice([0, 0, 1, 3, 70]))
+        assert cache.trim(t) == oc.trim(t) and c.trim(t) == o.trim(t)
+    check_quantized_state(cache, oc, dtype)
+    if c.offset > 0:
+        check_quantized_state(c.to_quantized(gs, bits), o.to_quantized(gs, bits), dtype)
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_ring_updates_trims_copies_and_restores(seed):
+    """Every update's presentation and metaState equal the reference's buffers through drawn widths (single
+    tokens, chunks up to twice the ring), trims, copies and state / metaState restores."""
+    rng = np.random.default_rng(7000 + seed)
+    M = int(rng.choice([5, 8, 16, 33, 64, 100, 300]))
+    keep = min(int(rng.choice([0, 1, 2, 4])), M - 1)
+    step = int(rng.choice([256, 3, 16]))
+    dtype = [torch.float16, torch.bfloat16, torch.float32][seed % 3]
+    c, o = kvhip.RotatingKVCache(M, keep=keep, step=step), O.RotatingKVCache(M, keep=keep, step=step, dtype=NAME[dtype])
+    pos = 0
+    for _ in range(int(rng.integers(5, 60))):
+        L = int(rng.choice([1, 1, 1, 1, 2, 3, M // 2 + 1, M, M + 3, 2 * M + 1]))
+        (k, v), _ = positioned(pos, pos + L, D=4)
+        k, v = O.round_to(k, NAME[dtype]), O.round_to(v, NAME[dtype])  # (positions past 256 / 2048 are not exact in 16 bits)
+        drive_pair(c, o, k, v, dtype)
+        pos += L
+        assert c.is_trimmable == o.is_trimmable
+        act = int(rng.integers(0, 10))
+        if act == 0 and o.is_trimmable:
+            t = int(rng.integers(0, 4))
+            assert c.trim(t) == o.trim(t) and c.meta_state == o.get_meta_state()
+            pos = o.offset
+        elif act == 1:
+            st = c.state
+            assert all(np.array_equal(np32(a), b) for a, b in zip(st, o.get_state()))
+            fresh = kvhip.RotatingKVCache(M)
+            fresh.state = st
+            fresh.meta_state = c.meta_state
+            c = fresh
+        elif act == 2:
+            c = c.copy()
+
+
+@pytest.mark.parametrize("seed", range(36))
+def test_decode_sequences_through_the_dispatcher(seed):
+    """A prompt, then single tokens and small chunks through `attentionWithCacheUpdate` (the steps whose row the
+    decode kernel writes itself, the ring's gather, trims in between): every step's output against the oracle's."""
+    rng = np.random.default_rng(11000 + seed)
+    kind = ["simple", "rotating", "quantized"][seed % 3]
+    dtype = [torch.float16, torch.bfloat16][(seed // 3) % 2]
+    if kind == "quantized":
+        Dk, Dv, gs = [(64, 64, 64), (128, 128, 64), (128, 128, 32), (96, 96, 32), (256, 256, 64), (192, 128, 64)][int(rng.integers(6))]
+        bits = int(rng.choice([4, 8]))
+        c, o = kvhip.QuantizedKVCache(gs, bits), O.QuantizedKVCache(gs, bits, NAME[dtype])
+    else:
+        Dk, Dv = [(64, 64), (128, 128), (256, 256), (96, 96), (80, 80), (192, 128)][int(rng.integers(6))]
+        if kind == "simple":
+            c, o = kvhip.KVCacheSimple(), O.KVCacheSimple(NAME[dtype])
+        else:
+            M, keep = int(rng.choice([64, 100, 300])), int(rng.choice([0, 4]))
+            c, o = kvhip.RotatingKVCache(M, keep=keep), O.RotatingKVCache(M, keep=keep, dtype=NAME[dtype])
+    B, Hkv, r = int(rng.integers(1, 4)), int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 4, 8]))
+    scale = Dk ** -0.5
+    steps = [int(rng.choice([1, 40, 70, 200, 330]))] + [int(rng.choice([1, 1, 1, 1, 1, 2, 4, 16])) for _ in range(int(rng.integers(4, 30)))]
+    for i, Lq in enumerate(steps):
+        k, kd = randn(rng, (B, Hkv, Lq, Dk), dtype)
+        v, vd = randn(rng, (B, Hkv, Lq, Dv), dtype)
+        q, qd = randn(rng, (B, Hkv * r, Lq, Dk), dtype)
+        if Lq == 1 and rng.random() < 0.7:
+            mask, om = kvhip.MaskMode.none(), O.Mask.NONE
+        else:
+            mask, om = kvhip.MaskMode.causal(), O.Mask.CAUSAL
+        out = np32(kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask))
+        ref = O.attention_with_cache_update(q, k, v, o, scale, om, NAME[dtype])
+        assert c.offset == o.offset and np.isfinite(out).all()
+        mx, mean = err_stats(out, ref)
+        # one step of the 16-bit output at the largest magnitude: with a handful of keys the outputs are as large as
+        # single V rows, and the oracle rounds the probabilities to the dtype where the kernels keep more bits
+        ulp = float(np.abs(ref).max()) * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10)
+        assert mx <= max(1e-2, 2 * ulp) and mean <= max(1e-3, ulp / 4), f"step {i} L={Lq} T={c.offset}: max-abs {mx:.3e} mean-abs {mean:.3e}"
+        if kind != "rotating" and rng.random() < 0.15:
+            t = int(rng.integers(0, 5))
+            assert c.trim(t) == o.trim(t)
