@@ -114,3 +114,32 @@ def test_decode_sequences_through_the_dispatcher(seed):
         if kind != "rotating" and rng.random() < 0.15:
             t = int(rng.integers(0, 5))
             assert c.trim(t) == o.trim(t)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_make_mask_between_drawn_updates(seed):
+    """`makeMask(n:windowSize:returnArray:)` (KVCache.swift:236-275, 834-871) of a ring or a simple cache at drawn
+    offsets: the same mode as the reference's, and the same array where it gives one."""
+    from kvhip import _lib as L
+    rng = np.random.default_rng(13000 + seed)
+    M = int(rng.choice([5, 8, 16, 33, 64]))
+    if seed % 4 != 3:
+        keep = min(int(rng.choice([0, 1, 4])), M - 1)
+        c, o = kvhip.RotatingKVCache(M, keep=keep), O.RotatingKVCache(M, keep=keep)
+    else:
+        c, o = kvhip.KVCacheSimple(), O.KVCacheSimple("float16")
+    pos = 0
+    for it in range(int(rng.integers(1, 40))):
+        n = int(rng.choice([1, 1, 2, 5, M, M + 2]))
+        w = [None, 1, 3, M // 2, M, 2 * M][int(rng.integers(6))]
+        ra = bool(rng.integers(2))
+        m, om = c.make_mask(n, w, ra), o.make_mask(n, w, ra)
+        what = f"update {it}, offset {o.offset}, n {n}, window {w}, returnArray {ra}"
+        if om.mode == "array":
+            assert np.array_equal(m.array.cpu().numpy(), om.array), what
+        else:
+            assert m.mode == (L.MASK_NONE if om.mode == "none" else L.MASK_CAUSAL), what
+        Lw = int(rng.choice([1, 1, 1, 2, M // 2 + 1, M + 1]))
+        (k, v), _ = positioned(pos, pos + Lw, D=4)
+        drive_pair(c, o, k, v, torch.float16)
+        pos += Lw
