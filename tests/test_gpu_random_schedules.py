@@ -143,3 +143,47 @@ def test_make_mask_between_drawn_updates(seed):
         (k, v), _ = positioned(pos, pos + Lw, D=4)
         drive_pair(c, o, k, v, torch.float16)
         pos += Lw
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_prompt_cache_files_of_drawn_cache_lists(seed, tmp_path):
+    """`savePromptCache` / `loadPromptCache` (KVCache.swift:1797-2249) over lists of caches of drawn kinds, dtypes,
+    head sizes and histories (never written, written, trimmed, trimmed back to empty): the loaded caches hold the
+    same state and metaState, and both lists continue alike."""
+    rng = np.random.default_rng(15000 + seed)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+
+    def rand(shape, dtype):
+        return torch.randn(*shape, generator=g, device="cuda").to(dtype)
+
+    caches = []
+    for _ in range(int(rng.integers(1, 6))):
+        kind = int(rng.integers(3))
+        dtype = [torch.float16, torch.bfloat16, torch.float32][int(rng.integers(3))]
+        B, H = int(rng.integers(1, 3)), int(rng.integers(1, 3))
+        Dk, Dv = [(64, 64), (128, 128), (96, 96), (192, 128), (64, 32)][int(rng.integers(5))]
+        if kind == 0:
+            c = kvhip.KVCacheSimple()
+        elif kind == 1:
+            c = kvhip.RotatingKVCache(int(rng.choice([8, 33, 64])), keep=int(rng.choice([0, 2])))
+        else:
+            c = kvhip.QuantizedKVCache(int(rng.choice([32, 64])), int(rng.choice([2, 3, 4, 5, 6, 8])))
+        for _ in range(int(rng.integers(0, 4))):
+            L = int(rng.choice([1, 3, 40, 70]))
+            (c.update_quantized if kind == 2 else c.update)(rand((B, H, L, Dk), dtype), rand((B, H, L, Dv), dtype), fetch=False)
+            if kind != 1 and rng.random() < 0.3:
+                c.trim(int(rng.choice([1, 2, 1000])))
+        caches.append((c, kind, dtype, B, H, Dk, Dv))
+    url = str(tmp_path / "drawn.safetensors")
+    kvhip.save_prompt_cache(url, [c[0] for c in caches], {"seed": str(seed)})
+    loaded, meta = kvhip.load_prompt_cache(url)
+    assert meta.get("seed") == str(seed) and len(loaded) == len(caches)
+    for (c, kind, dtype, B, H, Dk, Dv), r in zip(caches, loaded):
+        assert type(r) is type(c) and r.meta_state == c.meta_state and r.offset == c.offset
+        a, b = c.state, r.state
+        assert len(a) == len(b) and all(torch.equal(x, y) for x, y in zip(a, b))
+        k, v = rand((B, H, 2, Dk), dtype), rand((B, H, 2, Dv), dtype)
+        (c.update_quantized if kind == 2 else c.update)(k, v, fetch=False)
+        (r.update_quantized if kind == 2 else r.update)(k, v, fetch=False)
+        assert r.meta_state == c.meta_state and all(torch.equal(x, y) for x, y in zip(c.state, r.state))
