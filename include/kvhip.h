@@ -244,9 +244,12 @@ kvhip_status kvhip_cache_attend(kvhip_cache *cache, const void *queries, int32_t
  * reference.  Same arguments, same kernels and the same results as kvhip_cache_attend, but the
  * kernels' scratch (the partial results of the sequence spans) lives in a fixed array of
  * KVHIP_STATIC_SCRATCH_BYTES that every device the library was initialised on holds until the
- * process ends, and the call makes no hipMalloc / hipFree.  A call that needs more scratch than
- * that (the plain kernel on long sequences; every split-sequence decode shape fits) returns
- * KVHIP_ERR_UNSUPPORTED and enqueues nothing.  Nothing in the array has to start from zero:
+ * process ends, and the call makes no hipMalloc / hipFree.  The tuned kernels plan for that
+ * amount: they divide the sequence over fewer spans or key-range parts until the partials fit
+ * (a single span or part needs none), so they take every shape; where that gives another number of
+ * parts than kvhip_cache_attend would use, the float32 sums are formed in another order.  Only the
+ * plain kernel, which keeps one float per (query row, key), can need more than the array holds: such
+ * a call returns KVHIP_ERR_UNSUPPORTED and enqueues nothing.  Nothing in the array has to start from zero:
  * each span writes its partial before the merge reads it.  All calls on one device share the
  * array, so two calls whose device work can overlap (different streams, or a captured graph
  * replayed beside eager calls) race; calls on one stream are ordered and safe.

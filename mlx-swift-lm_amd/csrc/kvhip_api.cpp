@@ -72,6 +72,7 @@ static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
 struct Slab {
     void *base = nullptr;
     int64_t first_page = 0, pages = 0;
+    size_t bytes = 0;  // size of the allocation (at least what the pages need: it may come from the pool)
 };
 
 struct kvhip_cache {
@@ -113,7 +114,7 @@ struct kvhip_cache {
     size_t ws_bytes = 0;
     // buffers replaced by larger ones while work that reads them may still be in flight: kept
     // until the cache is freed (hipFree would wait for the whole device)
-    std::vector<void *> parked;
+    std::vector<std::pair<void *, size_t>> parked;
     // the stream the cache's device work was last enqueued on: freeing the cache releases its
     // memory behind that work instead of waiting for it
     mutable hipStream_t last_stream = nullptr;
@@ -126,44 +127,113 @@ namespace {
 
 // ---- page storage: slabs of pages behind a page table ------------------------------------------
 // Device buffers that work in flight may still read (page tables and page slabs that were
-// replaced) cannot be freed on the spot: hipFree waits for the whole device.  They are handed
-// over here and freed by the next call that is allowed to block (kvhip_sync, kvhip_cache_free,
-// kvhip_cache_reserve), each once an event recorded behind its last reader has completed.
+// replaced, the memory of a freed cache) cannot be freed on the spot: hipFree waits for the whole
+// device.  They are retired behind an event recorded on the stream of their last reader.  Once
+// that event has completed (hipEventQuery: no waiting) a buffer moves to a free list, from which
+// later allocations of a similar size are served instead of hipMalloc, so a loop that creates,
+// grows and frees caches without ever calling a blocking entry point neither waits nor keeps
+// growing the device's memory.  Buffers the free list holds beyond its limits, and everything on
+// it when a blocking call runs (kvhip_sync, kvhip_cache_reserve, a hipMalloc that failed), are
+// released with hipFree there.  Only the stream a cache was last used on is tracked: a caller who
+// reads one cache on several streams orders them before kvhip_cache_free.
+struct Buf {
+    void *p = nullptr;
+    size_t bytes = 0;  // 0: size not recorded, never reused
+    int dev = 0;
+};
 struct Retired {
     hipEvent_t done;
-    std::vector<void *> ptrs;
+    std::vector<Buf> bufs;
 };
 std::mutex g_retired_mu;
 std::vector<Retired> g_retired;
+std::vector<Buf> g_free;                          // finished with, kept for reuse
+constexpr size_t POOL_MAX_BUFS = 64;              // what the free list may hold after a blocking call
+constexpr size_t POOL_MAX_BYTES = (size_t)4 << 30;
 
-void retire(std::vector<void *> &&ptrs, hipStream_t stream) {
+int current_device() {
+    int d = 0;
+    if (hipGetDevice(&d) != hipSuccess) (void)hipGetLastError();
+    return d;
+}
+
+void retire(std::vector<std::pair<void *, size_t>> &&ptrs, hipStream_t stream) {
     if (ptrs.empty()) return;
     Retired r;
-    r.ptrs = std::move(ptrs);
+    const int dev = current_device();
+    for (auto &q : ptrs) r.bufs.push_back(Buf{q.first, q.second, dev});
     if (hipEventCreateWithFlags(&r.done, hipEventDisableTiming) != hipSuccess || hipEventRecord(r.done, stream) != hipSuccess) {
         (void)hipGetLastError();
         (void)hipDeviceSynchronize();
-        for (void *p : r.ptrs) (void)hipFree(p);
+        for (const Buf &b : r.bufs) (void)hipFree(b.p);
         return;
     }
     std::lock_guard<std::mutex> lock(g_retired_mu);
     g_retired.push_back(std::move(r));
 }
 
-// Frees what has been retired and is no longer in use.  Blocks (hipFree does): never on the hot path.
-void reap_retired() {
-    std::lock_guard<std::mutex> lock(g_retired_mu);
+// Moves retired buffers whose readers have finished to the free list.  Never waits.  (lock held)
+void harvest_locked() {
     for (size_t i = 0; i < g_retired.size();) {
         if (hipEventQuery(g_retired[i].done) != hipSuccess) {
             (void)hipGetLastError();
             ++i;
             continue;
         }
-        for (void *p : g_retired[i].ptrs) (void)hipFree(p);
+        for (const Buf &b : g_retired[i].bufs) g_free.push_back(b);
         (void)hipEventDestroy(g_retired[i].done);
         g_retired[i] = std::move(g_retired.back());
         g_retired.pop_back();
     }
+}
+
+// hipMalloc, or a finished buffer of at least `bytes` and at most 1.5 times that from the free list.
+// `got` receives the size of what was handed out.  Only enqueue-free work: usable on the hot path.
+hipError_t pool_alloc(void **out, size_t bytes, size_t *got) {
+    {
+        std::lock_guard<std::mutex> lock(g_retired_mu);
+        harvest_locked();
+        const int dev = current_device();
+        int best = -1;
+        for (size_t i = 0; i < g_free.size(); ++i) {
+            const Buf &b = g_free[i];
+            if (b.dev != dev || b.bytes < bytes || b.bytes > bytes + bytes / 2) continue;
+            if (best < 0 || b.bytes < g_free[best].bytes) best = (int)i;
+        }
+        if (best >= 0) {
+            *out = g_free[best].p;
+            *got = g_free[best].bytes;
+            g_free[best] = g_free.back();
+            g_free.pop_back();
+            return hipSuccess;
+        }
+    }
+    *got = bytes;
+    return hipMalloc(out, bytes);
+}
+
+// Releases what the free list holds beyond its limits (`all`: everything).  Blocks (hipFree does): never on
+// the hot path.
+void reap_retired(bool all = false) {
+    std::vector<Buf> drop;
+    {
+        std::lock_guard<std::mutex> lock(g_retired_mu);
+        harvest_locked();
+        size_t total = 0;
+        std::vector<Buf> keep;
+        // the most recently finished buffers are the likeliest to be asked for again
+        for (size_t i = g_free.size(); i-- > 0;) {
+            const Buf &b = g_free[i];
+            if (!all && b.bytes > 0 && keep.size() < POOL_MAX_BUFS && total + b.bytes <= POOL_MAX_BYTES) {
+                keep.push_back(b);
+                total += b.bytes;
+            } else {
+                drop.push_back(b);
+            }
+        }
+        g_free.swap(keep);
+    }
+    for (const Buf &b : drop) (void)hipFree(b.p);
 }
 
 // The same when `stream` has nothing in flight (then hipFree has little to wait for).
@@ -177,15 +247,15 @@ size_t align256(size_t n) { return (n + 255) / 256 * 256; }
 // Gives up the cache's pages and page table: freed at once when nothing in flight can read them
 // (`drained`), otherwise retired behind the work enqueued on `stream` so far.
 void drop_pages(kvhip_cache *c, hipStream_t stream, bool drained) {
-    std::vector<void *> ptrs;
-    for (const Slab &sl : c->slabs) ptrs.push_back(sl.base);
-    if (c->st.pt) ptrs.push_back(const_cast<PageEntry *>(c->st.pt));
+    std::vector<std::pair<void *, size_t>> ptrs;
+    for (const Slab &sl : c->slabs) ptrs.push_back({sl.base, sl.bytes});
+    if (c->st.pt) ptrs.push_back({const_cast<PageEntry *>(c->st.pt), (size_t)0});
     c->slabs.clear();
     c->st.pt = nullptr;
     c->cap_pages = 0;
     c->pt_cap = 0;
     if (drained) {
-        for (void *p : ptrs) (void)hipFree(p);
+        for (auto &q : ptrs) (void)hipFree(q.first);
     } else {
         retire(std::move(ptrs), stream);
     }
@@ -252,10 +322,10 @@ kvhip_status ensure_slots(kvhip_cache *c, int64_t slots, hipStream_t stream, boo
         int64_t cap = std::max<int64_t>(c->pt_cap * 2, 64);
         while (cap < pages) cap *= 2;
         void *npt = nullptr;
-        KV_HIP(hipMalloc(&npt, (size_t)cap * sizeof(PageEntry)));
+        KV_HIP(hipMalloc(&npt, (size_t)cap * sizeof(PageEntry)));  // (a few KB: not worth the pool)
         if (c->cap_pages > 0)
             KV_HIP_OR(launch_copy_bytes(npt, st.pt, (size_t)c->cap_pages * sizeof(PageEntry), stream), (void)hipFree(npt));
-        if (st.pt) retire({const_cast<PageEntry *>(st.pt)}, stream);
+        if (st.pt) retire({{const_cast<PageEntry *>(st.pt), (size_t)0}}, stream);
         c->st.pt = static_cast<PageEntry *>(npt);
         c->pt_cap = cap;
     }
@@ -265,11 +335,13 @@ kvhip_status ensure_slots(kvhip_cache *c, int64_t slots, hipStream_t stream, boo
     const size_t part[4] = {align256(stride[0] * add), align256(stride[1] * add), align256(stride[2] * add), align256(stride[3] * add)};
     const size_t bytes = part[0] + part[1] + part[2] + part[3];
     void *base = nullptr;
-    hipError_t e = hipMalloc(&base, bytes);
+    size_t got = bytes;
+    hipError_t e = pool_alloc(&base, bytes, &got);
     if (e != hipSuccess) {  // memory of freed caches may still be waiting for its release: wait for it and retry
         (void)hipGetLastError();
         (void)hipDeviceSynchronize();
-        reap_retired();
+        reap_retired(true);
+        got = bytes;
         e = hipMalloc(&base, bytes);
     }
     if (e != hipSuccess)
@@ -287,6 +359,7 @@ kvhip_status ensure_slots(kvhip_cache *c, int64_t slots, hipStream_t stream, boo
     sl.base = base;
     sl.first_page = c->cap_pages;
     sl.pages = add;
+    sl.bytes = got;
     c->slabs.push_back(sl);
     c->cap_pages = pages;
     if (c->kind == KVHIP_KIND_ROTATING) c->used.resize((size_t)c->cap_slots(), 0);
@@ -299,10 +372,11 @@ kvhip_status ensure_ws(kvhip_cache *c, size_t bytes, hipStream_t) {
     if (bytes <= c->ws_bytes) return KVHIP_OK;
     const size_t want = std::max(bytes + bytes / 4, 2 * c->ws_bytes);
     void *p = nullptr;
-    KV_HIP(hipMalloc(&p, want));
-    if (c->ws) c->parked.push_back(c->ws);
+    size_t got = want;
+    KV_HIP(pool_alloc(&p, want, &got));
+    if (c->ws) c->parked.push_back({c->ws, c->ws_bytes});
     c->ws = static_cast<float *>(p);
-    c->ws_bytes = want;
+    c->ws_bytes = got;
     return KVHIP_OK;
 }
 
@@ -717,19 +791,19 @@ void kvhip_cache_free(kvhip_cache *c) {
     // memory is handed to the retired list behind an event on that stream and released later,
     // so that dropping a cache (a conversion replacing it, the end of a round) does not make the
     // host wait for the device.
-    std::vector<void *> ptrs;
-    for (const Slab &sl : c->slabs) ptrs.push_back(sl.base);
-    if (c->st.pt) ptrs.push_back(const_cast<PageEntry *>(c->st.pt));
-    if (c->ws) ptrs.push_back(c->ws);
-    if (c->stage_tmp_k) ptrs.push_back(c->stage_tmp_k);
-    if (c->stage_tmp_v) ptrs.push_back(c->stage_tmp_v);
-    for (void *p : c->parked) ptrs.push_back(p);
+    std::vector<std::pair<void *, size_t>> ptrs;
+    for (const Slab &sl : c->slabs) ptrs.push_back({sl.base, sl.bytes});
+    if (c->st.pt) ptrs.push_back({const_cast<PageEntry *>(c->st.pt), (size_t)0});
+    if (c->ws) ptrs.push_back({c->ws, c->ws_bytes});
+    if (c->stage_tmp_k) ptrs.push_back({c->stage_tmp_k, (size_t)0});
+    if (c->stage_tmp_v) ptrs.push_back({c->stage_tmp_v, (size_t)0});
+    for (auto &q : c->parked) ptrs.push_back(q);
     const hipStream_t stream = c->last_stream;
     const bool used = c->used_stream;
     delete c;
     if (ptrs.empty()) return;
     if (!used) {  // no device work ever touched it
-        for (void *p : ptrs) (void)hipFree(p);
+        for (auto &q : ptrs) (void)hipFree(q.first);
         return;
     }
     retire(std::move(ptrs), stream);
@@ -941,6 +1015,7 @@ kvhip_status attend_impl(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, i
         }
     }
     hipStream_t s = S(c, stream);
+    a.workspace_cap = fixed ? fixed_bytes : 0;
     if (new_k) {
         if (g_policy == 0 && attend_decode_fuses_append(a)) {
             a.new_k = new_k;
@@ -1359,8 +1434,8 @@ kvhip_status kvhip_cache_stage_commit(kvhip_cache *c, int64_t retaining, void *s
         if ((size_t)keep > c->stage_tmp_rows) {
             // a larger pair replaces the old one, which an earlier commit's append may still read:
             // it stays allocated until the cache is freed (no wait for the device here)
-            if (c->stage_tmp_k) c->parked.push_back(c->stage_tmp_k);
-            if (c->stage_tmp_v) c->parked.push_back(c->stage_tmp_v);
+            if (c->stage_tmp_k) c->parked.push_back({c->stage_tmp_k, (size_t)0});
+            if (c->stage_tmp_v) c->parked.push_back({c->stage_tmp_v, (size_t)0});
             c->stage_tmp_k = c->stage_tmp_v = nullptr;
             c->stage_tmp_rows = 0;
             const size_t rows = (size_t)std::max<int64_t>(2 * keep, 16);

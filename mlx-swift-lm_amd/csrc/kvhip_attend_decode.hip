@@ -1041,7 +1041,7 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 // row and write the output row
 template <int D, int DT>
 __global__ void __launch_bounds__((D + 63) / 64 * 64)
-combine_kernel(AttendArgs a, int nsplit, int rr, int ragged) {
+combine_kernel(AttendArgs a, int nsplit, int rr) {
     constexpr int NT = (D + 63) / 64 * 64;
     __shared__ float w_s[512];  // weight of each span for this row (nsplit <= 512)
     __shared__ float red_s[4];
@@ -1050,12 +1050,7 @@ combine_kernel(AttendArgs a, int nsplit, int rr, int ragged) {
     const int r = a.Hq / a.Hkv;
     const int rep = i / a.L, l = i - rep * a.L;
     const size_t sstride = (size_t)rr * (D + 2);
-    size_t first_slot = (size_t)bh * nsplit;
-    if (ragged) {  // span slots shared over the batch in proportion to length: this row's are [first, first + count)
-        const RaggedSpan rs = ragged_span(a.mask, a.B, a.L, a.T, (a.slots + TILE - 1) / TILE, nsplit, -1, b, WAVES);
-        first_slot = (size_t)hk * nsplit + rs.first;
-        nsplit = rs.count;
-    }
+    const size_t first_slot = (size_t)bh * nsplit;
     const float *part = a.workspace + first_slot * sstride + (size_t)i * (D + 2);
     const int t = threadIdx.x;
     const int d = t < D ? t : 0;  // threads past the last column read column 0 and write nothing
@@ -1164,8 +1159,8 @@ Plan plan_for(const AttendArgs &a) {
     int want = (a.st.bits != 0 ? 256 * 2 : 256) / BH;
     if (want < 1) want = 1;
     int per = (p.tiles_total + want - 1) / want;
-    // KVHIP_DECODE_TILES (read once) forces the span size in tiles: a measurement aid
-    static const int forced_tiles = getenv("KVHIP_DECODE_TILES") ? atoi(getenv("KVHIP_DECODE_TILES")) : 0;
+    // KVHIP_DECODE_TILES forces the span size in tiles (timing builds only: measure_knob)
+    static const int forced_tiles = measure_knob("KVHIP_DECODE_TILES", 0);
     if (forced_tiles > 0) per = forced_tiles;
     // short sequences (up to 1024 quantized or 512 full-precision rows): one span per pair, so the
     // kernel writes the output rows itself and the merge launch, which costs more than the split
@@ -1187,17 +1182,9 @@ Plan plan_for(const AttendArgs &a) {
     const bool ident = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
     if (a.mask.mode == KVHIP_MASK_WINDOW && (a.mask.left_pad || a.mask.lengths) && forced_tiles <= 0 && ident) {
         p.tiles_per_wg = 0;
-        // KVHIP_RAGGED_SPANS (read once) forces the number of spans per batch row: a measurement aid
-        static const int forced_spans = getenv("KVHIP_RAGGED_SPANS") ? atoi(getenv("KVHIP_RAGGED_SPANS")) : 0;
+        // KVHIP_RAGGED_SPANS forces the number of spans per batch row (timing builds only: measure_knob)
+        static const int forced_spans = measure_knob("KVHIP_RAGGED_SPANS", 0);
         if (forced_spans > 0) p.nsplit = std::min(forced_spans, 512);
-        // the 16-row kernel goes further: a kv head's span slots are shared by its batch rows in
-        // proportion to their lengths (ragged_span), as many slots as workgroups are resident at once
-        static const bool prop_on = getenv("KVHIP_PROPORTIONAL_SPANS") != nullptr;
-        if (a.st.bits != 0 && p.rg >= 2 && a.B <= 64 && prop_on) {
-            p.tiles_per_wg = -1;
-            p.nsplit = std::max(512 / a.Hkv, 2 * a.B);
-            if (p.nsplit > 512) p.nsplit = 512;  // (more than 256 batch rows would be needed: not with B <= 64)
-        }
     } else if (a.st.bits != 0 && p.nsplit >= 2 && want <= 4 && p.rg == 1 && a.st.Dk != 96 && a.mask.mode != KVHIP_MASK_ARRAY &&
                forced_tiles <= 0) {
         // 128 pairs or more: workgroups of 8 wavefronts, one per CU -- the same wavefronts per CU
@@ -1211,6 +1198,19 @@ Plan plan_for(const AttendArgs &a) {
         per8 = (per8 + p.nw - 1) / p.nw * p.nw;
         p.tiles_per_wg = per8;
         p.nsplit = (p.tiles_total + per8 - 1) / per8;
+    }
+    // a caller with a fixed amount of scratch: fewer, longer spans until the partials fit (one span has none)
+    if (a.workspace_cap) {
+        const size_t per_span = (size_t)BH * (a.st.bits != 0 && (p.rg >= 2 || a.st.Dk == 96) ? 16 : 4 * p.rg) *
+                                (a.st.Dk + 2) * sizeof(float);
+        while (p.nsplit > 1 && per_span * p.nsplit > a.workspace_cap) {
+            if (p.tiles_per_wg > 0) {
+                p.tiles_per_wg *= 2;
+                p.nsplit = (p.tiles_total + p.tiles_per_wg - 1) / p.tiles_per_wg;
+            } else {
+                p.nsplit /= 2;
+            }
+        }
     }
     return p;
 }
@@ -1260,10 +1260,10 @@ hipError_t profile_read(int *launches, double *total_ms) {
     return hipSuccess;
 }
 
-hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s, int ragged) {
+hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s) {
     const int R = (a.Hq / a.Hkv) * a.L;
     dim3 grid(R, a.st.BH);
-    if (rows > 16 && !ragged && nsplit <= 8 && rows == R) {  // the prefill tiles' parts
+    if (rows > 16 && nsplit <= 8 && rows == R) {  // the prefill tiles' parts
         dim3 grid4((R + 3) / 4, a.st.BH);
 #define CMBR(D)                                                                                      \
     do {                                                                                             \
@@ -1280,8 +1280,8 @@ hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t
     }
 #define CMB(D)                                                                                       \
     do {                                                                                             \
-        if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL((combine_kernel<D, 0>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows, ragged); \
-        else hipLaunchKernelGGL((combine_kernel<D, 1>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows, ragged);       \
+        if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL((combine_kernel<D, 0>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows); \
+        else hipLaunchKernelGGL((combine_kernel<D, 1>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows);       \
     } while (0)
     // (the partials hold output columns: the head size of the values)
     if (a.st.Dv == 64) CMB(64);
@@ -1315,7 +1315,7 @@ bool attend_decode_supported(const AttendArgs &a) {
 // The 4-row quantized kernel and the full-precision decode kernel, without a mask, write the step's new row themselves.
 bool attend_decode_fuses_append(const AttendArgs &a) {
     if (!attend_decode_supported(a) || a.L != 1 || a.mask.mode != KVHIP_MASK_NONE) return false;
-    static const bool off = getenv("KVHIP_NO_FUSED_APPEND") != nullptr;  // measurement aid
+    static const bool off = measure_knob("KVHIP_NO_FUSED_APPEND", 0) != 0;  // (timing builds only)
     if (off) return false;
     if (a.st.bits == 0) return true;  // the full-precision decode kernel, any of its row counts
     return (a.Hq / a.Hkv) * a.L <= 4 && a.st.Dk != 96;
@@ -1331,8 +1331,8 @@ static bool use_decode16(const AttendArgs &a, const Plan &p) { return a.st.bits 
 size_t attend_decode_workspace(const AttendArgs &a) {
     const Plan p = plan_for(a);
     const int rows = use_decode16(a, p) ? 16 : 4 * p.rg;
-    const size_t slots = p.tiles_per_wg < 0 ? (size_t)a.Hkv * p.nsplit : (size_t)a.st.BH * p.nsplit;
-    return slots * rows * (a.st.Dk + 2) * sizeof(float);
+    if (p.nsplit == 1) return 0;  // a single span writes the output rows itself: no partials
+    return (size_t)a.st.BH * p.nsplit * rows * (a.st.Dk + 2) * sizeof(float);
 }
 
 hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
@@ -1340,7 +1340,6 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
     const Plan p = plan_for(a);
     const Store &st = a.st;
     dim3 grid(p.nsplit, st.BH), block(WAVES * 64);  // the quantized kernel sets its own block size
-    const int R = (a.Hq / a.Hkv) * a.L;
     const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
 #define DEC_K(BITS, D, GS, DT, RG, MM, NW)                                                                \
     hipLaunchKernelGGL((decode_kernel<BITS, D, GS, DT, RG, MM, NW>), grid, dim3(NW * 64), 0, s, a,        \
@@ -1360,7 +1359,7 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
         }                                                                                                 \
         profile_mark(s, false);                                                                           \
         if (p.nsplit > 1)                                                                                 \
-            (void)launch_combine(a, p.nsplit, 4 * RG, s, 0);                                             \
+            (void)launch_combine(a, p.nsplit, 4 * RG, s);                                                \
     } while (0)
 #define DEC_RG(BITS, D, GS, DT) DEC(BITS, D, GS, DT, 1) /* more rows: the 16-row kernel above */
     if (use_decode16(a_in, p)) {
@@ -1368,7 +1367,7 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
         hipError_t e = launch_attend_decode16(a_in, p.tiles_total, p.tiles_per_wg, p.nsplit, s);
         profile_mark(s, false);
         if (e != hipSuccess) return e;
-        if (p.nsplit > 1) return launch_combine(a_in, p.nsplit, 16, s, p.tiles_per_wg < 0 ? 1 : 0);
+        if (p.nsplit > 1) return launch_combine(a_in, p.nsplit, 16, s);
         return hipSuccess;
     }
 #define DEC_DT(BITS, D, GS)                                \
@@ -1394,7 +1393,7 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
                            p.tiles_per_wg, p.nsplit);                                                     \
         profile_mark(s, false);                                                                           \
         if (p.nsplit > 1)                                                                                 \
-            (void)launch_combine(a, p.nsplit, 4 * RG, s, 0);                                             \
+            (void)launch_combine(a, p.nsplit, 4 * RG, s);                                                \
     } while (0)
 #define FP_MI(D, DT, RG)                                          \
     do {                                                          \

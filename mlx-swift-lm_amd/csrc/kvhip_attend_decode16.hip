@@ -133,21 +133,6 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     __shared__ __attribute__((aligned(16))) uint32_t sbuf[WAVES][2][2][SB_WORDS];  // [wavefront][tile parity][K, V][pairs]
 
     // ---- span of this workgroup (as in the 4-row kernel) -----------------------------------
-    // tiles_per_wg < 0: a ragged batch, grid (nsplit span slots, kv heads): the slots of a kv head are
-    // shared by its batch rows in proportion to their lengths (ragged_span)
-    RaggedSpan rs;
-    rs.b = -1;
-    if constexpr (MM == 1) {
-        if (tiles_per_wg < 0) {
-            rs = ragged_span(a.mask, a.B, a.L, a.T, tiles_total, nsplit, blockIdx.x, -1, WAVES);
-            if (rs.b < 0) return;  // an unused slot (uniform over the workgroup)
-            hk = blockIdx.y;
-            b = rs.b;
-            bh = b * a.Hkv + hk;
-            split = blockIdx.x - rs.first;
-            part_slot = (size_t)hk * nsplit + blockIdx.x;
-        }
-    }
     if constexpr (MM == 1) {
         // a ragged batch whose rows divide their own ranges over the same number of spans: long and short
         // rows are paired on the CUs (balanced_row)
@@ -160,10 +145,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     const SymMask sym = sym_mask_init(a.mask, b, a.L, a.T);
     int tile_begin = split * tiles_per_wg;
     int tile_end = min(tiles_total, tile_begin + tiles_per_wg);
-    if (MM == 1 && rs.b >= 0) {
-        tile_begin = rs.t_lo + split * rs.q;
-        tile_end = min(rs.t_hi, tile_begin + rs.q);
-    } else if constexpr (MM == 1) {
+    if constexpr (MM == 1) {
         int vis_lo, vis_hi;
         sym_mask_row_range(sym, vis_lo, vis_hi);
         int t_lo = max(0, vis_lo) >> 6, t_hi = min(tiles_total, (min(vis_hi, a.T - 1) >> 6) + 1);
@@ -627,7 +609,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 // 4 wavefronts); the caller merges the partials when nsplit > 1.
 hipError_t launch_attend_decode16(const AttendArgs &a, int tiles_total, int tiles_per_wg, int nsplit, hipStream_t s) {
     const Store &st = a.st;
-    dim3 grid(nsplit, tiles_per_wg < 0 ? a.Hkv : st.BH), block(WAVES * 64);  // (< 0: span slots shared over the batch)
+    dim3 grid(nsplit, st.BH), block(WAVES * 64);
     const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
 #define D16_M(BITS, D, GS, DT)                                                                                  \
     do {                                                                                                        \

@@ -561,7 +561,7 @@ bool attend_prefill_supported(const AttendArgs &a) {
 // used when that would leave the grid too small to fill 256 CUs twice over.
 static bool prefill_wide(const AttendArgs &a) {
     const int R = (a.Hq / a.Hkv) * a.L;
-    static const int forced = getenv("KVHIP_PREFILL_WIDE") ? atoi(getenv("KVHIP_PREFILL_WIDE")) : -1;  // measurement aid
+    static const int forced = measure_knob("KVHIP_PREFILL_WIDE", -1);  // (timing builds only)
     if (forced >= 0) return forced != 0 && a.st.Dk <= 128;
     return (size_t)((R + 127) / 128) * a.st.BH >= 512 && a.st.Dk <= 128;
 }
@@ -574,14 +574,17 @@ static int prefill_splits(const AttendArgs &a) {
     const size_t wgs = (size_t)((R + (wide ? 127 : 63)) / (wide ? 128 : 64)) * a.st.BH;
     // as many workgroups as are resident at once: three per CU, two at D = 256 (LDS) -- a part more
     // than that starts a second round that leaves half the CUs idle
-    static const int forced = getenv("KVHIP_PREFILL_TARGET") ? atoi(getenv("KVHIP_PREFILL_TARGET")) : 0;  // measurement aid
+    static const int forced = measure_knob("KVHIP_PREFILL_TARGET", 0);  // (timing builds only)
     const int target = forced > 0 ? forced : (a.st.Dk >= 256 ? 512 : 768);
     int n = (int)(target / (wgs ? wgs : 1));
     const int tiles = (a.slots + BN - 1) / BN;
     if (n > tiles / 8) n = tiles / 8;
     if (n > 8) n = 8;
     if (n < 2) return 1;
-    if ((size_t)a.st.BH * n * R * (a.st.Dv + 2) * sizeof(float) > ((size_t)256 << 20)) return 1;
+    const size_t per_part = (size_t)a.st.BH * R * (a.st.Dv + 2) * sizeof(float);
+    if (per_part * n > ((size_t)256 << 20)) return 1;
+    // a caller with a fixed amount of scratch: fewer parts until they fit (one part has no partials)
+    while (a.workspace_cap && n > 1 && per_part * n > a.workspace_cap) --n;
     return n;
 }
 

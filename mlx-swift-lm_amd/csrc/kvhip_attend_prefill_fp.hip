@@ -673,12 +673,8 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         // iteration for it, so the wait is short, and no LDS read of the next iteration meets a load
         // in flight into its buffer.  A plain barrier instead of __syncthreads(): nothing but LDS
         // traffic (drained here) has to be ordered across it.
-#ifndef KVHIP_PROBE_NOWAIT  // (timing probe: results are wrong without the wait)
         wait_all_loads();
-#endif
-#ifndef KVHIP_PROBE_NOBARRIER
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-#endif
     };
 
     if (v_lo < v_hi) {
@@ -762,9 +758,6 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         }
     }
 
-#if defined(KVHIP_PROBE_NOWAIT)
-    wait_all_loads();
-#endif
     // ---- normalise and store: lane (n, jj) holds out[q = n][d = 16 dt + 4 jj + i] ------------
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {

@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "kvhip.h"
 
@@ -282,6 +283,9 @@ struct AttendArgs {
     const void *new_k = nullptr;
     const void *new_v = nullptr;
     int new_slot = -1;
+    // Upper bound on the scratch a launch may plan for (0: none).  The planners then split the sequence over
+    // fewer spans or key-range parts, down to one, which needs no scratch at all.
+    size_t workspace_cap = 0;
 };
 // Whether launch_attend_decode writes a.new_k / a.new_v itself for these arguments.
 bool attend_decode_fuses_append(const AttendArgs &a);
@@ -297,11 +301,20 @@ bool attend_prefill_supported(const AttendArgs &a);
 size_t attend_prefill_workspace(const AttendArgs &a);
 // Merge `nsplit` partials per query row, laid out [bh][split][rows][D+2] in a.workspace
 // (out[D] unnormalised, running max, running sum), and write the normalised rows to a.out.
-// ragged: the partials lie in span slots shared over the batch (ragged_span, kvhip_mask.hpp)
-hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s, int ragged = 0);
+hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s);
 hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s);
 hipError_t launch_attend_decode16(const AttendArgs &a, int tiles_total, int tiles_per_wg, int nsplit, hipStream_t s);
 hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, hipStream_t s);
+// Switches for timing experiments (forced span sizes and the like) are read from the environment only in a
+// library built with -DKVHIP_MEASURE; the shipped build compiles every one of them to its default.
+#ifdef KVHIP_MEASURE
+inline int measure_knob(const char *name, int dflt) {
+    const char *v = getenv(name);
+    return v ? atoi(v) : dflt;
+}
+#else
+constexpr int measure_knob(const char *, int dflt) { return dflt; }
+#endif
 // Event bracket around the dominant kernel while profiling is enabled.
 void profile_enable(int every);
 void profile_mark(hipStream_t s, bool begin);

@@ -112,73 +112,6 @@ __device__ __forceinline__ void sym_mask_full_range(const SymMask &s, int &lo, i
     if (s.window > 0) lo = max(lo, s.offset + s.L - s.window);
 }
 
-// ---- spans in proportion to length, for ragged batches ------------------------------------------
-// Under an index-only mask with per-batch bounds (left padding, lengths) every batch row sees its
-// own range of 64-token tiles.  A kv head's NS span slots are shared by its B batch rows in
-// proportion to those ranges: a span covers q tiles -- q the smallest multiple of `waves` with
-// sum_b ceil(tiles_b / q) <= NS -- so a long row gets many spans, a short one few, and the launch
-// ends when the longest span does rather than when the longest row does.  Row b owns span slots
-// [first, first + count).  Every lane takes one batch row (B <= 64), so the whole plan costs one
-// round of loads and a handful of cross-lane steps; the attention kernel and the merge kernel
-// compute the same plan from the same inputs.
-struct RaggedSpan {
-    int b;           // batch row of span slot w, or -1 if the slot is unused
-    int first, count;  // span slots of that row
-    int t_lo, t_hi;  // its visible tiles [t_lo, t_hi)
-    int q;           // tiles per span
-};
-// w >= 0: the row that owns span slot w.  w < 0: row `row`.
-__device__ __forceinline__ RaggedSpan ragged_span(const MaskDev &m, int B, int L, int T, int tiles_total, int NS, int w,
-                                                  int row, int waves) {
-    const int lane = threadIdx.x & 63;
-    int t_lo = 0, t_hi = 0;
-    if (lane < B) {
-        const SymMask s = sym_mask_init(m, lane, L, T);
-        int vis_lo, vis_hi;
-        sym_mask_row_range(s, vis_lo, vis_hi);
-        t_lo = max(0, vis_lo) >> 6;
-        t_hi = min(tiles_total, (min(vis_hi, T - 1) >> 6) + 1);
-        if (sym_mask_some_row_empty(s)) {  // a fully masked row averages over every key
-            t_lo = 0;
-            t_hi = tiles_total;
-        }
-        t_hi = max(t_hi, t_lo);
-    }
-    const int tiles = lane < B ? max(t_hi - t_lo, 1) : 0;
-    int total = tiles;
-    for (int off = 1; off < 64; off <<= 1) total += __shfl_xor(total, off);
-    const int room = max(NS - B, 1);
-    int q = (total + room - 1) / room;
-    q = max((q + waves - 1) / waves * waves, waves);
-    const int cnt = lane < B ? (tiles + q - 1) / q : 0;
-    int incl = cnt;  // inclusive prefix sum over the lanes
-    for (int off = 1; off < 64; off <<= 1) {
-        const int v = __shfl_up(incl, off);
-        if (lane >= off) incl += v;
-    }
-    const int first = incl - cnt;
-    int src = row;
-    if (w >= 0) {
-        const unsigned long long own = __ballot(lane < B && w >= first && w < first + cnt);
-        src = own ? __ffsll(own) - 1 : -1;
-    }
-    RaggedSpan r;
-    r.b = src;
-    r.q = q;
-    if (src < 0) {
-        r.first = r.count = r.t_lo = r.t_hi = 0;
-        return r;
-    }
-    // (wave-uniform values: kept in scalar registers)
-    r.b = __builtin_amdgcn_readfirstlane(src);
-    r.q = __builtin_amdgcn_readfirstlane(q);
-    r.first = __builtin_amdgcn_readfirstlane(__shfl(first, src));
-    r.count = __builtin_amdgcn_readfirstlane(__shfl(cnt, src));
-    r.t_lo = __builtin_amdgcn_readfirstlane(__shfl(t_lo, src));
-    r.t_hi = __builtin_amdgcn_readfirstlane(__shfl(t_hi, src));
-    return r;
-}
-
 // ---- which batch row a workgroup row takes, for ragged batches ------------------------------------
 // Workgroups are started in id order, one per CU and then a second one per CU, so rows v and v + B/2 of a
 // launch of 512 workgroups share CUs.  Taking the batch rows in order of their visible length -- the first

@@ -38,7 +38,13 @@ Parity status of each function
   code first) is likewise restated from that file and pinned only by byte patterns
   worked out by hand (tests/test_oracle_kat.py) and by the pack / unpack round trip:
   **parity unpinned** against the MLX binary.
-* `quantized_matmul` / `softmax_last` rounding points and accumulation order:
+* `sdpa`, `quantized_sdpa`, `softmax_last`, `_apply_mask`, `round_to`: what they compute -- which query
+  heads share a kv head, the lower-right alignment of `.causal` with fewer queries than keys, how
+  [L,T], [B,1,L,T] and [B,Hq,L,T] masks broadcast, exclusion against addition, the float16 / bfloat16
+  rounding itself -- is pinned against an implementation that shares no code with this file: torch's CPU
+  `scaled_dot_product_attention` on the dequantised cache, `torch.softmax` and torch's dtype casts
+  (tests/test_oracle_kat.py, float32 to 1e-5; the 16-bit paths inside the stated tolerance of it).
+* `quantized_matmul` / `softmax_last` rounding points and accumulation order inside MLX:
   **parity unpinned** (tolerance-level only).  `softmax(precise: false)`, which
   KVCache.swift:2416 calls, accumulates in the input dtype on MLX's CPU backend
   (`softmax<T, AccT = T>`, mlx/backend/cpu/softmax.cpp); this oracle exponentiates

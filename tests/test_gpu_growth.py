@@ -157,3 +157,38 @@ def test_reserve_then_append_on_another_stream():
         side.synchronize()
         for i, (a, b) in enumerate(zip(st, o.get_state())):
             assert np.array_equal(np32(a), b) if i % 3 == 0 else bits_equal(a, b, torch.float16)
+
+
+def test_created_grown_and_freed_caches_reuse_their_memory_without_a_blocking_call():
+    # A serving loop that never calls kvhip_sync / kvhip_cache_reserve: caches are created, grown page by page,
+    # read and dropped while their work may still be in flight.  Their pages go to the library's free list once the
+    # work behind them has finished and later caches are served from it, so the device's free memory settles
+    # instead of shrinking by one cache per iteration.
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    B, H, D = 4, 8, 128
+    k = torch.randn(B, H, 2048, D, generator=g, device="cuda").half()
+    q = torch.randn(B, 32, 1, D, generator=g, device="cuda").half()
+    one = torch.randn(B, H, 1, D, generator=g, device="cuda").half()
+    per_cache = 2 * B * H * 6144 * D * 2
+    outs = []
+
+    def serve():
+        c = kvhip.KVCacheSimple()
+        for _ in range(3):               # grows by slabs: 2048, 4096, 6144 rows
+            c.update(k, k, fetch=False)
+        outs.append(c.update_attend(q, one, one, D ** -0.5))
+        del c                            # kvhip_cache_free with the stream possibly still busy
+
+    for _ in range(4):
+        serve()
+    torch.cuda.current_stream().synchronize()   # torch's own wait: the library is not told
+    free_mid = torch.cuda.mem_get_info()[0]
+    for _ in range(24):
+        serve()
+    torch.cuda.current_stream().synchronize()
+    free_end = torch.cuda.mem_get_info()[0]
+    assert free_mid - free_end < 3 * per_cache, (free_mid - free_end, per_cache)
+    assert all(torch.isfinite(o).all() for o in outs)
+    # and the answers do not depend on whose memory a cache got
+    assert all(torch.equal(outs[0], o) for o in outs[1:])

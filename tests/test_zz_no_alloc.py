@@ -87,3 +87,54 @@ def test_static_scratch_rejects_what_does_not_fit():
     assert not out.any(), "a rejected call must enqueue nothing"
     # the allocating entry point still serves it
     assert torch.isfinite(c.attend(q[:, :, :2].contiguous(), 0.2)).all()
+
+
+def test_static_scratch_alone_on_a_fresh_cache_allocates_nothing():
+    # a cache that has never gone through the allocating entry point, so its own workspace does not exist: the
+    # result must come from the fixed array.  Device memory is observed around the calls (hipMemGetInfo), and the
+    # result is checked against the oracle rather than against another call of the library.
+    from oracle import c_oracle as CO
+    from oracle import kv_oracle as O
+    rng = np.random.default_rng(11)
+    B, Hq, Hkv, T, D = 2, 8, 2, 9000, 128
+    k = O.round_to(rng.standard_normal((B, Hkv, T, D)).astype(np.float32), "float16")
+    v = O.round_to(rng.standard_normal((B, Hkv, T, D)).astype(np.float32), "float16")
+    qn = O.round_to(rng.standard_normal((B, Hq, 1, D)).astype(np.float32), "float16")
+    cache = kvhip.QuantizedKVCache(64, 4)
+    cache.update_quantized(torch.from_numpy(k).half().cuda(), torch.from_numpy(v).half().cuda(), fetch=False)
+    q = torch.from_numpy(qn).half().cuda()
+    out = torch.full((B, Hq, 1, D), float("nan"), dtype=torch.float16, device="cuda")
+    q4 = torch.from_numpy(O.round_to(rng.standard_normal((B, Hq, 4, D)).astype(np.float32), "float16")).half().cuda()
+    out4 = torch.full((B, Hq, 4, D), float("nan"), dtype=torch.float16, device="cuda")
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    cache.attend(q, D ** -0.5, out=out, static_scratch=True)                     # 4-row kernel, many spans
+    cache.attend(q4, D ** -0.5, kvhip.MaskMode.causal(), out=out4, static_scratch=True)  # 16-row kernel
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the allocation-free entry point changed the device's free memory"
+    o = O.QuantizedKVCache(64, 4, "float16")
+    qk, qv = o.update_quantized(k, v)
+    ref = CO.qsdpa(qn, qk, qv, D ** -0.5, None, 64, 4, "float16")
+    d = np.abs(out.float().cpu().numpy() - ref)
+    assert d.max() <= 1e-2 and d.mean() <= 1e-3
+    ref4 = CO.qsdpa(q4.float().cpu().numpy(), qk, qv, D ** -0.5, "causal", 64, 4, "float16")
+    d = np.abs(out4.float().cpu().numpy() - ref4)
+    assert d.max() <= 1e-2 and d.mean() <= 1e-3
+
+
+def test_static_scratch_takes_large_batches_and_plans_fewer_parts_when_the_array_is_small():
+    # many (batch row, kv head) pairs: one span each, the kernel writes the output itself and needs no scratch,
+    # whatever the number of pairs (1024 pairs x 16 rows x 258 floats would be 16.9 MB of partials)
+    big, g = filled(kvhip.QuantizedKVCache, 128, 8, 200, 256, torch.float16, 6, group_size=64, bits=4)
+    q = torch.randn(128, 32, 4, 256, generator=g, device="cuda").half()
+    got, want, family = both(big, q, 256 ** -0.5, kvhip.MaskMode.causal())
+    assert family == 1 and torch.equal(got, want)
+    del big
+    # a prompt chunk whose two key-range parts would need 25.5 MB of partials: the allocating entry point splits the
+    # keys, the allocation-free one plans a single part (another summation order: compared within the tolerance)
+    c, g = filled(kvhip.KVCacheSimple, 1, 8, 1024, 128, torch.float16, 7)
+    q = torch.randn(1, 32, 768, 128, generator=g, device="cuda").half()
+    got, want, family = both(c, q, 128 ** -0.5, kvhip.MaskMode.causal())
+    assert family == 3
+    d = (got.float() - want.float()).abs()
+    assert float(d.max()) <= 2e-3 and float(d.mean()) <= 1e-4
