@@ -167,6 +167,11 @@ int64_t kvhip_cache_presented_length(const kvhip_cache *cache);/* key extent `up
 /* Rows the device pages allocated so far can hold (a multiple of 256).  No counterpart in the
  * reference, whose `capacity` above is the extent of its arrays; for tests and measurements. */
 int64_t kvhip_cache_device_rows(const kvhip_cache *cache);
+/* Device slots a decode launch walks: one past the highest slot that holds a presented row.  Equal to
+ * the presented length except for a RotatingKVCache whose prompt chunks left unused slots between its
+ * rows (they are squeezed out once when the full ring settles into single-token steps).  No counterpart
+ * in the reference; for tests and measurements. */
+int64_t kvhip_cache_slot_span(const kvhip_cache *cache);
 int32_t kvhip_cache_is_trimmable(const kvhip_cache *cache, int64_t after_positions); /* isTrimmable(after:) */
 int64_t kvhip_cache_trim(kvhip_cache *cache, int64_t n);       /* trim(_:) -> positions trimmed */
 /* `offset` is a settable stored property in the reference (KVCache.swift:185;

@@ -818,6 +818,13 @@ int32_t kvhip_cache_bits(const kvhip_cache *c) { return c ? c->bits : -1; }
 int64_t kvhip_cache_capacity(const kvhip_cache *c) { return c ? c->ref_len : -1; }
 int64_t kvhip_cache_presented_length(const kvhip_cache *c) { return c ? c->presented : -1; }
 int64_t kvhip_cache_device_rows(const kvhip_cache *c) { return c ? c->cap_slots() : -1; }
+int64_t kvhip_cache_slot_span(const kvhip_cache *c) {
+    if (!c) return -1;
+    if (c->kind != KVHIP_KIND_ROTATING) return c->presented;
+    int64_t span = 0;
+    for (int32_t slot : c->rows) span = std::max<int64_t>(span, (int64_t)slot + 1);
+    return span;
+}
 
 int32_t kvhip_cache_is_trimmable(const kvhip_cache *c, int64_t after) {
     if (!c) return 0;

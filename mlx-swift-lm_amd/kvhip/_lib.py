@@ -69,6 +69,7 @@ SIGNATURES = {
     "kvhip_cache_capacity": (_I64, [_P]),
     "kvhip_cache_presented_length": (_I64, [_P]),
     "kvhip_cache_device_rows": (_I64, [_P]),
+    "kvhip_cache_slot_span": (_I64, [_P]),
     "kvhip_cache_is_trimmable": (_I32, [_P, _I64]),
     "kvhip_cache_trim": (_I64, [_P, _I64]),
     "kvhip_cache_set_offset": (_I32, [_P, _I64]),

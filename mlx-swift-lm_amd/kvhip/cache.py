@@ -145,6 +145,11 @@ class _Cache:
         return self._lib.kvhip_cache_device_rows(self._h)
 
     @property
+    def slot_span(self):
+        """Device slots a decode launch walks (one past the highest slot holding a presented row)."""
+        return self._lib.kvhip_cache_slot_span(self._h)
+
+    @property
     def presented_length(self):
         return self._lib.kvhip_cache_presented_length(self._h)
 
