@@ -1,6 +1,7 @@
 // Chunked-prefill attention tile on the matrix cores (gfx950, v_mfma_f32_16x16x32_f16) for
-// quantized caches (full-precision caches take the kernel of kvhip_attend_prefill_fp.hip),
-// and the launcher of both.
+// quantized caches of head size 96 and of keys 192 with values 128 (head sizes 64 / 128 / 256 take the
+// pipelined tile of kvhip_attend_prefill_q.hip, full-precision caches the kernel of
+// kvhip_attend_prefill_fp.hip), and the launcher of all three.
 //
 // Many query rows per kv head (r = Hq/Hkv heads times L new tokens).  One workgroup
 // (4 wavefronts) owns 128 query rows of one (batch, kv-head) pair -- 32 per wavefront
@@ -554,6 +555,7 @@ bool attend_prefill_supported(const AttendArgs &a) {
     if (s.Dk != 64 && s.Dk != 128 && s.Dk != 256 && s.Dk != 96 && !(s.Dk == 80 && s.bits == 0)) return false;
     if (s.bits != 0 && s.bits != 4 && s.bits != 8) return false;
     if (s.bits != 0 && s.gs < 32) return false;
+    if (s.bits != 0 && s.Dk != 96) return attend_prefill_q_supported(a);  // the pipelined tile: slots in presented order
     return true;  // 16 rows or fewer come here only when the decode kernels do not take the shape
 }
 
@@ -566,12 +568,29 @@ static bool prefill_wide(const AttendArgs &a) {
     return (size_t)((R + 127) / 128) * a.st.BH >= 512 && a.st.Dk <= 128;
 }
 
+// Query rows per workgroup.  The pipelined tile for quantized caches (kvhip_attend_prefill_q.hip) takes 256 rows
+// on 8 wavefronts at head size 128, one workgroup per CU, whenever that still gives every CU a workgroup: four
+// times as many rows share each converted tile (B1, 2048 x 8192, 4 bits: 552 against 446 TFLOP/s; a square causal
+// 4096 x 4096, which would leave half the CUs empty, stays on 64 rows: 480 against 380).  Otherwise 128 or 64 rows
+// on 4 wavefronts as above (quantized: 64).
+static int prefill_block_rows(const AttendArgs &a) {
+    const int R = (a.Hq / a.Hkv) * a.L;
+    if (a.st.bits != 0 && attend_prefill_q_supported(a)) {
+        static const int forced = measure_knob("KVHIP_PREFILL_ROWS", 0);  // (timing builds only)
+        if (forced > 0 && a.st.Dk == 128) return forced;
+        // (head size 64 measured faster on 64 rows: 363 / 393 against 340 / 362 TFLOP/s at 8 / 4 bits, B4 2048 x 4096)
+        return ((size_t)((R + 255) / 256) * a.st.BH >= 256 && a.st.Dk == 128) ? 256 : 64;
+    }
+    return prefill_wide(a) ? 128 : 64;
+}
+
 // Key-range parts per query block: only when the grid would leave most CUs without a
 // second workgroup, and only while the partials stay small.
 static int prefill_splits(const AttendArgs &a) {
     const int R = (a.Hq / a.Hkv) * a.L;
-    const bool wide = prefill_wide(a);
-    const size_t wgs = (size_t)((R + (wide ? 127 : 63)) / (wide ? 128 : 64)) * a.st.BH;
+    const int bm = prefill_block_rows(a);
+    if (bm == 256) return 1;  // (chosen only when the grid fills the chip)
+    const size_t wgs = (size_t)((R + bm - 1) / bm) * a.st.BH;
     // as many workgroups as are resident at once: three per CU, two at D = 256 (LDS) -- a part more
     // than that starts a second round that leaves half the CUs idle
     static const int forced = measure_knob("KVHIP_PREFILL_TARGET", 0);  // (timing builds only)
@@ -599,8 +618,8 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
     const int R = (a.Hq / a.Hkv) * a.L;
     // 128 query rows per workgroup reuse each staged tile twice as often; 64 rows are used
     // when that would leave the grid too small to fill 256 CUs twice over
-    const bool wide = prefill_wide(a);
-    const int bm = wide ? 128 : 64;
+    const int bm = prefill_block_rows(a);
+    const bool wide = bm == 128;
     const int nsplit = prefill_splits(a);
     dim3 grid((unsigned)((R + bm - 1) / bm) * st.BH * nsplit), block(256);  // linear: the kernel maps ids to tiles
     const bool ident = a.runs.n == 1 && a.runs.row0[0] == 0 && a.runs.phys0[0] == 0;
@@ -647,13 +666,16 @@ hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s) {
     do {                                              \
         if (st.Dk == 192) { /* keys 192 / values 128: 64 query rows per workgroup */ \
             if (st.dtype == KVHIP_F16) PF_MLA(BITS, 0); else PF_MLA(BITS, 1);        \
-        } else if (st.Dk == 64) PF_DT(BITS, 64);             \
-        else if (st.Dk == 96) PF_DT(BITS, 96);        \
-        else if (st.Dk == 128) PF_DT(BITS, 128);      \
-        else if (st.dtype == KVHIP_F16) PF(BITS, 256, 0, 1); /* 64 query rows per workgroup only */ \
-        else PF(BITS, 256, 1, 1);                     \
+        } else if (st.Dk == 96) PF_DT(BITS, 96);      \
+        else return hipErrorInvalidValue; /* 64 / 128 / 256 are served above */ \
     } while (0)
-    if (st.bits == 4) PF_D(4);
+    if (st.bits != 0 && attend_prefill_q_supported(a)) {
+        // head sizes 64 / 128 / 256: the pipelined tile of kvhip_attend_prefill_q.hip
+        profile_mark(s, true);
+        hipError_t e = launch_attend_prefill_q(a, nsplit, bm, s);
+        profile_mark(s, false);
+        if (e != hipSuccess) return e;
+    } else if (st.bits == 4) PF_D(4);
     else if (st.bits == 8) PF_D(8);
     else {
         // full-precision caches have their own double-buffered kernel

@@ -305,6 +305,10 @@ hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t
 hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s);
 hipError_t launch_attend_decode16(const AttendArgs &a, int tiles_total, int tiles_per_wg, int nsplit, hipStream_t s);
 hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, hipStream_t s);
+// The pipelined tile for quantized caches (head sizes 64 / 128 / 256, slots in presented order).
+bool attend_prefill_q_supported(const AttendArgs &a);
+// rows: query rows per workgroup, 64 (4 wavefronts) or 256 (8 wavefronts; head size 128)
+hipError_t launch_attend_prefill_q(const AttendArgs &a, int nsplit, int rows, hipStream_t s);
 // Switches for timing experiments (forced span sizes and the like) are read from the environment only in a
 // library built with -DKVHIP_MEASURE; the shipped build compiles every one of them to its default.
 #ifdef KVHIP_MEASURE
