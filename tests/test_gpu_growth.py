@@ -35,7 +35,7 @@ def test_simple_cache_grows_from_empty_one_token_per_step(dtype):
             got = np32(c.update_attend(qd, kd, vd, scale))
             ref = O.attention_with_cache_update(q, k, v, o, scale, O.Mask.NONE, NAME[dtype])
             mx, mean = err_stats(got, ref)
-            assert mx <= (1e-2 if dtype == torch.float16 else 1.6e-2) and mean <= 1e-3, (t, mx, mean)
+            assert mx <= 1e-2 and mean <= 1e-3, (t, mx, mean)
         else:
             c.update(kd, vd, fetch=False)
             o.update(k, v)

@@ -9,7 +9,7 @@ import torch
 import kvhip
 from oracle import kv_oracle as O
 from tests.test_gpu_cache import check_quantized_state, drive_pair, positioned
-from tests.util import NAME, err_stats, np32, randn
+from tests.util import NAME, check_attention, err_stats, exact_attention, np32, presented_f64, randn
 
 pytestmark = pytest.mark.gpu
 
@@ -106,11 +106,8 @@ def test_decode_sequences_through_the_dispatcher(seed):
         out = np32(kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask))
         ref = O.attention_with_cache_update(q, k, v, o, scale, om, NAME[dtype])
         assert c.offset == o.offset and np.isfinite(out).all()
-        mx, mean = err_stats(out, ref)
-        # one step of the 16-bit output at the largest magnitude: with a handful of keys the outputs are as large as
-        # single V rows, and the oracle rounds the probabilities to the dtype where the kernels keep more bits
-        ulp = float(np.abs(ref).max()) * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10)
-        assert mx <= max(1e-2, 2 * ulp) and mean <= max(1e-3, ulp / 4), f"step {i} L={Lq} T={c.offset}: max-abs {mx:.3e} mean-abs {mean:.3e}"
+        # outside the 1e-2 / 1e-3 bound only where a float64 evaluation shows the device as close to exact as the oracle
+        check_attention(out, ref, dtype, f"step {i} L={Lq} T={c.offset}", lambda: exact_attention(q, *presented_f64(o), scale, om))
         if kind != "rotating" and rng.random() < 0.15:
             t = int(rng.integers(0, 5))
             assert c.trim(t) == o.trim(t)
