@@ -322,11 +322,13 @@ def other_workload(args, torch, kvhip, L, dev):
                 cache.update(k, v, fetch=False)
             q = torch.randn(Bn, Hq, Lq, Dk, generator=g, device=dev).to(dtype)
             mask = kvhip.MaskMode.causal()
-            for _ in range(12):  # (the first ten launches of a shape run up to 8 % slower than the later ones)
+            # 40 untimed launches: the chip's clocks take tens of milliseconds to settle under a new load, and the
+            # order of the shapes would otherwise show in the figures (runs then repeat within 1 %)
+            for _ in range(40):
                 cache.attend(q, Dk ** -0.5, mask)
             torch.cuda.synchronize()
             lib.kvhip_profile_enable(1)
-            for _ in range(args.steps if args.steps != 256 else 10):
+            for _ in range(args.steps if args.steps != 256 else 20):
                 cache.attend(q, Dk ** -0.5, mask)
             torch.cuda.synchronize()
             lib.kvhip_profile_enable(0)
