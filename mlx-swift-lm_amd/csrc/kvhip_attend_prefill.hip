@@ -553,9 +553,9 @@ bool attend_prefill_supported(const AttendArgs &a) {
     if (s.Dk != s.Dv) return false;
     // head sizes 80 (full precision only) and 96: every row count (no decode kernel is built for them)
     if (s.Dk != 64 && s.Dk != 128 && s.Dk != 256 && s.Dk != 96 && !(s.Dk == 80 && s.bits == 0)) return false;
-    if (s.bits != 0 && s.bits != 4 && s.bits != 8) return false;
     if (s.bits != 0 && s.gs < 32) return false;
-    if (s.bits != 0 && s.Dk != 96) return attend_prefill_q_supported(a);  // the pipelined tile: slots in presented order
+    if (s.bits != 0 && s.Dk != 96) return attend_prefill_q_supported(a);  // the pipelined tile (every code width): slots in presented order
+    if (s.bits != 0 && s.bits != 4 && s.bits != 8) return false;
     return true;  // 16 rows or fewer come here only when the decode kernels do not take the shape
 }
 
@@ -577,6 +577,7 @@ static int prefill_block_rows(const AttendArgs &a) {
     const int R = (a.Hq / a.Hkv) * a.L;
     if (a.st.bits != 0 && attend_prefill_q_supported(a)) {
         static const int forced = measure_knob("KVHIP_PREFILL_ROWS", 0);  // (timing builds only)
+        if (a.st.bits != 4 && a.st.bits != 8) return 64;
         if (forced > 0 && a.st.Dk == 128) return forced;
         // (head size 64 measured faster on 64 rows: 363 / 393 against 340 / 362 TFLOP/s at 8 / 4 bits, B4 2048 x 4096)
         return ((size_t)((R + 255) / 256) * a.st.BH >= 256 && a.st.Dk == 128) ? 256 : 64;

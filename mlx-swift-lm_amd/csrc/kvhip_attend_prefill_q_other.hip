@@ -1,0 +1,17 @@
+// The pipelined prefill tile for quantized caches (kvhip_attend_prefill_q.hpp): 2-, 3-, 5- and 6-bit codes, which
+// have no decode kernel of their own and take this tile at every row count.
+#include "kvhip_attend_prefill_q.hpp"
+
+namespace kvhip {
+
+hipError_t launch_attend_prefill_q_other(const AttendArgs &a, int nsplit, hipStream_t s) {
+    switch (a.st.bits) {
+    case 2: return launch_prefill_q_bits<2, false>(a, nsplit, 64, s);
+    case 3: return launch_prefill_q_bits<3, false>(a, nsplit, 64, s);
+    case 5: return launch_prefill_q_bits<5, false>(a, nsplit, 64, s);
+    case 6: return launch_prefill_q_bits<6, false>(a, nsplit, 64, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace kvhip

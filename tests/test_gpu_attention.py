@@ -510,3 +510,39 @@ def test_single_token_steps_write_their_row_inside_the_decode_kernel(dtype, bits
         for i, (a, b) in enumerate(zip(cache.state, ocache.get_state())):
             assert np.array_equal(np32(a), b) if i % 3 == 0 else bits_equal(a, b, dtype), (start, i)
         assert cache.trim(trim) == ocache.trim(trim)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bits,D,gs", [(2, 128, 64), (3, 128, 64), (5, 128, 32), (6, 128, 64), (3, 64, 32), (6, 64, 64), (2, 256, 64),
+                                        (5, 256, 128), (3, 256, 32)])
+def test_other_code_widths_on_the_pipelined_tile(dtype, bits, D, gs):
+    """2-, 3-, 5- and 6-bit codes (KVCacheConfiguration.swift:124 lists them beside 4 and 8) have no decode kernel of
+    their own: at head sizes 64 / 128 / 256 every row count runs on the pipelined prefill tile, which cuts the codes out
+    of the rows' bit streams.  Prompt chunks, single-token steps and a multi-token step against the oracle; codes and
+    pairs bit for bit."""
+    rng = np.random.default_rng(100 * bits + D + gs)
+    name = NAME[dtype]
+    B, Hkv, r = 2, 2, 4
+    scale = D ** -0.5
+    lib = kvhip.load()
+    c, o = kvhip.QuantizedKVCache(gs, bits), O.QuantizedKVCache(gs, bits, name)
+    for Lq, mode in [(200, "causal"), (1, "none"), (70, "causal"), (1, "none"), (4, "causal"), (1, "none")]:
+        k, kd = randn(rng, (B, Hkv, Lq, D), dtype)
+        v, vd = randn(rng, (B, Hkv, Lq, D), dtype)
+        q, qd = randn(rng, (B, Hkv * r, Lq, D), dtype)
+        mask, om = (kvhip.MaskMode.causal(), O.Mask.CAUSAL) if mode == "causal" else (kvhip.MaskMode.none(), O.Mask.NONE)
+        out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
+        assert lib.kvhip_last_attend_kernel() == 3
+        ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
+        check(out, ref, f"L={Lq}", lambda: exact_attention(q, *presented_f64(o), scale, om))
+    # a boolean array mask and a window evaluated from indices
+    T = c.offset
+    q, qd = randn(rng, (B, Hkv * r, 40, D), dtype)
+    m = O.create_causal_mask(40, T - 40, 33)
+    ref = O.quantized_sdpa(q, *o.get_quantized_state(), scale, O.Mask("array", m), o.group_size, bits, name)
+    exact = lambda: exact_attention(q, *presented_f64(o), scale, O.Mask("array", m))
+    check(c.attend(qd, scale, kvhip.MaskMode.from_array(torch.from_numpy(m).cuda())), ref, "bool array", exact)
+    check(c.attend(qd, scale, kvhip.MaskMode.window_mask(T - 40, 33)), ref, "window", exact)
+    assert lib.kvhip_last_attend_kernel() == 3
+    for i, (a, b) in enumerate(zip(c.state, o.get_state())):
+        assert np.array_equal(np32(a), b) if i % 3 == 0 else bits_equal(a, b, dtype), i
