@@ -249,6 +249,11 @@ hipError_t launch_compact_fp(const Store &src, const Runs &runs, const Store &ds
 // from pages to pages, no dense copy in between.
 hipError_t launch_requant_pages(const Store &src, const Store &dst, int rows, hipStream_t s);
 hipError_t launch_dequant_pages(const Store &q, const Store &dst, int rows, hipStream_t s);
+// The whole-tile quantizer for 2-, 3-, 5- and 6-bit codes (kvhip_quant_tile_other.hip): `tiles` tiles of dense rows
+// from row a0 on into the slots from b0 on, and tiles [0, tiles) of a full-precision page store into the same slots.
+hipError_t launch_quant_tiles_other(const Store &st, const void *keys, const void *values, int L, int a0, int b0, int tiles,
+                                    hipStream_t s, const RopeDev &r);
+hipError_t launch_requant_tiles_other(const Store &src, const Store &st, int tiles, hipStream_t s);
 hipError_t launch_affine_quantize(const void *src, int64_t rows, int D, int gs, int bits, int dtype,
                                   uint32_t *wq, void *scales, void *biases, hipStream_t s);
 hipError_t launch_affine_dequantize(const uint32_t *wq, const void *scales, const void *biases,

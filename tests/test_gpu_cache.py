@@ -169,12 +169,12 @@ def test_quantized_prompt_append_on_rounding_ties(bits):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
 @pytest.mark.parametrize("D,gs", [(64, 32), (64, 64), (96, 32), (128, 32), (128, 64), (128, 128), (256, 32), (256, 64), (256, 128)])
 def test_quantized_prompt_append_every_tile_shape(dtype, bits, D, gs):
-    """Whole 64-token tiles for every head size and group size the tile quantizer is built for (how
+    """Whole 64-token tiles for every head size, group size and code width the tile quantizer is built for (how
     many lanes share a group, and how many groups a lane works parameters out for, differ between
-    them), with a ragged head and tail around the tiles."""
+    them; 2-, 3-, 5- and 6-bit codes leave as bit streams), with a ragged head and tail around the tiles."""
     rng = np.random.default_rng(D + gs + bits)
     B, H = 2, 2
     cache = kvhip.QuantizedKVCache(gs, bits)
@@ -209,7 +209,7 @@ def test_keys_of_192_values_of_128_fill_and_convert_by_whole_tiles(dtype, bits, 
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("bits", [3, 4, 6, 8])
 def test_head_size_96_converts_by_whole_tiles(dtype, bits):
     """`toQuantized` of a full-precision cache of head size 96 (twelve 16-byte chunks per row: a row's
     threads do not divide the workgroup) gives the oracle's codes and pairs."""
