@@ -304,7 +304,8 @@ def other_workload(args, torch, kvhip, L, dev):
                   (1, 32, 8, 128, 4096, 4096, "f16"), (2, 16, 4, 64, 2048, 4096, "f16"), (4, 8, 4, 256, 512, 4608, "f16"),
                   (4, 8, 4, 256, 512, 4608, "bf16"), (1, 16, 16, "192/128", 2048, 8192, "f16"),
                   (1, 16, 16, "192/128", 2048, 8192, "bf16"), (1, 32, 8, 128, 2048, 8192, "q4"), (1, 32, 8, 128, 2048, 8192, "q8"),
-                  (4, 16, 4, 64, 2048, 4096, "q8"), (4, 8, 4, 256, 512, 4608, "q4"), (1, 32, 8, 96, 2048, 8192, "q4")]
+                  (4, 16, 4, 64, 2048, 4096, "q8"), (4, 8, 4, 256, 512, 4608, "q4"), (1, 32, 8, 96, 2048, 8192, "q4"),
+                  (1, 16, 16, "192/128", 2048, 8192, "q4"), (1, 16, 16, "192/128", 2048, 8192, "q8")]
         if args.prefill_shape:
             f = args.prefill_shape.split(",")
             shapes = [tuple(x if "/" in x else int(x) for x in f[:6]) + (f[6],)]
@@ -339,7 +340,7 @@ def other_workload(args, torch, kvhip, L, dev):
                          "kernel_ms": round(ms, 4), "TFLOPs": round(fl / ms / 1e9, 1),
                          "frac_of_2.5PF": round(fl / ms / 1e9 / 2500.0, 4)})
             del cache, k, v, q
-        return {"workload": "chunked-prefill tiles (prefill_fp_kernel, prefill_kernel for quantized caches) on their own", "results": rows}
+        return {"workload": "chunked-prefill tiles (prefill_fp_kernel, prefill_q_kernel for quantized caches) on their own", "results": rows}
 
     if args.workload == "cfg1":
         # the reference's own CPU-runnable case: B1, 16q/4kv, D64, fp16, 8-bit g64; prefill 512 under

@@ -1,5 +1,6 @@
 // Chunked-prefill attention for quantized caches on the matrix cores (gfx950,
-// v_mfma_f32_16x16x32_f16), head sizes 64 / 128 / 256, 4- or 8-bit codes, group size 32 and up.
+// v_mfma_f32_16x16x32_f16), head sizes 64 / 96 / 128 / 256 and keys of 192 with values of 128, every code width,
+// group size 32 and up.
 //
 // The loop is the one of the full-precision tile (kvhip_attend_prefill_fp.hip): a workgroup of 4
 // wavefronts owns 64 query rows of one (batch, kv-head) pair (QT = 1: 16 per wavefront), or one of 8
@@ -92,7 +93,7 @@ template <int DT> __device__ __forceinline__ void sb_h2(uint32_t raw, kv_h2 &s2,
 
 // NW wavefronts per workgroup: 4 (two workgroups per CU), or 8 (one per CU; 256 query rows share every
 // converted tile, which halves the conversion work per matrix-core instruction)
-template <int BITS, int D, int DT, int QT, int MM, int NW = 4>
+template <int BITS, int DK, int DV, int DT, int QT, int MM, int NW = 4>
 __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1)
 prefill_q_kernel(AttendArgs a, int nsplit) {
     constexpr int NT = 64 * NW;  // threads
@@ -100,17 +101,17 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
     // 2-, 3-, 5- and 6-bit codes: a row (and a V tile row) is a little-endian bit stream, code j at bit j BITS; a unit
     // is 32 codes (4 BITS bytes), its codes are cut out one by one (bit-field extracts) and paired in natural order
     constexpr bool GEN = BITS != 4 && BITS != 8;
-    static_assert(D == 64 || D == 128 || D == 256, "head size");
+    static_assert((DK == DV && (DK == 64 || DK == 96 || DK == 128 || DK == 256)) || (DK == 192 && DV == 128), "head sizes");
     constexpr int BM = 16 * QT * NW;
-    constexpr int S = D / 32;     // contraction steps over the head dim
-    constexpr int NDT = D / 16;   // 16-row tiles of out^T
-    constexpr int KSZ = BN * D, VSZ = BN * D;  // 16-bit elements of a tile's K and of its V
-    // units of UB bytes of packed codes: per tile UK for K (token-major: UPR per token row) and as many for V.
+    constexpr int S = DK / 32;    // contraction steps over the keys' head dim
+    constexpr int NDT = DV / 16;  // 16-row tiles of out^T
+    constexpr int KSZ = BN * DK, VSZ = BN * DV;  // 16-bit elements of a tile's K and of its V
+    // units of UB bytes of packed codes: per tile UK for K (token-major: UPR per token row) and UV for V.
     // 16 bytes, or 8 where that gives every thread of the workgroup a unit (4-bit codes on 8 wavefronts at D <= 128)
-    constexpr int UB = GEN ? 4 * BITS : ((32 * D * BITS / 8) * 2 / 16 < NT ? 8 : 16);
+    constexpr int UB = GEN ? 4 * BITS : ((32 * (DK + DV) * BITS / 8) / 16 < NT ? 8 : 16);
     constexpr int UWD = UB / 4;                // words per unit
-    constexpr int UK = 32 * D * BITS / 8 / UB, UPR = D * BITS / 8 / UB;
-    constexpr int NU = (2 * UK + NT - 1) / NT;   // units per thread
+    constexpr int UK = 32 * DK * BITS / 8 / UB, UPR = DK * BITS / 8 / UB, UV = 32 * DV * BITS / 8 / UB;
+    constexpr int NU = (UK + UV + NT - 1) / NT;  // units per thread
     constexpr int CPU = UB * 8 / BITS / 8;     // 8-element chunks a unit yields
     constexpr int TOK16 = 16 / UPR > 0 ? 16 / UPR : 1;  // tokens that 16 adjacent lanes of a K write cover
     __shared__ __attribute__((aligned(16))) uint16_t KV0[KSZ + VSZ], KV1[KSZ + VSZ];
@@ -123,7 +124,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, jj = lane >> 4;
-    const int G = D / st.gs;  // groups per row (1 .. 8)
+    const int G = DV / st.gs;  // groups per V row (1 .. 8)
     // workgroup ids -> (query block, pair, key-range part): all query blocks of a pair on one XCD (one L2)
     const int r = a.Hq / a.Hkv;
     const int R = r * a.L;
@@ -174,7 +175,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
         q_h[qt] = hk * r + rep;
         // rows past R read row (rep 0, l 0), which is in bounds, and are zeroed
         const u4 *qp = reinterpret_cast<const u4 *>(
-            reinterpret_cast<const uint16_t *>(a.q) + ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D + 8 * jj);
+            reinterpret_cast<const uint16_t *>(a.q) + ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * DK + 8 * jj);
         u4 raw[S];
 #pragma unroll
         for (int s = 0; s < S; ++s) raw[s] = qp[4 * s];
@@ -198,7 +199,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
     float m_run[QT], l_run[QT];
     // the denominators ride on the matrix cores up to D = 128 (lacc = ones . P^T sums the rounded probabilities
     // the numerator uses); D = 256 has no registers to spare
-    constexpr bool LM = D <= 128;
+    constexpr bool LM = DV <= 128;
     f4 lacc[LM ? QT : 1];
     Op8 ones;
     ones.v = u4{0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u};
@@ -252,7 +253,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
 
     // ---- units of packed codes: requests into registers, conversion into LDS ---------------------
     // unit u = tid + NT e: a K unit (u < UK: token u / UPR, part u % UPR of its row) or a V unit
-    // (u - UK = h * D + column: the h-th UB bytes of the column's 32-token half of a tile row)
+    // (u - UK = h * DV + column: the h-th UB bytes of the column's 32-token half of a tile row)
     uint32_t codes[NU][UWD];
     uint32_t ksb[NU];
     uint32_t vsb_raw[2] = {0u, 0u};  // table entries of a token pair (threads below 16 G)
@@ -269,7 +270,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
     // Everything about a thread's units that does not change from tile to tile is worked out once (group sizes
     // are powers of two: shifts, no divisions in the loop): byte offsets of the unit's (scale, bias) word and of
     // its V codes in global memory, of its first chunk in the LDS buffer, and of its table row.
-    const int gsh = __builtin_ctz((unsigned)st.gs), Gsh = __builtin_ctz((unsigned)G);
+    const int gsh = __builtin_ctz((unsigned)st.gs);
     uint32_t u_goff[NU], u_lds[NU], u_tab[NU];
 #pragma unroll
     for (int e = 0; e < NU; ++e) {
@@ -281,16 +282,16 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
             u_lds[e] = (uint32_t)(((part * CPU) * BN + ((pos + TOK16 * part) & (BN - 1))) * 16);
             u_tab[e] = 0;
         } else {
-            const int uv = u - UK, d = uv % D, h = uv / D;
+            const int uv = u - UK, d = uv % DV, h = uv / DV;
             u_goff[e] = (uint32_t)(d * (TILE * BITS / 8) + h * UB);
-            u_lds[e] = (uint32_t)(((h * CPU) * D + d) * 16);
+            u_lds[e] = (uint32_t)(((h * CPU) * DV + d) * 16);
             u_tab[e] = (uint32_t)(((d >> gsh) * (BN / 2) + 4 * h * CPU) * 4);
         }
     }
-    const bool tab_thread = tid < ((BN / 2) << Gsh);
-    const int tab_tp = tid >> Gsh, tab_g = tid & (G - 1);
-    const uint32_t tab_goff0 = (uint32_t)(((2 * tab_tp) << Gsh) + tab_g) * 4u, tab_goff1 = tab_goff0 + 4u * (uint32_t)G;
-    auto unit_is_v = [&](int e) __attribute__((always_inline)) -> bool { return tid + NT * e >= UK && tid + NT * e < 2 * UK; };
+    const bool tab_thread = tid < (BN / 2) * G;  // (G = 3 at head size 96: a division, once)
+    const int tab_tp = tid / G, tab_g = tid - tab_tp * G;
+    const uint32_t tab_goff0 = (uint32_t)(2 * tab_tp * G + tab_g) * 4u, tab_goff1 = tab_goff0 + 4u * (uint32_t)G;
+    auto unit_is_v = [&](int e) __attribute__((always_inline)) -> bool { return tid + NT * e >= UK && tid + NT * e < UK + UV; };
     auto load_unit = [&](uint32_t (&dst)[UWD], gptr p) __attribute__((always_inline)) {
         if constexpr (GEN) {  // 4-byte aligned: words one by one
 #pragma unroll
@@ -329,7 +330,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
         if (do_v) {
             const int slot0 = tile_v * BN;
             const PageEntry &pe = page_v.at(st, slot0);
-            gptr vb = as_global(pe.v + cell_v + (size_t)((slot0 & (PAGE - 1)) >> 6) * D * (TILE * BITS / 8) +
+            gptr vb = as_global(pe.v + cell_v + (size_t)((slot0 & (PAGE - 1)) >> 6) * DV * (TILE * BITS / 8) +
                                 ((slot0 & 32) ? BN * BITS / 8 : 0));
 #pragma unroll
             for (int e = 0; e < NU; ++e)
@@ -408,7 +409,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
             o.z = deq_pair((w1 & 0x00ff00ffu) | 0x64006400u, m1024, s2, b2);
             o.w = deq_pair(((w1 >> 8) & 0x00ff00ffu) | 0x64006400u, m1024, s3, b3);
         }
-        *reinterpret_cast<u4 *>(reinterpret_cast<char *>(Vs(par)) + u_lds[e] + c * (D * 16)) = o;
+        *reinterpret_cast<u4 *>(reinterpret_cast<char *>(Vs(par)) + u_lds[e] + c * (DV * 16)) = o;
     };
     // piece p (0 .. NU CPU - 1) of this thread's conversions: K units go to Ks(kpar), V units to Vs(vpar)
     constexpr int NPIECE = NU * CPU;
@@ -576,7 +577,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
 #pragma unroll
             for (int x = 0; x < VG; ++x)
                 if (VG * g + x < NDT)  // tokens 8 jj .. 8 jj + 7 of column 16 (VG g + x) + n: one chunk
-                    dst[x].v = *reinterpret_cast<const u4 *>(&Vs(PAR)[(jj * D + 16 * (VG * g + x) + n) * 8]);
+                    dst[x].v = *reinterpret_cast<const u4 *>(&Vs(PAR)[(jj * DV + 16 * (VG * g + x) + n) * 8]);
         };
         if (k2) write_table(PAR);  // of tile + 2: this buffer's last reader was the previous iteration
         if constexpr (HAS_NEXT) {
@@ -727,17 +728,17 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
         if (!q_ok[qt]) continue;
         if (nsplit > 1) {
             const int i = row0 + 16 * qt + n;
-            float *part = a.workspace + (((size_t)bh * nsplit + split) * R + i) * (D + 2);
+            float *part = a.workspace + (((size_t)bh * nsplit + split) * R + i) * (DV + 2);
 #pragma unroll
             for (int dt = 0; dt < NDT; ++dt) *reinterpret_cast<f4 *>(part + 16 * dt + 4 * jj) = oacc[qt][dt];
             if (jj == 0) {
-                part[D] = m_run[qt] * 0.6931471805599453f;  // back from the log2 domain
-                part[D + 1] = l;
+                part[DV] = m_run[qt] * 0.6931471805599453f;  // back from the log2 domain
+                part[DV + 1] = l;
             }
             continue;
         }
         const float inv = l > 0.f ? 1.0f / l : 0.f;
-        const size_t ooff = ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * D;
+        const size_t ooff = ((size_t)(b * a.Hq + q_h[qt]) * a.L + q_l[qt]) * DV;
 #pragma unroll
         for (int dt = 0; dt < NDT; ++dt) {
             const float o0 = oacc[qt][dt][0] * inv, o1 = oacc[qt][dt][1] * inv;
@@ -755,37 +756,45 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
     }
 }
 
-// Launch for one code width: 64 query rows on 4 wavefronts, or (4- and 8-bit codes at head size 128) 256 rows on 8.
-template <int BITS, bool BIG_TOO>
+// Launch for one code width: `rows` query rows per workgroup -- 64 on 4 wavefronts; keys of 192 with values of 128 also
+// 128 on 8 wavefronts (one workgroup per CU, twice as many rows share each converted tile: 454 against 366 TFLOP/s at
+// B1, 16 heads, 2048 x 8192, 4 bits; the other head sizes measured no faster or slower that way); WIDE (4- and 8-bit
+// codes) at head size 128 also 256 rows on 8 wavefronts.
+template <int BITS, bool WIDE>
 hipError_t launch_prefill_q_bits(const AttendArgs &a, int nsplit, int rows, hipStream_t s) {
     const Store &st = a.st;
     const int R = (a.Hq / a.Hkv) * a.L;
-    const bool big = BIG_TOO && rows == 256 && st.Dk == 128;
-    const int bm = big ? 256 : 64;
-    dim3 grid((unsigned)((R + bm - 1) / bm) * st.BH * nsplit), block(big ? 512 : 256);
+    if (rows != 64 && !(rows == 128 && st.Dk == 192) && !(WIDE && rows == 256 && st.Dk == 128)) return hipErrorInvalidValue;
+    dim3 grid((unsigned)((R + rows - 1) / rows) * st.BH * nsplit), block(rows == 64 ? 256 : 512);
     const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
-#define PQ_M(D, DT, QT, NW)                                                                            \
-    do {                                                                                               \
-        if (mm == 0) hipLaunchKernelGGL((prefill_q_kernel<BITS, D, DT, QT, 0, NW>), grid, block, 0, s, a, nsplit);      \
-        else if (mm == 1) hipLaunchKernelGGL((prefill_q_kernel<BITS, D, DT, QT, 1, NW>), grid, block, 0, s, a, nsplit); \
-        else hipLaunchKernelGGL((prefill_q_kernel<BITS, D, DT, QT, 2, NW>), grid, block, 0, s, a, nsplit);              \
+#define PQ_M(DK, DV, DT, QT, NW)                                                                                 \
+    do {                                                                                                         \
+        if (mm == 0) hipLaunchKernelGGL((prefill_q_kernel<BITS, DK, DV, DT, QT, 0, NW>), grid, block, 0, s, a, nsplit);      \
+        else if (mm == 1) hipLaunchKernelGGL((prefill_q_kernel<BITS, DK, DV, DT, QT, 1, NW>), grid, block, 0, s, a, nsplit); \
+        else hipLaunchKernelGGL((prefill_q_kernel<BITS, DK, DV, DT, QT, 2, NW>), grid, block, 0, s, a, nsplit);              \
     } while (0)
-#define PQ_DT(D, QT, NW)                              \
-    do {                                              \
-        if (st.dtype == KVHIP_F16) PQ_M(D, 0, QT, NW); \
-        else PQ_M(D, 1, QT, NW);                      \
+#define PQ_DT(DK, DV, QT, NW)                              \
+    do {                                                   \
+        if (st.dtype == KVHIP_F16) PQ_M(DK, DV, 0, QT, NW); \
+        else PQ_M(DK, DV, 1, QT, NW);                      \
     } while (0)
     if (st.Dk == 64) {
-        PQ_DT(64, 1, 4);
+        PQ_DT(64, 64, 1, 4);
+    } else if (st.Dk == 96) {
+        PQ_DT(96, 96, 1, 4);
     } else if (st.Dk == 128) {
-        if constexpr (BIG_TOO) {
-            if (big) PQ_DT(128, 2, 8);
-            else PQ_DT(128, 1, 4);
-        } else {
-            PQ_DT(128, 1, 4);
+        if constexpr (WIDE) {
+            if (rows == 256) {
+                PQ_DT(128, 128, 2, 8);
+                return hipGetLastError();
+            }
         }
+        PQ_DT(128, 128, 1, 4);
+    } else if (st.Dk == 192) {
+        if (rows == 128) PQ_DT(192, 128, 1, 8);
+        else PQ_DT(192, 128, 1, 4);
     } else {
-        PQ_DT(256, 1, 4);
+        PQ_DT(256, 256, 1, 4);
     }
 #undef PQ_DT
 #undef PQ_M

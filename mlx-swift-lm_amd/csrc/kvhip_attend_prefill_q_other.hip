@@ -4,12 +4,12 @@
 
 namespace kvhip {
 
-hipError_t launch_attend_prefill_q_other(const AttendArgs &a, int nsplit, hipStream_t s) {
+hipError_t launch_attend_prefill_q_other(const AttendArgs &a, int nsplit, int rows, hipStream_t s) {
     switch (a.st.bits) {
-    case 2: return launch_prefill_q_bits<2, false>(a, nsplit, 64, s);
-    case 3: return launch_prefill_q_bits<3, false>(a, nsplit, 64, s);
-    case 5: return launch_prefill_q_bits<5, false>(a, nsplit, 64, s);
-    case 6: return launch_prefill_q_bits<6, false>(a, nsplit, 64, s);
+    case 2: return launch_prefill_q_bits<2, false>(a, nsplit, rows, s);
+    case 3: return launch_prefill_q_bits<3, false>(a, nsplit, rows, s);
+    case 5: return launch_prefill_q_bits<5, false>(a, nsplit, rows, s);
+    case 6: return launch_prefill_q_bits<6, false>(a, nsplit, rows, s);
     default: return hipErrorInvalidValue;
     }
 }

@@ -314,7 +314,7 @@ hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, 
 bool attend_prefill_q_supported(const AttendArgs &a);
 // rows: query rows per workgroup, 64 (4 wavefronts) or 256 (8 wavefronts; head size 128)
 hipError_t launch_attend_prefill_q(const AttendArgs &a, int nsplit, int rows, hipStream_t s);
-hipError_t launch_attend_prefill_q_other(const AttendArgs &a, int nsplit, hipStream_t s);  // 2-, 3-, 5- and 6-bit codes
+hipError_t launch_attend_prefill_q_other(const AttendArgs &a, int nsplit, int rows, hipStream_t s);  // 2-, 3-, 5- and 6-bit codes
 // Switches for timing experiments (forced span sizes and the like) are read from the environment only in a
 // library built with -DKVHIP_MEASURE; the shipped build compiles every one of them to its default.
 #ifdef KVHIP_MEASURE

@@ -232,7 +232,8 @@ def test_keys_of_192_values_of_128_on_the_prefill_tile(dtype):
         check(out, ref, f"ring step {i}", lambda: exact_attention(q, *presented_f64(o), scale, om))
 
 
-@pytest.mark.parametrize("dtype,bits,gs", [(torch.float16, 4, 64), (torch.bfloat16, 8, 64), (torch.float16, 8, 32)])
+@pytest.mark.parametrize("dtype,bits,gs", [(torch.float16, 4, 64), (torch.bfloat16, 8, 64), (torch.float16, 8, 32), (torch.bfloat16, 4, 32),
+                                           (torch.float16, 3, 64), (torch.bfloat16, 5, 32), (torch.float16, 6, 32), (torch.bfloat16, 2, 64)])
 def test_quantized_keys_of_192_values_of_128_on_the_prefill_tile(dtype, bits, gs):
     """The same head sizes in a QuantizedKVCache (group sizes 32 and 64 divide both): every row count runs on
     the quantized prefill tile; codes and pairs equal the oracle's, outputs are the oracle's within the bound."""
@@ -514,10 +515,10 @@ def test_single_token_steps_write_their_row_inside_the_decode_kernel(dtype, bits
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("bits,D,gs", [(2, 128, 64), (3, 128, 64), (5, 128, 32), (6, 128, 64), (3, 64, 32), (6, 64, 64), (2, 256, 64),
-                                        (5, 256, 128), (3, 256, 32)])
+                                        (5, 256, 128), (3, 256, 32), (3, 96, 32), (6, 96, 32), (2, 96, 32), (5, 96, 32)])
 def test_other_code_widths_on_the_pipelined_tile(dtype, bits, D, gs):
     """2-, 3-, 5- and 6-bit codes (KVCacheConfiguration.swift:124 lists them beside 4 and 8) have no decode kernel of
-    their own: at head sizes 64 / 128 / 256 every row count runs on the pipelined prefill tile, which cuts the codes out
+    their own: at head sizes 64 / 96 / 128 / 256 every row count runs on the pipelined prefill tile, which cuts the codes out
     of the rows' bit streams.  Prompt chunks, single-token steps and a multi-token step against the oracle; codes and
     pairs bit for bit."""
     rng = np.random.default_rng(100 * bits + D + gs)
