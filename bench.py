@@ -64,7 +64,7 @@ def main():
                     help="cfg3 (default) is the configuration the metric is quoted on; the others are the "
                          "remaining BASELINE.json configs (reported as one JSON object each)")
     ap.add_argument("--prefill-shape", default=None,
-                    help="with --workload prefill: one shape B,Hq,Hkv,D,L,T,dtype (dtype f16, bf16, q4 or q8; D may be 192/128) instead of the table")
+                    help="with --workload prefill: one shape B,Hq,Hkv,D,L,T,dtype (dtype f16, bf16, or q2 / q3 / q4 / q5 / q6 / q8; D may be 192/128) instead of the table")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy 4 times (reference point for rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -298,7 +298,7 @@ def other_workload(args, torch, kvhip, L, dev):
     if args.workload == "prefill":
         # the chunked-prefill tile on its own: L new rows attending causally over T cached keys (the new rows
         # included); flops = 2 * B * Hq * (Dk + Dv) * (keys each row sees)
-        # dtype field: f16 / bf16 full precision; q4 / q8 a float16 QuantizedKVCache (group 64; 32 at D 96);
+        # dtype field: f16 / bf16 full precision; qN a float16 QuantizedKVCache of N-bit codes (group 64; 32 at D 96);
         # a head size "192/128" is keys of 192 with values of 128
         shapes = [(1, 32, 8, 128, 2048, 8192, "f16"), (1, 32, 8, 128, 2048, 8192, "bf16"), (4, 32, 8, 128, 512, 4096, "f16"),
                   (1, 32, 8, 128, 4096, 4096, "f16"), (2, 16, 4, 64, 2048, 4096, "f16"), (4, 8, 4, 256, 512, 4608, "f16"),
@@ -315,7 +315,7 @@ def other_workload(args, torch, kvhip, L, dev):
             dtype = torch.bfloat16 if dn == "bf16" else torch.float16
             k = torch.randn(Bn, Hkv, T, Dk, generator=g, device=dev).to(dtype)
             v = k.flip(-1)[..., :Dv].contiguous()
-            if dn in ("q4", "q8"):
+            if dn[0] == "q":
                 cache = kvhip.QuantizedKVCache(64, int(dn[1]))
                 cache.update_quantized(k, v, fetch=False)
             else:

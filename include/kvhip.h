@@ -235,8 +235,9 @@ kvhip_status kvhip_cache_fetch(const kvhip_cache *cache, void *dst_keys, void *d
  * queries [B,Hq,L,Dk] and out [B,Hq,L,Dv] in the cache's dtype.
  * Every dtype, bit width, head size, group size and mask is accepted.  The tuned kernels take
  * float16 / bfloat16 caches with Dk == Dv in {64, 96, 128, 256}, keys of 192 with values of 128 (also
- * 80 when not quantized; quantized: 4 or 8 bits, group size 32, 64 or 128); anything else
- * (float32, 2-, 3-, 5- and 6-bit codes, other head sizes) runs on a plain kernel
+ * 80 when not quantized; quantized: every code width, group size 32, 64 or 128; 2-, 3-, 5- and
+ * 6-bit codes have no decode kernel and run single-token steps on the prefill tile); anything else
+ * (float32, other head sizes) runs on a plain kernel
  * that is 50-75 times slower at 8k keys.  kvhip_last_attend_kernel() tells which one ran.
  */
 kvhip_status kvhip_cache_attend(kvhip_cache *cache, const void *queries, int32_t B, int32_t Hq,
