@@ -31,16 +31,22 @@ static bool prefill_wide(const AttendArgs &a) {
 
 // Query rows per workgroup.  The pipelined tile for quantized caches (kvhip_attend_prefill_q.hpp) takes 256 rows
 // on 8 wavefronts at head size 128, one workgroup per CU, whenever that still gives every CU a workgroup: four
-// times as many rows share each converted tile (B1, 2048 x 8192, 4 bits: 552 against 446 TFLOP/s; a square causal
-// 4096 x 4096, which would leave half the CUs empty, stays on 64 rows: 480 against 380).  Otherwise 128 or 64 rows
-// on 4 wavefronts as above (quantized: 64).
+// times as many rows share each converted tile (B1, 2048 x 8192, 4 bits: 600 against 457 TFLOP/s).  Otherwise 128 or
+// 64 rows on 4 wavefronts as above (quantized: 64; keys of 192 with values of 128: 128 rows on 8 wavefronts).
 static int prefill_block_rows(const AttendArgs &a) {
     const int R = (a.Hq / a.Hkv) * a.L;
     if (a.st.bits != 0) {
         static const int forced = measure_knob("KVHIP_PREFILL_ROWS", 0);  // (timing builds only)
         if (forced == 64 || (forced == 128 && a.st.Dk == 192) || (forced == 256 && a.st.Dk == 128 && (a.st.bits == 4 || a.st.bits == 8))) return forced;
         // (head size 64 measured faster on 64 rows: 363 / 393 against 340 / 362 TFLOP/s at 8 / 4 bits, B4 2048 x 4096)
-        if ((a.st.bits == 4 || a.st.bits == 8) && a.st.Dk == 128 && (size_t)((R + 255) / 256) * a.st.BH >= 256) return 256;
+        if ((a.st.bits == 4 || a.st.bits == 8) && a.st.Dk == 128) {
+            // 256 rows need a workgroup for every CU.  Under a causal or window mask the query blocks differ in work and a
+            // CU holds one such workgroup at a time, so beyond a single round the gain depends on the shape (4-bit, B1, 8 kv
+            // heads, TFLOP/s on 64 / 256 rows: 2048 x 4096 411 / 483, 2048 x 8192 457 / 600, 8192 x 8192 563 / 617,
+            // 4096 x 8192 543 / 532, but 4096 x 4096 457 / 384 and B4 2048 x 2048 435 / 362): one round, or long sequences
+            const size_t wgs = (size_t)((R + 255) / 256) * a.st.BH;
+            if (wgs >= 256 && (a.mask.mode == KVHIP_MASK_NONE || wgs <= 320 || a.T >= 8192)) return 256;
+        }
         // keys of 192 with values of 128: 128 rows on 8 wavefronts (head sizes 96 / 128 / 256 measured 4-20 % slower on it)
         return (a.st.Dk == 192 && (size_t)((R + 127) / 128) * a.st.BH >= 256) ? 128 : 64;
     }

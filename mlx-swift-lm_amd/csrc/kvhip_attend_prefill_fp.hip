@@ -551,12 +551,26 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         return ef * fmaxf(fmaxf(fmaxf(sc[qt][0][0], sc[qt][0][1]), fmaxf(sc[qt][0][2], sc[qt][0][3])),
                           fmaxf(fmaxf(sc[qt][1][0], sc[qt][1][1]), fmaxf(sc[qt][1][2], sc[qt][1][3])));
     };
+    // The same maximum in four instructions, for the end of an iteration.  `fmaxf` on values the compiler has not
+    // seen an arithmetic instruction produce (matrix-core results, selects) first quiets each operand with a
+    // maximum of its own: eleven instructions for eight values, on the path every wavefront runs before the
+    // barrier.  Written as assembly, which the compiler's hazard handling does not look into: the caller keeps it
+    // behind a scheduling barrier that follows the out^T matrix-core instructions, so the score registers, written
+    // by matrix-core instructions a whole block earlier (or by the mask's selects), are long complete.
+    auto tile_max_raw = [&](const f4 (&sc)[QT][2], int qt) __attribute__((always_inline)) -> float {
+        float m;  // (one statement per instruction: the result may then share a register with a finished operand)
+        asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(m) : "v"(sc[qt][0][0]), "v"(sc[qt][0][1]), "v"(sc[qt][0][2]));
+        asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(m) : "v"(m), "v"(sc[qt][0][3]), "v"(sc[qt][1][0]));
+        asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(m) : "v"(m), "v"(sc[qt][1][1]), "v"(sc[qt][1][2]));
+        asm volatile("v_max_f32 %0, %1, %2" : "=v"(m) : "v"(m), "v"(sc[qt][1][3]));
+        return ef * m;
+    };
     // whether the tile whose scores are in `sc` exceeds some query's reference maximum by more than
     // RAISE (wavefront-uniform; a handful of times per query)
     auto needs_raise = [&](const f4 (&sc)[QT][2]) __attribute__((always_inline)) -> bool {
         bool need = false;
 #pragma unroll
-        for (int qt = 0; qt < QT; ++qt) need = need || tile_max(sc, qt) > m_run[qt] + RAISE;
+        for (int qt = 0; qt < QT; ++qt) need = need || tile_max_raw(sc, qt) > m_run[qt] + RAISE;
         return __any(need);
     };
     auto do_raise = [&](const f4 (&sc)[QT][2]) __attribute__((always_inline)) {
@@ -667,6 +681,7 @@ prefill_fp_kernel(AttendArgs a, int nsplit) {
         need = false;
         if constexpr (HAS_NEXT) {
             if constexpr (MASKED) apply_mask(PAR ^ 1, sn);
+            KV_SB;  // (tile_max_raw: not before the matrix-core instructions above)
             need = needs_raise(sn);
         }
         // What was requested at the top has to land before the barrier: it has had the whole

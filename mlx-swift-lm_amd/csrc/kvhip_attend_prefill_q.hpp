@@ -351,6 +351,16 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
         }
     };
     const kv_h2 m1024 = kv_h2{(_Float16)1024.f, (_Float16)1024.f}, m64 = kv_h2{(_Float16)64.f, (_Float16)64.f};
+    // The float16 constants the codes are OR-ed into, held in vector registers the compiler cannot rematerialise:
+    // (w & mask) | constant is then one v_and_or_b32 (mask in a scalar register, constant in a vector register; with
+    // both as literals the instruction, which may read one scalar operand, is not formed), and an 8-bit pair is one
+    // v_perm_b32 that takes bytes 0 and 2 (or 1 and 3) of the word beside the constant's high bytes.
+    uint32_t mag = 0x64006400u, mag_hi = 0x54005400u;
+    asm volatile("" : "+v"(mag), "+v"(mag_hi));
+    auto nib_lo = [&](uint32_t w) __attribute__((always_inline)) -> uint32_t { return (w & 0x000f000fu) | mag; };
+    auto nib_hi = [&](uint32_t w) __attribute__((always_inline)) -> uint32_t { return (w & 0x00f000f0u) | mag_hi; };
+    auto bytes_even = [&](uint32_t w) __attribute__((always_inline)) -> uint32_t { return __builtin_amdgcn_perm(mag, w, 0x05020500u); };
+    auto bytes_odd = [&](uint32_t w) __attribute__((always_inline)) -> uint32_t { return __builtin_amdgcn_perm(mag, w, 0x05030501u); };
     // chunk c (0 .. CPU-1) of K unit e -> LDS
     auto convert_k = [&](int e, int c, int par) __attribute__((always_inline)) {
         kv_h2 s2, b2;
@@ -364,16 +374,16 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
             o.w = deq_pair(x.w, m1024, s2, b2);
         } else if constexpr (BITS == 4) {  // elements (0,4) (1,5) (2,6) (3,7) of the word's 8
             const uint32_t w = codes[e][c], w8 = w >> 8;
-            o.x = deq_pair((w & 0x000f000fu) | 0x64006400u, m1024, s2, b2);
-            o.y = deq_pair((w & 0x00f000f0u) | 0x54005400u, m64, s2, b2);
-            o.z = deq_pair((w8 & 0x000f000fu) | 0x64006400u, m1024, s2, b2);
-            o.w = deq_pair((w8 & 0x00f000f0u) | 0x54005400u, m64, s2, b2);
+            o.x = deq_pair(nib_lo(w), m1024, s2, b2);
+            o.y = deq_pair(nib_hi(w), m64, s2, b2);
+            o.z = deq_pair(nib_lo(w8), m1024, s2, b2);
+            o.w = deq_pair(nib_hi(w8), m64, s2, b2);
         } else {  // elements (0,2) (1,3) of each word's 4
             const uint32_t w0 = codes[e][2 * c], w1 = codes[e][2 * c + 1];
-            o.x = deq_pair((w0 & 0x00ff00ffu) | 0x64006400u, m1024, s2, b2);
-            o.y = deq_pair(((w0 >> 8) & 0x00ff00ffu) | 0x64006400u, m1024, s2, b2);
-            o.z = deq_pair((w1 & 0x00ff00ffu) | 0x64006400u, m1024, s2, b2);
-            o.w = deq_pair(((w1 >> 8) & 0x00ff00ffu) | 0x64006400u, m1024, s2, b2);
+            o.x = deq_pair(bytes_even(w0), m1024, s2, b2);
+            o.y = deq_pair(bytes_odd(w0), m1024, s2, b2);
+            o.z = deq_pair(bytes_even(w1), m1024, s2, b2);
+            o.w = deq_pair(bytes_odd(w1), m1024, s2, b2);
         }
         *reinterpret_cast<u4 *>(reinterpret_cast<char *>(Ks(par)) + u_lds[e] + c * (BN * 16)) = o;
     };
@@ -398,16 +408,16 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
             o.w = deq_pair(x.w, m1024, s3, b3);
         } else if constexpr (BITS == 4) {  // the word's tokens two at a time, in token order (the V tile's nibble order)
             const uint32_t w = codes[e][c], w8 = w >> 8;
-            o.x = deq_pair((w & 0x000f000fu) | 0x64006400u, m1024, s0, b0);
-            o.y = deq_pair((w & 0x00f000f0u) | 0x54005400u, m64, s1, b1);
-            o.z = deq_pair((w8 & 0x000f000fu) | 0x64006400u, m1024, s2, b2);
-            o.w = deq_pair((w8 & 0x00f000f0u) | 0x54005400u, m64, s3, b3);
+            o.x = deq_pair(nib_lo(w), m1024, s0, b0);
+            o.y = deq_pair(nib_hi(w), m64, s1, b1);
+            o.z = deq_pair(nib_lo(w8), m1024, s2, b2);
+            o.w = deq_pair(nib_hi(w8), m64, s3, b3);
         } else {
             const uint32_t w0 = codes[e][2 * c], w1 = codes[e][2 * c + 1];
-            o.x = deq_pair((w0 & 0x00ff00ffu) | 0x64006400u, m1024, s0, b0);
-            o.y = deq_pair(((w0 >> 8) & 0x00ff00ffu) | 0x64006400u, m1024, s1, b1);
-            o.z = deq_pair((w1 & 0x00ff00ffu) | 0x64006400u, m1024, s2, b2);
-            o.w = deq_pair(((w1 >> 8) & 0x00ff00ffu) | 0x64006400u, m1024, s3, b3);
+            o.x = deq_pair(bytes_even(w0), m1024, s0, b0);
+            o.y = deq_pair(bytes_odd(w0), m1024, s1, b1);
+            o.z = deq_pair(bytes_even(w1), m1024, s2, b2);
+            o.w = deq_pair(bytes_odd(w1), m1024, s3, b3);
         }
         *reinterpret_cast<u4 *>(reinterpret_cast<char *>(Vs(par)) + u_lds[e] + c * (DV * 16)) = o;
     };
@@ -528,10 +538,24 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
         return ef * fmaxf(fmaxf(fmaxf(sc[qt][0][0], sc[qt][0][1]), fmaxf(sc[qt][0][2], sc[qt][0][3])),
                           fmaxf(fmaxf(sc[qt][1][0], sc[qt][1][1]), fmaxf(sc[qt][1][2], sc[qt][1][3])));
     };
+    // The same maximum in four instructions, for the end of an iteration.  `fmaxf` on values the compiler has not
+    // seen an arithmetic instruction produce (matrix-core results, selects) first quiets each operand with a
+    // maximum of its own: eleven instructions for eight values, on the path every wavefront runs before the
+    // barrier.  Written as assembly, which the compiler's hazard handling does not look into: the caller keeps it
+    // behind a scheduling barrier that follows the out^T matrix-core instructions, so the score registers, written
+    // by matrix-core instructions a whole block earlier (or by the mask's selects), are long complete.
+    auto tile_max_raw = [&](const f4 (&sc)[QT][2], int qt) __attribute__((always_inline)) -> float {
+        float m;  // (one statement per instruction: the result may then share a register with a finished operand)
+        asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(m) : "v"(sc[qt][0][0]), "v"(sc[qt][0][1]), "v"(sc[qt][0][2]));
+        asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(m) : "v"(m), "v"(sc[qt][0][3]), "v"(sc[qt][1][0]));
+        asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(m) : "v"(m), "v"(sc[qt][1][1]), "v"(sc[qt][1][2]));
+        asm volatile("v_max_f32 %0, %1, %2" : "=v"(m) : "v"(m), "v"(sc[qt][1][3]));
+        return ef * m;
+    };
     auto needs_raise = [&](const f4 (&sc)[QT][2]) __attribute__((always_inline)) -> bool {
         bool need = false;
 #pragma unroll
-        for (int qt = 0; qt < QT; ++qt) need = need || tile_max(sc, qt) > m_run[qt] + RAISE;
+        for (int qt = 0; qt < QT; ++qt) need = need || tile_max_raw(sc, qt) > m_run[qt] + RAISE;
         return __any(need);
     };
     auto do_raise = [&](const f4 (&sc)[QT][2]) __attribute__((always_inline)) {
@@ -635,6 +659,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
         need = false;
         if constexpr (HAS_NEXT) {
             if constexpr (MASKED) apply_mask((tile + 1) * BN, sn);
+            KV_SB;  // (tile_max_raw: not before the matrix-core instructions above)
             need = needs_raise(sn);
         }
         // the conversions' LDS writes have to land before any wavefront reads the buffers
