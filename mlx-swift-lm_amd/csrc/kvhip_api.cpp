@@ -93,6 +93,13 @@ struct kvhip_cache {
     bool has_geom = false;
     int B = 0, Hkv = 0;
     Store st;                  // st.pt = the page table in device memory
+    // Head sizes of the caller's arrays.  The pages hold st.Dk / st.Dv, which are larger when the tuned kernels are
+    // not built for the caller's sizes: rows are then stored zero-padded (zero key columns add nothing to a score,
+    // zero value columns give output columns nobody reads), arrays are widened on the way in and narrowed on the
+    // way out, and everything between works on the stored sizes.
+    int Dk_user = 0, Dv_user = 0;
+    void *pad_buf[4] = {nullptr, nullptr, nullptr, nullptr};  // widened keys, values, queries; outputs before narrowing
+    size_t pad_bytes[4] = {0, 0, 0, 0};
     std::vector<Slab> slabs;   // the allocations behind the pages, in page order
     int64_t cap_pages = 0;     // pages allocated (= page-table entries in use)
     int64_t pt_cap = 0;        // entries the device page table has room for
@@ -121,6 +128,7 @@ struct kvhip_cache {
     mutable bool used_stream = false;
 
     int64_t cap_slots() const { return cap_pages * PAGE; }
+    bool padded() const { return has_geom && (Dk_user != st.Dk || Dv_user != st.Dv); }
 };
 
 namespace {
@@ -261,6 +269,26 @@ void drop_pages(kvhip_cache *c, hipStream_t stream, bool drained) {
     }
 }
 
+// The head sizes a cache stores for the caller's (Dk, Dv).  The tuned attention kernels are built for 16-bit caches
+// with one head size of 64, 96, 128 or 256 (80 too when not quantized) and for keys of 192 with values of 128; any
+// other pair up to 256 is stored zero-padded to the next of 64 / 96 / 128 / 256 that holds both (and that the
+// group size divides).  float32 caches and head sizes above 256 are stored as they are (plain kernel).
+void stored_head_sizes(int kind, int gs, int dtype, int Dk, int Dv, int &Pk, int &Pv) {
+    Pk = Dk;
+    Pv = Dv;
+    if (dtype != KVHIP_F16 && dtype != KVHIP_BF16) return;
+    if (Dk == 192 && Dv == 128) return;
+    const bool q = kind == KVHIP_KIND_QUANTIZED;
+    if (Dk == Dv && (Dk == 64 || Dk == 96 || Dk == 128 || Dk == 256 || (!q && Dk == 80))) return;
+    const int m = std::max(Dk, Dv);
+    for (int p : {64, 96, 128, 256})
+        if (p >= m && (!q || (gs > 0 && p % gs == 0))) {
+            Pk = Pv = p;
+            return;
+        }
+}
+
+// Dk / Dv: the head sizes of the caller's arrays
 kvhip_status set_geometry(kvhip_cache *c, int B, int Hkv, int Dk, int Dv, int dtype) {
     if (B <= 0 || Hkv <= 0 || Dk <= 0 || Dv <= 0) return fail(KVHIP_ERR_INVALID_ARG, "non-positive shape");
     if (dtype != KVHIP_F16 && dtype != KVHIP_BF16 && dtype != KVHIP_F32)
@@ -268,14 +296,19 @@ kvhip_status set_geometry(kvhip_cache *c, int B, int Hkv, int Dk, int Dv, int dt
     if ((int64_t)B * Hkv > 65535) return fail(KVHIP_ERR_UNSUPPORTED, "B * Hkv above 65535");
     if (c->has_geom) {
         const Store &s = c->st;
-        if (s.BH != B * Hkv || c->B != B || s.Dk != Dk || s.Dv != Dv || s.dtype != dtype)
+        if (s.BH != B * Hkv || c->B != B || c->Dk_user != Dk || c->Dv_user != Dv || s.dtype != dtype)
             return fail(KVHIP_ERR_INVALID_ARG, "shape or dtype differs from what this cache already holds");
         return KVHIP_OK;
     }
+    if (c->kind == KVHIP_KIND_QUANTIZED && c->gs > 0 && (Dk % c->gs || Dv % c->gs))
+        return fail(KVHIP_ERR_INVALID_ARG, "head dim not divisible by the group size");
     Store &s = c->st;
     s = Store();
     c->B = B;
     c->Hkv = Hkv;
+    c->Dk_user = Dk;
+    c->Dv_user = Dv;
+    stored_head_sizes(c->kind, c->gs, dtype, Dk, Dv, Dk, Dv);  // from here on: the stored sizes
     s.BH = B * Hkv;
     s.Dk = Dk;
     s.Dv = Dv;
@@ -380,6 +413,29 @@ kvhip_status ensure_ws(kvhip_cache *c, size_t bytes, hipStream_t) {
     return KVHIP_OK;
 }
 
+// A cache that stores padded rows: the caller's dense array `src` (rows of `user_d` elements) widened into the
+// cache's buffer number `which` (rows of `stored_d` elements, the added columns zero); `*out` is what the kernels read.
+kvhip_status ensure_pad_buf(kvhip_cache *c, int which, size_t need) {
+    if (need <= c->pad_bytes[which]) return KVHIP_OK;
+    void *p = nullptr;
+    size_t got = need;
+    KV_HIP(pool_alloc(&p, std::max(need + need / 4, 2 * c->pad_bytes[which]), &got));
+    if (c->pad_buf[which]) c->parked.push_back({c->pad_buf[which], c->pad_bytes[which]});  // (work in flight may read it)
+    c->pad_buf[which] = p;
+    c->pad_bytes[which] = got;
+    return KVHIP_OK;
+}
+
+kvhip_status widen_rows(kvhip_cache *c, int which, const void *src, size_t rows, int user_d, int stored_d,
+                        hipStream_t s, const void **out) {
+    *out = src;
+    if (user_d == stored_d) return KVHIP_OK;
+    KV_TRY(ensure_pad_buf(c, which, rows * (size_t)stored_d * c->st.es));
+    KV_HIP(launch_repitch_rows(c->pad_buf[which], (size_t)stored_d * c->st.es, src, (size_t)user_d * c->st.es, rows, s));
+    *out = c->pad_buf[which];
+    return KVHIP_OK;
+}
+
 // ---- run tables ------------------------------------------------------------
 struct RunList {
     std::vector<int32_t> row0, phys0, len;
@@ -422,8 +478,9 @@ Runs identity_runs(int64_t n) {
 }
 
 // Dense export of the rows named by `slots` (any order) into [BH, n, D] arrays.
-kvhip_status export_slots(const kvhip_cache *c, const int32_t *slots, int64_t n, void *dk, void *dv,
-                          hipStream_t stream) {
+// dense arrays of the stored head sizes
+kvhip_status export_slots_stored(const kvhip_cache *c, const int32_t *slots, int64_t n, void *dk, void *dv,
+                                 hipStream_t stream) {
     const RunList rl = runs_of(slots, n);
     for (size_t first = 0; first < rl.size(); first += MAXRUNS) {
         const size_t cnt = std::min((size_t)MAXRUNS, rl.size() - first);
@@ -433,6 +490,35 @@ kvhip_status export_slots(const kvhip_cache *c, const int32_t *slots, int64_t n,
         KV_HIP(launch_export_fp(c->st, r, begin, end - begin, 0, (int)n, dk, dv, stream));
     }
     return KVHIP_OK;
+}
+
+// dense arrays of the caller's head sizes (a cache that stores padded rows exports into a buffer of the stored
+// width first and narrows that; the buffer is handed back behind the stream's work)
+kvhip_status export_slots(const kvhip_cache *c, const int32_t *slots, int64_t n, void *dk, void *dv,
+                          hipStream_t stream) {
+    if (!c->padded() || n <= 0) return export_slots_stored(c, slots, n, dk, dv, stream);
+    const Store &st = c->st;
+    const size_t rows = (size_t)st.BH * (size_t)n;
+    void *tk = nullptr, *tv = nullptr;
+    size_t gk = 0, gv = 0;
+    if (dk) KV_HIP(pool_alloc(&tk, rows * st.Dk * st.es, &gk));
+    if (dv) {
+        const hipError_t e = pool_alloc(&tv, rows * st.Dv * st.es, &gv);
+        if (e != hipSuccess) {
+            if (tk) (void)hipFree(tk);
+            KV_HIP(e);
+        }
+    }
+    kvhip_status r = export_slots_stored(c, slots, n, tk, tv, stream);
+    if (r == KVHIP_OK && tk && launch_repitch_rows(dk, (size_t)c->Dk_user * st.es, tk, (size_t)st.Dk * st.es, rows, stream) != hipSuccess)
+        r = fail(KVHIP_ERR_HIP, "narrowing the exported keys failed");
+    if (r == KVHIP_OK && tv && launch_repitch_rows(dv, (size_t)c->Dv_user * st.es, tv, (size_t)st.Dv * st.es, rows, stream) != hipSuccess)
+        r = fail(KVHIP_ERR_HIP, "narrowing the exported values failed");
+    std::vector<std::pair<void *, size_t>> tmp;
+    if (tk) tmp.push_back({tk, gk});
+    if (tv) tmp.push_back({tv, gv});
+    retire(std::move(tmp), stream);
+    return r;
 }
 
 // ---- rotating: physical slot management ---------------------------------------
@@ -795,6 +881,8 @@ void kvhip_cache_free(kvhip_cache *c) {
     for (const Slab &sl : c->slabs) ptrs.push_back({sl.base, sl.bytes});
     if (c->st.pt) ptrs.push_back({const_cast<PageEntry *>(c->st.pt), (size_t)0});
     if (c->ws) ptrs.push_back({c->ws, c->ws_bytes});
+    for (int i = 0; i < 4; ++i)
+        if (c->pad_buf[i]) ptrs.push_back({c->pad_buf[i], c->pad_bytes[i]});
     if (c->stage_tmp_k) ptrs.push_back({c->stage_tmp_k, (size_t)0});
     if (c->stage_tmp_v) ptrs.push_back({c->stage_tmp_v, (size_t)0});
     for (auto &q : c->parked) ptrs.push_back(q);
@@ -891,6 +979,11 @@ kvhip_status kvhip_cache_update(kvhip_cache *c, const void *keys, const void *va
         }
     }
     KV_TRY(set_geometry(c, B, Hkv, Dk, Dv, dtype));
+    if (c->padded()) {  // rows of the stored head sizes, the added columns zero (a rotation reads its partners inside Dk)
+        const size_t rows = (size_t)B * Hkv * L;
+        KV_TRY(widen_rows(c, 0, keys, rows, Dk, c->st.Dk, S(c, stream), &keys));
+        KV_TRY(widen_rows(c, 1, values, rows, Dv, c->st.Dv, S(c, stream), &values));
+    }
     if (c->staging) return stage_update(c, keys, values, L, S(c, stream));
     if (c->kind == KVHIP_KIND_ROTATING) return update_rotating(c, keys, values, L, S(c, stream));
     return update_simple(c, keys, values, L, S(c, stream));
@@ -985,9 +1078,34 @@ kvhip_status attend_impl(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, i
     const bool staged_view = c->staging && !c->stage_view.empty();
     if (!c->has_geom || (!c->has_buffers && !staged_view) || c->presented <= 0)
         return fail(KVHIP_ERR_STATE, "attention over an empty cache");
-    if (B != c->B || D != c->st.Dk) return fail(KVHIP_ERR_INVALID_ARG, "query shape does not match the cache");
+    if (B != c->B || D != c->Dk_user) return fail(KVHIP_ERR_INVALID_ARG, "query shape does not match the cache");
     if (Hq <= 0 || Hq % c->Hkv) return fail(KVHIP_ERR_INVALID_ARG, "query heads must be a multiple of KV heads");
     if (L <= 0 || L > 65535) return fail(KVHIP_ERR_INVALID_ARG, "query length out of range");
+    // A cache that stores padded rows: the queries are widened with zero columns and the kernels write output rows of
+    // the stored width, which are narrowed at the end.  The allocation-free entry takes both buffers from the front of
+    // its scratch.
+    void *user_out = nullptr;
+    const size_t q_rows = (size_t)B * Hq * L;
+    if (c->padded()) {
+        const size_t es = c->st.es;
+        if (fixed) {
+            const size_t qb = align256(q_rows * c->st.Dk * es), ob = align256(q_rows * c->st.Dv * es);
+            if (qb + ob > fixed_bytes / 2)
+                return fail(KVHIP_ERR_UNSUPPORTED, "the padded queries and outputs of this call do not fit the allocation-free entry point's scratch");
+            char *base = reinterpret_cast<char *>(fixed);
+            KV_HIP(launch_repitch_rows(base, (size_t)c->st.Dk * es, q, (size_t)D * es, q_rows, S(c, stream)));
+            q = base;
+            user_out = out;
+            out = base + qb;
+            fixed = reinterpret_cast<float *>(base + qb + ob);
+            fixed_bytes -= qb + ob;
+        } else {
+            KV_TRY(widen_rows(c, 2, q, q_rows, D, c->st.Dk, S(c, stream), &q));
+            KV_TRY(ensure_pad_buf(c, 3, q_rows * c->st.Dv * es));
+            user_out = out;
+            out = c->pad_buf[3];
+        }
+    }
     AttendArgs a;
     a.st = c->st;
     KV_TRY(presented_runs(c, a.runs, a.slots));
@@ -1047,6 +1165,8 @@ kvhip_status attend_impl(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, i
         g_last_kernel = 0;
         KV_HIP(launch_attend_generic(a, s));
     }
+    if (user_out)
+        KV_HIP(launch_repitch_rows(user_out, (size_t)c->Dv_user * c->st.es, out, (size_t)c->st.Dv * c->st.es, q_rows, s));
     return KVHIP_OK;
 }
 }  // namespace
@@ -1073,7 +1193,7 @@ kvhip_status kvhip_cache_update_attend(kvhip_cache *c, const void *q, const void
     // step is a single launch.  The bookkeeping of `updateQuantized` runs here as usual.
     if (c && k && v && q && out && L == 1 && c->kind == KVHIP_KIND_QUANTIZED && !c->staging && !c->rope &&
         (dtype == KVHIP_F16 || dtype == KVHIP_BF16) && (!mask || mask->mode == KVHIP_MASK_NONE) && c->has_geom &&
-        c->has_buffers && c->B == B && c->Hkv == Hkv && c->st.Dk == Dk && c->st.Dv == Dv && c->st.dtype == dtype) {
+        c->has_buffers && !c->padded() && c->B == B && c->Hkv == Hkv && c->st.Dk == Dk && c->st.Dv == Dv && c->st.dtype == dtype) {
         KV_TRY(update_simple(c, k, v, 1, S(c, stream), false));
         const kvhip_status st = attend_impl(c, q, B, Hq, L, Dk, scale, mask, out, stream, nullptr, 0, k, v, (int32_t)c->offset - 1);
         if (st != KVHIP_OK) {  // nothing was written: take the row back
@@ -1088,7 +1208,7 @@ kvhip_status kvhip_cache_update_attend(kvhip_cache *c, const void *q, const void
     // the cache holds what its counters say.
     if (c && k && v && q && out && L == 1 && (c->kind == KVHIP_KIND_SIMPLE || c->kind == KVHIP_KIND_ROTATING) &&
         !c->staging && !c->rope && (dtype == KVHIP_F16 || dtype == KVHIP_BF16) && (!mask || mask->mode == KVHIP_MASK_NONE) &&
-        c->has_geom && c->has_buffers && c->B == B && c->Hkv == Hkv && c->st.Dk == Dk && c->st.Dv == Dv && c->st.dtype == dtype) {
+        c->has_geom && c->has_buffers && !c->padded() && c->B == B && c->Hkv == Hkv && c->st.Dk == Dk && c->st.Dv == Dv && c->st.dtype == dtype) {
         int32_t slot = -1;
         if (c->kind == KVHIP_KIND_SIMPLE) {
             KV_TRY(update_simple(c, k, v, 1, S(c, stream), false));
@@ -1177,11 +1297,11 @@ kvhip_status kvhip_cache_state_desc(const kvhip_cache *c, int32_t i, int64_t sha
     shape[1] = c->Hkv;
     shape[2] = state_rows(c);
     if (c->kind != KVHIP_KIND_QUANTIZED) {
-        shape[3] = i == 0 ? s.Dk : s.Dv;
+        shape[3] = i == 0 ? c->Dk_user : c->Dv_user;
         *dtype = s.dtype;
         return KVHIP_OK;
     }
-    const int D = i < 3 ? s.Dk : s.Dv;
+    const int D = i < 3 ? c->Dk_user : c->Dv_user;
     if (i % 3 == 0) {
         shape[3] = D * s.bits / 32;
         *dtype = KVHIP_U32;
@@ -1199,7 +1319,25 @@ kvhip_status kvhip_cache_state_export(const kvhip_cache *c, int32_t i, void *dst
     if (n == 0) return KVHIP_OK;  // (an array of no rows -- a cache trimmed back to empty -- has no address)
     if (!dst) return fail(KVHIP_ERR_INVALID_ARG, "null argument");
     if (c->kind == KVHIP_KIND_QUANTIZED) {
-        KV_HIP(launch_export_quant(c->st, i, (int)n, dst, S(c, stream)));
+        if (!c->padded()) {
+            KV_HIP(launch_export_quant(c->st, i, (int)n, dst, S(c, stream)));
+            return KVHIP_OK;
+        }
+        // the array of the stored width first, then its leading columns (codes are a bit stream from column 0 on,
+        // pairs come one per group: the caller's columns are a prefix of every row)
+        const Store &st = c->st;
+        const int Ds = i < 3 ? st.Dk : st.Dv, Du = i < 3 ? c->Dk_user : c->Dv_user;
+        const size_t wide = i % 3 == 0 ? (size_t)Ds * st.bits / 8 : (size_t)(Ds / st.gs) * st.es;
+        const size_t narrow = i % 3 == 0 ? (size_t)Du * st.bits / 8 : (size_t)(Du / st.gs) * st.es;
+        const size_t rows = (size_t)st.BH * (size_t)n;
+        void *tmp = nullptr;
+        size_t got = 0;
+        KV_HIP(pool_alloc(&tmp, rows * wide, &got));
+        hipError_t e = launch_export_quant(st, i, (int)n, tmp, S(c, stream));
+        if (e == hipSuccess) e = launch_repitch_rows(dst, narrow, tmp, wide, rows, S(c, stream));
+        std::vector<std::pair<void *, size_t>> t{{tmp, got}};
+        retire(std::move(t), S(c, stream));
+        KV_HIP(e);
         return KVHIP_OK;
     }
     std::vector<int32_t> ident;
@@ -1259,8 +1397,37 @@ kvhip_status kvhip_cache_state_import(kvhip_cache *c, int32_t count, const void 
     KV_TRY(set_geometry(c, (int)B, (int)H, Dk, Dv, dtype));
     hipStream_t s = S(c, stream);
     KV_TRY(ensure_slots(c, std::max<int64_t>(n, 1), s, true));
-    if (q) KV_HIP(launch_import_quant(c->st, srcs, (int)n, s));
-    else KV_HIP(launch_import_fp(c->st, srcs[0], srcs[1], (int)n, s));
+    const void *wide_srcs[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+    std::vector<std::pair<void *, size_t>> tmp;
+    if (c->padded() && n > 0) {
+        // arrays of the stored widths, the added columns zero (codes 0 with scale 0 and bias 0 are zero values)
+        const Store &st = c->st;
+        const size_t rows = (size_t)st.BH * (size_t)n;
+        hipError_t e = hipSuccess;
+        for (int a = 0; a < count && e == hipSuccess; ++a) {
+            const bool keys = q ? a < 3 : a == 0;
+            const int Ds = keys ? st.Dk : st.Dv, Du = keys ? c->Dk_user : c->Dv_user;
+            const size_t wide = !q ? (size_t)Ds * st.es : (a % 3 == 0 ? (size_t)Ds * st.bits / 8 : (size_t)(Ds / st.gs) * st.es);
+            const size_t narrow = !q ? (size_t)Du * st.es : (a % 3 == 0 ? (size_t)Du * st.bits / 8 : (size_t)(Du / st.gs) * st.es);
+            void *p = nullptr;
+            size_t got = 0;
+            e = pool_alloc(&p, rows * wide, &got);
+            if (e != hipSuccess) break;
+            tmp.push_back({p, got});
+            e = launch_repitch_rows(p, wide, srcs[a], narrow, rows, s);
+            wide_srcs[a] = p;
+        }
+        if (e != hipSuccess) {
+            retire(std::move(tmp), s);
+            KV_HIP(e);
+        }
+        srcs = wide_srcs;
+    }
+    {
+        const hipError_t e = q ? launch_import_quant(c->st, srcs, (int)n, s) : launch_import_fp(c->st, srcs[0], srcs[1], (int)n, s);
+        retire(std::move(tmp), s);
+        KV_HIP(e);
+    }
     c->has_buffers = true;
     c->ref_len = n;
     c->presented = n;
@@ -1362,7 +1529,7 @@ kvhip_status kvhip_cache_copy(const kvhip_cache *c, void *stream, kvhip_cache **
     if (c->has_buffers) {
         // `new.state = self.state`: the copy's buffers hold exactly the exported rows
         n->has_geom = false;
-        kvhip_status st = set_geometry(n, c->B, c->Hkv, c->st.Dk, c->st.Dv, c->st.dtype);
+        kvhip_status st = set_geometry(n, c->B, c->Hkv, c->Dk_user, c->Dv_user, c->st.dtype);
         if (st == KVHIP_OK) st = ensure_slots(n, std::max<int64_t>(rows, 1), s, true);
         if (st != KVHIP_OK) { kvhip_cache_free(n); return st; }
         if (c->kind == KVHIP_KIND_QUANTIZED) {
@@ -1450,7 +1617,7 @@ kvhip_status kvhip_cache_stage_commit(kvhip_cache *c, int64_t retaining, void *s
             KV_HIP(hipMalloc(&c->stage_tmp_v, (size_t)c->st.BH * rows * c->st.Dv * c->st.es));
             c->stage_tmp_rows = rows;
         }
-        st = export_slots(c, c->staged.data(), keep, c->stage_tmp_k, c->stage_tmp_v, s);
+        st = export_slots_stored(c, c->staged.data(), keep, c->stage_tmp_k, c->stage_tmp_v, s);
     }
     for (int32_t slot : c->staged) c->used[(size_t)slot] = 0;
     c->staged.clear();
@@ -1490,7 +1657,7 @@ kvhip_status kvhip_cache_to_quantized(const kvhip_cache *c, int32_t group_size, 
         (*out)->offset = c->offset;
         return KVHIP_OK;
     }
-    const int eff = kvhip_resolved_group_size(group_size, c->st.Dk, c->st.Dv);
+    const int eff = kvhip_resolved_group_size(group_size, c->Dk_user, c->Dv_user);
     if (!eff)
         return fail(KVHIP_ERR_STATE,
                     "KV cache quantization requires head dimensions divisible by one of the supported group sizes (32, 64, 128).");
@@ -1498,7 +1665,10 @@ kvhip_status kvhip_cache_to_quantized(const kvhip_cache *c, int32_t group_size, 
     kvhip_cache *n = nullptr;
     KV_TRY(kvhip_cache_create(&cfg, &n));
     const int64_t rows = std::max<int64_t>(c->offset, 0);
-    kvhip_status st = set_geometry(n, c->B, c->Hkv, c->st.Dk, c->st.Dv, c->st.dtype);
+    kvhip_status st = set_geometry(n, c->B, c->Hkv, c->Dk_user, c->Dv_user, c->st.dtype);
+    // (the conversion goes from pages to pages: both caches have to store the same head sizes)
+    if (st == KVHIP_OK && (n->st.Dk != c->st.Dk || n->st.Dv != c->st.Dv))
+        st = fail(KVHIP_ERR_UNSUPPORTED, "a quantized cache of this group size stores other head sizes than the cache being converted");
     if (st == KVHIP_OK) st = ensure_slots(n, std::max<int64_t>(rows, 1), s, true);
     if (st != KVHIP_OK) { kvhip_cache_free(n); return st; }
     // one pass from the full-precision pages into the new cache's pages, enqueued on the stream
@@ -1524,7 +1694,9 @@ kvhip_status kvhip_cache_to_unquantized(const kvhip_cache *c, void *stream, kvhi
     if (!c->has_buffers) { *out = n; return KVHIP_OK; }
     const int64_t rows = std::max<int64_t>(std::min(c->offset, c->ref_len), 0);
     const Store &q = c->st;
-    kvhip_status st = set_geometry(n, c->B, c->Hkv, q.Dk, q.Dv, q.dtype);
+    kvhip_status st = set_geometry(n, c->B, c->Hkv, c->Dk_user, c->Dv_user, q.dtype);
+    if (st == KVHIP_OK && (n->st.Dk != q.Dk || n->st.Dv != q.Dv))
+        st = fail(KVHIP_ERR_UNSUPPORTED, "a full-precision cache stores other head sizes than the quantized cache being converted");
     if (st == KVHIP_OK) st = ensure_slots(n, std::max<int64_t>(rows, 1), s, true);
     if (st != KVHIP_OK) { kvhip_cache_free(n); return st; }
     if (rows > 0) KV_HIP_OR(launch_dequant_pages(q, n->st, (int)rows, s), kvhip_cache_free(n));

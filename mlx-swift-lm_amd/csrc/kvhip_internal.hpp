@@ -263,6 +263,8 @@ hipError_t launch_mask_materialize(const kvhip_mask_plan_t &plan, uint8_t *dst, 
 // Zero / copy `bytes` of device memory with a kernel (16-byte aligned pointers and sizes).
 hipError_t launch_fill_zero(void *dst, size_t bytes, hipStream_t s);
 hipError_t launch_copy_bytes(void *dst, const void *src, size_t bytes, hipStream_t s);
+// `rows` dense rows of src_pitch bytes into rows of dst_pitch bytes (both even): common prefix copied, rest zero-filled
+hipError_t launch_repitch_rows(void *dst, size_t dst_pitch, const void *src, size_t src_pitch, size_t rows, hipStream_t s);
 // Page-table entries [first, first + count): page first + i keeps its cells at base.x + i * stride.x
 // for each plane x (pages backed by one allocation lie at a regular stride).
 hipError_t launch_set_pages(PageEntry *pt, int first, int count, PageEntry base, const size_t stride[4], hipStream_t s);

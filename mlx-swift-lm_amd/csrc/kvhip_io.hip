@@ -763,6 +763,34 @@ hipError_t launch_copy_bytes(void *dst, const void *src, size_t bytes, hipStream
     return hipGetLastError();
 }
 
+// Dense rows of one pitch into dense rows of another: the common prefix of every row is copied, what is left of a
+// wider destination row is zero-filled.  (How arrays of a head size the tuned kernels are not built for are widened
+// to the size the cache stores, and narrowed again on the way out.)
+template <typename U>
+__global__ void __launch_bounds__(256) repitch_rows_kernel(U *dst, uint32_t dst_units, const U *src, uint32_t src_units, size_t rows) {
+    const size_t total = rows * dst_units;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const size_t row = i / dst_units;
+        const uint32_t u = (uint32_t)(i - row * dst_units);
+        dst[i] = u < src_units ? src[row * src_units + u] : (U)0;
+    }
+}
+
+hipError_t launch_repitch_rows(void *dst, size_t dst_pitch, const void *src, size_t src_pitch, size_t rows, hipStream_t s) {
+    if (rows == 0 || dst_pitch == 0) return hipSuccess;
+    if ((dst_pitch | src_pitch) & 1) return hipErrorInvalidValue;
+    const bool words = ((dst_pitch | src_pitch) & 3) == 0;
+    const size_t units = rows * (dst_pitch / (words ? 4 : 2));
+    const unsigned blocks = (unsigned)std::min<size_t>((units + 255) / 256, 4096);
+    if (words)
+        hipLaunchKernelGGL(repitch_rows_kernel<uint32_t>, dim3(blocks), dim3(256), 0, s, (uint32_t *)dst, (uint32_t)(dst_pitch / 4),
+                           (const uint32_t *)src, (uint32_t)(src_pitch / 4), rows);
+    else
+        hipLaunchKernelGGL(repitch_rows_kernel<uint16_t>, dim3(blocks), dim3(256), 0, s, (uint16_t *)dst, (uint32_t)(dst_pitch / 2),
+                           (const uint16_t *)src, (uint32_t)(src_pitch / 2), rows);
+    return hipGetLastError();
+}
+
 hipError_t launch_mask_materialize(const kvhip_mask_plan_t &plan, uint8_t *dst, hipStream_t s) {
     if (plan.cols <= 0) return hipSuccess;
     dim3 grid((plan.cols + 255) / 256, plan.rolled ? 1 : (plan.rows < 1024 ? plan.rows : 1024)), block(256);
