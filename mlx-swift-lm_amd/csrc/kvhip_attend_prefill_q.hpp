@@ -71,12 +71,27 @@ template <int BITS, int N> __device__ __forceinline__ uint32_t stream_code_at(co
     if (sh + BITS > 32) v |= w[wi + 1 < N ? wi + 1 : wi] << ((32 - sh) & 31);
     return v & ((1u << BITS) - 1u);
 }
-// codes 8 c .. 8 c + 7 of such a unit as four (1024 + code, 1024 + code) float16 pairs
-template <int BITS, int N> __device__ __forceinline__ u4 stream_chunk(const uint32_t (&w)[N], int c) {
+// codes 8 c .. 8 c + 7 of such a unit as four (1024 + code, 1024 + code) float16 pairs; `mag` is 0x64006400 in a
+// vector register.  A pair of adjacent codes is cut out as one field of 2 BITS bits; for 2, 3 and 5 bits the field
+// times (1 + 2^(16 - BITS)) has the first code at bit 0 and the second at bit 16 (what else the product holds lies
+// between them and cannot carry into bit 16: the low part stays below 2^16), so one 24-bit multiply and one
+// mask-and-OR finish the pair.  Six-bit codes would carry (63 + 63 * 64 + 63 * 1024 > 2^16) and are placed one by one.
+template <int BITS, int N> __device__ __forceinline__ u4 stream_chunk(const uint32_t (&w)[N], int c, uint32_t mag) {
     u4 o;
+    constexpr uint32_t M1 = (1u << BITS) - 1u;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-        o[i] = stream_code_at<BITS, N>(w, 8 * c + 2 * i) | (stream_code_at<BITS, N>(w, 8 * c + 2 * i + 1) << 16) | 0x64006400u;
+    for (int i = 0; i < 4; ++i) {
+        if constexpr (BITS == 6) {
+            o[i] = stream_code_at<BITS, N>(w, 8 * c + 2 * i) | (stream_code_at<BITS, N>(w, 8 * c + 2 * i + 1) << 16) | mag;
+        } else {
+            const int bit = (8 * c + 2 * i) * BITS, wi = bit >> 5, sh = bit & 31;
+            uint32_t x = w[wi] >> sh;
+            if (sh + 2 * BITS > 32) x = __builtin_amdgcn_alignbit(w[wi + 1 < N ? wi + 1 : wi], w[wi], sh);
+            x &= (1u << (2 * BITS)) - 1u;
+            const uint32_t y = __umul24(x, 1u + (1u << (16 - BITS)));
+            o[i] = (y & (M1 | (M1 << 16))) | mag;
+        }
+    }
     return o;
 }
 // (scale, bias) pair of dtype DT in one dword -> float16 (scale, scale) and (bias, bias)
@@ -367,7 +382,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
         sb_h2<DT>(ksb[e], s2, b2);
         u4 o;
         if constexpr (GEN) {
-            const u4 x = stream_chunk<BITS, UWD>(codes[e], c);
+            const u4 x = stream_chunk<BITS, UWD>(codes[e], c, mag);
             o.x = deq_pair(x.x, m1024, s2, b2);
             o.y = deq_pair(x.y, m1024, s2, b2);
             o.z = deq_pair(x.z, m1024, s2, b2);
@@ -401,7 +416,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
         const kv_h2 b2 = __builtin_bit_cast(kv_h2, bw[2]), b3 = __builtin_bit_cast(kv_h2, bw[3]);
         u4 o;
         if constexpr (GEN) {  // a plain bit stream over the tile's tokens
-            const u4 x = stream_chunk<BITS, UWD>(codes[e], c);
+            const u4 x = stream_chunk<BITS, UWD>(codes[e], c, mag);
             o.x = deq_pair(x.x, m1024, s0, b0);
             o.y = deq_pair(x.y, m1024, s1, b1);
             o.z = deq_pair(x.z, m1024, s2, b2);
