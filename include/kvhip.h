@@ -144,7 +144,9 @@ kvhip_status kvhip_profile_read(int32_t *out_launches, double *out_total_ms);
 kvhip_status kvhip_cache_create(const kvhip_config *config, kvhip_cache **out_cache);
 /* Safe with NULL.  Does not wait for the device: the cache's memory is released once the work
  * enqueued on the stream it was last used with has run (by a later kvhip_sync / kvhip_cache_reserve,
- * or at once if that stream is idle). */
+ * or at once if that stream is idle), and is then kept for reuse by later allocations of a similar size.
+ * Only the last stream is tracked: a caller that reads one cache from several streams has to order them
+ * (an event wait on the last one) before it frees the cache. */
 void kvhip_cache_free(kvhip_cache *cache);
 /* `copy()` (KVCache.swift:525-533, :877-885, :1177-1185): independent deep copy. */
 kvhip_status kvhip_cache_copy(const kvhip_cache *cache, void *stream, kvhip_cache **out_cache);
