@@ -562,17 +562,25 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     }
     __syncthreads();
     // ---- merge the 4 wavefronts; a single span writes the output rows, several leave partials ---
+    // the weights of a row's four parts once per row (not once per column: an exponential each)
+    __shared__ float wrow[WAVES][RR], mrow[RR];
+    if (threadIdx.x < WAVES * RR) {
+        const int i = threadIdx.x / WAVES, w = threadIdx.x - i * WAVES;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int w2 = 0; w2 < WAVES; ++w2) mx = fmaxf(mx, cbuf[w2][i][D]);
+        const float mw = cbuf[w][i][D];
+        wrow[w][i] = (mw == -INFINITY) ? 0.f : fast_exp2((mw - mx) * LOG2E);
+        if (w == 0) mrow[i] = mx;
+    }
+    __syncthreads();
     if (nsplit == 1) {
         for (int idx = threadIdx.x; idx < R * D; idx += WAVES * 64) {
             const int i = idx / D, c = idx - i * D;
-            float mx = -INFINITY;
-#pragma unroll
-            for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, cbuf[w][i][D]);
             float v = 0.f, l = 0.f;
 #pragma unroll
             for (int w = 0; w < WAVES; ++w) {
-                const float mw = cbuf[w][i][D];
-                const float wgt = (mw == -INFINITY) ? 0.f : fast_exp2((mw - mx) * LOG2E);
+                const float wgt = wrow[w][i];
                 v += wgt * cbuf[w][i][c];
                 l += wgt * cbuf[w][i][D + 1];
             }
@@ -584,20 +592,13 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     float *part = a.workspace + part_slot * RR * (D + 2);
     for (int idx = threadIdx.x; idx < RR * (D + 2); idx += WAVES * 64) {
         const int i = idx / (D + 2), c = idx - i * (D + 2);
-        float mx = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < WAVES; ++w) mx = fmaxf(mx, cbuf[w][i][D]);
         float v;
         if (c == D) {
-            v = mx;
+            v = mrow[i];
         } else {
             v = 0.f;
 #pragma unroll
-            for (int w = 0; w < WAVES; ++w) {
-                const float mw = cbuf[w][i][D];
-                const float wgt = (mw == -INFINITY) ? 0.f : fast_exp2((mw - mx) * LOG2E);
-                v += wgt * cbuf[w][i][c];
-            }
+            for (int w = 0; w < WAVES; ++w) v += wrow[w][i] * cbuf[w][i][c];
         }
         part[idx] = v;
     }
