@@ -91,17 +91,64 @@ __device__ __forceinline__ uint32_t affine_code(float w, float scale, float bias
     return (uint32_t)q;
 }
 
-// Min/max over a group of `width` (<= 64, power of two) adjacent lanes.
+// Min/max over GL (4, 8 or 16) adjacent lanes without LDS round trips: two quad permutes, then
+// the mirror of each half row and of each row (the lanes of a quad, then of a half row, already
+// agree, so the mirrored lane holds the other half's result).  Minimum and maximum do not depend
+// on the order of the reduction.
+// Each step is one instruction per value, the permute being an operand modifier (through the
+// permuting-move builtin a step came out as a copy, the move, a quieting maximum and the minimum:
+// 24 instructions per reduction of two values at GL = 8 instead of 6).  A register written by a
+// vector instruction may be read through a permute two wait states later at the earliest: the
+// other value's instruction and one s_nop stand between; the leading s_nop covers whatever wrote
+// the inputs (and a write of the execution mask, five wait states).
+#define KV_MINMAX_STEP(CTRL)                                                \
+    "v_min_f32_dpp %0, %0, %0 " CTRL " row_mask:0xf bank_mask:0xf\n\t"      \
+    "v_max_f32_dpp %1, %1, %1 " CTRL " row_mask:0xf bank_mask:0xf\n\t"      \
+    "s_nop 0\n\t"
+template <int GL> __device__ __forceinline__ void group_minmax_dpp(float &mn, float &mx) {
+    static_assert(GL == 4 || GL == 8 || GL == 16, "lanes per quantization group");
+    if constexpr (GL == 4)
+        asm volatile("s_nop 4\n\t" KV_MINMAX_STEP("quad_perm:[1,0,3,2]") KV_MINMAX_STEP("quad_perm:[2,3,0,1]") : "+v"(mn), "+v"(mx));
+    else if constexpr (GL == 8)
+        asm volatile("s_nop 4\n\t" KV_MINMAX_STEP("quad_perm:[1,0,3,2]") KV_MINMAX_STEP("quad_perm:[2,3,0,1]")
+                     KV_MINMAX_STEP("row_half_mirror") : "+v"(mn), "+v"(mx));
+    else
+        asm volatile("s_nop 4\n\t" KV_MINMAX_STEP("quad_perm:[1,0,3,2]") KV_MINMAX_STEP("quad_perm:[2,3,0,1]")
+                     KV_MINMAX_STEP("row_half_mirror") KV_MINMAX_STEP("row_mirror") : "+v"(mn), "+v"(mx));
+}
+#undef KV_MINMAX_STEP
+
+// Min/max over a group of `width` (32 or 64) adjacent lanes of a wavefront; every lane gets its group's values.
+// Rows of 16 lanes are reduced with the permutes above; the four rows' results are then read into scalar registers
+// and combined there (twelve LDS permutes with their latencies, which is what the reduction cost as a butterfly of
+// __shfl_xor, held a single-row append up for a microsecond per 64 elements).  Minimum and maximum do not depend on
+// the order of the reduction.
 __device__ __forceinline__ void group_minmax(float &mn, float &mx, int width) {
-    for (int off = 1; off < width; off <<= 1) {
-        mn = fminf(mn, __shfl_xor(mn, off));
-        mx = fmaxf(mx, __shfl_xor(mx, off));
+    group_minmax_dpp<16>(mn, mx);
+    const int mi = __builtin_bit_cast(int, mn), xi = __builtin_bit_cast(int, mx);
+    const float n0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(mi, 0)), n1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(mi, 16));
+    const float n2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(mi, 32)), n3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(mi, 48));
+    const float x0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 0)), x1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 16));
+    const float x2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 32)), x3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(xi, 48));
+    const float nlo = fminf(n0, n1), nhi = fminf(n2, n3), xlo = fmaxf(x0, x1), xhi = fmaxf(x2, x3);
+    if (width >= 64) {
+        mn = fminf(nlo, nhi);
+        mx = fmaxf(xlo, xhi);
+    } else {  // 32: lanes 0..31 and 32..63 are two groups
+        const bool upper = (threadIdx.x & 32) != 0;
+        mn = upper ? nhi : nlo;
+        mx = upper ? xhi : xlo;
     }
 }
 
-// OR-combine `v` across `width` adjacent lanes (power of two).
+// OR-combine `v` across `width` (2, 4, 8 or 16) adjacent lanes: one instruction per step, the permute an operand modifier.
 __device__ __forceinline__ uint32_t group_or(uint32_t v, int width) {
-    for (int off = 1; off < width; off <<= 1) v |= __shfl_xor(v, off);
+#define KV_OR_STEP(CTRL) "v_or_b32_dpp %0, %0, %0 " CTRL " row_mask:0xf bank_mask:0xf\n\ts_nop 1\n\t"
+    if (width >= 2) asm volatile("s_nop 4\n\t" KV_OR_STEP("quad_perm:[1,0,3,2]") : "+v"(v));
+    if (width >= 4) asm volatile(KV_OR_STEP("quad_perm:[2,3,0,1]") : "+v"(v));
+    if (width >= 8) asm volatile(KV_OR_STEP("row_half_mirror") : "+v"(v));
+    if (width >= 16) asm volatile(KV_OR_STEP("row_mirror") : "+v"(v));
+#undef KV_OR_STEP
     return v;
 }
 

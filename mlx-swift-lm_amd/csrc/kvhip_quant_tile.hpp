@@ -70,33 +70,6 @@ __device__ __forceinline__ void unpack8(const u4v &raw, const void *row, int d0,
     }
 }
 
-// Min/max over GL (4, 8 or 16) adjacent lanes without LDS round trips: two quad permutes, then
-// the mirror of each half row and of each row (the lanes of a quad, then of a half row, already
-// agree, so the mirrored lane holds the other half's result).  Minimum and maximum do not depend
-// on the order of the reduction, so the values are those of group_minmax.
-// Each step is one instruction per value, the permute being an operand modifier (through the
-// permuting-move builtin a step came out as a copy, the move, a quieting maximum and the minimum:
-// 24 instructions per reduction of two values at GL = 8 instead of 6).  A register written by a
-// vector instruction may be read through a permute two wait states later at the earliest: the
-// other value's instruction and one s_nop stand between; the leading s_nop covers whatever wrote
-// the inputs (and a write of the execution mask, five wait states).
-#define KV_MINMAX_STEP(CTRL)                                                \
-    "v_min_f32_dpp %0, %0, %0 " CTRL " row_mask:0xf bank_mask:0xf\n\t"      \
-    "v_max_f32_dpp %1, %1, %1 " CTRL " row_mask:0xf bank_mask:0xf\n\t"      \
-    "s_nop 0\n\t"
-template <int GL> __device__ __forceinline__ void group_minmax_dpp(float &mn, float &mx) {
-    static_assert(GL == 4 || GL == 8 || GL == 16, "lanes per quantization group");
-    if constexpr (GL == 4)
-        asm volatile("s_nop 4\n\t" KV_MINMAX_STEP("quad_perm:[1,0,3,2]") KV_MINMAX_STEP("quad_perm:[2,3,0,1]") : "+v"(mn), "+v"(mx));
-    else if constexpr (GL == 8)
-        asm volatile("s_nop 4\n\t" KV_MINMAX_STEP("quad_perm:[1,0,3,2]") KV_MINMAX_STEP("quad_perm:[2,3,0,1]")
-                     KV_MINMAX_STEP("row_half_mirror") : "+v"(mn), "+v"(mx));
-    else
-        asm volatile("s_nop 4\n\t" KV_MINMAX_STEP("quad_perm:[1,0,3,2]") KV_MINMAX_STEP("quad_perm:[2,3,0,1]")
-                     KV_MINMAX_STEP("row_half_mirror") KV_MINMAX_STEP("row_mirror") : "+v"(mn), "+v"(mx));
-}
-#undef KV_MINMAX_STEP
-
 // Codes of the eight elements a thread holds, as integer-valued floats in [0, 2^BITS - 1], from
 // the parameters of their group; `inv` is the hardware reciprocal of `scale`.
 // code = rint((w - bias) / scale), clamped.  The quotient is first formed with the reciprocal
