@@ -1185,7 +1185,7 @@ Plan plan_for(const AttendArgs &a) {
         // KVHIP_RAGGED_SPANS forces the number of spans per batch row (timing builds only: measure_knob)
         static const int forced_spans = measure_knob("KVHIP_RAGGED_SPANS", 0);
         if (forced_spans > 0) p.nsplit = std::min(forced_spans, 512);
-    } else if (a.st.bits != 0 && p.nsplit >= 2 && want <= 4 && p.rg == 1 && a.st.Dk != 96 && a.mask.mode != KVHIP_MASK_ARRAY &&
+    } else if (a.st.bits != 0 && p.nsplit >= 2 && want <= 4 && p.rg == 1 && a.st.Dk != 96 && a.st.Dk != 192 && a.mask.mode != KVHIP_MASK_ARRAY &&
                forced_tiles <= 0) {
         // 128 pairs or more: workgroups of 8 wavefronts, one per CU -- the same wavefronts per CU
         // with half the spans.  With 256 pairs a workgroup takes its pair's whole sequence: the
@@ -1201,8 +1201,8 @@ Plan plan_for(const AttendArgs &a) {
     }
     // a caller with a fixed amount of scratch: fewer, longer spans until the partials fit (one span has none)
     if (a.workspace_cap) {
-        const size_t per_span = (size_t)BH * (a.st.bits != 0 && (p.rg >= 2 || a.st.Dk == 96) ? 16 : 4 * p.rg) *
-                                (a.st.Dk + 2) * sizeof(float);
+        const size_t per_span = (size_t)BH * (a.st.bits != 0 && (p.rg >= 2 || a.st.Dk == 96 || a.st.Dk == 192) ? 16 : 4 * p.rg) *
+                                (a.st.Dv + 2) * sizeof(float);
         while (p.nsplit > 1 && per_span * p.nsplit > a.workspace_cap) {
             if (p.tiles_per_wg > 0) {
                 p.tiles_per_wg *= 2;
@@ -1296,7 +1296,9 @@ hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t
 bool attend_decode_supported(const AttendArgs &a) {
     const Store &s = a.st;
     if (s.dtype != KVHIP_F16 && s.dtype != KVHIP_BF16) return false;
-    if (s.Dk != s.Dv) return false;
+    // keys of 192 with values of 128 (the multi-head latent attention models): quantized caches, on the 16-row kernel
+    const bool mla = s.Dk == 192 && s.Dv == 128 && s.bits != 0;
+    if (s.Dk != s.Dv && !mla) return false;
     const int R = (a.Hq / a.Hkv) * a.L;
     if (R > 16) return false;
     // full precision: more than 8 rows (4 at D = 256) are faster on the prefill tile than on further
@@ -1307,6 +1309,7 @@ bool attend_decode_supported(const AttendArgs &a) {
     if (s.bits != 4 && s.bits != 8) return false;
     if (s.Dk == 64) return s.gs == 32 || s.gs == 64;
     if (s.Dk == 96) return s.gs == 32;  // every row count on the 16-row kernel
+    if (mla) return s.gs == 32 || s.gs == 64;  // likewise
     if (s.Dk == 128) return s.gs == 32 || s.gs == 64 || s.gs == 128;
     if (s.Dk == 256) return s.gs == 64 || s.gs == 128;
     return false;
@@ -1318,21 +1321,24 @@ bool attend_decode_fuses_append(const AttendArgs &a) {
     static const bool off = measure_knob("KVHIP_NO_FUSED_APPEND", 0) != 0;  // (timing builds only)
     if (off) return false;
     if (a.st.bits == 0) return true;  // the full-precision decode kernel, any of its row counts
-    return (a.Hq / a.Hkv) * a.L <= 4 && a.st.Dk != 96;
+    return (a.Hq / a.Hkv) * a.L <= 4 && a.st.Dk != 96 && a.st.Dk != 192;
 }
 
 // 5..16 rows per kv head of a quantized cache go to the 16x16x32 kernel
 // (kvhip_attend_decode16.hip), which always carries 16 rows: measured faster than the 4-row
 // broadcast contraction from 8 rows up (B16, 8 kv heads, 8192 tokens: 37 us against 43 us at
 // 8 rows, 36 us against 87 us at 16).
-// Head size 96 (a row and a half of the 4-row kernel's 64-column halves) takes it for every row count.
-static bool use_decode16(const AttendArgs &a, const Plan &p) { return a.st.bits != 0 && (p.rg >= 2 || a.st.Dk == 96); }
+// Head size 96 (a row and a half of the 4-row kernel's 64-column halves) and keys of 192 with values of 128 take it
+// for every row count.
+static bool use_decode16(const AttendArgs &a, const Plan &p) {
+    return a.st.bits != 0 && (p.rg >= 2 || a.st.Dk == 96 || a.st.Dk == 192);
+}
 
 size_t attend_decode_workspace(const AttendArgs &a) {
     const Plan p = plan_for(a);
     const int rows = use_decode16(a, p) ? 16 : 4 * p.rg;
     if (p.nsplit == 1) return 0;  // a single span writes the output rows itself: no partials
-    return (size_t)a.st.BH * p.nsplit * rows * (a.st.Dk + 2) * sizeof(float);
+    return (size_t)a.st.BH * p.nsplit * rows * (a.st.Dv + 2) * sizeof(float);  // (partials hold output columns)
 }
 
 hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {

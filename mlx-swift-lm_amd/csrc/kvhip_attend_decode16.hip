@@ -100,25 +100,28 @@ template <int BITS> __device__ __forceinline__ constexpr bool hi_of(int p) { ret
 
 // MM: 0 no mask, 1 index-only mask (causal / window with per-batch bounds), 2 array mask.
 // (8-bit codes at D = 256 take more than 256 registers: one workgroup per CU)
-template <int BITS, int D, int GS, int DT, int MM>
-__global__ void __launch_bounds__(WAVES * 64, (D >= 256 && BITS == 8) ? 1 : 2)
+// DK / DV: head sizes of keys / queries and of values / outputs (192 and 128 for the multi-head latent attention
+// models, equal otherwise).
+template <int BITS, int DK, int DV, int GS, int DT, int MM>
+__global__ void __launch_bounds__(WAVES * 64, (DK >= 256 && BITS == 8) ? 1 : 2)
 decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     using CD = Codes<BITS>;
-    constexpr int G = D / GS;                    // quantization groups per row
+    constexpr int GK = DK / GS, GV = DV / GS;    // quantization groups per K row and per V row
     constexpr int SPG = GS / 32;                 // contraction steps per group
     constexpr int KWL = GS * BITS / 8 / 16;      // words per lane, group and K row (segment of GS/4 codes)
-    constexpr int NDB = D / 16;                  // 16-row blocks of out^T
+    constexpr int NDB = DV / 16;                 // 16-row blocks of out^T
     constexpr int VWL = 16 * BITS / 32;          // words per lane and V row: its 16 tokens
     constexpr int VROW = 64 * BITS / 8;          // bytes of one V tile row
     constexpr int RR = 16;
     // Three or four groups per row (group size 32 at D = 96 / 128, 64 at D = 256), and D = 256 with two: the (scale, bias) pairs of a tile -- 64 tokens
     // x G pairs per side, 2 G registers per token of the lane group if held in registers -- go from global memory
     // straight into LDS one tile ahead and are read from there four tokens at a time when they are used.
-    constexpr bool SB_LDS = G >= 3 || D >= 256;  // (D = 256: the accumulators alone take 64 registers)
+    constexpr bool SB_LDS = GK >= 3 || GV >= 3 || DK >= 256;  // (D = 256: the accumulators alone take 64 registers)
     // words between the 64-word pieces the pairs arrive in (G = 2, 4: no lane group's pairs straddle two pieces;
     // the gap keeps the four lane groups' reads on different banks)
-    constexpr int SB_PAD = (G == 4 || G == 2) ? 4 : 0;
-    constexpr int SB_WORDS = SB_LDS ? G * (64 + SB_PAD) : 4;
+    constexpr int SB_PAD_K = (GK == 4 || GK == 2) ? 4 : 0, SB_PAD_V = (GV == 4 || GV == 2) ? 4 : 0;
+    constexpr int SB_WORDS_K = GK * (64 + SB_PAD_K), SB_WORDS_V = GV * (64 + SB_PAD_V);
+    constexpr int SB_WORDS = SB_LDS ? (SB_WORDS_K > SB_WORDS_V ? SB_WORDS_K : SB_WORDS_V) : 4;
     const Store &st = a.st;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -129,7 +132,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     const int R = r * a.L;
     size_t part_slot = (size_t)bh * nsplit + split;  // where this workgroup's partial goes
 
-    __shared__ float cbuf[WAVES][RR][D + 2];
+    __shared__ float cbuf[WAVES][RR][DV + 2];
     __shared__ __attribute__((aligned(16))) uint32_t sbuf[WAVES][2][2][SB_WORDS];  // [wavefront][tile parity][K, V][pairs]
 
     // ---- span of this workgroup (as in the 4-row kernel) -----------------------------------
@@ -177,7 +180,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     int page_k = my_tiles > 0 ? tile0 >> 2 : 0, page_v = page_k;
     const size_t k_off = (size_t)bh * st.k_cell + (size_t)tip * TILE * st.k_row
                          + (size_t)(16 * (n >> 2) + (n & 3)) * st.k_row + jj * (KWL * 4);
-    const size_t v_off = (size_t)bh * st.v_cell + (size_t)tip * D * VROW + (size_t)n * VROW + jj * (VWL * 4);
+    const size_t v_off = (size_t)bh * st.v_cell + (size_t)tip * DV * VROW + (size_t)n * VROW + jj * (VWL * 4);
     // (scale, bias) pairs of this lane group's 16 tokens, 16 jj .. 16 jj + 15
     const size_t ksb_off = (size_t)bh * st.ksb_cell + (size_t)(tip * TILE + 16 * jj) * st.ksb_row;
     const size_t vsb_off = (size_t)bh * st.vsb_cell + (size_t)(tip * TILE + 16 * jj) * st.vsb_row;
@@ -190,9 +193,9 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     int base_next = tile0 * TILE;
 
     struct Tile {
-        uint32_t k[4][G][KWL];
+        uint32_t k[4][GK][KWL];
         uint32_t v[NDB][VWL];
-        uint32_t ksb[SB_LDS ? 1 : 16][G], vsb[SB_LDS ? 1 : 16][G];  // raw (scale, bias) pairs per token of the lane group
+        uint32_t ksb[SB_LDS ? 1 : 16][GK], vsb[SB_LDS ? 1 : 16][GV];  // raw (scale, bias) pairs per token of the lane group
         int base;                          // first slot of the tile
     };
     // (SB_LDS) the pairs of the wavefront's tile number `i`, both sides, into the buffer of that parity; the plane
@@ -205,10 +208,9 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         const gptr vs = vsb_n + (size_t)bh * st.vsb_cell + tile_off * st.vsb_row;
         const int par = sb_issued & 1;
 #pragma unroll
-        for (int c = 0; c < G; ++c) {
-            load_dword_to_lds(ks, (uint32_t)(c * 256 + lane * 4), &sbuf[wave][par][0][c * (64 + SB_PAD)]);
-            load_dword_to_lds(vs, (uint32_t)(c * 256 + lane * 4), &sbuf[wave][par][1][c * (64 + SB_PAD)]);
-        }
+        for (int c = 0; c < GK; ++c) load_dword_to_lds(ks, (uint32_t)(c * 256 + lane * 4), &sbuf[wave][par][0][c * (64 + SB_PAD_K)]);
+#pragma unroll
+        for (int c = 0; c < GV; ++c) load_dword_to_lds(vs, (uint32_t)(c * 256 + lane * 4), &sbuf[wave][par][1][c * (64 + SB_PAD_V)]);
         ++sb_issued;
         if (sb_issued < my_tiles) {
             ++page_sb;
@@ -216,10 +218,12 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             vsb_n = as_global(st.pt[page_sb].vsb);
         }
     };
-    // (SB_LDS) the pairs of tokens 4 tb .. 4 tb + 3 of the lane group, `side` 0 K / 1 V: out[i * G + g]
-    auto sb_quad = [&](int par, int side, int tb, uint32_t (&out)[4 * G]) __attribute__((always_inline)) {
+    // (SB_LDS) the pairs of tokens 4 tb .. 4 tb + 3 of the lane group, side 0 K (G = GK) / 1 V (G = GV): out[i * G + g]
+    auto sb_quad = [&](int par, auto SIDE_, int tb, auto &out) __attribute__((always_inline)) {
+        constexpr int side = decltype(SIDE_)::value;
+        constexpr int G = side == 0 ? GK : GV, PAD = side == 0 ? SB_PAD_K : SB_PAD_V;
         const int first = 16 * G * jj;  // the lane group's first word among the tile's 64 G
-        const u4 *p = reinterpret_cast<const u4 *>(&sbuf[wave][par][side][first + SB_PAD * (first >> 6) + 4 * G * tb]);
+        const u4 *p = reinterpret_cast<const u4 *>(&sbuf[wave][par][side][first + PAD * (first >> 6) + 4 * G * tb]);
 #pragma unroll
         for (int e = 0; e < G; ++e) {
             const u4 w = p[e];
@@ -233,7 +237,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
 #pragma unroll
         for (int tb = 0; tb < 4; ++tb)
 #pragma unroll
-            for (int g = 0; g < G; ++g) {
+            for (int g = 0; g < GK; ++g) {
                 const gptr p = kp + (size_t)(4 * tb) * st.k_row + g * (GS * BITS / 8);
                 if constexpr (KWL == 1) {
                     t.k[tb][g][0] = ld_global<uint32_t>(p);
@@ -252,7 +256,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         // 16 tokens x G pairs of 4 bytes: contiguous rows of G * 4 bytes
         if constexpr (!SB_LDS) {
 #pragma unroll
-            for (int e = 0; e < 16 * G / 4; ++e) {
+            for (int e = 0; e < 16 * GK / 4; ++e) {
                 const u4 w = ld_global<u4>(ksp, e);
                 (&t.ksb[0][0])[4 * e] = w.x; (&t.ksb[0][0])[4 * e + 1] = w.y;
                 (&t.ksb[0][0])[4 * e + 2] = w.z; (&t.ksb[0][0])[4 * e + 3] = w.w;
@@ -282,7 +286,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         }
         if constexpr (!SB_LDS) {
 #pragma unroll
-            for (int e = 0; e < 16 * G / 4; ++e) {
+            for (int e = 0; e < 16 * GV / 4; ++e) {
                 const u4 w = ld_global<u4>(vsp, e);
                 (&t.vsb[0][0])[4 * e] = w.x; (&t.vsb[0][0])[4 * e + 1] = w.y;
                 (&t.vsb[0][0])[4 * e + 2] = w.z; (&t.vsb[0][0])[4 * e + 3] = w.w;
@@ -297,21 +301,21 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     };
 
     // ---- query operands (B of S^T) and the group sums of each query row ------------------------
-    Op8 qb[G][SPG];
-    float qsum[G];
+    Op8 qb[GK][SPG];
+    float qsum[GK];
     auto load_queries = [&]() __attribute__((always_inline)) {
         // rows past R read row 0 (in bounds) and are zeroed: no branch around the loads, which
         // are one 16-byte piece per contraction step
         const int rep = row_ok ? row_rep : 0, lq = row_ok ? row_l : 0;
-        const uint16_t *qrow = reinterpret_cast<const uint16_t *>(a.q) + ((size_t)(b * a.Hq + hk * r + rep) * a.L + lq) * D;
-        u4 raw[G][SPG];
+        const uint16_t *qrow = reinterpret_cast<const uint16_t *>(a.q) + ((size_t)(b * a.Hq + hk * r + rep) * a.L + lq) * DK;
+        u4 raw[GK][SPG];
 #pragma unroll
-        for (int g = 0; g < G; ++g)
+        for (int g = 0; g < GK; ++g)
 #pragma unroll
             for (int h = 0; h < SPG; ++h)
                 raw[g][h] = *reinterpret_cast<const u4 *>(qrow + GS * g + (GS / 4) * jj + 8 * h);
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
+        for (int g = 0; g < GK; ++g) {
             float part = 0.f;
 #pragma unroll
             for (int h = 0; h < SPG; ++h) {
@@ -338,23 +342,23 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     // (float16 caches, 4-bit codes: the probabilities that meet high nibbles are formed already divided by 16
     // and summed apart -- `l_hi`, `bacc_hi` -- so that no multiply brings them down; they rejoin at the end)
     constexpr bool SPLIT_HI = DT == 0 && BITS == 4;
-    float m_run = -INFINITY, l_part = 0.f, bacc[G], l_hi = 0.f, bacc_hi[G];
+    float m_run = -INFINITY, l_part = 0.f, bacc[GV], l_hi = 0.f, bacc_hi[GV];
     f4 oacc[NDB];
 #pragma unroll
-    for (int g = 0; g < G; ++g) bacc[g] = bacc_hi[g] = 0.f;
+    for (int g = 0; g < GV; ++g) bacc[g] = bacc_hi[g] = 0.f;
 #pragma unroll
     for (int db = 0; db < NDB; ++db) oacc[db] = f4{0.f, 0.f, 0.f, 0.f};
     const float fill = finfo_min_dt(DT);
 
-    Op8 pb[G][2];  // probabilities of the tile in flight: per group (pre-scaled by V's scale), step u
+    Op8 pb[GV][2];  // probabilities of the tile in flight: per group (pre-scaled by V's scale), step u
 
     auto compute_qk_softmax = [&](const Tile &t, int par) __attribute__((always_inline)) {
         // ---- S^T blocks --------------------------------------------------------------------
-        f4 sacc[4][G];
+        f4 sacc[4][GK];
 #pragma unroll
         for (int tb = 0; tb < 4; ++tb)
 #pragma unroll
-            for (int g = 0; g < G; ++g) {
+            for (int g = 0; g < GK; ++g) {
                 sacc[tb][g] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int h = 0; h < SPG; ++h) {
@@ -369,8 +373,8 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         XT x[16];
 #pragma unroll
         for (int tb = 0; tb < 4; ++tb) {
-            uint32_t kq[4 * G];
-            if constexpr (SB_LDS) sb_quad(par, 0, tb, kq);
+            uint32_t kq[4 * GK];
+            if constexpr (SB_LDS) sb_quad(par, std::integral_constant<int, 0>{}, tb, kq);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int tl = 4 * tb + i;
@@ -378,8 +382,8 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 // taken out of the sum over the groups (one multiply-add instead of one multiply per group)
                 float sc_ = 0.f, sb_ = 0.f;
 #pragma unroll
-                for (int g = 0; g < G; ++g) {
-                    const uint32_t raw = SB_LDS ? kq[i * G + g] : t.ksb[SB_LDS ? 0 : tl][g];
+                for (int g = 0; g < GK; ++g) {
+                    const uint32_t raw = SB_LDS ? kq[i * GK + g] : t.ksb[SB_LDS ? 0 : tl][g];
                     sc_ = __builtin_fmaf(sb_scale<DT>(raw), sacc[tb][g][i], sc_);
                     sb_ = __builtin_fmaf(sb_bias<DT>(raw), qsum[g], sb_);
                 }
@@ -446,7 +450,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             l_part *= alpha;
             l_hi *= alpha;
 #pragma unroll
-            for (int g = 0; g < G; ++g) {
+            for (int g = 0; g < GV; ++g) {
                 bacc[g] *= alpha;
                 bacc_hi[g] *= alpha;
             }
@@ -457,11 +461,11 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         }
         const float mu = (m_run == -INFINITY) ? 0.f : m_run;
         const float nmu = -mu * LOG2E;  // (float16: |mu| <= 65504, the product is finite)
-        float pv[G][16];
+        float pv[GV][16];
 #pragma unroll
         for (int tb = 0; tb < 4; ++tb) {
-            uint32_t vq[4 * G];
-            if constexpr (SB_LDS) sb_quad(par, 1, tb, vq);
+            uint32_t vq[4 * GV];
+            if constexpr (SB_LDS) sb_quad(par, std::integral_constant<int, 1>{}, tb, vq);
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int tl = 4 * tb + i;
@@ -480,8 +484,8 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
                 if (SPLIT_HI && hi) l_hi += p;
                 else l_part += p;
 #pragma unroll
-                for (int g = 0; g < G; ++g) {
-                    const uint32_t raw = SB_LDS ? vq[i * G + g] : t.vsb[SB_LDS ? 0 : tl][g];
+                for (int g = 0; g < GV; ++g) {
+                    const uint32_t raw = SB_LDS ? vq[i * GV + g] : t.vsb[SB_LDS ? 0 : tl][g];
                     if (SPLIT_HI && hi) bacc_hi[g] = __builtin_fmaf(p, sb_bias<DT>(raw), bacc_hi[g]);
                     else bacc[g] = __builtin_fmaf(p, sb_bias<DT>(raw), bacc[g]);
                     // (float16: written as a multiply-add so that the widening of the scale folds into it)
@@ -491,7 +495,7 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             }
         }
 #pragma unroll
-        for (int g = 0; g < G; ++g)
+        for (int g = 0; g < GV; ++g)
 #pragma unroll
             for (int u = 0; u < 2; ++u)
                 pb[g][u].v = u4{pack_h2(pv[g][8 * u], pv[g][8 * u + 1]), pack_h2(pv[g][8 * u + 2], pv[g][8 * u + 3]),
@@ -533,19 +537,19 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         }
     } else {
 #pragma unroll
-        for (int g = 0; g < G; ++g) qsum[g] = 0.f;
+        for (int g = 0; g < GK; ++g) qsum[g] = 0.f;
     }
 
     // ---- wavefront partial -> LDS: lane (n, jj) holds out^T[d = 16 db + 4 jj + i][row n] ---------
     if constexpr (SPLIT_HI) {
         l_part = __builtin_fmaf(l_hi, 16.f, l_part);
 #pragma unroll
-        for (int g = 0; g < G; ++g) bacc[g] = __builtin_fmaf(bacc_hi[g], 16.f, bacc[g]);
+        for (int g = 0; g < GV; ++g) bacc[g] = __builtin_fmaf(bacc_hi[g], 16.f, bacc[g]);
     }
     l_part += __shfl_xor(l_part, 16);
     l_part += __shfl_xor(l_part, 32);
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
+    for (int g = 0; g < GV; ++g) {
         bacc[g] += __shfl_xor(bacc[g], 16);
         bacc[g] += __shfl_xor(bacc[g], 32);
     }
@@ -557,8 +561,8 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
             cbuf[wave][n][16 * db + 4 * jj + i] = oacc[db][i] * TWO24 + bacc[g];
     }
     if (jj == 0) {
-        cbuf[wave][n][D] = m_run;
-        cbuf[wave][n][D + 1] = l_part;
+        cbuf[wave][n][DV] = m_run;
+        cbuf[wave][n][DV + 1] = l_part;
     }
     __syncthreads();
     // ---- merge the 4 wavefronts; a single span writes the output rows, several leave partials ---
@@ -568,32 +572,32 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
         const int i = threadIdx.x / WAVES, w = threadIdx.x - i * WAVES;
         float mx = -INFINITY;
 #pragma unroll
-        for (int w2 = 0; w2 < WAVES; ++w2) mx = fmaxf(mx, cbuf[w2][i][D]);
-        const float mw = cbuf[w][i][D];
+        for (int w2 = 0; w2 < WAVES; ++w2) mx = fmaxf(mx, cbuf[w2][i][DV]);
+        const float mw = cbuf[w][i][DV];
         wrow[w][i] = (mw == -INFINITY) ? 0.f : fast_exp2((mw - mx) * LOG2E);
         if (w == 0) mrow[i] = mx;
     }
     __syncthreads();
     if (nsplit == 1) {
-        for (int idx = threadIdx.x; idx < R * D; idx += WAVES * 64) {
-            const int i = idx / D, c = idx - i * D;
+        for (int idx = threadIdx.x; idx < R * DV; idx += WAVES * 64) {
+            const int i = idx / DV, c = idx - i * DV;
             float v = 0.f, l = 0.f;
 #pragma unroll
             for (int w = 0; w < WAVES; ++w) {
                 const float wgt = wrow[w][i];
                 v += wgt * cbuf[w][i][c];
-                l += wgt * cbuf[w][i][D + 1];
+                l += wgt * cbuf[w][i][DV + 1];
             }
             const int rep = i / a.L, lq = i - rep * a.L;
-            Elem<DT>::store(a.out, ((size_t)(b * a.Hq + hk * r + rep) * a.L + lq) * D + c, l > 0.f ? v / l : 0.f);
+            Elem<DT>::store(a.out, ((size_t)(b * a.Hq + hk * r + rep) * a.L + lq) * DV + c, l > 0.f ? v / l : 0.f);
         }
         return;
     }
-    float *part = a.workspace + part_slot * RR * (D + 2);
-    for (int idx = threadIdx.x; idx < RR * (D + 2); idx += WAVES * 64) {
-        const int i = idx / (D + 2), c = idx - i * (D + 2);
+    float *part = a.workspace + part_slot * RR * (DV + 2);
+    for (int idx = threadIdx.x; idx < RR * (DV + 2); idx += WAVES * 64) {
+        const int i = idx / (DV + 2), c = idx - i * (DV + 2);
         float v;
-        if (c == D) {
+        if (c == DV) {
             v = mrow[i];
         } else {
             v = 0.f;
@@ -612,27 +616,29 @@ hipError_t launch_attend_decode16(const AttendArgs &a, int tiles_total, int tile
     const Store &st = a.st;
     dim3 grid(nsplit, st.BH), block(WAVES * 64);
     const int mm = a.mask.mode == KVHIP_MASK_NONE ? 0 : (a.mask.mode == KVHIP_MASK_ARRAY ? 2 : 1);
-#define D16_M(BITS, D, GS, DT)                                                                                  \
+#define D16_M(BITS, DK, DV, GS, DT)                                                                             \
     do {                                                                                                        \
-        if (mm == 0) hipLaunchKernelGGL((decode16_kernel<BITS, D, GS, DT, 0>), grid, block, 0, s, a, tiles_total, tiles_per_wg, nsplit); \
-        else if (mm == 1) hipLaunchKernelGGL((decode16_kernel<BITS, D, GS, DT, 1>), grid, block, 0, s, a, tiles_total, tiles_per_wg, nsplit); \
-        else hipLaunchKernelGGL((decode16_kernel<BITS, D, GS, DT, 2>), grid, block, 0, s, a, tiles_total, tiles_per_wg, nsplit); \
+        if (mm == 0) hipLaunchKernelGGL((decode16_kernel<BITS, DK, DV, GS, DT, 0>), grid, block, 0, s, a, tiles_total, tiles_per_wg, nsplit); \
+        else if (mm == 1) hipLaunchKernelGGL((decode16_kernel<BITS, DK, DV, GS, DT, 1>), grid, block, 0, s, a, tiles_total, tiles_per_wg, nsplit); \
+        else hipLaunchKernelGGL((decode16_kernel<BITS, DK, DV, GS, DT, 2>), grid, block, 0, s, a, tiles_total, tiles_per_wg, nsplit); \
     } while (0)
-#define D16_DT(BITS, D, GS)                             \
-    do {                                                \
-        if (st.dtype == KVHIP_F16) D16_M(BITS, D, GS, 0); \
-        else D16_M(BITS, D, GS, 1);                     \
+#define D16_DT(BITS, DK, DV, GS)                             \
+    do {                                                     \
+        if (st.dtype == KVHIP_F16) D16_M(BITS, DK, DV, GS, 0); \
+        else D16_M(BITS, DK, DV, GS, 1);                     \
     } while (0)
 #define D16_Q(BITS)                                     \
     do {                                                \
-        if (st.Dk == 64 && st.gs == 32) D16_DT(BITS, 64, 32);        \
-        else if (st.Dk == 64) D16_DT(BITS, 64, 64);                  \
-        else if (st.Dk == 96) D16_DT(BITS, 96, 32);                  \
-        else if (st.Dk == 256 && st.gs == 64) D16_DT(BITS, 256, 64); \
-        else if (st.Dk == 256) D16_DT(BITS, 256, 128);               \
-        else if (st.gs == 32) D16_DT(BITS, 128, 32);                 \
-        else if (st.gs == 64) D16_DT(BITS, 128, 64);                 \
-        else D16_DT(BITS, 128, 128);                                 \
+        if (st.Dk == 64 && st.gs == 32) D16_DT(BITS, 64, 64, 32);         \
+        else if (st.Dk == 64) D16_DT(BITS, 64, 64, 64);                   \
+        else if (st.Dk == 96) D16_DT(BITS, 96, 96, 32);                   \
+        else if (st.Dk == 192 && st.gs == 32) D16_DT(BITS, 192, 128, 32); \
+        else if (st.Dk == 192) D16_DT(BITS, 192, 128, 64);                \
+        else if (st.Dk == 256 && st.gs == 64) D16_DT(BITS, 256, 256, 64); \
+        else if (st.Dk == 256) D16_DT(BITS, 256, 256, 128);               \
+        else if (st.gs == 32) D16_DT(BITS, 128, 128, 32);                 \
+        else if (st.gs == 64) D16_DT(BITS, 128, 128, 64);                 \
+        else D16_DT(BITS, 128, 128, 128);                                 \
     } while (0)
     // (head size 96 only divides by group size 32; D = 256 keeps 66 KB of partials in LDS -- one workgroup per
     // CU at group size 64, whose instances also need more than 256 registers)

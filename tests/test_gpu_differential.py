@@ -156,8 +156,9 @@ def test_quantized_shapes_against_generic(seed):
 
 @pytest.mark.parametrize("seed", range(48))
 def test_keys_of_192_values_of_128_against_generic(seed):
-    """Keys of 192 with values of 128 (multi-head latent attention) in all three cache kinds, every row
-    count on the prefill tiles: the tuned result against the generic kernel's."""
+    """Keys of 192 with values of 128 (multi-head latent attention) in all three cache kinds, on the prefill tiles
+    (quantized caches: up to 16 query rows per kv head on the 16-row decode kernel): the tuned result against the
+    generic kernel's."""
     rng = np.random.default_rng(5000 + seed)
     kind = ["simple", "rotating", "quantized"][seed % 3]
     dtype = [torch.float16, torch.bfloat16][(seed // 3) % 2]
@@ -215,7 +216,8 @@ def test_keys_of_192_values_of_128_against_generic(seed):
         chosen = lib.kvhip_last_attend_kernel()
     finally:
         lib.kvhip_set_kernel_policy(0)
-    assert chosen == 3 and out.shape == (B, Hkv * r, Lq, Dv)
+    # (up to 16 query rows per kv head of a quantized cache: the 16-row decode kernel)
+    assert chosen == (1 if kind == "quantized" and r * Lq <= 16 else 3) and out.shape == (B, Hkv * r, Lq, Dv)
     assert np.isfinite(ref).all() and np.isfinite(out).all()
     d = np.abs(out.astype(np.float64) - ref.astype(np.float64))
     ulp = float(np.abs(ref).max()) * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10)
