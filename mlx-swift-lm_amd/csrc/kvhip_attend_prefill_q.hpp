@@ -445,12 +445,23 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
     };
 
     // ---- S^T = K . Q^T operands: K slot (chunk 4 s + jj, position 16 mt + n) ------------------------
+    // (chunk cc = 4 s + jj is rotated by TOK16 (cc / CPU) positions; CPU divides 4, so that is a per-lane part,
+    // TOK16 (jj / CPU), plus a constant of the step.  The eight addresses of an iteration are then three
+    // instructions each from two lane constants.  The 256-row shape, which has no registers to keep eight
+    // addresses in -- held across the loop they were spilled to scratch memory and reloaded in front of every
+    // operand read, on the path to the matrix-core instruction that waits for it -- forms them anew every time.)
+    static_assert(4 % CPU == 0, "a contraction step's four chunks are whole units");
+    const int k_pos0 = n + TOK16 * (jj / CPU);        // position of this lane's row before the step's rotation
+    const int k_byte0 = jj * (BN * 16);               // byte offset of chunk jj
     auto read_k = [&](int par, int s, Op8 (&ka)[2]) __attribute__((always_inline)) {
-        const int cc = 4 * s + jj;
-        const int rot = TOK16 * (cc / CPU);
+        int pos0 = k_pos0;
+        if constexpr (NW == 8 && QT == 2) asm volatile("" : "+v"(pos0));  // (not hoisted out of the loop)
+        const char *base = reinterpret_cast<const char *>(Ks(par)) + k_byte0 + s * (4 * BN * 16);
 #pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-            ka[mt].v = *reinterpret_cast<const u4 *>(&Ks(par)[(cc * BN + ((16 * mt + n + rot) & (BN - 1))) * 8]);
+        for (int mt = 0; mt < 2; ++mt) {
+            const int pos = (pos0 + 16 * mt + TOK16 * (4 / CPU) * s) & (BN - 1);
+            ka[mt].v = *reinterpret_cast<const u4 *>(base + pos * 16);
+        }
     };
 
     // ---- mask of the tile at slot0 whose raw scores are in `sc` ------------------------------------
