@@ -118,6 +118,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
     constexpr bool GEN = BITS != 4 && BITS != 8;
     static_assert((DK == DV && (DK == 64 || DK == 96 || DK == 128 || DK == 256)) || (DK == 192 && DV == 128), "head sizes");
     constexpr int BM = 16 * QT * NW;
+    constexpr bool TIGHT = (NW == 8 && QT == 2) || DK >= 256;  // the shapes that have no registers to spare
     constexpr int S = DK / 32;    // contraction steps over the keys' head dim
     constexpr int NDT = DV / 16;  // 16-row tiles of out^T
     constexpr int KSZ = BN * DK, VSZ = BN * DV;  // 16-bit elements of a tile's K and of its V
@@ -305,7 +306,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
     }
     const bool tab_thread = tid < (BN / 2) * G;  // (G = 3 at head size 96: a division, once)
     const int tab_tp = tid / G, tab_g = tid - tab_tp * G;
-    const uint32_t tab_goff0 = (uint32_t)(2 * tab_tp * G + tab_g) * 4u, tab_goff1 = tab_goff0 + 4u * (uint32_t)G;
+    const uint32_t tab_goff0 = (uint32_t)(2 * tab_tp * G + tab_g) * 4u;  // (the pair's second token: one row of G words further)
     auto unit_is_v = [&](int e) __attribute__((always_inline)) -> bool { return tid + NT * e >= UK && tid + NT * e < UK + UV; };
     auto load_unit = [&](uint32_t (&dst)[UWD], gptr p) __attribute__((always_inline)) {
         if constexpr (GEN) {  // 4-byte aligned: words one by one
@@ -333,13 +334,19 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
 #pragma unroll
             for (int e = 0; e < NU; ++e)
                 if (unit_is_k(e)) {
-                    load_unit(codes[e], kb + (size_t)(tid + NT * e) * UB);  // the tile's K rows are one contiguous block
-                    ksb[e] = ld_global<uint32_t>(sbb + u_goff[e]);
+                    // (TIGHT: the 32-bit lane offsets are handed over as they are -- held across the loop the compiler
+                    // keeps each as a zero-extended 64-bit pair, twice the registers, and spills them)
+                    uint32_t ko = (uint32_t)((tid + NT * e) * UB), go = u_goff[e];
+                    if constexpr (TIGHT) asm volatile("" : "+v"(ko), "+v"(go));
+                    load_unit(codes[e], kb + ko);  // the tile's K rows are one contiguous block
+                    ksb[e] = ld_global<uint32_t>(sbb + go);
                 }
             if (tab_thread) {  // thread (token pair, group): the two tokens' (scale, bias) words
                 gptr vsbb = as_global(pe.vsb + cell_vsb + (size_t)in_page * st.vsb_row);
-                vsb_raw[0] = ld_global<uint32_t>(vsbb + tab_goff0);
-                vsb_raw[1] = ld_global<uint32_t>(vsbb + tab_goff1);
+                uint32_t t0 = tab_goff0;
+                if constexpr (TIGHT) asm volatile("" : "+v"(t0));
+                vsb_raw[0] = ld_global<uint32_t>(vsbb + t0);
+                vsb_raw[1] = ld_global<uint32_t>(vsbb + t0 + 4u * (uint32_t)G);
             }
         }
         if (do_v) {
@@ -349,7 +356,11 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
                                 ((slot0 & 32) ? BN * BITS / 8 : 0));
 #pragma unroll
             for (int e = 0; e < NU; ++e)
-                if (unit_is_v(e)) load_unit(codes[e], vb + u_goff[e]);
+                if (unit_is_v(e)) {
+                    uint32_t go = u_goff[e];
+                    if constexpr (TIGHT) asm volatile("" : "+v"(go));
+                    load_unit(codes[e], vb + go);
+                }
         }
     };
     // the table of the V rows' (scale, bias) pairs of the tile whose entry `request` fetched
@@ -455,7 +466,7 @@ prefill_q_kernel(AttendArgs a, int nsplit) {
     const int k_byte0 = jj * (BN * 16);               // byte offset of chunk jj
     auto read_k = [&](int par, int s, Op8 (&ka)[2]) __attribute__((always_inline)) {
         int pos0 = k_pos0;
-        if constexpr (NW == 8 && QT == 2) asm volatile("" : "+v"(pos0));  // (not hoisted out of the loop)
+        if constexpr (TIGHT) asm volatile("" : "+v"(pos0));  // (not hoisted out of the loop)
         const char *base = reinterpret_cast<const char *>(Ks(par)) + k_byte0 + s * (4 * BN * 16);
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt) {
