@@ -1145,6 +1145,13 @@ struct Plan {
     int tiles_total, tiles_per_wg, nsplit, rg, nw;
 };
 
+// Quantized shapes that run on the 16-row kernel at every row count: head size 96 (a row and a half of the 4-row
+// kernel's 64-column halves), keys of 192 with values of 128, and 2-, 3-, 5- and 6-bit codes (bit streams, which
+// the 4-row kernel's whole-word operands do not read).
+static bool only_decode16(const Store &s) {
+    return s.bits != 0 && (s.Dk == 96 || s.Dk == 192 || (s.bits != 4 && s.bits != 8));
+}
+
 Plan plan_for(const AttendArgs &a) {
     Plan p;
     p.tiles_total = (a.slots + TILE - 1) / TILE;
@@ -1185,7 +1192,7 @@ Plan plan_for(const AttendArgs &a) {
         // KVHIP_RAGGED_SPANS forces the number of spans per batch row (timing builds only: measure_knob)
         static const int forced_spans = measure_knob("KVHIP_RAGGED_SPANS", 0);
         if (forced_spans > 0) p.nsplit = std::min(forced_spans, 512);
-    } else if (a.st.bits != 0 && p.nsplit >= 2 && want <= 4 && p.rg == 1 && a.st.Dk != 96 && a.st.Dk != 192 && a.mask.mode != KVHIP_MASK_ARRAY &&
+    } else if (a.st.bits != 0 && p.nsplit >= 2 && want <= 4 && p.rg == 1 && !only_decode16(a.st) && a.mask.mode != KVHIP_MASK_ARRAY &&
                forced_tiles <= 0) {
         // 128 pairs or more: workgroups of 8 wavefronts, one per CU -- the same wavefronts per CU
         // with half the spans.  With 256 pairs a workgroup takes its pair's whole sequence: the
@@ -1201,7 +1208,7 @@ Plan plan_for(const AttendArgs &a) {
     }
     // a caller with a fixed amount of scratch: fewer, longer spans until the partials fit (one span has none)
     if (a.workspace_cap) {
-        const size_t per_span = (size_t)BH * (a.st.bits != 0 && (p.rg >= 2 || a.st.Dk == 96 || a.st.Dk == 192) ? 16 : 4 * p.rg) *
+        const size_t per_span = (size_t)BH * (a.st.bits != 0 && (p.rg >= 2 || only_decode16(a.st)) ? 16 : 4 * p.rg) *
                                 (a.st.Dv + 2) * sizeof(float);
         while (p.nsplit > 1 && per_span * p.nsplit > a.workspace_cap) {
             if (p.tiles_per_wg > 0) {
@@ -1306,7 +1313,7 @@ bool attend_decode_supported(const AttendArgs &a) {
     // 164 us; B8 D 256 8 rows about 105 us against 133 us)
     if (s.bits == 0) return (s.Dk == 64 || s.Dk == 128 || s.Dk == 256) && R <= (s.Dk == 256 ? 4 : 8);
     if (a.runs.n != 1 || a.runs.row0[0] != 0 || a.runs.phys0[0] != 0) return false;
-    if (s.bits != 4 && s.bits != 8) return false;
+    if (s.bits != 4 && s.bits != 8) return decode16_stream_shape(s);  // every row count on the 16-row kernel
     if (s.Dk == 64) return s.gs == 32 || s.gs == 64;
     if (s.Dk == 96) return s.gs == 32;  // every row count on the 16-row kernel
     if (mla) return s.gs == 32 || s.gs == 64;  // likewise
@@ -1321,17 +1328,16 @@ bool attend_decode_fuses_append(const AttendArgs &a) {
     static const bool off = measure_knob("KVHIP_NO_FUSED_APPEND", 0) != 0;  // (timing builds only)
     if (off) return false;
     if (a.st.bits == 0) return true;  // the full-precision decode kernel, any of its row counts
-    return (a.Hq / a.Hkv) * a.L <= 4 && a.st.Dk != 96 && a.st.Dk != 192;
+    return (a.Hq / a.Hkv) * a.L <= 4 && !only_decode16(a.st);
 }
 
 // 5..16 rows per kv head of a quantized cache go to the 16x16x32 kernel
 // (kvhip_attend_decode16.hip), which always carries 16 rows: measured faster than the 4-row
 // broadcast contraction from 8 rows up (B16, 8 kv heads, 8192 tokens: 37 us against 43 us at
 // 8 rows, 36 us against 87 us at 16).
-// Head size 96 (a row and a half of the 4-row kernel's 64-column halves) and keys of 192 with values of 128 take it
-// for every row count.
+// The shapes of only_decode16() take it for every row count.
 static bool use_decode16(const AttendArgs &a, const Plan &p) {
-    return a.st.bits != 0 && (p.rg >= 2 || a.st.Dk == 96 || a.st.Dk == 192);
+    return a.st.bits != 0 && (p.rg >= 2 || only_decode16(a.st));
 }
 
 size_t attend_decode_workspace(const AttendArgs &a) {

@@ -220,4 +220,36 @@ __device__ __forceinline__ void quantize_row_wave_from(LOAD load, int D, int gs,
     }
 }
 
+typedef uint32_t kv_u4 __attribute__((ext_vector_type(4)));
+// code j of a unit whose words hold a little-endian bit stream (j and BITS constant once unrolled)
+template <int BITS, int N> __device__ __forceinline__ uint32_t stream_code_at(const uint32_t (&w)[N], int j) {
+    const int bit = j * BITS, wi = bit >> 5, sh = bit & 31;
+    uint32_t v = w[wi] >> sh;
+    if (sh + BITS > 32) v |= w[wi + 1 < N ? wi + 1 : wi] << ((32 - sh) & 31);
+    return v & ((1u << BITS) - 1u);
+}
+// codes 8 c .. 8 c + 7 of such a unit as four float16 pairs with `mag` OR-ed over them: 0x64006400 (in a vector
+// register) gives (1024 + code, 1024 + code), 0 leaves the codes as the subnormals code * 2^-24.  A pair of adjacent codes is cut out as one field of 2 BITS bits; for 2, 3 and 5 bits the field
+// times (1 + 2^(16 - BITS)) has the first code at bit 0 and the second at bit 16 (what else the product holds lies
+// between them and cannot carry into bit 16: the low part stays below 2^16), so one 24-bit multiply and one
+// mask-and-OR finish the pair.  Six-bit codes would carry (63 + 63 * 64 + 63 * 1024 > 2^16) and are placed one by one.
+template <int BITS, int N> __device__ __forceinline__ kv_u4 stream_chunk(const uint32_t (&w)[N], int c, uint32_t mag) {
+    kv_u4 o;
+    constexpr uint32_t M1 = (1u << BITS) - 1u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if constexpr (BITS == 6) {
+            o[i] = stream_code_at<BITS, N>(w, 8 * c + 2 * i) | (stream_code_at<BITS, N>(w, 8 * c + 2 * i + 1) << 16) | mag;
+        } else {
+            const int bit = (8 * c + 2 * i) * BITS, wi = bit >> 5, sh = bit & 31;
+            uint32_t x = w[wi] >> sh;
+            if (sh + 2 * BITS > 32) x = __builtin_amdgcn_alignbit(w[wi + 1 < N ? wi + 1 : wi], w[wi], sh);
+            x &= (1u << (2 * BITS)) - 1u;
+            const uint32_t y = __umul24(x, 1u + (1u << (16 - BITS)));
+            o[i] = (y & (M1 | (M1 << 16))) | mag;
+        }
+    }
+    return o;
+}
+
 }  // namespace kvhip

@@ -311,6 +311,10 @@ size_t attend_prefill_workspace(const AttendArgs &a);
 hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s);
 hipError_t launch_attend_prefill(const AttendArgs &a, hipStream_t s);
 hipError_t launch_attend_decode16(const AttendArgs &a, int tiles_total, int tiles_per_wg, int nsplit, hipStream_t s);
+// (2- / 3-bit and 5- / 6-bit instances of the same kernel, and the shapes they are built for)
+hipError_t launch_attend_decode16_low(const AttendArgs &a, int tiles_total, int tiles_per_wg, int nsplit, hipStream_t s);
+hipError_t launch_attend_decode16_high(const AttendArgs &a, int tiles_total, int tiles_per_wg, int nsplit, hipStream_t s);
+bool decode16_stream_shape(const Store &s);
 hipError_t launch_attend_prefill_fp(const AttendArgs &a, int nsplit, bool wide, hipStream_t s);
 // The pipelined tile for quantized caches (head sizes 64 / 128 / 256, slots in presented order).
 bool attend_prefill_q_supported(const AttendArgs &a);

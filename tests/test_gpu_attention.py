@@ -394,7 +394,7 @@ def test_cfg5_ragged_speculative_rollback_reduced(policy):
             assert np.array_equal(np32(a), b)
 
 
-@pytest.mark.parametrize("kind,Lq", [("q4", 1), ("q4", 4), ("q8", 2), ("fp16", 1), ("bf16", 2)])
+@pytest.mark.parametrize("kind,Lq", [("q4", 1), ("q4", 4), ("q8", 2), ("fp16", 1), ("bf16", 2), ("q3", 1), ("q5", 4), ("q2", 2), ("q6", 1)])
 def test_ragged_batch_spans(policy, kind, Lq):
     """Per-batch lengths and left padding far apart (1 .. 3000 rows visible): the decode kernels
     divide each row's own visible range over the spans; every row must come out as under the
@@ -444,7 +444,9 @@ def test_ragged_batch_spans(policy, kind, Lq):
             first = False
         else:
             out = c.attend(qd, scale, mask)
-            if kind[0] == "q":
+            if kind[0] == "q" and int(kind[1]) in (3, 5, 6):  # (the C oracle unpacks whole-word code widths only)
+                ref = O.quantized_sdpa(q, *o.get_quantized_state(), scale, O.Mask("array", m), 64, int(kind[1]), name)
+            elif kind[0] == "q":
                 ref = CO.qsdpa(q, *o.get_quantized_state(), scale, m, 64, int(kind[1]), name)
             else:
                 ref = CO.sdpa(q, o.keys[:, :, :T], o.values[:, :, :T], scale, m, name)
@@ -516,14 +518,19 @@ def test_single_token_steps_write_their_row_inside_the_decode_kernel(dtype, bits
         assert cache.trim(trim) == ocache.trim(trim)
 
 
+def stream_decode_shape(D, gs):
+    """Head and group sizes the 16-row decode kernel has 2- / 3- / 5- / 6-bit instances for."""
+    return (D == 64 and gs in (32, 64)) or D == 128 or (D == 256 and gs == 64)
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("bits,D,gs", [(2, 128, 64), (3, 128, 64), (5, 128, 32), (6, 128, 64), (3, 64, 32), (6, 64, 64), (2, 256, 64),
                                         (5, 256, 128), (3, 256, 32), (3, 96, 32), (6, 96, 32), (2, 96, 32), (5, 96, 32)])
 def test_other_code_widths_on_the_pipelined_tile(dtype, bits, D, gs):
-    """2-, 3-, 5- and 6-bit codes (KVCacheConfiguration.swift:124 lists them beside 4 and 8) have no decode kernel of
-    their own: at head sizes 64 / 96 / 128 / 256 every row count runs on the pipelined prefill tile, which cuts the codes out
-    of the rows' bit streams.  Prompt chunks, single-token steps and a multi-token step against the oracle; codes and
-    pairs bit for bit."""
+    """2-, 3-, 5- and 6-bit codes (KVCacheConfiguration.swift:124 lists them beside 4 and 8): prompt chunks run on the
+    pipelined prefill tile, which cuts the codes out of the rows' bit streams; up to 16 query rows per kv head run on
+    the 16-row decode kernel where it has an instance for the shape (`stream_decode_shape`), on the tile otherwise.
+    Prompt chunks, single-token steps and a multi-token step against the oracle; codes and pairs bit for bit."""
     rng = np.random.default_rng(100 * bits + D + gs)
     name = NAME[dtype]
     B, Hkv, r = 2, 2, 4
@@ -536,7 +543,7 @@ def test_other_code_widths_on_the_pipelined_tile(dtype, bits, D, gs):
         q, qd = randn(rng, (B, Hkv * r, Lq, D), dtype)
         mask, om = (kvhip.MaskMode.causal(), O.Mask.CAUSAL) if mode == "causal" else (kvhip.MaskMode.none(), O.Mask.NONE)
         out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
-        assert lib.kvhip_last_attend_kernel() == 3
+        assert lib.kvhip_last_attend_kernel() == (1 if r * Lq <= 16 and stream_decode_shape(D, gs) else 3)
         ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
         check(out, ref, f"L={Lq}", lambda: exact_attention(q, *presented_f64(o), scale, om))
     # a boolean array mask and a window evaluated from indices
@@ -548,5 +555,66 @@ def test_other_code_widths_on_the_pipelined_tile(dtype, bits, D, gs):
     check(c.attend(qd, scale, kvhip.MaskMode.from_array(torch.from_numpy(m).cuda())), ref, "bool array", exact)
     check(c.attend(qd, scale, kvhip.MaskMode.window_mask(T - 40, 33)), ref, "window", exact)
     assert lib.kvhip_last_attend_kernel() == 3
+    for i, (a, b) in enumerate(zip(c.state, o.get_state())):
+        assert np.array_equal(np32(a), b) if i % 3 == 0 else bits_equal(a, b, dtype), i
+
+
+STREAM_DECODE_CASES = [(torch.float16, b, 128, g) for b in (2, 3, 5, 6) for g in (32, 64, 128)] + [
+    (torch.bfloat16, 3, 128, 64), (torch.bfloat16, 6, 128, 32), (torch.bfloat16, 2, 128, 128), (torch.bfloat16, 5, 128, 64),
+    (torch.float16, 3, 64, 32), (torch.bfloat16, 5, 64, 32), (torch.float16, 2, 64, 64), (torch.bfloat16, 6, 64, 64),
+    (torch.float16, 2, 256, 64), (torch.bfloat16, 3, 256, 64), (torch.float16, 5, 256, 64), (torch.float16, 6, 256, 64)]
+
+
+@pytest.mark.parametrize("dtype,bits,D,gs", STREAM_DECODE_CASES)
+def test_other_code_widths_on_the_16_row_decode_kernel(dtype, bits, D, gs):
+    """Decode steps of 2-, 3-, 5- and 6-bit caches: a lane of the 16-row kernel cuts its segment of every group out
+    of the row's bit stream (every segment width and alignment the head and group sizes give is a case here).  A
+    cache long enough for several spans and the merge launch; 1, 3, 8, 13 and 16 query rows per kv head; no mask,
+    causal, boolean and additive arrays, per-batch lengths and left padding -- against the oracle, and the kernel
+    family asserted."""
+    rng = np.random.default_rng(1000 * bits + D + gs)
+    name = NAME[dtype]
+    B, Hkv = 3, 2
+    scale = D ** -0.5
+    lib = kvhip.load()
+    c, o = kvhip.QuantizedKVCache(gs, bits), O.QuantizedKVCache(gs, bits, name)
+    T0 = 2900 + bits
+    k, kd = randn(rng, (B, Hkv, T0, D), dtype)
+    v, vd = randn(rng, (B, Hkv, T0, D), dtype)
+    c.update_quantized(kd, vd, fetch=False)
+    o.update_quantized(k, v)
+    for r, Lq, mode in [(4, 1, "none"), (1, 1, "none"), (1, 3, "causal"), (4, 4, "causal"), (8, 1, "none"), (13, 1, "none"),
+                        (2, 4, "bool"), (4, 2, "additive"), (4, 3, "lengths"), (2, 8, "left_pad"), (1, 16, "causal")]:
+        k, kd = randn(rng, (B, Hkv, Lq, D), dtype)
+        v, vd = randn(rng, (B, Hkv, Lq, D), dtype)
+        q, qd = randn(rng, (B, Hkv * r, Lq, D), dtype)
+        T = c.offset + Lq
+        j = np.arange(T)[None, None, None, :]
+        causal = np.broadcast_to(O.create_causal_mask(Lq, T - Lq)[None, None], (B, 1, Lq, T))
+        if mode == "none":
+            mask, om = kvhip.MaskMode.none(), O.Mask.NONE
+        elif mode == "causal":
+            mask, om = kvhip.MaskMode.causal(), O.Mask.CAUSAL
+        elif mode == "bool":
+            m = causal & (rng.random((B, 1, Lq, T)) < 0.8)
+            m[..., 0] = True
+            mask, om = kvhip.MaskMode.from_array(torch.from_numpy(m).cuda()), O.Mask("array", m)
+        elif mode == "additive":
+            add = np.where(causal, rng.standard_normal((B, 1, Lq, T)) * 0.5, -30000.0).astype(np.float32)
+            add = O.round_to(add, name)
+            mask = kvhip.MaskMode.from_array(torch.from_numpy(add).to(dtype).cuda())
+            om = O.Mask("array", add)
+        elif mode == "lengths":
+            lengths = np.array([T, 70, 1500], np.int32)
+            m = causal & (j < lengths[:, None, None, None])
+            mask, om = kvhip.MaskMode.window_mask(T - Lq, 0, lengths=torch.from_numpy(lengths)), O.Mask("array", m)
+        else:
+            pad = np.array([0, T - Lq - 3, 1000], np.int32)
+            m = causal & (j >= pad[:, None, None, None])
+            mask, om = kvhip.MaskMode.window_mask(T - Lq, 0, left_pad=torch.from_numpy(pad)), O.Mask("array", m)
+        out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
+        assert lib.kvhip_last_attend_kernel() == 1 and tuple(out.shape) == (B, Hkv * r, Lq, D)
+        ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
+        check(out, ref, f"r={r} L={Lq} {mode}", lambda: exact_attention(q, *presented_f64(o), scale, om))
     for i, (a, b) in enumerate(zip(c.state, o.get_state())):
         assert np.array_equal(np32(a), b) if i % 3 == 0 else bits_equal(a, b, dtype), i

@@ -155,6 +155,67 @@ def test_quantized_shapes_against_generic(seed):
 
 
 @pytest.mark.parametrize("seed", range(48))
+def test_other_code_widths_against_generic(seed):
+    """2-, 3-, 5- and 6-bit caches, mostly at decode row counts: up to 16 query rows per kv head run on the 16-row
+    decode kernel where it has an instance for the head and group size, everything else on the prefill tile."""
+    rng = np.random.default_rng(7000 + seed)
+    bits = [2, 3, 5, 6][seed % 4]
+    D = [64, 128, 256][(seed // 4) % 3]
+    gs = [32, 64, 128][(seed // 12) % 3]
+    if gs > D:
+        gs = 32
+    dtype = [torch.float16, torch.bfloat16][(seed // 2) % 2]
+    B, Hkv, r = int(rng.integers(1, 4)), int(rng.choice([1, 2])), int(rng.choice([1, 3, 4, 8]))
+    Lq = int(rng.choice([1, 1, 1, 2, 4, 5, 40]))
+    T0 = int(rng.choice([1, 31, 64, 200, 257, 700, 1300, 3100]))
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+
+    def rand(*shape):
+        return torch.randn(*shape, generator=g, device="cuda").to(dtype)
+
+    c = kvhip.QuantizedKVCache(gs, bits)
+    c.update_quantized(rand(B, Hkv, T0, D), rand(B, Hkv, T0, D), fetch=False)
+    c.update_quantized(rand(B, Hkv, Lq, D), rand(B, Hkv, Lq, D), fetch=False)
+    assert c.group_size == gs
+    T = c.offset
+    q = rand(B, Hkv * r, Lq, D)
+    which = rng.choice(["none", "causal", "left_pad", "lengths", "bool"])
+    if which == "none":
+        mask = kvhip.MaskMode.none()
+    elif which == "causal":
+        mask = kvhip.MaskMode.causal()
+    elif which == "left_pad":
+        pad = torch.from_numpy(rng.integers(0, max(T - Lq, 1), size=B).astype(np.int32))
+        mask = kvhip.MaskMode.window_mask(T - Lq, 0, left_pad=pad)
+    elif which == "lengths":
+        lengths = torch.from_numpy(rng.integers(1, T + 1, size=B).astype(np.int32))
+        mask = kvhip.MaskMode.window_mask(T - Lq, 0, lengths=lengths)
+    else:
+        keep = rng.random((B, 1, Lq, T)) < 0.7
+        keep[..., int(rng.integers(T))] = True
+        mask = kvhip.MaskMode.from_array(torch.from_numpy(keep).cuda())
+    scale = D ** -0.5
+    print(f"seed {seed}: {dtype} D{D} g{gs} {bits}-bit B{B} Hkv{Hkv} r{r} L{Lq} T{T} mask {which}", flush=True)
+    lib = kvhip.load()
+    try:
+        lib.kvhip_set_kernel_policy(1)
+        ref = np32(c.attend(q, scale, mask))
+        lib.kvhip_set_kernel_policy(0)
+        out = np32(c.attend(q, scale, mask))
+        chosen = lib.kvhip_last_attend_kernel()
+    finally:
+        lib.kvhip_set_kernel_policy(0)
+    decode_shape = (D == 64 and gs in (32, 64)) or D == 128 or (D == 256 and gs == 64)
+    assert chosen == (1 if r * Lq <= 16 and decode_shape else 3), chosen
+    assert np.isfinite(ref).all() and np.isfinite(out).all(), f"kernel {chosen}"
+    d = np.abs(out.astype(np.float64) - ref.astype(np.float64))
+    ulp = float(np.abs(ref).max()) * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10)
+    assert d.max() <= max(MAX_ABS, 2 * ulp) and d.mean() <= max(MEAN_ABS, ulp / 4), \
+        f"kernel {chosen}: max-abs {d.max():.3e} mean-abs {d.mean():.3e}"
+
+
+@pytest.mark.parametrize("seed", range(48))
 def test_keys_of_192_values_of_128_against_generic(seed):
     """Keys of 192 with values of 128 (multi-head latent attention) in all three cache kinds, on the prefill tiles
     (quantized caches: up to 16 query rows per kv head on the 16-row decode kernel): the tuned result against the
