@@ -52,7 +52,7 @@ def main():
                     help="new tokens per step of the cfg3-shaped run (more than 1: a causal multi-token step, "
                          "as a speculative verify makes; needs --cpu-steps 0)")
     ap.add_argument("--group-size", type=int, default=64, help="quantization group size (32, 64, 128)")
-    ap.add_argument("--bits", type=int, default=4, help="code width (4, 8)")
+    ap.add_argument("--bits", type=int, default=4, help="code width (2, 3, 4, 5, 6, 8; the CPU baseline only takes 2, 4 and 8: pass --cpu-steps 0 otherwise)")
     ap.add_argument("--cpu-steps", type=int, default=5, help="decode steps timed on the CPU baseline after one warm-up (0 = skip)")
     ap.add_argument("--settle", type=int, default=256,
                     help="untimed launches of the attention kernel alone (no append, the cache is left as it is) in front "
@@ -94,6 +94,8 @@ def main():
     D, GS, BITS, NT = args.head_dim, args.group_size, args.bits, args.tokens
     if NT > 1 and args.cpu_steps > 0:
         sys.exit("bench.py: --tokens above 1 is timed on the GPU only; pass --cpu-steps 0")
+    if BITS in (3, 5, 6) and args.cpu_steps > 0:
+        sys.exit("bench.py: the C oracle of the CPU baseline unpacks whole-word code widths only; pass --cpu-steps 0")
     # per cached token and kv head: K and V codes + (scale, bias) pairs of 2 x 2 bytes per group
     ROW_BYTES = 2 * (D * BITS // 8 + (D // GS) * 4)
     headline = (nb, ctx, D, GS, BITS, NT) == (32, 32768, 128, 64, 4, 1)
@@ -180,7 +182,7 @@ def main():
         kernel_ms = kms.value / launches.value
         achieved = alg_bytes / (kernel_ms * 1e-3) / 1e9
         rows = (HQ // HKV) * NT
-        kname = "decode16_kernel" if (rows > 4 or D == 96) else "decode_kernel"
+        kname = "decode16_kernel" if (rows > 4 or D == 96 or BITS not in (4, 8)) else "decode_kernel"
         roofline = {"bound": "hbm", "kernel": f"{kname}<{BITS},{D},{GS},f16>", "achieved": round(achieved, 1),
                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                     "kernel_ms": round(kernel_ms, 5), "algorithmic_bytes": int(alg_bytes),

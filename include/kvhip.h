@@ -237,8 +237,7 @@ kvhip_status kvhip_cache_fetch(const kvhip_cache *cache, void *dst_keys, void *d
  * queries [B,Hq,L,Dk] and out [B,Hq,L,Dv] in the cache's dtype.
  * Every dtype, bit width, head size, group size and mask is accepted.  The tuned kernels take
  * float16 / bfloat16 caches with Dk == Dv in {64, 96, 128, 256}, keys of 192 with values of 128 (also
- * 80 when not quantized; quantized: every code width, group size 32, 64 or 128; 2-, 3-, 5- and
- * 6-bit codes have no decode kernel and run single-token steps on the prefill tile).  A 16-bit cache
+ * 80 when not quantized; quantized: every code width, group size 32, 64 or 128).  A 16-bit cache
  * of other head sizes up to 256 stores its rows zero-padded to the next of those sizes (112 as 128,
  * 160 as 256) and runs the same kernels; every array that crosses this interface keeps the caller's
  * head sizes.  float32 caches and head sizes above 256 run on a plain kernel that is 50-75 times

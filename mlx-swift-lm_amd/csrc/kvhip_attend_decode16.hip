@@ -4,11 +4,14 @@
 
 namespace kvhip {
 
-// 2-, 3-, 5- and 6-bit codes: equal head sizes of 64 (groups of 32 / 64), 128 (32 / 64 / 128) and 256 (64)
+// 2-, 3-, 5- and 6-bit codes: equal head sizes of 64 (groups of 32 / 64), 96 (32), 128 (32 / 64 / 128) and 256 (64),
+// keys of 192 with values of 128 (64)
 bool decode16_stream_shape(const Store &s) {
     if (s.bits != 2 && s.bits != 3 && s.bits != 5 && s.bits != 6) return false;
+    if (s.Dk == 192 && s.Dv == 128) return s.gs == 64;
     if (s.Dk != s.Dv) return false;
     if (s.Dk == 64) return s.gs == 32 || s.gs == 64;
+    if (s.Dk == 96) return s.gs == 32;
     if (s.Dk == 128) return s.gs == 32 || s.gs == 64 || s.gs == 128;
     if (s.Dk == 256) return s.gs == 64;
     return false;

@@ -715,6 +715,8 @@ hipError_t launch_decode16_bits(const AttendArgs &a, int tiles_total, int tiles_
         // the other code widths: the shapes decode16_stream_shape() lists
         if (st.Dk == 64 && st.gs == 32) D16_DT(64, 64, 32);
         else if (st.Dk == 64) D16_DT(64, 64, 64);
+        else if (st.Dk == 96) D16_DT(96, 96, 32);
+        else if (st.Dk == 192) D16_DT(192, 128, 64);
         else if (st.Dk == 256) D16_DT(256, 256, 64);
         else if (st.gs == 32) D16_DT(128, 128, 32);
         else if (st.gs == 64) D16_DT(128, 128, 64);

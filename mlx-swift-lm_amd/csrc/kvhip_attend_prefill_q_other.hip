@@ -1,5 +1,5 @@
-// The pipelined prefill tile for quantized caches (kvhip_attend_prefill_q.hpp): 2-, 3-, 5- and 6-bit codes, which
-// have no decode kernel of their own and take this tile at every row count.
+// The pipelined prefill tile for quantized caches (kvhip_attend_prefill_q.hpp): 2-, 3-, 5- and 6-bit codes (more than
+// 16 query rows per kv head, and every row count of the shapes the 16-row decode kernel has no instance for).
 #include "kvhip_attend_prefill_q.hpp"
 
 namespace kvhip {

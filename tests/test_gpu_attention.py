@@ -235,9 +235,9 @@ def test_keys_of_192_values_of_128_on_the_prefill_tile(dtype):
 @pytest.mark.parametrize("dtype,bits,gs", [(torch.float16, 4, 64), (torch.bfloat16, 8, 64), (torch.float16, 8, 32), (torch.bfloat16, 4, 32),
                                            (torch.float16, 3, 64), (torch.bfloat16, 5, 32), (torch.float16, 6, 32), (torch.bfloat16, 2, 64)])
 def test_quantized_keys_of_192_values_of_128_on_the_prefill_tile(dtype, bits, gs):
-    """The same head sizes in a QuantizedKVCache (group sizes 32 and 64 divide both): decode steps of 4- / 8-bit caches run
-    on the 16-row decode kernel, everything else on the quantized prefill tile; codes and pairs equal the oracle's,
-    outputs are the oracle's within the bound."""
+    """The same head sizes in a QuantizedKVCache (group sizes 32 and 64 divide both): decode steps run on the 16-row
+    decode kernel, everything else on the quantized prefill tile; codes and pairs equal the oracle's, outputs are the
+    oracle's within the bound."""
     rng = np.random.default_rng(bits + gs)
     name, Dk, Dv = NAME[dtype], 192, 128
     scale = Dk ** -0.5
@@ -250,8 +250,9 @@ def test_quantized_keys_of_192_values_of_128_on_the_prefill_tile(dtype, bits, gs
         q, qd = randn(rng, (B, H * r, Lq, Dk), dtype)
         mask, om = (kvhip.MaskMode.causal(), O.Mask.CAUSAL) if mode == "causal" else (kvhip.MaskMode.none(), O.Mask.NONE)
         out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
-        # up to 16 query rows per kv head of a 4- / 8-bit cache: the 16-row decode kernel; otherwise the prefill tile
-        want = 1 if (bits in (4, 8) and r * Lq <= 16) else 3
+        # up to 16 query rows per kv head: the 16-row decode kernel (other code widths than 4 / 8 bits: its instances
+        # are built for group size 64); otherwise the prefill tile
+        want = 1 if ((bits in (4, 8) or gs == 64) and r * Lq <= 16) else 3
         assert lib.kvhip_last_attend_kernel() == want and tuple(out.shape) == (B, H * r, Lq, Dv)
         ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
         check(out, ref, f"L={Lq}", lambda: exact_attention(q, *presented_f64(o), scale, om))
@@ -520,7 +521,7 @@ def test_single_token_steps_write_their_row_inside_the_decode_kernel(dtype, bits
 
 def stream_decode_shape(D, gs):
     """Head and group sizes the 16-row decode kernel has 2- / 3- / 5- / 6-bit instances for."""
-    return (D == 64 and gs in (32, 64)) or D == 128 or (D == 256 and gs == 64)
+    return (D == 64 and gs in (32, 64)) or (D == 96 and gs == 32) or D == 128 or (D == 256 and gs == 64)
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -562,7 +563,9 @@ def test_other_code_widths_on_the_pipelined_tile(dtype, bits, D, gs):
 STREAM_DECODE_CASES = [(torch.float16, b, 128, g) for b in (2, 3, 5, 6) for g in (32, 64, 128)] + [
     (torch.bfloat16, 3, 128, 64), (torch.bfloat16, 6, 128, 32), (torch.bfloat16, 2, 128, 128), (torch.bfloat16, 5, 128, 64),
     (torch.float16, 3, 64, 32), (torch.bfloat16, 5, 64, 32), (torch.float16, 2, 64, 64), (torch.bfloat16, 6, 64, 64),
-    (torch.float16, 2, 256, 64), (torch.bfloat16, 3, 256, 64), (torch.float16, 5, 256, 64), (torch.float16, 6, 256, 64)]
+    (torch.float16, 2, 256, 64), (torch.bfloat16, 3, 256, 64), (torch.float16, 5, 256, 64), (torch.float16, 6, 256, 64),
+    (torch.float16, 2, 96, 32), (torch.bfloat16, 3, 96, 32), (torch.float16, 5, 96, 32), (torch.bfloat16, 6, 96, 32),
+    (torch.float16, 2, (192, 128), 64), (torch.float16, 3, (192, 128), 64), (torch.bfloat16, 5, (192, 128), 64), (torch.float16, 6, (192, 128), 64)]
 
 
 @pytest.mark.parametrize("dtype,bits,D,gs", STREAM_DECODE_CASES)
@@ -572,6 +575,7 @@ def test_other_code_widths_on_the_16_row_decode_kernel(dtype, bits, D, gs):
     cache long enough for several spans and the merge launch; 1, 3, 8, 13 and 16 query rows per kv head; no mask,
     causal, boolean and additive arrays, per-batch lengths and left padding -- against the oracle, and the kernel
     family asserted."""
+    D, Dv = D if isinstance(D, tuple) else (D, D)  # (keys of 192 with values of 128)
     rng = np.random.default_rng(1000 * bits + D + gs)
     name = NAME[dtype]
     B, Hkv = 3, 2
@@ -580,13 +584,13 @@ def test_other_code_widths_on_the_16_row_decode_kernel(dtype, bits, D, gs):
     c, o = kvhip.QuantizedKVCache(gs, bits), O.QuantizedKVCache(gs, bits, name)
     T0 = 2900 + bits
     k, kd = randn(rng, (B, Hkv, T0, D), dtype)
-    v, vd = randn(rng, (B, Hkv, T0, D), dtype)
+    v, vd = randn(rng, (B, Hkv, T0, Dv), dtype)
     c.update_quantized(kd, vd, fetch=False)
     o.update_quantized(k, v)
     for r, Lq, mode in [(4, 1, "none"), (1, 1, "none"), (1, 3, "causal"), (4, 4, "causal"), (8, 1, "none"), (13, 1, "none"),
                         (2, 4, "bool"), (4, 2, "additive"), (4, 3, "lengths"), (2, 8, "left_pad"), (1, 16, "causal")]:
         k, kd = randn(rng, (B, Hkv, Lq, D), dtype)
-        v, vd = randn(rng, (B, Hkv, Lq, D), dtype)
+        v, vd = randn(rng, (B, Hkv, Lq, Dv), dtype)
         q, qd = randn(rng, (B, Hkv * r, Lq, D), dtype)
         T = c.offset + Lq
         j = np.arange(T)[None, None, None, :]
@@ -613,7 +617,7 @@ def test_other_code_widths_on_the_16_row_decode_kernel(dtype, bits, D, gs):
             m = causal & (j >= pad[:, None, None, None])
             mask, om = kvhip.MaskMode.window_mask(T - Lq, 0, left_pad=torch.from_numpy(pad)), O.Mask("array", m)
         out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
-        assert lib.kvhip_last_attend_kernel() == 1 and tuple(out.shape) == (B, Hkv * r, Lq, D)
+        assert lib.kvhip_last_attend_kernel() == 1 and tuple(out.shape) == (B, Hkv * r, Lq, Dv)
         ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
         check(out, ref, f"r={r} L={Lq} {mode}", lambda: exact_attention(q, *presented_f64(o), scale, om))
     for i, (a, b) in enumerate(zip(c.state, o.get_state())):
