@@ -1416,11 +1416,12 @@ hipError_t launch_attend_decode(const AttendArgs &a_in, hipStream_t s) {
         else if (ident) FP(D, DT, RG, 2, true);                   \
         else FP(D, DT, RG, 2, false);                             \
     } while (0)
-#define FP_RG(D, DT)                              \
-    do {                                          \
-        if (p.rg == 1) FP_MI(D, DT, 1);           \
-        else if (p.rg == 2) FP_MI(D, DT, 2);      \
-        else FP_MI(D, DT, 4);                     \
+    // (up to 8 query rows per kv head, 4 at D = 256: attend_decode_supported() sends more to the prefill tile)
+#define FP_RG(D, DT)                                           \
+    do {                                                       \
+        if (p.rg == 1) FP_MI(D, DT, 1);                        \
+        else if (p.rg == 2 && D < 256) FP_MI(D, DT, (D < 256 ? 2 : 1)); \
+        else return hipErrorInvalidValue;                      \
     } while (0)
 #define FP_DT(D)                                  \
     do {                                          \
