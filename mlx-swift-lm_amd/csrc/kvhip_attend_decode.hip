@@ -1322,13 +1322,12 @@ bool attend_decode_supported(const AttendArgs &a) {
     return false;
 }
 
-// The 4-row quantized kernel and the full-precision decode kernel, without a mask, write the step's new row themselves.
+// The decode kernels -- the 4-row and the 16-row quantized kernel and the full-precision one --, without a mask, write
+// a single-token step's new row themselves.
 bool attend_decode_fuses_append(const AttendArgs &a) {
     if (!attend_decode_supported(a) || a.L != 1 || a.mask.mode != KVHIP_MASK_NONE) return false;
     static const bool off = measure_knob("KVHIP_NO_FUSED_APPEND", 0) != 0;  // (timing builds only)
-    if (off) return false;
-    if (a.st.bits == 0) return true;  // the full-precision decode kernel, any of its row counts
-    return (a.Hq / a.Hkv) * a.L <= 4 && !only_decode16(a.st);
+    return !off;
 }
 
 // 5..16 rows per kv head of a quantized cache go to the 16x16x32 kernel

@@ -214,6 +214,38 @@ decode16_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     const int row_l = n % a.L, row_rep = n / a.L;  // this lane's query row n = (head rep, position l)
     const bool row_ok = n < R;
 
+    // ---- the step's new row, when it is still to be written (unmasked single-token step) --------
+    // Its slot lies in the last tile, which exactly one wavefront of one workgroup reads: that wavefront
+    // quantizes the row into the cache before it requests any tile, with the arithmetic of the append kernel,
+    // so its own later loads of the tile (and of the tile's scale / bias pairs) see it.  A lane owns the V
+    // columns it quantizes; their codes go into the columns' tile rows read-modify-write (a code of a bit
+    // stream may lie across two dwords).
+    if constexpr (MM == 0) {
+        if (a.new_k != nullptr) {  // wave-uniform
+            const int slot = a.new_slot, tl = slot >> 6;
+            if (tl >= tile_begin && tl < tile_end && ((tl - tile_begin) % WAVES) == wave) {
+                const char *krow = static_cast<const char *>(a.new_k) + (size_t)bh * DK * 2;
+                const char *vrow = static_cast<const char *>(a.new_v) + (size_t)bh * DV * 2;
+                quantize_row_wave_from<DT, BITS>([&](int d) { return Elem<DT>::load(krow, d); }, DK, GS, lane,
+                                                 reinterpret_cast<uint32_t *>(const_cast<char *>(k_row_ptr(st, bh, slot))),
+                                                 [](int, uint32_t) {}, const_cast<char *>(ksb_row_ptr(st, bh, slot)), nullptr, nullptr);
+                char *vcell = const_cast<char *>(v_cell_ptr(st, bh, slot));
+                const int bp = v_bitpos<BITS>(slot & (TILE - 1)), sh = bp & 31;
+                constexpr uint32_t M = (1u << BITS) - 1u;
+                quantize_row_wave_from<DT, BITS>(
+                    [&](int d) { return Elem<DT>::load(vrow, d); }, DV, GS, lane, nullptr,
+                    [&](int d, uint32_t code) {
+                        uint32_t *p = reinterpret_cast<uint32_t *>(vcell + v_row_off(st, slot, d)) + (bp >> 5);
+                        p[0] = (p[0] & ~(M << sh)) | (code << sh);
+                        if ((32 % BITS) != 0 && sh + BITS > 32) p[1] = (p[1] & ~(M >> (32 - sh))) | (code >> (32 - sh));
+                    },
+                    const_cast<char *>(vsb_row_ptr(st, bh, slot)), nullptr, nullptr);
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            }
+        }
+    }
+
     // ---- per-lane addresses inside a tile; tiles of one wavefront are a page apart -----------
     // K block tb, lane (n, jj): row of token tok(tb, n) = 16 (n / 4) + 4 tb + n % 4, segment jj
     // each page is found through the page table (a scalar load per plane pair); the offsets below are

@@ -486,12 +486,19 @@ def test_ring_in_temporal_order_with_lengths(policy):
     (torch.float16, 4, 64, 128, 3, 8, 2), (torch.bfloat16, 4, 64, 128, 2, 4, 4), (torch.float16, 8, 64, 64, 1, 16, 4),
     (torch.float16, 4, 32, 128, 2, 8, 2), (torch.float16, 8, 128, 256, 1, 4, 2), (torch.bfloat16, 8, 32, 64, 2, 6, 2),
     (torch.float16, 4, 64, 256, 2, 8, 4),
+    # the 16-row kernel: more than 4 query heads per kv head, head size 96, keys of 192 with values of 128, bit streams
+    (torch.float16, 4, 64, 128, 2, 16, 2), (torch.bfloat16, 8, 64, 64, 1, 16, 1), (torch.bfloat16, 8, 32, 96, 2, 4, 2),
+    (torch.float16, 4, 32, 96, 1, 8, 1), (torch.float16, 4, 64, (192, 128), 2, 4, 4), (torch.bfloat16, 8, 32, (192, 128), 1, 16, 2),
+    (torch.float16, 3, 64, 128, 2, 8, 2), (torch.bfloat16, 5, 32, 128, 1, 4, 4), (torch.float16, 6, 64, 64, 2, 4, 2),
+    (torch.float16, 2, 128, 128, 2, 16, 2), (torch.bfloat16, 3, 64, 256, 1, 4, 2), (torch.float16, 5, 32, 96, 2, 6, 2),
+    (torch.bfloat16, 6, 64, (192, 128), 1, 8, 2), (torch.float16, 3, 32, 64, 2, 2, 2),
 ])
 def test_single_token_steps_write_their_row_inside_the_decode_kernel(dtype, bits, gs, D, B, Hq, Hkv):
     """`attentionWithCacheUpdate` with one new token and no mask on a quantized cache is one launch: the decode
     kernel quantizes the new row into the cache itself.  Codes, scale / bias pairs and offsets must be the
     append kernel's (the oracle's) bit for bit after every step -- across octets, 64-token tiles, pages and
     trims -- and the outputs the oracle's within the bound."""
+    D, Dv = D if isinstance(D, tuple) else (D, D)
     rng = np.random.default_rng(bits * 7 + D + gs)
     cache = kvhip.QuantizedKVCache(gs, bits)
     ocache = O.QuantizedKVCache(gs, bits, NAME[dtype])
@@ -501,13 +508,13 @@ def test_single_token_steps_write_their_row_inside_the_decode_kernel(dtype, bits
         n = start - ocache.offset
         if n > 0:
             k, kd = randn(rng, (B, Hkv, n, D), dtype, 1.5)
-            v, vd = randn(rng, (B, Hkv, n, D), dtype, 0.7)
+            v, vd = randn(rng, (B, Hkv, n, Dv), dtype, 0.7)
             cache.update_quantized(kd, vd, fetch=False)
             ocache.update_quantized(k, v)
         for _ in range(steps):
             q, qd = randn(rng, (B, Hq, 1, D), dtype)
             k, kd = randn(rng, (B, Hkv, 1, D), dtype, 1.5)
-            v, vd = randn(rng, (B, Hkv, 1, D), dtype, 0.7)
+            v, vd = randn(rng, (B, Hkv, 1, Dv), dtype, 0.7)
             got = np32(cache.update_attend(qd, kd, vd, scale))
             assert kvhip.load().kvhip_last_attend_kernel() == 1
             ref = O.attention_with_cache_update(q, k, v, ocache, scale, O.Mask.NONE, NAME[dtype])
