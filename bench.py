@@ -65,6 +65,9 @@ def main():
                          "remaining BASELINE.json configs (reported as one JSON object each)")
     ap.add_argument("--prefill-shape", default=None,
                     help="with --workload prefill: one shape B,Hq,Hkv,D,L,T,dtype (dtype f16, bf16, or q2 / q3 / q4 / q5 / q6 / q8; D may be 192/128) instead of the table")
+    ap.add_argument("--policy", type=int, default=0, choices=[0, 2, 3],
+                    help="kvhip_set_kernel_policy for the run: 0 the library's choice, 2 quantized prompt chunks always on "
+                         "the quantized tile, 3 dequantize-first whenever the shape allows")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy 4 times (reference point for rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings)")
@@ -87,6 +90,7 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
     dev = torch.device("cuda:0")
+    kvhip.load().kvhip_set_kernel_policy(args.policy)
     if args.workload != "cfg3":
         print(json.dumps(other_workload(args, torch, kvhip, L, dev)))
         return
@@ -331,18 +335,30 @@ def other_workload(args, torch, kvhip, L, dev):
                 cache.attend(q, Dk ** -0.5, mask)
             torch.cuda.synchronize()
             lib.kvhip_profile_enable(1)
-            for _ in range(args.steps if args.steps != 256 else 20):
+            nrun = args.steps if args.steps != 256 else 20
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(nrun):
                 cache.attend(q, Dk ** -0.5, mask)
+            e1.record()
             torch.cuda.synchronize()
             lib.kvhip_profile_enable(0)
+            family = lib.kvhip_last_attend_kernel()
             ms, n = kernel_ms()
+            call_ms = e0.elapsed_time(e1) / nrun
             keys = sum(T - Lq + i + 1 for i in range(Lq))
             fl = 2.0 * Bn * Hq * keys * (Dk + Dv)
+            # kernel_ms: the tile kernel alone (the library's event bracket); call_ms: a whole call, the calls enqueued
+            # back to back -- for a quantized cache that runs dequantize-first (family 4) it holds the conversion pass
+            # in front of the tile, and the rate of the call is the one that counts
             rows.append({"shape": f"B{Bn} {Hq}q/{Hkv}kv D{D} {dn}, {Lq} new rows over {T} keys, causal", "launches": n,
-                         "kernel_ms": round(ms, 4), "TFLOPs": round(fl / ms / 1e9, 1),
-                         "frac_of_2.5PF": round(fl / ms / 1e9 / 2500.0, 4)})
+                         "family": family, "kernel_ms": round(ms, 4), "call_ms": round(call_ms, 4),
+                         "TFLOPs": round(fl / ms / 1e9, 1), "TFLOPs_call": round(fl / call_ms / 1e9, 1),
+                         "frac_of_2.5PF": round(fl / (call_ms if family == 4 else ms) / 1e9 / 2500.0, 4)})
             del cache, k, v, q
-        return {"workload": "chunked-prefill tiles (prefill_fp_kernel, prefill_q_kernel for quantized caches) on their own", "results": rows}
+        return {"workload": "chunked-prefill tiles on their own (prefill_fp_kernel; quantized caches: prefill_q_kernel, or "
+                            "dequantize-first + prefill_fp_kernel from 1024 query rows per kv head; --policy 2 keeps them on prefill_q_kernel)",
+                "results": rows}
 
     if args.workload == "cfg1":
         # the reference's own CPU-runnable case: B1, 16q/4kv, D64, fp16, 8-bit g64; prefill 512 under

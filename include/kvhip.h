@@ -120,7 +120,9 @@ kvhip_status kvhip_init(int32_t device);
 /* Blocks until all work enqueued on `stream` is done (tests; `eval(cache)` LLMModel.swift:56-58).
  * Also releases device memory of freed caches and replaced buffers whose last readers are done. */
 kvhip_status kvhip_sync(void *stream);
-/* 0 = choose the fastest kernel for the shape (default); 1 = always the generic kernel.
+/* 0 = choose the fastest kernel for the shape (default); 1 = always the generic kernel; 2 and 3 = as 0, but a
+ * prompt chunk over a quantized cache never (2) or whenever the shape allows (3) runs dequantize-first -- the
+ * cached rows converted once into scratch pages, then the full-precision tile -- instead of by row count.
  * The setting, kvhip_last_attend_kernel and the profile record below belong to the calling thread. */
 void kvhip_set_kernel_policy(int32_t policy);
 /*
@@ -134,7 +136,8 @@ void kvhip_set_kernel_policy(int32_t policy);
  */
 /* Which kernel family the last attention call on this thread's library state used:
  * 0 generic, 1 matrix-core decode (quantized), 2 matrix-core decode (full precision),
- * 3 matrix-core chunked-prefill tile; -1 before the first call.  For tests and reports. */
+ * 3 matrix-core chunked-prefill tile, 4 the same tile over scratch pages a quantized cache was dequantized into
+ * first; -1 before the first call.  For tests and reports. */
 int32_t kvhip_last_attend_kernel(void);
 void kvhip_profile_enable(int32_t every);
 kvhip_status kvhip_profile_read(int32_t *out_launches, double *out_total_ms);
@@ -270,8 +273,8 @@ kvhip_status kvhip_cache_attend_static(kvhip_cache *cache, const void *queries, 
                                        void *out, void *stream);
 
 /* `attentionWithCacheUpdate` (AttentionUtils.swift:37-95): update, then attend.  A single new token without a
- * mask is written by the decode kernel itself where one of them serves the call (quantized caches up to four
- * query rows per kv head, 16-bit full-precision caches): the step then has no launch for the append. */
+ * mask is written by the decode kernel itself where one of them serves the call (quantized caches up to sixteen
+ * query heads per kv head, 16-bit full-precision caches up to eight): the step then has no launch for the append. */
 kvhip_status kvhip_cache_update_attend(kvhip_cache *cache, const void *queries, const void *keys,
                                        const void *values, int32_t B, int32_t Hq, int32_t Hkv,
                                        int32_t L, int32_t Dk, int32_t Dv, int32_t dtype, float scale,

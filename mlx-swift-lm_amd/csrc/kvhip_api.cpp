@@ -151,6 +151,7 @@ struct Buf {
 };
 struct Retired {
     hipEvent_t done;
+    hipStream_t stream;  // where `done` was recorded: work enqueued there later runs after the buffers' last reader
     std::vector<Buf> bufs;
 };
 std::mutex g_retired_mu;
@@ -168,6 +169,7 @@ int current_device() {
 void retire(std::vector<std::pair<void *, size_t>> &&ptrs, hipStream_t stream) {
     if (ptrs.empty()) return;
     Retired r;
+    r.stream = stream;
     const int dev = current_device();
     for (auto &q : ptrs) r.bufs.push_back(Buf{q.first, q.second, dev});
     if (hipEventCreateWithFlags(&r.done, hipEventDisableTiming) != hipSuccess || hipEventRecord(r.done, stream) != hipSuccess) {
@@ -197,11 +199,35 @@ void harvest_locked() {
 
 // hipMalloc, or a finished buffer of at least `bytes` and at most 1.5 times that from the free list.
 // `got` receives the size of what was handed out.  Only enqueue-free work: usable on the hot path.
-hipError_t pool_alloc(void **out, size_t bytes, size_t *got) {
+// `same_stream`: the buffer will only be touched by work enqueued on that stream from now on, so a buffer retired
+// behind earlier work of the same stream may be handed out before that work has finished (stream order keeps the
+// new user behind the old reader): scratch that every call takes and gives back is then one buffer per stream
+// however far the host runs ahead.
+hipError_t pool_alloc(void **out, size_t bytes, size_t *got, const hipStream_t *same_stream = nullptr) {
     {
         std::lock_guard<std::mutex> lock(g_retired_mu);
         harvest_locked();
         const int dev = current_device();
+        if (same_stream) {
+            for (size_t i = 0; i < g_retired.size(); ++i) {
+                Retired &r = g_retired[i];
+                if (r.stream != *same_stream) continue;
+                for (size_t j = 0; j < r.bufs.size(); ++j) {
+                    const Buf &b = r.bufs[j];
+                    if (b.dev != dev || b.bytes < bytes || b.bytes > bytes + bytes / 2) continue;
+                    *out = b.p;
+                    *got = b.bytes;
+                    r.bufs[j] = r.bufs.back();
+                    r.bufs.pop_back();
+                    if (r.bufs.empty()) {
+                        (void)hipEventDestroy(r.done);
+                        g_retired[i] = std::move(g_retired.back());
+                        g_retired.pop_back();
+                    }
+                    return hipSuccess;
+                }
+            }
+        }
         int best = -1;
         for (size_t i = 0; i < g_free.size(); ++i) {
             const Buf &b = g_free[i];
@@ -1068,6 +1094,51 @@ kvhip_status bind_workspace(kvhip_cache *c, AttendArgs &a, size_t need, float *f
     return KVHIP_OK;
 }
 
+// A prompt chunk with many query rows per kv head over a quantized cache (attend_prefill_dequant_first): the cached
+// rows are dequantized once into scratch pages of the cache dtype -- `MLX.dequantized`'s values, scale * code + bias
+// in float32 rounded once -- and the chunk runs on the full-precision prefill tile, which needs no conversions in
+// its loop.  The scratch (a page table, K pages, V pages) comes from the pool and goes back to it behind the call:
+// calls on one stream share one buffer.  Returns KVHIP_ERR_HIP only for launch failures; when the scratch cannot be
+// had, `*done` stays false and the caller runs the quantized tile.
+kvhip_status attend_dequant_first(kvhip_cache *c, const AttendArgs &a, hipStream_t s, bool *done) {
+    *done = false;
+    Store t;
+    t.BH = a.st.BH;
+    t.Dk = a.st.Dk;
+    t.Dv = a.st.Dv;
+    t.dtype = a.st.dtype;
+    t.es = a.st.es;
+    t.k_row = (uint32_t)((t.Dk * t.es + 15) / 16 * 16);
+    t.k_cell = t.k_row * PAGE;
+    t.v_cell = (uint32_t)(t.Dv * t.es) * PAGE;
+    const int64_t pages = ((int64_t)a.slots + PAGE - 1) / PAGE;
+    const size_t BH = t.BH;
+    const size_t ptb = align256((size_t)pages * sizeof(PageEntry)), kb = align256(BH * t.k_cell * pages), vb = align256(BH * t.v_cell * pages);
+    void *base = nullptr;
+    size_t got = 0;
+    if (pool_alloc(&base, ptb + kb + vb, &got, &s) != hipSuccess) {
+        (void)hipGetLastError();
+        return KVHIP_OK;
+    }
+    std::vector<std::pair<void *, size_t>> give_back{{base, got}};
+    PageEntry first;
+    first.k = static_cast<char *>(base) + ptb;
+    first.v = static_cast<char *>(base) + ptb + kb;
+    const size_t stride[2] = {BH * t.k_cell, BH * t.v_cell};
+    t.pt = static_cast<PageEntry *>(base);
+    AttendArgs a2 = a;
+    a2.st = t;
+    kvhip_status st = KVHIP_OK;
+    hipError_t e = launch_dequant_scratch(a.st, t, a.T, (int)pages, first, stride[0], stride[1], s);
+    if (e == hipSuccess) st = bind_workspace(c, a2, attend_prefill_workspace(a2), nullptr, 0, s);
+    if (e == hipSuccess && st == KVHIP_OK) e = launch_attend_prefill(a2, s);
+    retire(std::move(give_back), s);
+    if (e != hipSuccess) return fail(KVHIP_ERR_HIP, std::string("dequantize-first prefill: ") + hipGetErrorString(e));
+    if (st != KVHIP_OK) return st;
+    *done = true;
+    return KVHIP_OK;
+}
+
 // new_k / new_v: the rows of a single-token step whose bookkeeping is done but whose write into physical
 // slot `new_slot` is still owed; the decode kernel takes them along when it can, else they are
 // appended by a launch of their own first.
@@ -1142,7 +1213,7 @@ kvhip_status attend_impl(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, i
     hipStream_t s = S(c, stream);
     a.workspace_cap = fixed ? fixed_bytes : 0;
     if (new_k) {
-        if (g_policy == 0 && attend_decode_fuses_append(a)) {
+        if (g_policy != 1 && attend_decode_fuses_append(a)) {
             a.new_k = new_k;
             a.new_v = new_v;
             a.new_slot = new_slot;
@@ -1152,14 +1223,18 @@ kvhip_status attend_impl(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, i
             KV_HIP(launch_append_fp(c->st, new_k, new_v, 1, 0, new_slot, 1, s, nullptr));
         }
     }
-    if (g_policy == 0 && attend_decode_supported(a)) {
+    if (g_policy != 1 && attend_decode_supported(a)) {
         KV_TRY(bind_workspace(c, a, attend_decode_workspace(a), fixed, fixed_bytes, s));
         KV_HIP(launch_attend_decode(a, s));
         g_last_kernel = a.st.bits ? 1 : 2;
-    } else if (g_policy == 0 && attend_prefill_supported(a)) {
-        KV_TRY(bind_workspace(c, a, attend_prefill_workspace(a), fixed, fixed_bytes, s));
-        KV_HIP(launch_attend_prefill(a, s));
-        g_last_kernel = 3;
+    } else if (g_policy != 1 && attend_prefill_supported(a)) {
+        bool done = false;
+        if (!fixed && g_policy != 2 && attend_prefill_dequant_first(a, g_policy == 3)) KV_TRY(attend_dequant_first(c, a, s, &done));
+        if (!done) {
+            KV_TRY(bind_workspace(c, a, attend_prefill_workspace(a), fixed, fixed_bytes, s));
+            KV_HIP(launch_attend_prefill(a, s));
+        }
+        g_last_kernel = done ? 4 : 3;
     } else {
         KV_TRY(bind_workspace(c, a, attend_generic_workspace(a), fixed, fixed_bytes, s));
         g_last_kernel = 0;

@@ -20,6 +20,28 @@ bool attend_prefill_supported(const AttendArgs &a) {
     return s.Dk == 64 || s.Dk == 80 || s.Dk == 96 || s.Dk == 128 || s.Dk == 256;
 }
 
+// A prompt chunk over a quantized cache converts every cached row once per workgroup that reads it.  With many query
+// rows per kv head it is cheaper to convert the rows once for all of them: the cache is dequantized into scratch
+// pages of its dtype and the full-precision tile, whose loop has no conversions, runs over those.  The scratch costs
+// 2 (Dk + Dv) bytes per cached row and kv head written and read again; the tile gains about a third of its time.
+bool attend_prefill_dequant_first(const AttendArgs &a, bool always) {
+    const Store &s = a.st;
+    if (s.bits == 0 || (s.dtype != KVHIP_F16 && s.dtype != KVHIP_BF16)) return false;
+    if (a.runs.n != 1 || a.runs.row0[0] != 0 || a.runs.phys0[0] != 0) return false;
+    if (s.Dk % 8 != 0 || s.Dv % 8 != 0) return false;
+    AttendArgs fp = a;
+    fp.st.bits = 0;
+    if (!attend_prefill_supported(fp)) return false;
+    if (always) return true;
+    // the conversion pass and its page table are two launches more: the chunk must be worth them
+    const int R = (a.Hq / a.Hkv) * a.L;
+    const double flops = 2.0 * s.BH * R * (double)a.T * (s.Dk + s.Dv);
+    static const int min_rows = measure_knob("KVHIP_DEQUANT_FIRST_ROWS", 1024);  // (timing builds only)
+    // (measured equal at 1024 rows per kv head and ahead beyond -- the more so for the shapes the quantized tile is
+    // slowest on; keys of 192 with values of 128 are ahead from 512 rows)
+    return R >= (s.Dk == 192 ? min_rows / 2 : min_rows) && flops >= 4e10;
+}
+
 // 128 query rows per workgroup reuse each staged tile twice as often as 64; 64 rows are
 // used when that would leave the grid too small to fill 256 CUs twice over.
 static bool prefill_wide(const AttendArgs &a) {

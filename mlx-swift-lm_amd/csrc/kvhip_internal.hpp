@@ -249,6 +249,8 @@ hipError_t launch_compact_fp(const Store &src, const Runs &runs, const Store &ds
 // from pages to pages, no dense copy in between.
 hipError_t launch_requant_pages(const Store &src, const Store &dst, int rows, hipStream_t s);
 hipError_t launch_dequant_pages(const Store &q, const Store &dst, int rows, hipStream_t s);
+hipError_t launch_dequant_scratch(const Store &q, const Store &dst, int rows, int pages, const PageEntry &page0, size_t sk, size_t sv,
+                                  hipStream_t s);
 // The whole-tile quantizer for 2-, 3-, 5- and 6-bit codes (kvhip_quant_tile_other.hip): `tiles` tiles of dense rows
 // from row a0 on into the slots from b0 on, and tiles [0, tiles) of a full-precision page store into the same slots.
 hipError_t launch_quant_tiles_other(const Store &st, const void *keys, const void *values, int L, int a0, int b0, int tiles,
@@ -306,6 +308,10 @@ hipError_t launch_attend_decode(const AttendArgs &a, hipStream_t s);
 // Matrix-core chunked-prefill tile (many query rows per kv head).
 bool attend_prefill_supported(const AttendArgs &a);
 size_t attend_prefill_workspace(const AttendArgs &a);
+// Whether a prompt chunk over a quantized cache is faster with the cache dequantized into scratch pages first and the
+// full-precision tile run over them (many query rows per kv head share the one conversion of every cached row).
+// (`always`: whenever the shape allows it, whatever the row count)
+bool attend_prefill_dequant_first(const AttendArgs &a, bool always);
 // Merge `nsplit` partials per query row, laid out [bh][split][rows][D+2] in a.workspace
 // (out[D] unnormalised, running max, running sum), and write the normalised rows to a.out.
 hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s);

@@ -199,6 +199,111 @@ __global__ void __launch_bounds__(256) dequant_pages_kernel(Store q, Store dst, 
     }
 }
 
+// The same for 16-bit dtypes and head sizes that are multiples of 8, in whole tiles and 16-byte pieces: a thread forms
+// eight adjacent elements of a K row, or one column's values for eight adjacent tokens, which is one 16-byte chunk of
+// the interleaved full-precision tile; consecutive threads write consecutive chunks.  grid (tiles, BH, 2): K and V of a
+// tile are separate workgroups; a thread requests the codes and (scale, bias) pairs of up to four chunks before it
+// converts the first.  Eight codes lie inside two adjacent dwords for every code width (a V tile row's octet of
+// tokens likewise, in the order v_bitpos gives).  Rows past the cache's length in the last tile come out as
+// whatever their slots hold (zeros, or rows trimmed earlier): finite values nobody presents.
+template <int DT> __device__ __forceinline__ void pair_of(uint32_t raw, float &sc, float &bi) {
+    if (DT == 0) {
+        sc = (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+        bi = (float)__builtin_bit_cast(_Float16, (uint16_t)(raw >> 16));
+    } else {
+        sc = __uint_as_float(raw << 16);
+        bi = __uint_as_float(raw & 0xffff0000u);
+    }
+}
+// `dst_pt` non-null: the destination is scratch whose page p lies at `page0` + p * (sk, sv) and whose page table
+// `dst_pt` is still unwritten -- the first workgroup writes its `pages` entries for the kernels that follow, and
+// nobody here reads them.
+template <int DT, int BITS>
+__global__ void __launch_bounds__(256) dequant_tiles16_kernel(Store q, Store dst, PageEntry *dst_pt, int pages, PageEntry page0, size_t sk, size_t sv) {
+    typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+    constexpr uint32_t M = (1u << BITS) - 1u;
+    constexpr int NB = 4;  // chunks in flight per thread
+    const int bh = blockIdx.y, lo = blockIdx.x * TILE;
+    auto pack = [](float a, float b) { return DT == 0 ? pk_h2(a, b) : pk_bf2(a, b); };
+    if (dst_pt != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0) {
+        for (int p = threadIdx.x; p < pages; p += 256) {
+            PageEntry e;
+            e.k = page0.k + (size_t)p * sk;
+            e.v = page0.v + (size_t)p * sv;
+            dst_pt[p] = e;
+        }
+    }
+    const PageEntry de = dst_pt != nullptr ? PageEntry{page0.k + (size_t)(lo >> PAGE_SHIFT) * sk, nullptr, page0.v + (size_t)(lo >> PAGE_SHIFT) * sv, nullptr}
+                                           : dst.pt[lo >> PAGE_SHIFT];
+    if (blockIdx.z == 0) {
+        char *kdst = de.k + (size_t)bh * dst.k_cell + kfp_off(dst, lo, 0);
+        const int items = (q.Dk / 8) * TILE, last = (int)q.k_row / 4 - 1;
+        for (int base = threadIdx.x; base < items; base += 256 * NB) {
+            uint32_t w0[NB], w1[NB], sb[NB];
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                const int item = base + 256 * u;
+                if (item < items) {
+                    const int c = item >> 6, slot = lo + (item & 63), wi = (8 * c * BITS) >> 5;
+                    const uint32_t *row = reinterpret_cast<const uint32_t *>(k_row_ptr(q, bh, slot));
+                    w0[u] = row[wi];
+                    w1[u] = row[min(wi + 1, last)];
+                    sb[u] = reinterpret_cast<const uint32_t *>(ksb_row_ptr(q, bh, slot))[(8 * c) / q.gs];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                const int item = base + 256 * u;
+                if (item < items) {
+                    const int off = ((item >> 6) * 8 * BITS) & 31;
+                    const uint64_t bits = (((uint64_t)w1[u] << 32) | w0[u]) >> off;
+                    float sc, bi, x[8];
+                    pair_of<DT>(sb[u], sc, bi);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) x[j] = __fadd_rn(__fmul_rn(sc, (float)((uint32_t)(bits >> (j * BITS)) & M)), bi);
+                    *reinterpret_cast<u4v *>(kdst + (size_t)item * 16) = u4v{pack(x[0], x[1]), pack(x[2], x[3]), pack(x[4], x[5]), pack(x[6], x[7])};
+                }
+            }
+        }
+        return;
+    }
+    const char *vcell = v_cell_ptr(q, bh, lo);
+    char *vdst = de.v + (size_t)bh * dst.v_cell + vfp_off(dst, lo, 0);
+    const int items = 8 * q.Dv, last = TILE * BITS / 32 - 1;
+    for (int base = threadIdx.x; base < items; base += 256 * NB) {
+        uint32_t w0[NB], w1[NB], sb[NB][8];
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int item = base + 256 * u;
+            if (item < items) {
+                const int tc = item / q.Dv, d = item - tc * q.Dv, wi = v_bitpos<BITS>(8 * tc) >> 5;
+                const uint32_t *row = reinterpret_cast<const uint32_t *>(vcell + v_row_off(q, lo, d));
+                w0[u] = row[wi];
+                w1[u] = row[min(wi + 1, last)];
+                const int g = d / q.gs;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) sb[u][j] = reinterpret_cast<const uint32_t *>(vsb_row_ptr(q, bh, lo + 8 * tc + j))[g];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int item = base + 256 * u;
+            if (item < items) {
+                const int tc = item / q.Dv, first = v_bitpos<BITS>(8 * tc) & ~31;
+                const uint64_t bits = ((uint64_t)w1[u] << 32) | w0[u];
+                float x[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    float sc, bi;
+                    pair_of<DT>(sb[u][j], sc, bi);
+                    x[j] = __fadd_rn(__fmul_rn(sc, (float)((uint32_t)(bits >> (v_bitpos<BITS>(8 * tc + j) - first)) & M)), bi);
+                }
+                *reinterpret_cast<u4v *>(vdst + (size_t)item * 16) = u4v{pack(x[0], x[1]), pack(x[2], x[3]), pack(x[4], x[5]), pack(x[6], x[7])};
+            }
+        }
+    }
+}
+
 // grid (whole tiles, BH), 256 threads; 16-bit dtypes, Dk == 32 NCK, Dv == 32 NCV
 template <int NCK, int NCV>
 __global__ void __launch_bounds__(256)
@@ -599,7 +704,30 @@ hipError_t launch_requant_pages(const Store &src, const Store &st, int rows, hip
 hipError_t launch_dequant_pages(const Store &q, const Store &dst, int rows, hipStream_t s) {
     if (rows <= 0) return hipSuccess;
     dim3 grid((rows + TILE - 1) / TILE, q.BH), block(256);
+    if (q.es == 2 && q.Dk % 8 == 0 && q.Dv % 8 == 0) {
+#define CALL(DT, BITS)                                                                                                  \
+    hipLaunchKernelGGL((dequant_tiles16_kernel<(DT == 2 ? 0 : DT), BITS>), dim3(grid.x, grid.y, 2), block, 0, s, q, dst, \
+                       (PageEntry *)nullptr, 0, PageEntry(), (size_t)0, (size_t)0)
+        KV_DISPATCH_DT_BITS(q.dtype, q.bits, CALL);
+#undef CALL
+        return hipGetLastError();
+    }
 #define CALL(DT, BITS) hipLaunchKernelGGL((dequant_pages_kernel<DT, BITS>), grid, block, 0, s, q, dst, rows)
+    KV_DISPATCH_DT_BITS(q.dtype, q.bits, CALL);
+#undef CALL
+    return hipGetLastError();
+}
+
+// The same into scratch pages whose table the launch writes itself (16-bit dtypes, head sizes that are multiples of 8):
+// page p of the scratch at `page0` + p * (sk, sv), `dst.pt` the table to fill, `dst` otherwise only geometry.
+hipError_t launch_dequant_scratch(const Store &q, const Store &dst, int rows, int pages, const PageEntry &page0, size_t sk, size_t sv,
+                                  hipStream_t s) {
+    if (rows <= 0) return hipSuccess;
+    if (q.es != 2 || q.Dk % 8 != 0 || q.Dv % 8 != 0) return hipErrorInvalidValue;
+    dim3 grid((rows + TILE - 1) / TILE, q.BH, 2), block(256);
+#define CALL(DT, BITS)                                                                                          \
+    hipLaunchKernelGGL((dequant_tiles16_kernel<(DT == 2 ? 0 : DT), BITS>), grid, block, 0, s, q, dst,              \
+                       const_cast<PageEntry *>(dst.pt), pages, page0, sk, sv)
     KV_DISPATCH_DT_BITS(q.dtype, q.bits, CALL);
 #undef CALL
     return hipGetLastError();

@@ -335,7 +335,8 @@ def test_cfg1_quantized_prefill_then_decode(policy):
     qk, qv = o.update_quantized(k, v)
     ref = CO.qsdpa(q, qk, qv, scale, "causal", 64, 8, "float16")
     check(out, ref, "prefill")
-    assert kvhip.load().kvhip_last_attend_kernel() == (3 if policy == 0 else 0)  # MFMA prefill tile
+    # (the quantized MFMA prefill tile: a chunk this small is not worth a conversion pass of its own)
+    assert kvhip.load().kvhip_last_attend_kernel() == (3 if policy == 0 else 0)
     # the same causal mask handed over as a boolean array
     tri = torch.ones(512, 512, dtype=torch.bool, device="cuda").tril()
     out = c.attend(qd, scale, kvhip.MaskMode.from_array(tri))
@@ -629,3 +630,86 @@ def test_other_code_widths_on_the_16_row_decode_kernel(dtype, bits, D, gs):
         check(out, ref, f"r={r} L={Lq} {mode}", lambda: exact_attention(q, *presented_f64(o), scale, om))
     for i, (a, b) in enumerate(zip(c.state, o.get_state())):
         assert np.array_equal(np32(a), b) if i % 3 == 0 else bits_equal(a, b, dtype), i
+
+
+@pytest.mark.parametrize("dtype,bits,gs,D", [
+    (torch.float16, 4, 64, 128), (torch.bfloat16, 4, 64, 128), (torch.float16, 8, 32, 64), (torch.bfloat16, 8, 64, 256),
+    (torch.float16, 4, 32, 96), (torch.float16, 4, 64, (192, 128)), (torch.bfloat16, 8, 32, (192, 128)),
+    (torch.float16, 2, 64, 128), (torch.bfloat16, 3, 32, 96), (torch.float16, 5, 128, 256), (torch.bfloat16, 6, 64, 64),
+])
+def test_quantized_prompt_chunks_dequantize_first(dtype, bits, gs, D):
+    """A prompt chunk with many query rows per kv head over a quantized cache is not converted tile by tile: the
+    cached rows are dequantized once into scratch pages (`MLX.dequantized`'s values) and the full-precision tile runs
+    over them (kernel family 4).  Forced here on small chunks (policy 3) under every mask kind; against the oracle,
+    and the cache's state untouched."""
+    D, Dv = D if isinstance(D, tuple) else (D, D)
+    rng = np.random.default_rng(31 * bits + D + gs)
+    name = NAME[dtype]
+    B, Hkv, r = 2, 2, 4
+    scale = D ** -0.5
+    lib = kvhip.load()
+    c, o = kvhip.QuantizedKVCache(gs, bits), O.QuantizedKVCache(gs, bits, name)
+    try:
+        for Lq, mode, policy in [(150, "causal", 3), (70, "bool", 3), (40, "additive", 3), (33, "window", 3), (64, "lengths", 3),
+                                 (300, "causal", 3), (20, "causal", 3)]:
+            lib.kvhip_set_kernel_policy(policy)
+            k, kd = randn(rng, (B, Hkv, Lq, D), dtype)
+            v, vd = randn(rng, (B, Hkv, Lq, Dv), dtype)
+            q, qd = randn(rng, (B, Hkv * r, Lq, D), dtype)
+            T = c.offset + Lq
+            j = np.arange(T)[None, None, None, :]
+            causal = np.broadcast_to(O.create_causal_mask(Lq, T - Lq)[None, None], (B, 1, Lq, T))
+            if mode == "causal":
+                mask, om = kvhip.MaskMode.causal(), O.Mask.CAUSAL
+            elif mode == "bool":
+                m = causal & (rng.random((B, 1, Lq, T)) < 0.8)
+                m[..., 0] = True
+                mask, om = kvhip.MaskMode.from_array(torch.from_numpy(m).cuda()), O.Mask("array", m)
+            elif mode == "additive":
+                add = O.round_to(np.where(causal, rng.standard_normal((B, 1, Lq, T)) * 0.5, -30000.0).astype(np.float32), name)
+                mask, om = kvhip.MaskMode.from_array(dev(add, dtype)), O.Mask("array", add)
+            elif mode == "window":
+                m = np.broadcast_to(O.create_causal_mask(Lq, T - Lq, 48)[None, None], (B, 1, Lq, T))
+                mask, om = kvhip.MaskMode.window_mask(T - Lq, 48), O.Mask("array", m)
+            else:
+                lengths = np.array([T, T - 90], np.int32)
+                m = causal & (j < lengths[:, None, None, None])
+                mask, om = kvhip.MaskMode.window_mask(T - Lq, 0, lengths=torch.from_numpy(lengths)), O.Mask("array", m)
+            out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
+            assert lib.kvhip_last_attend_kernel() == 4 and tuple(out.shape) == (B, Hkv * r, Lq, Dv), (Lq, mode)
+            ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
+            check(out, ref, f"L={Lq} {mode}", lambda: exact_attention(q, *presented_f64(o), scale, om))
+    finally:
+        lib.kvhip_set_kernel_policy(0)
+    for i, (a, b) in enumerate(zip(c.state, o.get_state())):
+        assert np.array_equal(np32(a), b) if i % 3 == 0 else bits_equal(a, b, dtype), i
+
+
+@pytest.mark.parametrize("dtype,bits,D", [(torch.float16, 4, 128), (torch.bfloat16, 8, 128), (torch.float16, 3, 96), (torch.bfloat16, 4, (192, 128))])
+def test_large_quantized_chunks_run_dequantize_first_by_the_librarys_choice(dtype, bits, D):
+    """From 1024 query rows per kv head (512 with keys of 192 and values of 128) and 4e10 floating-point operations a
+    chunk over a quantized cache runs dequantize-first without being told to; a chunk below either bound stays on the
+    quantized tile.  The two paths agree to within the rounding of their intermediates (both are checked against the
+    oracle at sizes it covers)."""
+    D, Dv = D if isinstance(D, tuple) else (D, D)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(bits + D)
+    B, Hkv, r, L, T = 1, 8, 4, 1024, 4096
+    c = kvhip.QuantizedKVCache(32 if D == 96 else 64, bits)
+    c.update_quantized(torch.randn(B, Hkv, T, D, generator=g, device="cuda").to(dtype), torch.randn(B, Hkv, T, Dv, generator=g, device="cuda").to(dtype), fetch=False)
+    lib = kvhip.load()
+    scale = D ** -0.5
+    try:
+        for Lq, want in ((L, 4), (128, 3)):
+            q = torch.randn(B, Hkv * r, Lq, D, generator=g, device="cuda").to(dtype)
+            for mask in (kvhip.MaskMode.causal(), kvhip.MaskMode.window_mask(T - Lq, 1000)):
+                lib.kvhip_set_kernel_policy(0)
+                out = np32(c.attend(q, scale, mask))
+                assert lib.kvhip_last_attend_kernel() == want
+                lib.kvhip_set_kernel_policy(2)
+                tile = np32(c.attend(q, scale, mask))
+                assert lib.kvhip_last_attend_kernel() == 3
+                d = np.abs(out.astype(np.float64) - tile.astype(np.float64))
+                assert np.isfinite(out).all() and d.max() <= (4e-3 if dtype == torch.float16 else 2e-2) and d.mean() <= 2e-4, (Lq, d.max(), d.mean())
+    finally:
+        lib.kvhip_set_kernel_policy(0)
