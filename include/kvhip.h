@@ -259,7 +259,9 @@ kvhip_status kvhip_cache_attend(kvhip_cache *cache, const void *queries, int32_t
  * process ends, and the call makes no hipMalloc / hipFree.  The tuned kernels plan for that
  * amount: they divide the sequence over fewer spans or key-range parts until the partials fit
  * (a single span or part needs none), so they take every shape; where that gives another number of
- * parts than kvhip_cache_attend would use, the float32 sums are formed in another order.  Only the
+ * parts than kvhip_cache_attend would use, the float32 sums are formed in another order; and a large
+ * prompt chunk over a quantized cache, which kvhip_cache_attend runs over a dequantized copy in pooled
+ * scratch pages, runs on the quantized tile here (the same result within the rounding of intermediates).  Only the
  * plain kernel, which keeps one float per (query row, key), can need more than the array holds: such
  * a call returns KVHIP_ERR_UNSUPPORTED and enqueues nothing.  Nothing in the array has to start from zero:
  * each span writes its partial before the merge reads it.  All calls on one device share the
