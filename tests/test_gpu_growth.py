@@ -192,3 +192,36 @@ def test_created_grown_and_freed_caches_reuse_their_memory_without_a_blocking_ca
     assert all(torch.isfinite(o).all() for o in outs)
     # and the answers do not depend on whose memory a cache got
     assert all(torch.equal(outs[0], o) for o in outs[1:])
+
+
+def test_dequantize_first_scratch_is_one_buffer_per_stream():
+    """A large prompt chunk over a quantized cache runs over scratch pages the cache is dequantized into.  The scratch
+    is taken from the pool at the call and retired behind it, and a call may take a buffer retired on its own stream
+    without waiting for it: twelve layers' calls enqueued back to back, three rounds of them with no wait in between,
+    hold one scratch buffer, not thirty-six -- and every layer's result is what it is when computed alone."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(3)
+    B, Hkv, r, D, T, Lq = 1, 8, 4, 128, 4096, 1024
+    lib = kvhip.load()
+    caches = []
+    for _ in range(12):
+        c = kvhip.QuantizedKVCache(64, 4)
+        c.update_quantized(torch.randn(B, Hkv, T, D, generator=g, device="cuda").half(), torch.randn(B, Hkv, T, D, generator=g, device="cuda").half(), fetch=False)
+        caches.append(c)
+    q = torch.randn(B, Hkv * r, Lq, D, generator=g, device="cuda").half()
+    outs = [torch.empty_like(q) for _ in caches]
+    scratch = B * Hkv * T * 2 * D * 2
+    causal = kvhip.MaskMode.causal()
+    alone = []
+    for c in caches:                       # each layer alone (this also brings the pool to its working size)
+        alone.append(c.attend(q, D ** -0.5, causal))
+        assert lib.kvhip_last_attend_kernel() == 4
+        torch.cuda.current_stream().synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        for c, o in zip(caches, outs):
+            c.attend(q, D ** -0.5, causal, out=o)
+    torch.cuda.current_stream().synchronize()
+    free_after = torch.cuda.mem_get_info()[0]
+    assert free_before - free_after < 2 * scratch, (free_before - free_after, scratch)
+    assert all(torch.equal(a, o) for a, o in zip(alone, outs))
