@@ -1037,61 +1037,83 @@ decode_fp_kernel(AttendArgs a, int tiles_total, int tiles_per_wg, int nsplit) {
     }
 }
 
-// grid (R, BH), D rounded up to whole wavefronts of threads: merge the span partials of one query
-// row and write the output row
+// grid (R, BH), 256 threads: merge the span partials of one query row and write the output row.
+// A launch with few rows and many spans (a single sequence: 8 pairs, 32 to 512 spans each) lasts as long as its
+// chain of memory round trips, so everything is asked for at once: a thread is (column pair, span group) and
+// requests its first eight partial pairs before anything else, then the (max, sum) of up to two spans; the weights
+// are formed while the columns are in flight, go through LDS, and the span groups' sums meet there at the end.
 template <int D, int DT>
-__global__ void __launch_bounds__((D + 63) / 64 * 64)
-combine_kernel(AttendArgs a, int nsplit, int rr) {
-    constexpr int NT = (D + 63) / 64 * 64;
-    __shared__ float w_s[512];  // weight of each span for this row (nsplit <= 512)
-    __shared__ float red_s[4];
+__global__ void __launch_bounds__(256) combine_kernel(AttendArgs a, int nsplit, int rr) {
+    constexpr int CP = D / 2;     // column pairs
+    constexpr int NG = 256 / CP;  // span groups: 8 (D 64), 6, 5, 4 (D 128), 2 (D 256)
+    constexpr int UN = 8;         // loads in flight per thread and round
+    __shared__ float w_s[512];    // weight of each span for this row (nsplit <= 512)
+    __shared__ float red_s[2][4];
+    __shared__ kv_f2 acc_s[NG][CP];
     const int i = blockIdx.x, bh = blockIdx.y;
     const int b = bh / a.Hkv, hk = bh - b * a.Hkv;
     const int r = a.Hq / a.Hkv;
     const int rep = i / a.L, l = i - rep * a.L;
     const size_t sstride = (size_t)rr * (D + 2);
     const size_t first_slot = (size_t)bh * nsplit;
+    // (rows of D + 2 floats, D even: every pair below is 8-byte aligned)
     const float *part = a.workspace + first_slot * sstride + (size_t)i * (D + 2);
     const int t = threadIdx.x;
-    const int d = t < D ? t : 0;  // threads past the last column read column 0 and write nothing
-    // every span's (max, sum) in one parallel round of loads, reduced through LDS
-    float mloc = -INFINITY;
-    for (int s = t; s < nsplit; s += NT) {
-        const float m = part[s * sstride + D];
-        w_s[s] = m;
-        mloc = fmaxf(mloc, m);
-    }
-    mloc = wave_max(mloc);
-    if ((t & 63) == 0) red_s[t >> 6] = mloc;
-    __syncthreads();
-    float mx = red_s[0];
+    const int g = t / CP, cp = t - g * CP;
+    const bool col = g < NG;
+    auto pair_at = [&](int s, int c) { return *reinterpret_cast<const kv_f2 *>(part + (size_t)s * sstride + c); };
+    kv_f2 v[UN];
 #pragma unroll
-    for (int w = 1; w < NT / 64; ++w) mx = fmaxf(mx, red_s[w]);
+    for (int u = 0; u < UN; ++u) {
+        const int s = g + NG * u;
+        v[u] = (col && s < nsplit) ? pair_at(s, 2 * cp) : kv_f2{0.f, 0.f};
+    }
+    kv_f2 ml[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) ml[u] = t + 256 * u < nsplit ? pair_at(t + 256 * u, D) : kv_f2{-INFINITY, 0.f};
+    float mloc = wave_max(fmaxf(ml[0].x, ml[1].x));
+    if ((t & 63) == 0) red_s[0][t >> 6] = mloc;
     __syncthreads();
+    const float mx = fmaxf(fmaxf(red_s[0][0], red_s[0][1]), fmaxf(red_s[0][2], red_s[0][3]));
     float dloc = 0.f;
-    for (int s = t; s < nsplit; s += NT) {
-        const float m = w_s[s];
-        const float w = (m == -INFINITY) ? 0.f : fast_exp2((m - mx) * LOG2E);
-        w_s[s] = w;
-        dloc += w * part[s * sstride + D + 1];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const float w = (ml[u].x == -INFINITY) ? 0.f : fast_exp2((ml[u].x - mx) * LOG2E);
+        if (t + 256 * u < nsplit) w_s[t + 256 * u] = w;
+        dloc += w * ml[u].y;
     }
     dloc = wave_sum(dloc);
-    if ((t & 63) == 0) red_s[t >> 6] = dloc;
+    if ((t & 63) == 0) red_s[1][t >> 6] = dloc;
     __syncthreads();
-    float den = red_s[0];
+    const float den = (red_s[1][0] + red_s[1][1]) + (red_s[1][2] + red_s[1][3]);
+    kv_f2 num{0.f, 0.f};
 #pragma unroll
-    for (int w = 1; w < NT / 64; ++w) den += red_s[w];
-    // the column sums: independent loads, issued several at a time
-    float num = 0.f;
-    int s = 0;
-    for (; s + 4 <= nsplit; s += 4) {
-        const float p0 = part[(s + 0) * sstride + d], p1 = part[(s + 1) * sstride + d];
-        const float p2 = part[(s + 2) * sstride + d], p3 = part[(s + 3) * sstride + d];
-        num += w_s[s] * p0 + w_s[s + 1] * p1 + w_s[s + 2] * p2 + w_s[s + 3] * p3;
+    for (int u = 0; u < UN; ++u) {
+        const int s = g + NG * u;
+        if (col && s < nsplit) num += w_s[s] * v[u];
     }
-    for (; s < nsplit; ++s) num += w_s[s] * part[s * sstride + d];
-    const float o = den > 0.f ? num / den : 0.f;
-    if (t < D) Elem<DT>::store(a.out, ((size_t)(b * a.Hq + hk * r + rep) * a.L + l) * D + d, o);
+    for (int s0 = g + NG * UN; col && s0 < nsplit; s0 += NG * UN) {  // more than 8 NG spans: further rounds
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int s = s0 + NG * u;
+            v[u] = s < nsplit ? pair_at(s, 2 * cp) : kv_f2{0.f, 0.f};
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int s = s0 + NG * u;
+            if (s < nsplit) num += w_s[s] * v[u];
+        }
+    }
+    if (col) acc_s[g][cp] = num;
+    __syncthreads();
+    if (t < CP) {
+        kv_f2 o = acc_s[0][t];
+#pragma unroll
+        for (int k = 1; k < NG; ++k) o += acc_s[k][t];
+        const float o0 = den > 0.f ? o.x / den : 0.f, o1 = den > 0.f ? o.y / den : 0.f;
+        uint32_t *dst = reinterpret_cast<uint32_t *>(static_cast<char *>(a.out) + (((size_t)(b * a.Hq + hk * r + rep) * a.L + l) * D + 2 * t) * 2);
+        *dst = DT == 0 ? pk_h2(o0, o1) : pk_bf2(o0, o1);
+    }
 }
 
 // The same merge for the prefill tiles' key-range parts: many query rows, at most 8 parts.  One wavefront per
@@ -1287,8 +1309,8 @@ hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t
     }
 #define CMB(D)                                                                                       \
     do {                                                                                             \
-        if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL((combine_kernel<D, 0>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows); \
-        else hipLaunchKernelGGL((combine_kernel<D, 1>), grid, dim3((D + 63) / 64 * 64), 0, s, a, nsplit, rows);       \
+        if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL((combine_kernel<D, 0>), grid, dim3(256), 0, s, a, nsplit, rows); \
+        else hipLaunchKernelGGL((combine_kernel<D, 1>), grid, dim3(256), 0, s, a, nsplit, rows);       \
     } while (0)
     // (the partials hold output columns: the head size of the values)
     if (a.st.Dv == 64) CMB(64);
