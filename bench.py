@@ -311,7 +311,8 @@ def other_workload(args, torch, kvhip, L, dev):
                   (4, 8, 4, 256, 512, 4608, "bf16"), (1, 16, 16, "192/128", 2048, 8192, "f16"),
                   (1, 16, 16, "192/128", 2048, 8192, "bf16"), (1, 32, 8, 128, 2048, 8192, "q4"), (1, 32, 8, 128, 2048, 8192, "q8"),
                   (4, 16, 4, 64, 2048, 4096, "q8"), (4, 8, 4, 256, 512, 4608, "q4"), (1, 32, 8, 96, 2048, 8192, "q4"),
-                  (1, 16, 16, "192/128", 2048, 8192, "q4"), (1, 16, 16, "192/128", 2048, 8192, "q8")]
+                  (1, 16, 16, "192/128", 2048, 8192, "q4"), (1, 16, 16, "192/128", 2048, 8192, "q8"), (1, 32, 8, 128, 2048, 8192, "q3"),
+                  (1, 32, 8, 128, 512, 8192, "q4"), (1, 32, 8, 128, 128, 8192, "q4")]
         if args.prefill_shape:
             f = args.prefill_shape.split(",")
             shapes = [tuple(x if "/" in x else int(x) for x in f[:6]) + (f[6],)]
