@@ -225,3 +225,32 @@ def test_dequantize_first_scratch_is_one_buffer_per_stream():
     free_after = torch.cuda.mem_get_info()[0]
     assert free_before - free_after < 2 * scratch, (free_before - free_after, scratch)
     assert all(torch.equal(a, o) for a, o in zip(alone, outs))
+
+
+def test_dequantize_first_on_two_streams():
+    """Calls on different streams never share a scratch buffer that is still in use: two caches attended in turn on
+    two streams (default priority), ten times each with nothing waited for, give what each gives alone."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(4)
+    B, Hkv, r, D, T, Lq = 1, 8, 4, 128, 4096, 1024
+    lib = kvhip.load()
+    caches, alone = [], []
+    q = torch.randn(B, Hkv * r, Lq, D, generator=g, device="cuda").half()
+    causal = kvhip.MaskMode.causal()
+    for _ in range(2):
+        c = kvhip.QuantizedKVCache(64, 4)
+        c.update_quantized(torch.randn(B, Hkv, T, D, generator=g, device="cuda").half(), torch.randn(B, Hkv, T, D, generator=g, device="cuda").half(), fetch=False)
+        caches.append(c)
+        alone.append(c.attend(q, D ** -0.5, causal))
+        assert lib.kvhip_last_attend_kernel() == 4
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[torch.empty_like(q) for _ in range(10)] for _ in range(2)]
+    for i in range(10):
+        for k in range(2):
+            with torch.cuda.stream(streams[k]):
+                caches[k].attend(q, D ** -0.5, causal, out=outs[k][i])
+    for st in streams:
+        st.synchronize()
+    for k in range(2):
+        assert all(torch.equal(alone[k], o) for o in outs[k])
