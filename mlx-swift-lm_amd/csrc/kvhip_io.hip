@@ -304,6 +304,92 @@ __global__ void __launch_bounds__(256) dequant_tiles16_kernel(Store q, Store dst
     }
 }
 
+// The same for head sizes that are multiples of 32, by units of 32 codes (4 BITS bytes: whole dwords for every code
+// width).  A thread loads one unit -- the units of a tile's K rows, and of its V tile rows, are one contiguous run, so
+// the loads of a workgroup are too --, converts it and writes four 16-byte chunks of the interleaved full-precision
+// tile; for each of the four, the threads of a wavefront write runs of 256 bytes (K: sixteen tokens of one chunk
+// column) or 512 bytes (V: thirty-two columns of one token octet).  A K unit has one (scale, bias) pair, loaded with
+// it; a V unit needs the pairs of its 32 tokens, which the workgroup stages in LDS once ([group][token]).
+// code j (0..31) of a unit held in N dwords, at unit-relative bit `pos` (constant once unrolled)
+template <int BITS, int N> __device__ __forceinline__ uint32_t unit_code(const uint32_t (&w)[N], int pos) {
+    const int wi = pos >> 5, sh = pos & 31;
+    uint32_t v = w[wi] >> sh;
+    if (sh + BITS > 32) v |= w[wi + 1 < N ? wi + 1 : wi] << ((32 - sh) & 31);
+    return v & ((1u << BITS) - 1u);
+}
+template <int DT, int BITS>
+__global__ void __launch_bounds__(256) dequant_units_kernel(Store q, Store dst, PageEntry *dst_pt, int pages, PageEntry page0, size_t sk, size_t sv) {
+    typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+    const int bh = blockIdx.y, lo = blockIdx.x * TILE;
+    auto pack = [](float a, float b) { return DT == 0 ? pk_h2(a, b) : pk_bf2(a, b); };
+    if (dst_pt != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0) {
+        for (int p = threadIdx.x; p < pages; p += 256) {
+            PageEntry e;
+            e.k = page0.k + (size_t)p * sk;
+            e.v = page0.v + (size_t)p * sv;
+            dst_pt[p] = e;
+        }
+    }
+    const PageEntry de = dst_pt != nullptr ? PageEntry{page0.k + (size_t)(lo >> PAGE_SHIFT) * sk, nullptr, page0.v + (size_t)(lo >> PAGE_SHIFT) * sv, nullptr}
+                                           : dst.pt[lo >> PAGE_SHIFT];
+    if (blockIdx.z == 0) {
+        char *kdst = de.k + (size_t)bh * dst.k_cell + kfp_off(dst, lo, 0);
+        const int upr = q.Dk / 32;  // units per row
+        const uint32_t *krows = reinterpret_cast<const uint32_t *>(k_row_ptr(q, bh, lo));  // the tile's 64 rows are contiguous
+        for (int u = threadIdx.x; u < upr * TILE; u += 256) {
+            const int t = u / upr, p = u - t * upr;
+            uint32_t w[BITS];
+#pragma unroll
+            for (int e = 0; e < BITS; ++e) w[e] = krows[(size_t)u * BITS + e];
+            float sc, bi;
+            pair_of<DT>(reinterpret_cast<const uint32_t *>(ksb_row_ptr(q, bh, lo + t))[(32 * p) / q.gs], sc, bi);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                uint32_t o[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float x0 = __fadd_rn(__fmul_rn(sc, (float)unit_code<BITS, BITS>(w, (8 * k + 2 * j) * BITS)), bi);
+                    const float x1 = __fadd_rn(__fmul_rn(sc, (float)unit_code<BITS, BITS>(w, (8 * k + 2 * j + 1) * BITS)), bi);
+                    o[j] = pack(x0, x1);
+                }
+                *reinterpret_cast<u4v *>(kdst + ((size_t)(4 * p + k) * TILE + t) * 16) = u4v{o[0], o[1], o[2], o[3]};
+            }
+        }
+        return;
+    }
+    // V: the pairs of the tile's 64 tokens, [group][token], through LDS
+    extern __shared__ uint32_t sbv[];
+    const int G = q.Dv / q.gs;
+    for (int i = threadIdx.x; i < G * TILE; i += 256) {
+        const int t = i / G, g = i - t * G;
+        sbv[g * TILE + t] = reinterpret_cast<const uint32_t *>(vsb_row_ptr(q, bh, lo + t))[g];
+    }
+    __syncthreads();
+    const uint32_t *vrows = reinterpret_cast<const uint32_t *>(v_cell_ptr(q, bh, lo) + v_row_off(q, lo, 0));  // Dv rows of 2 BITS dwords
+    char *vdst = de.v + (size_t)bh * dst.v_cell + vfp_off(dst, lo, 0);
+    for (int u = threadIdx.x; u < 2 * q.Dv; u += 256) {
+        const int d = u >> 1, half = u & 1;
+        uint32_t w[BITS];
+#pragma unroll
+        for (int e = 0; e < BITS; ++e) w[e] = vrows[(size_t)u * BITS + e];
+        const uint32_t *sb = sbv + (d / q.gs) * TILE + 32 * half;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            uint32_t o[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float s0, b0, s1, b1;
+                pair_of<DT>(sb[8 * k + 2 * j], s0, b0);
+                pair_of<DT>(sb[8 * k + 2 * j + 1], s1, b1);
+                const float x0 = __fadd_rn(__fmul_rn(s0, (float)unit_code<BITS, BITS>(w, v_bitpos<BITS>(8 * k + 2 * j))), b0);
+                const float x1 = __fadd_rn(__fmul_rn(s1, (float)unit_code<BITS, BITS>(w, v_bitpos<BITS>(8 * k + 2 * j + 1))), b1);
+                o[j] = pack(x0, x1);
+            }
+            *reinterpret_cast<u4v *>(vdst + ((size_t)(4 * half + k) * q.Dv + d) * 16) = u4v{o[0], o[1], o[2], o[3]};
+        }
+    }
+}
+
 // grid (whole tiles, BH), 256 threads; 16-bit dtypes, Dk == 32 NCK, Dv == 32 NCV
 template <int NCK, int NCV>
 __global__ void __launch_bounds__(256)
@@ -705,9 +791,16 @@ hipError_t launch_dequant_pages(const Store &q, const Store &dst, int rows, hipS
     if (rows <= 0) return hipSuccess;
     dim3 grid((rows + TILE - 1) / TILE, q.BH), block(256);
     if (q.es == 2 && q.Dk % 8 == 0 && q.Dv % 8 == 0) {
+        const size_t lds = (size_t)(q.Dv / q.gs) * TILE * 4;
 #define CALL(DT, BITS)                                                                                                  \
-    hipLaunchKernelGGL((dequant_tiles16_kernel<(DT == 2 ? 0 : DT), BITS>), dim3(grid.x, grid.y, 2), block, 0, s, q, dst, \
-                       (PageEntry *)nullptr, 0, PageEntry(), (size_t)0, (size_t)0)
+    do {                                                                                                                \
+        if (q.Dk % 32 == 0 && q.Dv % 32 == 0)                                                                           \
+            hipLaunchKernelGGL((dequant_units_kernel<(DT == 2 ? 0 : DT), BITS>), dim3(grid.x, grid.y, 2), block, lds, s, q, dst, \
+                               (PageEntry *)nullptr, 0, PageEntry(), (size_t)0, (size_t)0);                             \
+        else                                                                                                            \
+            hipLaunchKernelGGL((dequant_tiles16_kernel<(DT == 2 ? 0 : DT), BITS>), dim3(grid.x, grid.y, 2), block, 0, s, q, dst, \
+                               (PageEntry *)nullptr, 0, PageEntry(), (size_t)0, (size_t)0);                             \
+    } while (0)
         KV_DISPATCH_DT_BITS(q.dtype, q.bits, CALL);
 #undef CALL
         return hipGetLastError();
@@ -725,9 +818,16 @@ hipError_t launch_dequant_scratch(const Store &q, const Store &dst, int rows, in
     if (rows <= 0) return hipSuccess;
     if (q.es != 2 || q.Dk % 8 != 0 || q.Dv % 8 != 0) return hipErrorInvalidValue;
     dim3 grid((rows + TILE - 1) / TILE, q.BH, 2), block(256);
+    const size_t lds = (size_t)(q.Dv / q.gs) * TILE * 4;
 #define CALL(DT, BITS)                                                                                          \
-    hipLaunchKernelGGL((dequant_tiles16_kernel<(DT == 2 ? 0 : DT), BITS>), grid, block, 0, s, q, dst,              \
-                       const_cast<PageEntry *>(dst.pt), pages, page0, sk, sv)
+    do {                                                                                                        \
+        if (q.Dk % 32 == 0 && q.Dv % 32 == 0)                                                                   \
+            hipLaunchKernelGGL((dequant_units_kernel<(DT == 2 ? 0 : DT), BITS>), grid, block, lds, s, q, dst,    \
+                               const_cast<PageEntry *>(dst.pt), pages, page0, sk, sv);                          \
+        else                                                                                                    \
+            hipLaunchKernelGGL((dequant_tiles16_kernel<(DT == 2 ? 0 : DT), BITS>), grid, block, 0, s, q, dst,    \
+                               const_cast<PageEntry *>(dst.pt), pages, page0, sk, sv);                          \
+    } while (0)
     KV_DISPATCH_DT_BITS(q.dtype, q.bits, CALL);
 #undef CALL
     return hipGetLastError();
