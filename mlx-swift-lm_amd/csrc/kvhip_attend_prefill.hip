@@ -42,13 +42,16 @@ bool attend_prefill_dequant_first(const AttendArgs &a, bool always) {
     return R >= (s.Dk == 192 ? min_rows / 2 : min_rows) && flops >= 4e10;
 }
 
-// 128 query rows per workgroup reuse each staged tile twice as often as 64; 64 rows are
-// used when that would leave the grid too small to fill 256 CUs twice over.
+// 128 query rows per workgroup reuse each staged tile twice as often as 64, and measured ahead of 64 rows on every
+// grid from two such blocks per kv head up -- also where they leave the grid small, which key-range parts then fill
+// (TFLOP/s of the call, 64 / 128 rows, fp16 D 128 32q/8kv causal: B1 512 x 8192 542 / 598, 512 x 32768 709 / 855,
+// 1024 x 8192 590 / 714, 256 x 32768 643 / 754, B2 512 x 8192 603 / 712, B7 256 x 4096 547 / 695, B3 512 x 8192
+// 693 / 708; D 64 B1 2048 x 8192 334 / 446; equal at 128 rows of 4 heads).
 static bool prefill_wide(const AttendArgs &a) {
     const int R = (a.Hq / a.Hkv) * a.L;
     static const int forced = measure_knob("KVHIP_PREFILL_WIDE", -1);  // (timing builds only)
     if (forced >= 0) return forced != 0 && a.st.Dk <= 128;
-    return (size_t)((R + 127) / 128) * a.st.BH >= 512 && a.st.Dk <= 128;
+    return R >= 256 && a.st.Dk <= 128;
 }
 
 // Query rows per workgroup.  The pipelined tile for quantized caches (kvhip_attend_prefill_q.hpp) takes 256 rows
@@ -82,10 +85,10 @@ static int prefill_splits(const AttendArgs &a) {
     const int bm = prefill_block_rows(a);
     if (a.st.bits != 0 && bm > 64) return 1;  // (chosen only when the grid fills the chip)
     const size_t wgs = (size_t)((R + bm - 1) / bm) * a.st.BH;
-    // as many workgroups as are resident at once: three per CU, two at D = 256 (LDS) -- a part more
-    // than that starts a second round that leaves half the CUs idle
+    // as many workgroups as are resident at once: three per CU, two at D = 256 (LDS) and for 128-row workgroups
+    // (registers) -- a part more than that starts a second round that leaves half the CUs idle
     static const int forced = measure_knob("KVHIP_PREFILL_TARGET", 0);  // (timing builds only)
-    const int target = forced > 0 ? forced : (a.st.Dk >= 256 ? 512 : 768);
+    const int target = forced > 0 ? forced : ((a.st.Dk >= 256 || (a.st.bits == 0 && bm == 128)) ? 512 : 768);
     int n = (int)(target / (wgs ? wgs : 1));
     const int tiles = (a.slots + BN - 1) / BN;
     if (n > tiles / 8) n = tiles / 8;
