@@ -687,10 +687,10 @@ def test_quantized_prompt_chunks_dequantize_first(dtype, bits, gs, D):
 
 @pytest.mark.parametrize("dtype,bits,D", [(torch.float16, 4, 128), (torch.bfloat16, 8, 128), (torch.float16, 3, 96), (torch.bfloat16, 4, (192, 128))])
 def test_large_quantized_chunks_run_dequantize_first_by_the_librarys_choice(dtype, bits, D):
-    """From 1024 query rows per kv head (512 with keys of 192 and values of 128) and 4e10 floating-point operations a
-    chunk over a quantized cache runs dequantize-first without being told to; a chunk below either bound stays on the
-    quantized tile.  The two paths agree to within the rounding of their intermediates (both are checked against the
-    oracle at sizes it covers)."""
+    """From 1024 query rows per kv head (512 with keys of 192 and values of 128) and 4e10 floating-point operations,
+    or 512 rows over 4096 keys and more, a chunk over a quantized cache runs dequantize-first without being told to;
+    a chunk of fewer rows stays on the quantized tile.  The two paths agree to within the rounding of their
+    intermediates (both are checked against the oracle at sizes it covers)."""
     D, Dv = D if isinstance(D, tuple) else (D, D)
     g = torch.Generator(device="cuda")
     g.manual_seed(bits + D)
@@ -700,7 +700,7 @@ def test_large_quantized_chunks_run_dequantize_first_by_the_librarys_choice(dtyp
     lib = kvhip.load()
     scale = D ** -0.5
     try:
-        for Lq, want in ((L, 4), (128, 3)):
+        for Lq, want in ((L, 4), (128, 4), (64, 3)):
             q = torch.randn(B, Hkv * r, Lq, D, generator=g, device="cuda").to(dtype)
             for mask in (kvhip.MaskMode.causal(), kvhip.MaskMode.window_mask(T - Lq, 1000)):
                 lib.kvhip_set_kernel_policy(0)
