@@ -60,7 +60,7 @@ def main():
                          "shader clock for some 30 ms; reported as settle_launches (0 = none)")
     ap.add_argument("--reserve", action="store_true",
                     help="pre-size the cache's pages (default: grow from empty, as the reference does)")
-    ap.add_argument("--workload", default="cfg3", choices=["cfg3", "cfg1", "cfg2", "cfg4", "cfg5", "prefill"],
+    ap.add_argument("--workload", default="cfg3", choices=["cfg3", "cfg1", "cfg2", "cfg4", "cfg5", "prefill", "prompt"],
                     help="cfg3 (default) is the configuration the metric is quoted on; the others are the "
                          "remaining BASELINE.json configs (reported as one JSON object each)")
     ap.add_argument("--prefill-shape", default=None,
@@ -359,6 +359,44 @@ def other_workload(args, torch, kvhip, L, dev):
             del cache, k, v, q
         return {"workload": "chunked-prefill tiles on their own (prefill_fp_kernel; quantized caches: prefill_q_kernel, or "
                             "dequantize-first + prefill_fp_kernel from 512-1024 query rows per kv head; --policy 2 keeps them on prefill_q_kernel)",
+                "results": rows}
+
+    if args.workload == "prompt":
+        # one sequence's prompt through one layer's cache the way the reference feeds it (prefillStepSize 512,
+        # PrefillParameters.swift): chunks of 512 rows, each appended (quantized caches: quantized) and attended
+        # causally over everything cached so far; 32q/8kv, D 128.  The chunks are enqueued back to back; the time is
+        # that of the whole prompt, HIP events around all chunks, the median of five prompts after two untimed ones.
+        Hq, Hkv, D, chunk = 32, 8, 128, 512
+        rows = []
+        for T in (8192, 32768):
+            for dn in ("f16", "bf16", "q4", "q8"):
+                dtype = torch.bfloat16 if dn == "bf16" else torch.float16
+                k = torch.randn(1, Hkv, T, D, generator=g, device=dev).to(dtype)
+                v = k.flip(-1).contiguous()
+                q = torch.randn(1, Hq, T, D, generator=g, device=dev).to(dtype)
+                ks, vs, qs = [[x[:, :, t0:t0 + chunk].contiguous() for t0 in range(0, T, chunk)] for x in (k, v, q)]
+                out = torch.empty(1, Hq, chunk, D, dtype=dtype, device=dev)
+                times = []
+                for rep in range(7):
+                    cache = kvhip.QuantizedKVCache(64, int(dn[1])) if dn[0] == "q" else kvhip.KVCacheSimple()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for kc, vc, qc in zip(ks, vs, qs):
+                        if dn[0] == "q":
+                            cache.update_quantized(kc, vc, fetch=False)
+                        else:
+                            cache.update(kc, vc, fetch=False)
+                        cache.attend(qc, D ** -0.5, kvhip.MaskMode.causal(), out=out)
+                    e1.record()
+                    torch.cuda.synchronize()
+                    times.append(e0.elapsed_time(e1))
+                    del cache
+                ms = sorted(times[2:])[2]
+                fl = 4.0 * Hq * D * sum(t0 + (chunk + 1) / 2 for t0 in range(0, T, chunk)) * chunk
+                rows.append({"prompt": T, "cache": dn, "ms_per_layer": round(ms, 3), "prompt_tokens_per_s_per_layer": round(T / ms * 1e3),
+                             "TFLOPs": round(fl / ms / 1e9, 1)})
+                del k, v, q, ks, vs, qs
+        return {"workload": "one sequence's prompt in 512-row chunks through one layer: append + causal attention per chunk, 32q/8kv D128",
                 "results": rows}
 
     if args.workload == "cfg1":
