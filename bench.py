@@ -358,7 +358,7 @@ def other_workload(args, torch, kvhip, L, dev):
                          "frac_of_2.5PF": round(fl / (call_ms if family == 4 else ms) / 1e9 / 2500.0, 4)})
             del cache, k, v, q
         return {"workload": "chunked-prefill tiles on their own (prefill_fp_kernel; quantized caches: prefill_q_kernel, or "
-                            "dequantize-first + prefill_fp_kernel from 512-1024 query rows per kv head; --policy 2 keeps them on prefill_q_kernel)",
+                            "dequantize-first + prefill_fp_kernel from 512 query rows per kv head and rows x keys x (Dk + Dv) = 2^30; --policy 2 keeps them on prefill_q_kernel)",
                 "results": rows}
 
     if args.workload == "prompt":

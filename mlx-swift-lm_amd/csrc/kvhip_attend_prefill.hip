@@ -20,8 +20,6 @@ bool attend_prefill_supported(const AttendArgs &a) {
     return s.Dk == 64 || s.Dk == 80 || s.Dk == 96 || s.Dk == 128 || s.Dk == 256;
 }
 
-static int prefill_block_rows(const AttendArgs &a);
-
 // A prompt chunk over a quantized cache converts every cached row once per workgroup that reads it.  With many query
 // rows per kv head it is cheaper to convert the rows once for all of them: the cache is dequantized into scratch
 // pages of its dtype and the full-precision tile, whose loop has no conversions, runs over those.  The scratch costs
@@ -35,18 +33,17 @@ bool attend_prefill_dequant_first(const AttendArgs &a, bool always) {
     fp.st.bits = 0;
     if (!attend_prefill_supported(fp)) return false;
     if (always) return true;
-    // The conversion pass is a launch more and 2 (Dk + Dv) bytes per cached row and kv head written and read again:
-    // the chunk must be worth it.  Measured ahead (10-40 %) from 1024 query rows per kv head (512 for keys of 192 with
-    // values of 128) once the chunk has 4 x 10^10 operations, and over 4096 keys and more from 512 rows -- except
-    // where a chunk of exactly 512 rows fills the chip with 256-row workgroups of the quantized tile, which then is
-    // the faster one (B16, 128 x 4096: 198 against 234 us; at 768 rows, B16 192 x 8192, it is behind again: 752
-    // against 675 us).  Behind: few rows (B8, 64 x 8192: 189 against 144 us), few keys (a
-    // single sequence's 512 x 512: 37 against 33 us).
+    // The conversion pass is a launch more and 2 (Dk + Dv) bytes per cached row and kv head written and read again,
+    // the same for any number of query rows: what it buys grows with the rows per kv head that share a converted
+    // key.  Per kv head both costs scale alike with batch and heads, so the bound is one on rows x keys x head
+    // sizes: measured ahead by 5-40 % from 512 rows and rows x keys = 4 M at D 128 (2048 x 2048, 1024 x 4096,
+    // 512 x 8192; B1 to B16) over 2048 keys and more, equal or behind below that (1024 x 2048: 44 against 40 us,
+    // 2048 x 1024: 44 against 42, 4096 x 1024: 50 against 41,
+    // B16 512 x 4096, where 256-row workgroups of the quantized tile fill the chip: 231 against 197) and with
+    // fewer rows whatever the keys (B8, 256 x 8192: 185 against 141 us).
     const int R = (a.Hq / a.Hkv) * a.L;
-    const double flops = 2.0 * s.BH * R * (double)a.T * (s.Dk + s.Dv);
-    static const int min_rows = measure_knob("KVHIP_DEQUANT_FIRST_ROWS", 1024);  // (timing builds only)
-    if (R >= (s.Dk == 192 ? min_rows / 2 : min_rows) && flops >= 4e10) return true;
-    return a.T >= 4096 && R >= min_rows / 2 && !(R == min_rows / 2 && prefill_block_rows(a) == 256);
+    static const int min_rows = measure_knob("KVHIP_DEQUANT_FIRST_ROWS", 512);  // (timing builds only)
+    return R >= min_rows && a.T >= 2048 && (double)R * a.T * (s.Dk + s.Dv) >= 1073741824.0;
 }
 
 // 128 query rows per workgroup reuse each staged tile twice as often as 64, and measured ahead of 64 rows on every

@@ -687,9 +687,9 @@ def test_quantized_prompt_chunks_dequantize_first(dtype, bits, gs, D):
 
 @pytest.mark.parametrize("dtype,bits,D", [(torch.float16, 4, 128), (torch.bfloat16, 8, 128), (torch.float16, 3, 96), (torch.bfloat16, 4, (192, 128))])
 def test_large_quantized_chunks_run_dequantize_first_by_the_librarys_choice(dtype, bits, D):
-    """From 1024 query rows per kv head (512 with keys of 192 and values of 128) and 4e10 floating-point operations,
-    or 512 rows over 4096 keys and more, a chunk over a quantized cache runs dequantize-first without being told to;
-    a chunk of fewer rows stays on the quantized tile.  The two paths agree to within the rounding of their
+    """From 512 query rows per kv head, 2048 keys and rows x keys x (Dk + Dv) = 2^30 (1024 rows over 4096 keys at head
+    size 128) a chunk over a quantized cache runs dequantize-first without being told to; a smaller one stays on the
+    quantized tile.  The two paths agree to within the rounding of their
     intermediates (both are checked against the oracle at sizes it covers)."""
     D, Dv = D if isinstance(D, tuple) else (D, D)
     g = torch.Generator(device="cuda")
@@ -700,7 +700,8 @@ def test_large_quantized_chunks_run_dequantize_first_by_the_librarys_choice(dtyp
     lib = kvhip.load()
     scale = D ** -0.5
     try:
-        for Lq, want in ((L, 4), (128, 4), (64, 3)):
+        for Lq in (L, 256, 128):
+            want = 4 if r * Lq >= 512 and T >= 2048 and r * Lq * T * (D + Dv) >= 2 ** 30 else 3
             q = torch.randn(B, Hkv * r, Lq, D, generator=g, device="cuda").to(dtype)
             for mask in (kvhip.MaskMode.causal(), kvhip.MaskMode.window_mask(T - Lq, 1000)):
                 lib.kvhip_set_kernel_policy(0)
