@@ -55,7 +55,13 @@ static bool prefill_wide(const AttendArgs &a) {
     const int R = (a.Hq / a.Hkv) * a.L;
     static const int forced = measure_knob("KVHIP_PREFILL_WIDE", -1);  // (timing builds only)
     if (forced >= 0) return forced != 0 && a.st.Dk <= 128;
-    return R >= 256 && a.st.Dk <= 128;
+    if (R < 256 || a.st.Dk > 128) return false;
+    // Few keys (a prompt's first chunks): where 128-row workgroups would need key-range parts to fill the chip and
+    // 64-row ones fill it without, the merge launch costs more than the wider tile gains (a single sequence's
+    // 512 x 512: 22 against 35 us; 512 x 1024: 33 against 43; equal from 2048 keys).
+    const size_t wide_wgs = (size_t)((R + 127) / 128) * a.st.BH, narrow_wgs = (size_t)((R + 63) / 64) * a.st.BH;
+    if (a.T <= 1024 && wide_wgs < 512 && narrow_wgs >= 256) return false;
+    return true;
 }
 
 // Query rows per workgroup.  The pipelined tile for quantized caches (kvhip_attend_prefill_q.hpp) takes 256 rows
@@ -89,6 +95,7 @@ static int prefill_splits(const AttendArgs &a) {
     const int bm = prefill_block_rows(a);
     if (a.st.bits != 0 && bm > 64) return 1;  // (chosen only when the grid fills the chip)
     const size_t wgs = (size_t)((R + bm - 1) / bm) * a.st.BH;
+    if (a.st.bits == 0 && a.T <= 1024 && wgs >= 256) return 1;  // (few keys and a workgroup per CU: see prefill_wide)
     // as many workgroups as are resident at once: three per CU, two at D = 256 (LDS) and for 128-row workgroups
     // (registers) -- a part more than that starts a second round that leaves half the CUs idle
     static const int forced = measure_knob("KVHIP_PREFILL_TARGET", 0);  // (timing builds only)
