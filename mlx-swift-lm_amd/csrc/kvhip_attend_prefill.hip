@@ -95,7 +95,9 @@ static int prefill_splits(const AttendArgs &a) {
     const int bm = prefill_block_rows(a);
     if (a.st.bits != 0 && bm > 64) return 1;  // (chosen only when the grid fills the chip)
     const size_t wgs = (size_t)((R + bm - 1) / bm) * a.st.BH;
-    if (a.st.bits == 0 && a.T <= 1024 && wgs >= 256) return 1;  // (few keys and a workgroup per CU: see prefill_wide)
+    // (few keys and a workgroup per CU: see prefill_wide; the quantized tile likewise -- a single sequence's 512 x 512
+    // 4-bit chunk 33 -> 30 us undivided, 512 x 1024 at 8 bits 55 -> 47 us, at 4 bits 47 either way)
+    if (a.T <= 1024 && wgs >= 256) return 1;
     // as many workgroups as are resident at once: three per CU, two at D = 256 (LDS) and for 128-row workgroups
     // (registers) -- a part more than that starts a second round that leaves half the CUs idle
     static const int forced = measure_knob("KVHIP_PREFILL_TARGET", 0);  // (timing builds only)
