@@ -105,11 +105,11 @@ static int prefill_splits(const AttendArgs &a) {
     int n = (int)(target / (wgs ? wgs : 1));
     const int tiles = (a.slots + BN - 1) / BN;
     if (n > tiles / 8) n = tiles / 8;
-    // (a multi-token step of a few sequences -- 17 to 256 query rows per kv head, one to four 64-row blocks -- is a
-    // grid of a handful of workgroups: up to 64 parts instead of 8, merged by the decode path's many-part kernel.  A
+    // (a multi-token step or a short chunk of a few sequences -- up to 4096 query rows in all -- is a grid of a
+    // handful of workgroups: up to 64 parts instead of 8, merged by the decode path's many-part kernel.  A
     // single sequence, 32q/8kv, 5 new tokens: over 8192 keys 43 -> 18 us at 4 bits and 31 -> 15 us in float16, over
     // 32768 keys 152 -> 31 us and 97 -> 28 us; 32 new tokens over 32768 keys 154 -> 50 us and 97 -> 39 us)
-    const int cap = R <= 256 ? 64 : 8;
+    const int cap = (size_t)R * a.st.BH <= 4096 ? 64 : 8;  // (the many-part merge takes a workgroup per query row)
     if (n > cap) n = cap;
     if (n < 2) return 1;
     const size_t per_part = (size_t)a.st.BH * R * (a.st.Dv + 2) * sizeof(float);
