@@ -64,7 +64,7 @@ def main():
                     help="cfg3 (default) is the configuration the metric is quoted on; the others are the "
                          "remaining BASELINE.json configs (reported as one JSON object each)")
     ap.add_argument("--prefill-shape", default=None,
-                    help="with --workload prefill: one shape B,Hq,Hkv,D,L,T,dtype (dtype f16, bf16, or q2 / q3 / q4 / q5 / q6 / q8; D may be 192/128) instead of the table")
+                    help="with --workload prefill: one shape B,Hq,Hkv,D,L,T,dtype (dtype f16, bf16, f32, or q2 / q3 / q4 / q5 / q6 / q8; D may be 192/128) instead of the table")
     ap.add_argument("--policy", type=int, default=0, choices=[0, 2, 3],
                     help="kvhip_set_kernel_policy for the run: 0 the library's choice, 2 quantized prompt chunks always on "
                          "the quantized tile, 3 dequantize-first whenever the shape allows")
@@ -304,7 +304,8 @@ def other_workload(args, torch, kvhip, L, dev):
     if args.workload == "prefill":
         # the chunked-prefill tile on its own: L new rows attending causally over T cached keys (the new rows
         # included); flops = 2 * B * Hq * (Dk + Dv) * (keys each row sees)
-        # dtype field: f16 / bf16 full precision; qN a float16 QuantizedKVCache of N-bit codes (group 64; 32 at D 96);
+        # dtype field: f16 / bf16 / f32 full precision (f32: the vector-ALU kernel, its rate is float32 FMAs, not
+        # matrix-core work); qN a float16 QuantizedKVCache of N-bit codes (group 64; 32 at D 96);
         # a head size "192/128" is keys of 192 with values of 128
         shapes = [(1, 32, 8, 128, 2048, 8192, "f16"), (1, 32, 8, 128, 2048, 8192, "bf16"), (4, 32, 8, 128, 512, 4096, "f16"),
                   (1, 32, 8, 128, 4096, 4096, "f16"), (2, 16, 4, 64, 2048, 4096, "f16"), (4, 8, 4, 256, 512, 4608, "f16"),
@@ -319,7 +320,7 @@ def other_workload(args, torch, kvhip, L, dev):
         rows = []
         for Bn, Hq, Hkv, D, Lq, T, dn in shapes:
             Dk, Dv = (int(x) for x in D.split("/")) if isinstance(D, str) else (D, D)
-            dtype = torch.bfloat16 if dn == "bf16" else torch.float16
+            dtype = torch.bfloat16 if dn == "bf16" else torch.float32 if dn == "f32" else torch.float16
             k = torch.randn(Bn, Hkv, T, Dk, generator=g, device=dev).to(dtype)
             v = k.flip(-1)[..., :Dv].contiguous()
             if dn[0] == "q":
@@ -355,6 +356,7 @@ def other_workload(args, torch, kvhip, L, dev):
             rows.append({"shape": f"B{Bn} {Hq}q/{Hkv}kv D{D} {dn}, {Lq} new rows over {T} keys, causal", "launches": n,
                          "family": family, "kernel_ms": round(ms, 4), "call_ms": round(call_ms, 4),
                          "TFLOPs": round(fl / ms / 1e9, 1), "TFLOPs_call": round(fl / call_ms / 1e9, 1),
+                         "cache_TBps": round(Bn * Hkv * T * (Dk + Dv) * (int(dn[1]) / 8 if dn[0] == "q" else 4 if dn == "f32" else 2) / ms / 1e9, 2),
                          "frac_of_2.5PF": round(fl / (call_ms if family == 4 else ms) / 1e9 / 2500.0, 4)})
             del cache, k, v, q
         return {"workload": "chunked-prefill tiles on their own (prefill_fp_kernel; quantized caches: prefill_q_kernel, or "
