@@ -1235,9 +1235,9 @@ kvhip_status attend_impl(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, i
             KV_HIP(launch_attend_prefill(a, s));
         }
         g_last_kernel = done ? 4 : 3;
-    } else if (g_policy != 1 && attend_f32_supported(a)) {
-        KV_TRY(bind_workspace(c, a, attend_f32_workspace(a), fixed, fixed_bytes, s));
-        KV_HIP(launch_attend_f32(a, s));
+    } else if (g_policy != 1 && attend_valu_supported(a)) {
+        KV_TRY(bind_workspace(c, a, attend_valu_workspace(a), fixed, fixed_bytes, s));
+        KV_HIP(launch_attend_valu(a, s));
         g_last_kernel = 5;
     } else {
         KV_TRY(bind_workspace(c, a, attend_generic_workspace(a), fixed, fixed_bytes, s));

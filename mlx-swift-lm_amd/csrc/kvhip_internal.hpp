@@ -301,10 +301,11 @@ bool attend_decode_fuses_append(const AttendArgs &a);
 // Bytes of scratch each kernel family needs for these arguments.
 size_t attend_generic_workspace(const AttendArgs &a);
 hipError_t launch_attend_generic(const AttendArgs &a, hipStream_t s);
-// float32 caches on the vector ALUs (head sizes up to 512 / 256): any row count, any mask.
-bool attend_f32_supported(const AttendArgs &a);
-size_t attend_f32_workspace(const AttendArgs &a);
-hipError_t launch_attend_f32(const AttendArgs &a, hipStream_t s);
+// Full-precision caches on the vector ALUs (float32 caches; 16-bit ones of head sizes above 256, which the matrix-core
+// kernels are not built for; keys up to 1024 wide, values up to 512): any row count, any mask.
+bool attend_valu_supported(const AttendArgs &a);
+size_t attend_valu_workspace(const AttendArgs &a);
+hipError_t launch_attend_valu(const AttendArgs &a, hipStream_t s);
 // Fast split-sequence decode kernels; `supported` says whether the shape is covered.
 bool attend_decode_supported(const AttendArgs &a);
 size_t attend_decode_workspace(const AttendArgs &a);

@@ -155,13 +155,13 @@ def test_allocation_free_entry_on_a_padded_cache():
         assert family() == fam and fam in (2, 3) and torch.equal(got, want)
 
 
-def test_float32_has_its_own_kernel_and_head_sizes_above_256_stay_on_the_plain_one():
+def test_float32_and_head_sizes_above_256_run_on_the_vector_alu_kernel():
     rng = np.random.default_rng(9)
     for dtype, D in ((torch.float32, 72), (torch.float16, 320)):
         c, o = kvhip.KVCacheSimple(), O.KVCacheSimple(NAME[dtype])
         k, kd = randn(rng, (1, 2, 50, D), dtype)
         q, qd = randn(rng, (1, 4, 50, D), dtype)
         out = kvhip.attention_with_cache_update(qd, kd, kd, c, D ** -0.5, kvhip.MaskMode.causal())
-        assert family() == (5 if dtype == torch.float32 else 0)
+        assert family() == 5
         ref = O.attention_with_cache_update(q, k, k, o, D ** -0.5, O.Mask.CAUSAL, NAME[dtype])
         check_attention(out, ref, dtype, f"D={D}", lambda: exact_attention(q, *presented_f64(o), D ** -0.5, O.Mask.CAUSAL))

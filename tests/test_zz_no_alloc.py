@@ -76,8 +76,9 @@ def test_static_scratch_full_precision_and_ring(dtype):
 
 
 def test_static_scratch_rejects_what_does_not_fit():
-    # the plain kernel materialises one float per (query row, key): 4 * 32 * 64 * 40000 * 4 bytes > 16 MiB
-    c, g = filled(kvhip.KVCacheSimple, 4, 8, 40000, 32, torch.float32, 5)
+    # the plain kernel (here: a quantized cache whose scales are float32) materialises one float per (query row, key):
+    # 4 * 32 * 64 * 40000 * 4 bytes > 16 MiB
+    c, g = filled(kvhip.QuantizedKVCache, 4, 8, 40000, 32, torch.float32, 5, group_size=32, bits=8)
     q = torch.randn(4, 32, 64, 32, generator=g, device="cuda")
     out = torch.zeros(4, 32, 64, 32, device="cuda")
     with pytest.raises(L.KVHipError) as e:
