@@ -1132,6 +1132,7 @@ kvhip_status attend_dequant_first(kvhip_cache *c, const AttendArgs &a, hipStream
     hipError_t e = launch_dequant_scratch(a.st, t, a.T, (int)pages, first, stride[0], stride[1], s);
     if (e == hipSuccess) st = bind_workspace(c, a2, attend_prefill_workspace(a2), nullptr, 0, s);
     if (e == hipSuccess && st == KVHIP_OK) e = launch_attend_prefill(a2, s);
+    if (e == hipSuccess && st == KVHIP_OK && mask_may_leave_rows_without_keys(a2)) e = launch_rows_without_keys(a2, s);
     retire(std::move(give_back), s);
     if (e != hipSuccess) return fail(KVHIP_ERR_HIP, std::string("dequantize-first prefill: ") + hipGetErrorString(e));
     if (st != KVHIP_OK) return st;

@@ -7,6 +7,8 @@
 // finfo(T).min fill (or T(scores + mask)), p = T(softmax), out = T(p . V^).
 // Full-precision caches follow the fused op (AttentionUtils.swift:86-93):
 // float32 inside, excluded keys contribute nothing, one rounding at the output.
+#include <algorithm>
+
 #include "kvhip_mask.hpp"
 
 namespace kvhip {
@@ -138,7 +140,104 @@ attend_generic_kernel(AttendArgs a, int slots_pad) {
     }
 }
 
+// ---- rows that see no key, after the full-precision tile ran over a dequantized copy of a quantized cache ----
+// The reference's quantized sequence fills masked scores with finfo(T).min (KVCache.swift:2441-2445), so a query row
+// whose mask excludes every key -- a batch row that is all padding -- weighs all T keys alike: p = T(1 / T), out =
+// T(p . V^).  The full-precision tile drops excluded keys and leaves such a row at zero.  This kernel finds those rows
+// (boolean arrays: 16 mask bytes per lane and load; index masks: from the bounds) and writes them.
+// a.st: the dequantized pages (slots in presented order); grid (row blocks of 64, BH), 256 threads.
+template <int DT>
+__global__ void __launch_bounds__(GT)
+rows_without_keys_kernel(AttendArgs a) {
+    __shared__ int empty_s[64];
+    __shared__ int any_s;
+    const Store &st = a.st;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bh = blockIdx.y, b = bh / a.Hkv, h = bh % a.Hkv;
+    const int r = a.Hq / a.Hkv, R = r * a.L, row0 = blockIdx.x * 64;
+    if (tid == 0) any_s = 0;
+    __syncthreads();
+    for (int i = wave; i < 64; i += GT / 64) {  // one wavefront per query row
+        const int rr = row0 + i;
+        bool empty = false;
+        if (rr < R) {
+            const int hq = h * r + rr / a.L, l = rr % a.L;
+            if (a.mask.mode == KVHIP_MASK_ARRAY) {
+                const uint8_t *mrow = reinterpret_cast<const uint8_t *>(a.mask.data) + (size_t)(b * a.mask.sb + hq * a.mask.sh + l * a.mask.sl);
+                bool seen = false;
+                for (int base = 0; base < a.T; base += 64 * 16) {  // wave-uniform trips
+                    const int j0 = base + lane * 16;
+                    if (j0 + 16 <= a.T) {
+                        uint32_t w[4];
+                        mask_bool_words<4>(a.mask, b, hq, l, j0, w);
+                        seen = (w[0] | w[1] | w[2] | w[3]) != 0;
+                    } else {
+                        for (int j = j0; j < a.T; ++j) seen = seen || mrow[j] != 0;
+                    }
+                    if (__any(seen)) break;
+                }
+                empty = !__any(seen);
+            } else {
+                const SymMask sm = sym_mask_init(a.mask, b, a.L, a.T);
+                int lo, hi;
+                if (sm.mode == KVHIP_MASK_CAUSAL) {
+                    lo = 0;
+                    hi = a.T - a.L + l;
+                } else {
+                    lo = sm.pad_b;
+                    hi = min(sm.offset + l, sm.len_b - 1);
+                    if (sm.window > 0) lo = max(lo, sm.offset + l - sm.window + 1);
+                }
+                empty = max(lo, 0) > min(hi, a.T - 1);
+            }
+        }
+        if (lane == 0) {
+            empty_s[i] = empty;
+            if (empty) any_s = 1;
+        }
+    }
+    __syncthreads();
+    if (!any_s) return;
+    const float p = round_dt<DT>(1.0f / (float)a.T);
+    constexpr int EPC = 8;  // tokens per 16-byte chunk of a 16-bit V tile
+    for (int d = tid; d < st.Dv; d += GT) {
+        float sum = 0.f;
+        for (int slot0 = 0; slot0 < a.T; slot0 += EPC) {
+            const uint4 w = *reinterpret_cast<const uint4 *>(v_cell_ptr(st, bh, slot0) + vfp_off(st, slot0, d));  // 8 tokens of column d
+            const int n = min(EPC, a.T - slot0);
+            for (int e = 0; e < n; ++e) sum += Elem<DT>::load(&w, e);
+        }
+        const float v = p * sum;
+        for (int i = 0; i < 64; ++i) {
+            if (!empty_s[i]) continue;
+            const int rr = row0 + i, hq = h * r + rr / a.L, l = rr % a.L;
+            Elem<DT>::store(a.out, ((size_t)(b * a.Hq + hq) * a.L + l) * st.Dv + d, v);
+        }
+    }
+}
+
 }  // namespace
+
+bool mask_may_leave_rows_without_keys(const AttendArgs &a) {
+    const MaskDev &m = a.mask;
+    if (m.mode == KVHIP_MASK_NONE) return false;
+    if (m.mode == KVHIP_MASK_CAUSAL) return a.T < a.L;
+    if (m.mode == KVHIP_MASK_ARRAY) return m.dtype == KVHIP_BOOL;
+    if (m.lengths || m.left_pad) return true;  // per-batch bounds in device memory
+    for (int e = 0; e < 2; ++e) {  // the kept range [max(0, offset + l - window + 1), min(offset + l, T - 1)] is narrowest at an end
+        const int l = e ? a.L - 1 : 0;
+        const int lo = m.window > 0 ? std::max(0, m.offset + l - m.window + 1) : 0, hi = std::min(m.offset + l, a.T - 1);
+        if (lo > hi) return true;
+    }
+    return false;
+}
+
+hipError_t launch_rows_without_keys(const AttendArgs &a, hipStream_t s) {
+    const dim3 grid(((a.Hq / a.Hkv) * a.L + 63) / 64, a.st.BH), block(GT);
+    if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL(rows_without_keys_kernel<0>, grid, block, 0, s, a);
+    else hipLaunchKernelGGL(rows_without_keys_kernel<1>, grid, block, 0, s, a);
+    return hipGetLastError();
+}
 
 static int pad32(int n) { return (n + 31) & ~31; }
 

@@ -317,6 +317,11 @@ size_t attend_prefill_workspace(const AttendArgs &a);
 // full-precision tile run over them (many query rows per kv head share the one conversion of every cached row).
 // (`always`: whenever the shape allows it, whatever the row count)
 bool attend_prefill_dequant_first(const AttendArgs &a, bool always);
+// After the full-precision tile has run over a dequantized copy of a quantized cache: query rows whose mask excludes
+// every key take the reference's quantized answer, equal weights over all T keys (a.st: the dequantized pages).
+// `mask_may_...`: false when the mask provably leaves no such row, so the launch can be left out.
+bool mask_may_leave_rows_without_keys(const AttendArgs &a);
+hipError_t launch_rows_without_keys(const AttendArgs &a, hipStream_t s);
 // Merge `nsplit` partials per query row, laid out [bh][split][rows][D+2] in a.workspace
 // (out[D] unnormalised, running max, running sum), and write the normalised rows to a.out.
 hipError_t launch_combine(const AttendArgs &a, int nsplit, int rows, hipStream_t s);

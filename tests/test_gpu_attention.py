@@ -685,6 +685,65 @@ def test_quantized_prompt_chunks_dequantize_first(dtype, bits, gs, D):
         assert np.array_equal(np32(a), b) if i % 3 == 0 else bits_equal(a, b, dtype), i
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("mode", ["lengths", "left_pad", "bool"])
+def test_dequantize_first_gives_rows_without_keys_the_quantized_answer(dtype, mode):
+    """A query row whose mask excludes every key (a batch row that is all padding): the reference's quantized sequence
+    fills the scores with finfo.min, so the row weighs every key alike (KVCache.swift:2441-2445); the full-precision
+    tile that dequantize-first runs would leave it at zero.  Both policies against the oracle."""
+    rng = np.random.default_rng(77)
+    name = NAME[dtype]
+    B, Hkv, r, D, T0, Lq = 2, 2, 4, 128, 300, 70
+    scale = D ** -0.5
+    lib = kvhip.load()
+    try:
+        for policy, family in ((3, 4), (2, 3)):
+            lib.kvhip_set_kernel_policy(policy)
+            c, o = kvhip.QuantizedKVCache(64, 4), O.QuantizedKVCache(64, 4, name)
+            k, kd = randn(rng, (B, Hkv, T0, D), dtype)
+            v, vd = randn(rng, (B, Hkv, T0, D), dtype)
+            c.update_quantized(kd, vd, fetch=False)
+            o.update_quantized(k, v)
+            k, kd = randn(rng, (B, Hkv, Lq, D), dtype)
+            v, vd = randn(rng, (B, Hkv, Lq, D), dtype)
+            q, qd = randn(rng, (B, Hkv * r, Lq, D), dtype)
+            T = T0 + Lq
+            j = np.arange(T)[None, None, None, :]
+            causal = np.broadcast_to(O.create_causal_mask(Lq, T - Lq)[None, None], (B, 1, Lq, T))
+            if mode == "lengths":
+                lengths = np.array([0, T - 20], np.int32)
+                m = causal & (j < lengths[:, None, None, None])
+                mask = kvhip.MaskMode.window_mask(T - Lq, 0, lengths=torch.from_numpy(lengths))
+            elif mode == "left_pad":
+                pad = np.array([T0 + 30, 5], np.int32)  # batch row 0: its first 30 query positions are padding
+                m = causal & (j >= pad[:, None, None, None])
+                mask = kvhip.MaskMode.window_mask(T - Lq, 0, left_pad=torch.from_numpy(pad))
+            else:
+                m = causal & (rng.random((B, 1, Lq, T)) < 0.8)
+                m[..., 0] = True
+                m[0, 0, 3:9] = False   # rows without keys, in the middle of a block and ...
+                m[1, -1, -1] = False   # ... the last row of the last head
+                mask = kvhip.MaskMode.from_array(torch.from_numpy(np.ascontiguousarray(m)).cuda())
+            om = O.Mask("array", np.ascontiguousarray(m))
+            assert not m.any(axis=-1).all(), "the case needs a row without keys"
+            out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
+            assert lib.kvhip_last_attend_kernel() == family
+            ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
+            empty = ~np.broadcast_to(m, (B, Hkv * r, Lq, T)).any(axis=-1)
+
+            def exact():  # float64, the rows without keys at the mean of V over all keys
+                kk, vv = presented_f64(o)
+                with np.errstate(invalid="ignore"):
+                    ex = exact_attention(q, kk, vv, scale, om)
+                ex[empty] = np.broadcast_to(np.repeat(vv, r, axis=1).mean(axis=2)[:, :, None, :], ex.shape)[empty]
+                return ex
+            check(out, ref, f"policy {policy} {mode}", exact)
+            got = np32(out)
+            assert np.abs(got[empty]).max() > 0 and np.abs(got[empty] - ref[empty]).max() <= 2e-3
+    finally:
+        lib.kvhip_set_kernel_policy(0)
+
+
 @pytest.mark.parametrize("dtype,bits,D", [(torch.float16, 4, 128), (torch.bfloat16, 8, 128), (torch.float16, 3, 96), (torch.bfloat16, 4, (192, 128))])
 def test_large_quantized_chunks_run_dequantize_first_by_the_librarys_choice(dtype, bits, D):
     """From 512 query rows per kv head, 2048 keys and rows x keys x (Dk + Dv) = 2^30 (1024 rows over 4096 keys at head
