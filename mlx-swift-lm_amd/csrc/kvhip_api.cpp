@@ -1100,7 +1100,8 @@ kvhip_status bind_workspace(kvhip_cache *c, AttendArgs &a, size_t need, float *f
 // its loop.  The scratch (a page table, K pages, V pages) comes from the pool and goes back to it behind the call:
 // calls on one stream share one buffer.  Returns KVHIP_ERR_HIP only for launch failures; when the scratch cannot be
 // had, `*done` stays false and the caller runs the quantized tile.
-kvhip_status attend_dequant_first(kvhip_cache *c, const AttendArgs &a, hipStream_t s, bool *done) {
+// `valu`: head sizes above 256, which the tile is not built for -- the vector-ALU kernel runs over the scratch pages instead.
+kvhip_status attend_dequant_first(kvhip_cache *c, const AttendArgs &a, hipStream_t s, bool *done, bool valu = false) {
     *done = false;
     Store t;
     t.BH = a.st.BH;
@@ -1130,8 +1131,8 @@ kvhip_status attend_dequant_first(kvhip_cache *c, const AttendArgs &a, hipStream
     a2.st = t;
     kvhip_status st = KVHIP_OK;
     hipError_t e = launch_dequant_scratch(a.st, t, a.T, (int)pages, first, stride[0], stride[1], s);
-    if (e == hipSuccess) st = bind_workspace(c, a2, attend_prefill_workspace(a2), nullptr, 0, s);
-    if (e == hipSuccess && st == KVHIP_OK) e = launch_attend_prefill(a2, s);
+    if (e == hipSuccess) st = bind_workspace(c, a2, valu ? attend_valu_workspace(a2) : attend_prefill_workspace(a2), nullptr, 0, s);
+    if (e == hipSuccess && st == KVHIP_OK) e = valu ? launch_attend_valu(a2, s) : launch_attend_prefill(a2, s);
     if (e == hipSuccess && st == KVHIP_OK && mask_may_leave_rows_without_keys(a2)) e = launch_rows_without_keys(a2, s);
     retire(std::move(give_back), s);
     if (e != hipSuccess) return fail(KVHIP_ERR_HIP, std::string("dequantize-first prefill: ") + hipGetErrorString(e));
@@ -1241,9 +1242,15 @@ kvhip_status attend_impl(kvhip_cache *c, const void *q, int32_t B, int32_t Hq, i
         KV_HIP(launch_attend_valu(a, s));
         g_last_kernel = 5;
     } else {
-        KV_TRY(bind_workspace(c, a, attend_generic_workspace(a), fixed, fixed_bytes, s));
-        g_last_kernel = 0;
-        KV_HIP(launch_attend_generic(a, s));
+        // a 16-bit quantized cache of head sizes above 256: dequantized into scratch pages, every call, for the
+        // vector-ALU kernel (several times the bytes of a quantized decode kernel, a fiftieth of the plain kernel's time)
+        bool done = false;
+        if (!fixed && g_policy != 1 && attend_valu_dequant_first(a)) KV_TRY(attend_dequant_first(c, a, s, &done, true));
+        g_last_kernel = done ? 6 : 0;
+        if (!done) {
+            KV_TRY(bind_workspace(c, a, attend_generic_workspace(a), fixed, fixed_bytes, s));
+            KV_HIP(launch_attend_generic(a, s));
+        }
     }
     if (user_out)
         KV_HIP(launch_repitch_rows(user_out, (size_t)c->Dv_user * c->st.es, out, (size_t)c->st.Dv * c->st.es, q_rows, s));

@@ -373,6 +373,16 @@ bool attend_valu_supported(const AttendArgs &a) {
     return s.bits == 0 && s.Dk <= 1024 && s.Dv <= 512 && s.BH <= 65535 && plan_valu(a).lds <= 64 * 1024;
 }
 
+bool attend_valu_dequant_first(const AttendArgs &a) {
+    const Store &s = a.st;
+    if (s.bits == 0 || (s.dtype != KVHIP_F16 && s.dtype != KVHIP_BF16)) return false;
+    if (a.runs.n != 1 || a.runs.row0[0] != 0 || a.runs.phys0[0] != 0) return false;  // the scratch pages hold slots in presented order
+    if (s.Dk % 8 != 0 || s.Dv % 8 != 0) return false;
+    AttendArgs fp = a;
+    fp.st.bits = 0;
+    return attend_valu_supported(fp);
+}
+
 size_t attend_valu_workspace(const AttendArgs &a) {
     const PlanValu p = plan_valu(a);
     return p.nparts == 1 ? 0 : (size_t)a.st.BH * p.nparts * (a.Hq / a.Hkv) * a.L * (a.st.Dv + 2) * sizeof(float);

@@ -304,6 +304,9 @@ hipError_t launch_attend_generic(const AttendArgs &a, hipStream_t s);
 // Full-precision caches on the vector ALUs (float32 caches; 16-bit ones of head sizes above 256, which the matrix-core
 // kernels are not built for; keys up to 1024 wide, values up to 512): any row count, any mask.
 bool attend_valu_supported(const AttendArgs &a);
+// Whether a quantized cache none of the quantized kernels take (head sizes above 256) can be dequantized into scratch
+// pages for this kernel.
+bool attend_valu_dequant_first(const AttendArgs &a);
 size_t attend_valu_workspace(const AttendArgs &a);
 hipError_t launch_attend_valu(const AttendArgs &a, hipStream_t s);
 // Fast split-sequence decode kernels; `supported` says whether the shape is covered.

@@ -138,3 +138,51 @@ def test_against_the_plain_kernel(seed):
     d = np.abs(out.astype(np.float64) - ref.astype(np.float64))
     ulp = max(float(np.abs(ref).max()), 1e-3) * (2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10)
     assert d.max() <= ulp and d.mean() <= ulp / 8, f"max-abs {d.max():.3e} mean-abs {d.mean():.3e} (unit {ulp:.3e})"
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("bits,gs,Dk,Dv", [(4, 64, 512, 512), (8, 64, 512, 512), (4, 32, 320, 320), (3, 64, 512, 512), (6, 128, 384, 256)])
+def test_quantized_cache_is_dequantized_for_the_vector_alu_kernel(dtype, bits, gs, Dk, Dv):
+    """A quantized cache of such head sizes (Gemma 4 with kvBits): no quantized kernel takes it, so every call
+    dequantizes it into scratch pages and runs the vector-ALU kernel over them (family 6); against the oracle's
+    quantized sequence, a batch row that is all padding included, and the state untouched."""
+    rng = np.random.default_rng(bits + Dk + gs)
+    name = NAME[dtype]
+    B, Hkv, r = 2, 2, 4
+    scale = Dk ** -0.5
+    c, o = kvhip.QuantizedKVCache(gs, bits), O.QuantizedKVCache(gs, bits, name)
+    for Lq, mode in [(70, "causal"), (1, "none"), (3, "causal"), (1, "none"), (130, "lengths"), (1, "none"), (40, "bool")]:
+        k, kd = randn(rng, (B, Hkv, Lq, Dk), dtype)
+        v, vd = randn(rng, (B, Hkv, Lq, Dv), dtype)
+        q, qd = randn(rng, (B, Hkv * r, Lq, Dk), dtype)
+        T = o.offset + Lq
+        j = np.arange(T)[None, None, None, :]
+        causal = np.broadcast_to(O.create_causal_mask(Lq, T - Lq)[None, None], (B, 1, Lq, T))
+        m = None
+        if mode == "lengths":
+            lengths = np.array([0, T - 20], np.int32)
+            m = causal & (j < lengths[:, None, None, None])
+            mask, om = kvhip.MaskMode.window_mask(T - Lq, 0, lengths=torch.from_numpy(lengths)), O.Mask("array", m)
+        elif mode == "bool":
+            m = causal & (rng.random((B, 1, Lq, T)) < 0.8)
+            m[..., 0] = True
+            m[0, 0, 3:9] = False
+            mask, om = kvhip.MaskMode.from_array(torch.from_numpy(m).cuda()), O.Mask("array", m)
+        else:
+            mask = kvhip.MaskMode.causal() if mode == "causal" else kvhip.MaskMode.none()
+            om = O.Mask.CAUSAL if mode == "causal" else O.Mask.NONE
+        out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
+        assert tuple(out.shape) == (B, Hkv * r, Lq, Dv) and family() == 6, (Lq, mode)
+        ref = O.attention_with_cache_update(q, k, v, o, scale, om, name)
+
+        def exact():
+            kk, vv = presented_f64(o)
+            with np.errstate(invalid="ignore"):
+                ex = exact_attention(q, kk, vv, scale, om)
+            if m is not None:
+                empty = ~np.broadcast_to(m, (B, Hkv * r, Lq, T)).any(axis=-1)
+                ex[empty] = np.broadcast_to(np.repeat(vv, r, axis=1).mean(axis=2)[:, :, None, :], ex.shape)[empty]
+            return ex
+        check_attention(out, ref, dtype, f"L={Lq} {mode}", exact)
+    for i, (a, b) in enumerate(zip(c.state, o.get_state())):
+        assert np.array_equal(np32(a), b) if i % 3 == 0 else np.array_equal(np32(a), b.astype(np.float32)), i
