@@ -314,11 +314,13 @@ PlanValu plan_valu(const AttendArgs &a) {
     const int R = (a.Hq / a.Hkv) * a.L;
     p.nc = a.st.Dv <= 64 ? 1 : a.st.Dv <= 128 ? 2 : a.st.Dv <= 256 ? 4 : 8;
     // (16 rows per workgroup would read the keys half as often, but that instance holds one wavefront per SIMD
-    // and waits on its scalar loads: measured at 60 % of the 8-row one's rate on prompt chunks.  8 columns per
-    // lane leave registers for 4 rows.)
-    p.rb = (R <= 4 || p.nc == 8) ? 4 : 8;
-    p.row_blocks = (R + p.rb - 1) / p.rb;
+    // and waits on its scalar loads: measured at 60 % of the 8-row one's rate on prompt chunks)
+    p.rb = R <= 4 ? 4 : 8;
     p.tiles_total = (a.slots + TILE - 1) / TILE;
+    // a launch that cannot fill the chip even with every key range it may have is bound by latency: row blocks of
+    // 4 double its workgroups (one sequence, 2 kv heads of 512, 2 new tokens over 8192 keys: 51 us against 69)
+    if (p.rb == 8 && (long)((R + 7) / 8) * a.st.BH * std::min(64, std::max(1, p.tiles_total / FW)) < 256) p.rb = 4;
+    p.row_blocks = (R + p.rb - 1) / p.rb;
     p.sq = a.st.dtype == KVHIP_F32 && a.st.Dk % 4 == 0;
     const int n_el = a.st.dtype == KVHIP_F32 ? 4 : 8, nck = (a.st.Dk + n_el - 1) / n_el;
     p.lds = ((p.sq ? 0 : (size_t)p.rb * nck * n_el) + (size_t)std::max(FW, p.nc) * p.rb * 64 + (size_t)p.rb * 2) * sizeof(float);
@@ -349,7 +351,8 @@ void launch_instance(const AttendArgs &a, const PlanValu &p, hipStream_t s) {
 template <int DT>
 hipError_t launch_dt(const AttendArgs &a, const PlanValu &p, hipStream_t s) {
     profile_mark(s, true);
-    if (p.nc == 8) launch_instance<DT, 4, 8>(a, p, s);
+    if (p.nc == 8 && p.rb == 8) launch_instance<DT, 8, 8>(a, p, s);
+    else if (p.nc == 8) launch_instance<DT, 4, 8>(a, p, s);
     else if (p.rb == 4) {
         if (p.nc == 1) launch_instance<DT, 4, 1>(a, p, s);
         else if (p.nc == 2) launch_instance<DT, 4, 2>(a, p, s);
