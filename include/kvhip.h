@@ -138,7 +138,8 @@ void kvhip_set_kernel_policy(int32_t policy);
  * 0 generic, 1 matrix-core decode (quantized), 2 matrix-core decode (full precision),
  * 3 matrix-core chunked-prefill tile, 4 the same tile over scratch pages a quantized cache was dequantized into
  * first, 5 the vector-ALU kernel (float32 caches, 16-bit head sizes above 256), 6 the same over scratch pages a
- * quantized cache of such head sizes was dequantized into first; -1 before the first call.  For tests and reports. */
+ * quantized cache of such head sizes, or one with float32 scales, was dequantized into first; -1 before the first
+ * call.  For tests and reports. */
 int32_t kvhip_last_attend_kernel(void);
 void kvhip_profile_enable(int32_t every);
 kvhip_status kvhip_profile_read(int32_t *out_launches, double *out_total_ms);
@@ -246,10 +247,11 @@ kvhip_status kvhip_cache_fetch(const kvhip_cache *cache, void *dst_keys, void *d
  * 160 as 256) and runs the same kernels; every array that crosses this interface keeps the caller's
  * head sizes.  float32 caches and 16-bit caches of head sizes above 256 (not quantized; keys up to
  * 1024 wide, values up to 512) run on a vector-ALU kernel, bound by the memory system at a few query
- * rows per kv head and by float32 arithmetic on prompt chunks.  A quantized 16-bit cache of head sizes
- * above 256 is dequantized into pooled scratch pages at every call and runs the same kernel over them
- * (the allocation-free entry point does not: it uses the plain kernel).  Quantized caches with float32
- * scales run on a plain kernel that is 50-75 times slower than the tuned ones at 8k keys.  kvhip_last_attend_kernel() tells which one ran.
+ * rows per kv head and by float32 arithmetic on prompt chunks.  A quantized cache of head sizes above
+ * 256, or one with float32 scales, is dequantized into pooled scratch pages at every call and runs the
+ * same kernel over them (the allocation-free entry point does not: it uses the plain kernel, which is
+ * 50-75 times slower than the tuned ones at 8k keys and otherwise only serves head sizes above 1024 /
+ * 512 and kvhip_set_kernel_policy(1)).  kvhip_last_attend_kernel() tells which one ran.
  */
 kvhip_status kvhip_cache_attend(kvhip_cache *cache, const void *queries, int32_t B, int32_t Hq,
                                 int32_t L, int32_t D, float scale, const kvhip_mask *mask, void *out,

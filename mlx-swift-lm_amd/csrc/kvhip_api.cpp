@@ -1130,7 +1130,16 @@ kvhip_status attend_dequant_first(kvhip_cache *c, const AttendArgs &a, hipStream
     AttendArgs a2 = a;
     a2.st = t;
     kvhip_status st = KVHIP_OK;
-    hipError_t e = launch_dequant_scratch(a.st, t, a.T, (int)pages, first, stride[0], stride[1], s);
+    hipError_t e;
+    if (t.es == 2) {
+        e = launch_dequant_scratch(a.st, t, a.T, (int)pages, first, stride[0], stride[1], s);
+    } else {  // float32 scales: the page table, then the element-wise pass over whole tiles (what lies past the
+              // presented rows in the last tile is zeros or rows trimmed earlier: finite values the kernel weighs with 0)
+        const size_t stride4[4] = {stride[0], stride[1], 0, 0};
+        e = launch_set_pages(const_cast<PageEntry *>(t.pt), 0, (int)pages, first, stride4, s);
+        const int rows_up = (int)std::min<int64_t>(pages * PAGE, ((int64_t)a.T + TILE - 1) / TILE * TILE);
+        if (e == hipSuccess) e = launch_dequant_pages(a.st, t, rows_up, s);
+    }
     if (e == hipSuccess) st = bind_workspace(c, a2, valu ? attend_valu_workspace(a2) : attend_prefill_workspace(a2), nullptr, 0, s);
     if (e == hipSuccess && st == KVHIP_OK) e = valu ? launch_attend_valu(a2, s) : launch_attend_prefill(a2, s);
     if (e == hipSuccess && st == KVHIP_OK && mask_may_leave_rows_without_keys(a2)) e = launch_rows_without_keys(a2, s);

@@ -199,11 +199,11 @@ rows_without_keys_kernel(AttendArgs a) {
     __syncthreads();
     if (!any_s) return;
     const float p = round_dt<DT>(1.0f / (float)a.T);
-    constexpr int EPC = 8;  // tokens per 16-byte chunk of a 16-bit V tile
+    constexpr int EPC = DT == 2 ? 4 : 8;  // tokens per 16-byte chunk of a V tile
     for (int d = tid; d < st.Dv; d += GT) {
         float sum = 0.f;
         for (int slot0 = 0; slot0 < a.T; slot0 += EPC) {
-            const uint4 w = *reinterpret_cast<const uint4 *>(v_cell_ptr(st, bh, slot0) + vfp_off(st, slot0, d));  // 8 tokens of column d
+            const uint4 w = *reinterpret_cast<const uint4 *>(v_cell_ptr(st, bh, slot0) + vfp_off(st, slot0, d));  // EPC tokens of column d
             const int n = min(EPC, a.T - slot0);
             for (int e = 0; e < n; ++e) sum += Elem<DT>::load(&w, e);
         }
@@ -235,7 +235,8 @@ bool mask_may_leave_rows_without_keys(const AttendArgs &a) {
 hipError_t launch_rows_without_keys(const AttendArgs &a, hipStream_t s) {
     const dim3 grid(((a.Hq / a.Hkv) * a.L + 63) / 64, a.st.BH), block(GT);
     if (a.st.dtype == KVHIP_F16) hipLaunchKernelGGL(rows_without_keys_kernel<0>, grid, block, 0, s, a);
-    else hipLaunchKernelGGL(rows_without_keys_kernel<1>, grid, block, 0, s, a);
+    else if (a.st.dtype == KVHIP_BF16) hipLaunchKernelGGL(rows_without_keys_kernel<1>, grid, block, 0, s, a);
+    else hipLaunchKernelGGL(rows_without_keys_kernel<2>, grid, block, 0, s, a);
     return hipGetLastError();
 }
 

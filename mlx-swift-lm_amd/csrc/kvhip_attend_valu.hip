@@ -378,9 +378,9 @@ bool attend_valu_supported(const AttendArgs &a) {
 
 bool attend_valu_dequant_first(const AttendArgs &a) {
     const Store &s = a.st;
-    if (s.bits == 0 || (s.dtype != KVHIP_F16 && s.dtype != KVHIP_BF16)) return false;
+    if (s.bits == 0) return false;
     if (a.runs.n != 1 || a.runs.row0[0] != 0 || a.runs.phys0[0] != 0) return false;  // the scratch pages hold slots in presented order
-    if (s.Dk % 8 != 0 || s.Dv % 8 != 0) return false;
+    if (s.es == 2 && (s.Dk % 8 != 0 || s.Dv % 8 != 0)) return false;
     AttendArgs fp = a;
     fp.st.bits = 0;
     return attend_valu_supported(fp);

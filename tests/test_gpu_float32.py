@@ -162,3 +162,41 @@ def test_against_the_plain_kernel(seed):
     finally:
         lib.kvhip_set_kernel_policy(0)
     close(out, ref, "against the plain kernel")
+
+
+@pytest.mark.parametrize("bits,gs,Dk,Dv", [(8, 64, 64, 64), (4, 64, 128, 128), (4, 32, 96, 96), (3, 64, 128, 128), (6, 64, 64, 128), (2, 128, 256, 256), (5, 32, 32, 32)])
+def test_quantized_cache_with_float32_scales(bits, gs, Dk, Dv):
+    """A quantized cache built from float32 arrays (as KVCacheTests.swift builds them) keeps float32 scales and biases;
+    the matrix-core kernels take 16-bit ones.  Every call dequantizes it into scratch pages of float32 and runs the
+    vector-ALU kernel over them (family 6); against the oracle's quantized sequence, with a batch row that is all
+    padding and boolean rows of zeros, and the state untouched."""
+    from tests.util import check_attention
+    rng = np.random.default_rng(bits + Dk + gs)
+    B, Hkv, r = 2, 2, 4
+    scale = Dk ** -0.5
+    c, o = kvhip.QuantizedKVCache(gs, bits), O.QuantizedKVCache(gs, bits, "float32")
+    for Lq, mode in [(70, "causal"), (1, "none"), (3, "causal"), (1, "none"), (130, "lengths"), (1, "none"), (40, "bool"), (200, "causal")]:
+        k, kd = randn(rng, (B, Hkv, Lq, Dk), F32)
+        v, vd = randn(rng, (B, Hkv, Lq, Dv), F32)
+        q, qd = randn(rng, (B, Hkv * r, Lq, Dk), F32)
+        T = o.offset + Lq
+        j = np.arange(T)[None, None, None, :]
+        causal = np.broadcast_to(O.create_causal_mask(Lq, T - Lq)[None, None], (B, 1, Lq, T))
+        if mode == "lengths":
+            lengths = np.array([0, T - 20], np.int32)
+            m = causal & (j < lengths[:, None, None, None])
+            mask, om = kvhip.MaskMode.window_mask(T - Lq, 0, lengths=torch.from_numpy(lengths)), O.Mask("array", m)
+        elif mode == "bool":
+            m = causal & (rng.random((B, 1, Lq, T)) < 0.8)
+            m[..., 0] = True
+            m[0, 0, 3:9] = False
+            mask, om = kvhip.MaskMode.from_array(torch.from_numpy(m).cuda()), O.Mask("array", m)
+        else:
+            mask = kvhip.MaskMode.causal() if mode == "causal" else kvhip.MaskMode.none()
+            om = O.Mask.CAUSAL if mode == "causal" else O.Mask.NONE
+        out = kvhip.attention_with_cache_update(qd, kd, vd, c, scale, mask)
+        assert tuple(out.shape) == (B, Hkv * r, Lq, Dv) and out.dtype == F32 and family() == 6, (Lq, mode)
+        ref = O.attention_with_cache_update(q, k, v, o, scale, om, "float32")
+        close(out, ref.astype(np.float64), f"L={Lq} {mode}")
+    for i, (a, b) in enumerate(zip(c.state, o.get_state())):
+        assert np.array_equal(np32(a), b.astype(np.float32) if i % 3 else b), i
