@@ -313,7 +313,9 @@ def other_workload(args, torch, kvhip, L, dev):
                   (1, 16, 16, "192/128", 2048, 8192, "bf16"), (1, 32, 8, 128, 2048, 8192, "q4"), (1, 32, 8, 128, 2048, 8192, "q8"),
                   (4, 16, 4, 64, 2048, 4096, "q8"), (4, 8, 4, 256, 512, 4608, "q4"), (1, 32, 8, 96, 2048, 8192, "q4"),
                   (1, 16, 16, "192/128", 2048, 8192, "q4"), (1, 16, 16, "192/128", 2048, 8192, "q8"), (1, 32, 8, 128, 2048, 8192, "q3"),
-                  (1, 32, 8, 128, 512, 8192, "q4"), (1, 32, 8, 128, 128, 8192, "q4")]
+                  (1, 32, 8, 128, 512, 8192, "q4"), (1, 32, 8, 128, 128, 8192, "q4"),
+                  # the vector-ALU kernel (float32 caches, head size 512): a decode step each (cache_TBps is its figure) and a chunk
+                  (8, 32, 8, 128, 1, 8192, "f32"), (8, 16, 8, 512, 1, 4096, "bf16"), (1, 8, 2, 512, 512, 8192, "bf16")]
         if args.prefill_shape:
             f = args.prefill_shape.split(",")
             shapes = [tuple(x if "/" in x else int(x) for x in f[:6]) + (f[6],)]
@@ -357,7 +359,8 @@ def other_workload(args, torch, kvhip, L, dev):
                          "family": family, "kernel_ms": round(ms, 4), "call_ms": round(call_ms, 4),
                          "TFLOPs": round(fl / ms / 1e9, 1), "TFLOPs_call": round(fl / call_ms / 1e9, 1),
                          "cache_TBps": round(Bn * Hkv * T * (Dk + Dv) * (int(dn[1]) / 8 if dn[0] == "q" else 4 if dn == "f32" else 2) / ms / 1e9, 2),
-                         "frac_of_2.5PF": round(fl / (call_ms if family == 4 else ms) / 1e9 / 2500.0, 4)})
+                         # (families 5 and 6 run on the vector ALUs: no matrix-core fraction)
+                         "frac_of_2.5PF": None if family in (5, 6) else round(fl / (call_ms if family == 4 else ms) / 1e9 / 2500.0, 4)})
             del cache, k, v, q
         return {"workload": "chunked-prefill tiles on their own (prefill_fp_kernel; quantized caches: prefill_q_kernel, or "
                             "dequantize-first + prefill_fp_kernel from 512 query rows per kv head and rows x keys x (Dk + Dv) = 2^30; --policy 2 keeps them on prefill_q_kernel)",
